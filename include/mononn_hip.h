@@ -1,0 +1,120 @@
+/* C ABI of libmononn_hip.so: a fused XLA HLO module (text) in, one monolithic gfx950 kernel out.
+ *
+ * Each entry point names the reference interface it stands in for (paths relative to the
+ * reference checkout).  The reference exposes C++ classes to its TensorFlow fork and aborts the
+ * process on error; this boundary uses opaque handles, plain pointers and sizes, integer return
+ * codes (0 = success) and a thread-local error string.  A handle may be used from one thread at a
+ * time; different handles are independent.
+ */
+#ifndef MONONN_HIP_H_
+#define MONONN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mononn_module mononn_module;
+
+enum mononn_status {
+  MONONN_OK = 0,
+  MONONN_INVALID_ARGUMENT = 1,
+  MONONN_PARSE_ERROR = 2,      /* malformed HLO / JSON text */
+  MONONN_UNSUPPORTED = 3,      /* construct outside the accepted HLO dialect */
+  MONONN_SPEC_ERROR = 4,       /* tuning specification does not fit the graph or the device */
+  MONONN_COMPILE_ERROR = 5,    /* hipRTC rejected the generated source (log in the message) */
+  MONONN_RUNTIME_ERROR = 6,    /* HIP runtime failure, no usable GPU */
+  MONONN_RESOURCE_EXHAUSTED = 7, /* grid larger than co-resident capacity, LDS over budget */
+  MONONN_NOT_FOUND = 8,
+  MONONN_INTERNAL = 9
+};
+
+/* Message of the last failing call on this thread ("" when none). */
+const char* mononn_last_error(void);
+const char* mononn_version(void);
+
+/* Compile from an existing tuning specification.
+ * Replaces: MonoNNModule(hlo, spec, kernel_name, ...) + generate_code() + build_assembly()
+ *           (mononn_engine/module/mononn_module.h:31-59, mononn_module.cc:39-193) and the worker
+ *           path of CompilationThreadpool::post (mononn_engine/codegen/compilation_threadpool.cc:41-117).
+ * spec_json may be NULL: a default specification is derived (tuning_space_generator.cc:312-403).
+ * kernel_name may be NULL: "mononn_cluster_<id>" from the module name (README.md:186).
+ * build != 0 also runs hipRTC; build == 0 stops after code generation (no GPU or compiler needed). */
+int mononn_compile(const char* hlo_text, size_t hlo_len, const char* spec_json, const char* kernel_name,
+                   int build, mononn_module** out);
+
+/* Search the tuning space on `device` and return the best module.
+ * Replaces: MonoNNModuleTuner::tune(const Params&) (mononn_engine/module/mononn_module_tuner.h:27-37,
+ *           mononn_module_tuner.cc:620-991).  Honours TF_MONONN_DUMP_DIR (dump tree written when set or
+ *           when dump_dir != NULL) and TF_MONONN_THREADPOOL_SIZE.  budget: 0 = full, 1 = faster,
+ *           2 = fastest (Config::faster_tuning / fastest_tuning, mononn_engine/config/config.h:22-47). */
+int mononn_tune(const char* hlo_text, size_t hlo_len, int device, const char* dump_dir, int budget,
+                mononn_module** out);
+
+/* Load what a previous tuning run dumped: <spec_dir>/<cluster_N>/best_tuning_spec.json and, unless
+ * TF_MONONN_NO_USE_PTX_CACHE is true, the cached best_tuning_spec.hsaco next to it.
+ * Replaces: the TF_MONONN_EXISTING_TUNING_SPEC_DIR path of the reference's TensorFlow fork
+ *           (README.md:145-149, EnvVars.md:7,14).  spec_dir NULL = read that environment variable. */
+int mononn_compile_from_spec_dir(const char* hlo_text, size_t hlo_len, const char* spec_dir, mononn_module** out);
+
+void mononn_module_destroy(mononn_module* m);
+
+/* Replaces: kernel name / get_tuning_spec() / get_cuda_program() / get_ptx()+get_cubin()
+ *           (mononn_engine/module/mononn_module.h:60-74).  Returned memory belongs to the handle
+ *           and stays valid until the next call that regenerates it or until destroy. */
+const char* mononn_module_kernel_name(const mononn_module* m);
+int mononn_module_spec_json(mononn_module* m, const char** text, size_t* len);
+int mononn_module_source(const mononn_module* m, const char* file /* "main.hip" | "headers.h" */,
+                         const char** text, size_t* len);
+int mononn_module_code_object(const mononn_module* m, const void** data, size_t* len);
+int mononn_module_summary(mononn_module* m, const char** text, size_t* len);
+
+/* Replaces: the buffer summary the reference logs (README.md:189-196): parameter bytes in
+ *           parameter order, live-out bytes in root-tuple order, temp bytes.  Pass NULL to skip. */
+int mononn_module_buffer_info(const mononn_module* m, int* n_params, const int64_t** param_bytes,
+                              int* n_liveouts, const int64_t** liveout_bytes, int64_t* temp_bytes);
+/* grid / block / dynamic LDS of the launch (best_tuning_spec.json keys grid_dim, block_dim, smem_size;
+ * README.md:199-200) and the number of grid-wide barriers in the kernel. */
+int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int* smem, int* barriers);
+
+/* Non-scalar constants of the module ("buffer_for_<node>" globals that the host fills before
+ * launch: mononn_engine/codegen/graph_codegen.cc:71-86, :448-459). */
+int mononn_module_num_constants(const mononn_module* m);
+int mononn_module_constant_info(const mononn_module* m, int index, const char** hlo_name, const char** role,
+                                int64_t* bytes, int* needs_payload);
+int mononn_module_set_constant(mononn_module* m, const char* name, const void* host_data, size_t bytes);
+
+/* Load the code object on a GPU, size-check the grid against the co-resident capacity and upload
+ * the constants given so far.  Replaces: xla::gpu::CreateKernel + FuncSetAttribute of profile_kernel
+ * (mononn_engine/module/mononn_module_tuner.cc:99-131). */
+int mononn_module_load(mononn_module* m, int device);
+
+/* One forward pass = one cooperative launch.  device_ptrs: entry parameters in parameter order, then
+ * live-out buffers, then the temp buffer (argument order of mononn_engine/module/mononn_module.cc:91-143).
+ * Replaces: Launch(...) of profile_kernel (mononn_module_tuner.cc:135-139); the call is asynchronous
+ *           on `stream` (a hipStream_t, NULL = default stream). */
+int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);
+
+/* Time `iters` launches after `warmup` with HIP events on `stream`; avg_ms receives the mean,
+ * each_ms (may be NULL, else iters floats) the individual launches.
+ * Replaces: the CUPTI gpu__time_duration range of profile_in_batch
+ *           (mononn_engine/module/mononn_module_tuner.cc:250-372, tuning/profiler/cupti_profiling_session.h:20-78). */
+int mononn_time_kernel(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream, int warmup,
+                       int iters, float* avg_ms, float* each_ms);
+
+/* Write <dump_dir>/<cluster_N>/{<ctx>.json,<ctx>.hsaco,<ctx>_src/*,best_tuning_spec.{json,hsaco}}.
+ * Replaces: the dump half of final_tuning (mononn_engine/module/mononn_module_tuner.cc:457-603). */
+int mononn_module_dump(mononn_module* m, const char* dump_dir);
+
+/* Device query used for the default launch shape.
+ * Replaces: CUDADeviceContext::get_cuda_device_context (mononn_engine/core/context/cuda_device_context.cc:42-80). */
+int mononn_device_count(void);
+int mononn_device_info(int device, int* compute_units, int* wave_size, int* max_lds_per_block, char* arch,
+                       size_t arch_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MONONN_HIP_H_ */

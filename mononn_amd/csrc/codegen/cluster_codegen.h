@@ -1,0 +1,68 @@
+// Per-node device functions: fused memory-bound clusters (element-wise loops and row programs)
+// and GEMMs with their fused epilogues.
+//
+// Reference counterparts: ClusterElewise / ClusterReduce code shapes
+// (mononn_engine/core/op/cluster_elewise.cc:247-348, cluster_reduce.cc:249-497), loop schedules
+// T0..T2 (mononn_engine/core/schedule/schedule_factory.cc:29-89), GemmImpl::generate_impl
+// (mononn_engine/core/op_impl/gemm_impl.cc:55-141) and ClusterCodegen (codegen/cluster_codegen.cc:37-119).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "codegen/emitter.h"
+#include "graph/program.h"
+
+namespace mononn {
+namespace codegen {
+
+struct LaunchShape {
+  int block_size = 256;   // threads per workgroup (multiple of 64)
+  int waves() const { return block_size / 64; }
+};
+
+// per-cluster knobs; names follow the reference's cluster_*_spec fields
+// (tuning_space_generator.cc:151-160, :184-194)
+struct ClusterTuning {
+  int ilp_factor = 1;        // independent elements per thread per trip (element-wise clusters)
+  int locality_tier = 1;     // row programs: 1 = one wave per row, 2 = one workgroup per row
+};
+
+struct GemmTuning {
+  int bm = 32, bn = 32;      // workgroup tile
+  int wm = 1, wn = 1, wk = 4;   // wave arrangement; wm*wn*wk == waves per workgroup
+};
+
+struct NodeFunction {
+  std::string text;                            // device function, name written as @NAME@
+  std::vector<PointerTable::Entry> pointers;   // call arguments after `unit`, before `smem`
+  int64_t num_units = 0;                       // independent work units (one workgroup each)
+  int smem_bytes = 0;
+  std::vector<std::string> globals;            // device-global definitions the function needs
+};
+
+// fills has_reduce / row_program / rows / row_len
+void classify_cluster(const graph::Program& prog, graph::Node& node);
+
+NodeFunction generate_cluster(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls,
+                              const ClusterTuning& t);
+NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls,
+                           const GemmTuning& t);
+
+GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus);
+// throws Error(kSpecError) when the tile / wave arrangement cannot be generated for this GEMM
+void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t);
+bool gemm_uses_mfma(const graph::GemmDesc& g);
+
+// dry runs used by the merge passes
+bool can_merge_clusters(const graph::Program& prog, const std::vector<const hlo::Instr*>& producer,
+                        const std::vector<const hlo::Instr*>& consumer,
+                        const std::vector<const hlo::Instr*>& merged);
+bool can_fuse_epilogue(const graph::Program& prog, const std::vector<const hlo::Instr*>& gemm_members,
+                       const std::vector<const hlo::Instr*>& cluster_members);
+
+// entry-level values defined by `members` that somebody outside (another instruction or the
+// module root) reads, in definition order
+std::vector<const hlo::Instr*> external_outputs(const graph::Program& prog, const std::vector<const hlo::Instr*>& members);
+
+}  // namespace codegen
+}  // namespace mononn

@@ -1,0 +1,108 @@
+// Element-level expression emitter: given an instruction and a symbolic index, writes the HIP
+// statements that compute that one element and returns the name of the variable holding it.
+//
+// It plays the role of the reference's per-op implementations plus index tracer
+// (mononn_engine/core/op_impl/*.cc, mononn_engine/core/context/index_tracer.cc:67-456,
+// functors mononn_engine/core/gpu/functor.cc:42-88): broadcast / transpose / reshape / slice /
+// pad / concatenate / gather / dynamic-slice rewrite the index, element-wise ops combine operand
+// values, values produced by another member of the same cluster are recomputed in registers
+// instead of being re-read from memory (the on-chip hand-over of
+// mononn_engine/core/graph/cluster_util.cc:305-337).
+#pragma once
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "codegen/index.h"
+#include "graph/program.h"
+#include "hlo/hlo.h"
+
+namespace mononn {
+namespace codegen {
+
+class CodeBuffer {
+ public:
+  void line(const std::string& s);
+  void open(const std::string& header);   // "header {" and indent
+  void close(const std::string& tail = "");
+  const std::string& text() const { return text_; }
+  int indent() const { return indent_; }
+
+ private:
+  std::string text_;
+  int indent_ = 1;
+};
+
+using Index = std::vector<LinExpr>;
+
+// Pointer parameters of the function being generated, in order of first use.  Names are
+// positional (in0, in1, out0 ...) so that structurally identical nodes of different layers
+// generate identical text and can share one device function.
+struct PointerTable {
+  struct Entry {
+    const hlo::Instr* root;   // storage root
+    bool is_output;
+    std::string name;
+    hlo::DType dtype;
+  };
+  std::vector<Entry> entries;
+  std::string input(const hlo::Instr* root);
+  std::string output(const hlo::Instr* root);
+};
+
+class Emitter {
+ public:
+  Emitter(const graph::Program& prog, const std::vector<const hlo::Instr*>& members, CodeBuffer& out,
+          VarTable& vars, PointerTable& ptrs);
+
+  // value of `ins` (any computation reachable from the members) at multi-index `idx`
+  std::string value(const hlo::Instr* ins, const Index& idx);
+
+  // make a value available from a register when it is requested at exactly this index
+  void bind(const hlo::Instr* ins, const Index& idx, const std::string& expr);
+  void unbind(const hlo::Instr* ins);
+
+  void push_scope();
+  void pop_scope();
+  std::string fresh(const std::string& prefix = "v");
+
+  // all reduce instructions inside the members (fused computations and bare ops), dependency order
+  std::vector<const hlo::Instr*> collect_reduces() const;
+  // the instruction computing output `i` of an entry-level member (fusion root / tuple element)
+  const hlo::Instr* resolve_output(const hlo::Instr* entry_value) const;
+
+  static std::string literal(const hlo::Instr* c);                    // scalar constant as C literal
+  static std::string literal_of(hlo::DType t, const std::string& text);
+  static std::string reducer_expr(const hlo::Instr* reduce, const std::string& a, const std::string& b);
+  static std::string reducer_functor(const hlo::Instr* reduce);       // C++ lambda text
+  // device-global arrays for non-scalar literal constants met inside fused computations
+  const std::map<std::string, std::string>& literal_tables() const { return literal_tables_; }
+
+ private:
+  std::string emit(const hlo::Instr* ins, const Index& idx);
+  std::string load(const hlo::Instr* root, const Index& idx);
+  std::string serial_reduce(const hlo::Instr* ins, const Index& idx);
+  std::string key(const hlo::Instr* ins, const Index& idx) const;
+  std::string def(hlo::DType t, const std::string& rhs);
+  bool is_member(const hlo::Instr* v) const { return members_.count(v) > 0; }
+
+  const graph::Program& prog_;
+  std::set<const hlo::Instr*> members_;
+  std::vector<const hlo::Instr*> member_order_;
+  std::map<const hlo::Computation*, const hlo::Instr*> caller_;
+  CodeBuffer& out_;
+  VarTable& vars_;
+  PointerTable& ptrs_;
+  std::vector<std::map<std::string, std::string>> scopes_;
+  struct Bound {
+    Index idx;
+    std::string expr;
+  };
+  std::map<const hlo::Instr*, Bound> bound_;
+  std::map<std::string, std::string> literal_tables_;
+  int counter_ = 0;
+};
+
+}  // namespace codegen
+}  // namespace mononn

@@ -1,0 +1,239 @@
+#include "codegen/kernel_codegen.h"
+
+#include <algorithm>
+#include <set>
+#include <sstream>
+
+#include "codegen/cluster_codegen.h"
+#include "common/status.h"
+#include "common/env.h"
+#include "device/prelude_text.h"
+
+namespace mononn {
+namespace codegen {
+
+using graph::Buffer;
+using graph::Node;
+using graph::NodeKind;
+
+graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
+  graph::BuildOptions o;
+  o.merge_dependent = s.hip.merge_dependent;
+  o.fuse_gemm_epilogue = s.hip.gemm_epilogue_fusion;
+  o.transpose_constant_b = s.hip.transpose_constant_b;
+  for (auto& p : env::disabled_passes()) o.disabled_passes.insert(p);
+  return o;
+}
+
+namespace {
+std::string pointer_expr(const graph::Program& prog, const hlo::Instr* root, bool is_output, const std::map<const hlo::Instr*, std::string>& const_symbol) {
+  auto it = prog.buffers.find(root);
+  MONONN_CHECK(it != prog.buffers.end(), kInternal) << "no buffer for " << root->hlo_name;
+  const Buffer& b = it->second;
+  std::string T = std::string(is_output ? "" : "const ") + hlo::dtype_ctype(root->shape.dtype) + "*";
+  switch (b.kind) {
+    case Buffer::kParameter: return "(" + T + ")arg" + std::to_string(b.index);
+    case Buffer::kConstant: return "(" + T + ")" + const_symbol.at(root);
+    case Buffer::kLiveOut: return "(" + T + ")liveout_buffer_" + std::to_string(b.index);
+    case Buffer::kTemp: return "(" + T + ")((char*)temp_buffer + " + std::to_string(b.offset) + ")";
+  }
+  return "";
+}
+}  // namespace
+
+HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification& spec, const std::string& kernel_name) {
+  HipProgram hp;
+  hp.kernel_name = kernel_name;
+  LaunchShape ls;
+  ls.block_size = spec.runtime.block_dim.x;
+  hp.block = ls.block_size;
+  hp.grid = spec.runtime.grid_dim.x;
+  MONONN_CHECK(hp.grid <= hp.max_grid, kSpecError) << "grid of " << hp.grid << " workgroups exceeds the barrier capacity of " << hp.max_grid;
+
+  // every node named by the spec must exist (mononn_module.cc:83-85)
+  std::set<std::string> names;
+  for (auto& n : prog.nodes) names.insert(n.name);
+  auto check_known = [&](const std::string& n, const char* where) {
+    MONONN_CHECK(names.count(n), kSpecError) << where << " names node '" << n << "' which is not in the graph";
+  };
+  for (auto& kv : spec.cluster_elewise_spec) check_known(kv.first, "cluster_elewise_spec");
+  for (auto& kv : spec.cluster_reduce_spec) check_known(kv.first, "cluster_reduce_spec");
+  for (auto& kv : spec.gemm_spec_list) check_known(kv.first, "gemm_spec_list");
+  for (auto& n : spec.codegen_allow_list) check_known(n, "codegen_allow_list");
+  for (auto& n : spec.codegen_reject_list) check_known(n, "codegen_reject_list");
+  std::set<std::string> allow(spec.codegen_allow_list.begin(), spec.codegen_allow_list.end());
+  std::set<std::string> reject(spec.codegen_reject_list.begin(), spec.codegen_reject_list.end());
+
+  // constants
+  std::map<const hlo::Instr*, std::string> const_symbol;
+  for (auto* c : prog.constants) {
+    ConstantInfo ci;
+    ci.name = c->name;
+    ci.hlo_name = c->hlo_name;
+    ci.symbol = "buffer_for_" + c->name;
+    ci.bytes = c->shape.byte_size();
+    ci.dtype = c->shape.dtype;
+    ci.dims = c->shape.dims;
+    auto tr = prog.constant_transform.find(c);
+    if (tr != prog.constant_transform.end()) ci.transform = tr->second;
+    if (!c->literal_elided) ci.literal = c->literal;
+    auto md = c->attrs.find("metadata");
+    if (md != c->attrs.end()) {
+      size_t p = md->second.find("op_name=\"");
+      if (p != std::string::npos) {
+        size_t e = md->second.find('"', p + 9);
+        if (e != std::string::npos) ci.role = md->second.substr(p + 9, e - p - 9);
+      }
+    }
+    const_symbol[c] = ci.symbol;
+    hp.constants.push_back(ci);
+  }
+  for (auto* p : prog.parameters) hp.param_bytes.push_back(p->shape.byte_size());
+  for (auto* l : prog.live_outs) hp.liveout_bytes.push_back(l->shape.byte_size());
+  hp.temp_bytes = prog.temp_bytes;
+
+  // node functions, de-duplicated by text
+  std::map<std::string, std::string> fn_by_text;
+  std::vector<std::string> fn_defs;
+  std::set<std::string> globals;
+  struct Call {
+    const Node* node;
+    std::string fn;
+    std::vector<std::string> args;
+    int64_t units;
+  };
+  std::map<int, std::vector<Call>> by_stage;
+  int smem = 0;
+  for (auto& n : prog.nodes) {
+    NodeFunction f;
+    if (n.kind == NodeKind::kGemm) {
+      auto it = spec.gemm_spec_list.find(n.name);
+      GemmTuning t;
+      if (it == spec.gemm_spec_list.end()) {
+        t = default_gemm_tuning(n.gemm, ls, spec.device.sm_count);
+        spec::GemmSpec g;
+        g.tb_m = t.bm;
+        g.tb_n = t.bn;
+        g.wave_m = t.wm;
+        g.wave_n = t.wn;
+        g.wave_k = t.wk;
+        g.warp_m = t.bm / t.wm;
+        g.warp_n = t.bn / t.wn;
+        g.warp_k = static_cast<int>(n.gemm.K / t.wk);
+        if (!gemm_uses_mfma(n.gemm)) g.operator_class = "SIMT";
+        auto bc = n.members[0]->attrs.find("backend_config");
+        if (bc != n.members[0]->attrs.end()) g.backend_config = Json::parse(bc->second);
+        spec.gemm_spec_list[n.name] = g;
+      } else {
+        t.bm = it->second.tb_m;
+        t.bn = it->second.tb_n;
+        t.wm = it->second.wave_m;
+        t.wn = it->second.wave_n;
+        t.wk = it->second.wave_k;
+      }
+      f = generate_gemm(prog, n, ls, t);
+    } else {
+      ClusterTuning t;
+      if (n.has_reduce) {
+        auto it = spec.cluster_reduce_spec.find(n.name);
+        if (it == spec.cluster_reduce_spec.end()) {
+          spec::ClusterReduceSpec r;
+          r.name = n.name;
+          // long rows get a whole workgroup, short ones a wave (tiers 2 / 1 of schedule_factory.cc:42-79)
+          r.locality_tier = (n.row_program && n.row_len >= 512) ? 2 : 1;
+          spec.cluster_reduce_spec[n.name] = r;
+          it = spec.cluster_reduce_spec.find(n.name);
+        }
+        t.ilp_factor = it->second.ilp_factor;
+        t.locality_tier = it->second.locality_tier;
+      } else {
+        auto it = spec.cluster_elewise_spec.find(n.name);
+        if (it == spec.cluster_elewise_spec.end()) {
+          spec::ClusterElewiseSpec e;
+          e.name = n.name;
+          spec.cluster_elewise_spec[n.name] = e;
+          it = spec.cluster_elewise_spec.find(n.name);
+        }
+        t.ilp_factor = it->second.ilp_factor;
+      }
+      f = generate_cluster(prog, n, ls, t);
+    }
+    bool emit = (allow.empty() || allow.count(n.name)) && !reject.count(n.name);
+    std::string fn;
+    auto known = fn_by_text.find(f.text);
+    if (known != fn_by_text.end()) {
+      fn = known->second;
+    } else if (emit) {
+      fn = "node_fn_" + std::to_string(fn_by_text.size());
+      fn_by_text[f.text] = fn;
+      std::string def = f.text;
+      size_t pos;
+      while ((pos = def.find("@NAME@")) != std::string::npos) def.replace(pos, 6, fn);
+      fn_defs.push_back(def);
+      for (auto& g : f.globals) globals.insert(g);
+    }
+    NodeReport rep;
+    rep.name = n.name;
+    rep.kind = n.kind == NodeKind::kGemm ? "gemm" : (n.row_program ? "cluster_reduce" : "cluster_elewise");
+    rep.function = fn;
+    rep.stage = n.stage;
+    rep.units = f.num_units;
+    hp.nodes.push_back(rep);
+    if (!emit) continue;
+    smem = std::max(smem, f.smem_bytes);
+    Call c;
+    c.node = &n;
+    c.fn = fn;
+    c.units = f.num_units;
+    for (auto& e : f.pointers) c.args.push_back(pointer_expr(prog, e.root, e.is_output, const_symbol));
+    by_stage[n.stage].push_back(c);
+  }
+  hp.smem = smem;
+  spec.runtime.smem_size = smem;
+  MONONN_CHECK(smem <= spec.device.max_configurable_smem_size, kResourceExhausted)
+      << "kernel needs " << smem << " bytes of LDS, device offers " << spec.device.max_configurable_smem_size;
+
+  std::ostringstream src;
+  src << "// generated by mononn-hip for " << spec.device.cuda_arch << "; kernel " << kernel_name << "\n";
+  src << "#include \"headers.h\"\n\n";
+  for (auto& c : hp.constants)
+    src << "__device__ __attribute__((aligned(256))) unsigned char " << c.symbol << "[" << std::max<int64_t>(c.bytes, 1) << "];\n";
+  src << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];\n\n";
+  for (auto& g : globals) src << g << "\n";
+  for (auto& d : fn_defs) src << d << "\n";
+
+  src << "extern \"C\" __launch_bounds__(" << ls.block_size << ") __global__ void " << kernel_name << "(";
+  for (size_t i = 0; i < hp.param_bytes.size(); ++i) src << "void* arg" << i << ", ";
+  for (size_t i = 0; i < hp.liveout_bytes.size(); ++i) src << "void* liveout_buffer_" << i << ", ";
+  src << "void* temp_buffer) {\n";
+  src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
+  src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags);\n";
+  bool first = true;
+  for (auto& st : by_stage) {
+    if (!first) {
+      src << "  barrier.sync();\n";
+      ++hp.num_barriers;
+    }
+    first = false;
+    int64_t total = 0;
+    for (auto& c : st.second) total += c.units;
+    src << "  // stage " << st.first << "\n";
+    src << "  for (int u = blockIdx.x; u < " << total << "; u += gridDim.x) {\n";
+    int64_t base = 0;
+    for (size_t i = 0; i < st.second.size(); ++i) {
+      auto& c = st.second[i];
+      src << "    " << (i ? "else " : "") << "if (u < " << base + c.units << ") " << c.fn << "(u - " << base;
+      for (auto& a : c.args) src << ", " << a;
+      src << ", smem);\n";
+      base += c.units;
+    }
+    src << "  }\n";
+  }
+  src << "}\n";
+  hp.files["headers.h"] = device::kPreludeText;
+  hp.files["main.hip"] = src.str();
+  return hp;
+}
+
+}  // namespace codegen
+}  // namespace mononn

@@ -1,0 +1,60 @@
+// Whole-program code generation: one `extern "C" __global__` function for the module.
+//
+// Reference counterpart: GraphCodegen::generate (mononn_engine/codegen/graph_codegen.cc:637-842):
+// helper prelude, one device function per cluster, then the kernel whose body is buffer-pointer
+// setup followed by the nodes in topological order with grid barriers between dependent groups.
+// Argument order is the reference's (mononn_engine/module/mononn_module.cc:91-143): entry
+// parameters, one `liveout_buffer_<i>` per live-out, then `temp_buffer`; non-scalar constants are
+// `buffer_for_<node>` device globals that the host fills before launch (graph_codegen.cc:71-86).
+// Unlike the reference, node functions that come out textually identical (the same layer
+// repeated) are emitted once and called with different pointers, which keeps the instruction
+// working set of a 12-layer kernel at one layer's worth.
+#pragma once
+#include <map>
+#include <string>
+#include <vector>
+
+#include "graph/program.h"
+#include "spec/spec.h"
+
+namespace mononn {
+namespace codegen {
+
+struct ConstantInfo {
+  std::string name;        // canonical HLO name
+  std::string hlo_name;
+  std::string symbol;      // buffer_for_<name>
+  std::string role;        // metadata op_name when present
+  int64_t bytes = 0;
+  hlo::DType dtype = hlo::DType::kInvalid;
+  std::vector<int64_t> dims;
+  graph::ConstantTransform transform = graph::ConstantTransform::kNone;
+  std::string literal;     // payload text when the HLO carries it (not elided)
+};
+
+struct NodeReport {
+  std::string name, kind, function;
+  int stage = 0;
+  int64_t units = 0;
+};
+
+struct HipProgram {
+  std::string kernel_name;
+  std::map<std::string, std::string> files;   // "headers.h" (device runtime) and "main.hip"
+  std::vector<int64_t> param_bytes, liveout_bytes;
+  int64_t temp_bytes = 0;
+  std::vector<ConstantInfo> constants;
+  std::vector<NodeReport> nodes;
+  int num_barriers = 0;
+  int grid = 0, block = 0, smem = 0;
+  int max_grid = 4096;       // barrier flag capacity
+};
+
+// Fills `spec` with defaults for nodes it does not mention, validates the rest (a spec naming a
+// node the graph does not have is an error, cf. mononn_module.cc:83-85) and generates the source.
+HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification& spec, const std::string& kernel_name);
+
+graph::BuildOptions build_options_from(const spec::GraphSpecification& spec);
+
+}  // namespace codegen
+}  // namespace mononn

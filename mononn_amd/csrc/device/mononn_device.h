@@ -1,0 +1,236 @@
+// Device-side runtime of the generated monolithic kernel (gfx950 / CDNA4, wave64).
+//
+// This text is embedded into the host compiler and prepended to every generated program before it
+// goes to hipRTC.  It is the counterpart of the string prelude the reference assembles from
+// mononn_engine/core/gpu/{synchronization,reduction,memory,headers}.cc, re-designed for 64-wide
+// wavefronts, MFMA and a 256-CU / 8-XCD part:
+//   * grid_sync         <- synchronization.cc:45-82 (flag array; block 0 as master).  Here every
+//                          workgroup publishes a monotonically increasing epoch and polls all
+//                          flags itself, so there is no master round trip and nothing to clear.
+//   * wave/block reduce <- reduce_impl.cc:480-680 (32-lane shuffles) -> 64-lane butterflies.
+//   * gemm              <- gemm_impl.cc:42-141 (CUTLASS device GEMM, persistent tile swizzle)
+//                          -> register-resident MFMA 16x16x32 f16 tiles fed straight from
+//                          global memory, K split across the waves of a workgroup.
+#pragma once
+
+// hipRTC provides no <cstdint>; generated code uses these names for HLO integer types
+typedef signed char int8_t;
+typedef unsigned char uint8_t;
+typedef short int16_t;
+typedef unsigned short uint16_t;
+typedef int int32_t;
+typedef unsigned int uint32_t;
+typedef long long int64_t;
+typedef unsigned long long uint64_t;
+
+typedef _Float16 half_t;
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+
+namespace mononn_dev {
+
+constexpr int kWaveSize = 64;
+constexpr int kFlagStride = 16;   // one 64-byte line per workgroup flag
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWaveSize - 1); }
+__device__ __forceinline__ int wave_id() { return threadIdx.x / kWaveSize; }
+
+// ---------------------------------------------------------------------------------------------
+// grid-wide barrier
+// ---------------------------------------------------------------------------------------------
+struct GridBarrier {
+  unsigned* flags;   // [gridDim.x * kFlagStride]
+  unsigned epoch;    // last epoch this workgroup has published
+
+  __device__ __forceinline__ void init(unsigned* f) {
+    flags = f;
+    // all workgroups left the previous launch at the same epoch; pick it up from our own flag
+    epoch = __hip_atomic_load(&flags[blockIdx.x * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  __device__ __forceinline__ void sync() {
+    __syncthreads();
+    epoch += 1;
+    if (threadIdx.x == 0) {
+      __hip_atomic_store(&flags[blockIdx.x * kFlagStride], epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
+      while ((int)(__hip_atomic_load(&flags[b * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);   // agent scope: drop stale lines before the next stage reads
+    __syncthreads();
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// reductions (all lanes / all threads receive the result)
+// ---------------------------------------------------------------------------------------------
+template <class T, class Op>
+__device__ __forceinline__ T wave_all_reduce(T v, Op op) {
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWaveSize));
+  return v;
+}
+
+// `scratch` holds at least blockDim.x / 64 elements of T in LDS
+template <class T, class Op>
+__device__ __forceinline__ T block_all_reduce(T v, Op op, T* scratch) {
+  v = wave_all_reduce(v, op);
+  const int nw = blockDim.x / kWaveSize;
+  if (lane_id() == 0) scratch[wave_id()] = v;
+  __syncthreads();
+  T r = scratch[0];
+  for (int w = 1; w < nw; ++w) r = op(r, scratch[w]);
+  __syncthreads();
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------------
+// math helpers used by generated element-wise code
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float fast_tanh(float x) {
+  // tanh(x) = 1 - 2 / (exp(2x) + 1); exact enough in fp32 and safe for large |x|
+  float e = __expf(2.0f * x);
+  return 1.0f - 2.0f / (e + 1.0f);
+}
+template <class T>
+__device__ __forceinline__ T sign_of(T x) {
+  return (T)((x > (T)0) - (x < (T)0));
+}
+
+// ---------------------------------------------------------------------------------------------
+// GEMM:  D[m][n] = sum_k A[m][k] * Bt[n][k]      (both operands contiguous along k)
+// ---------------------------------------------------------------------------------------------
+// One workgroup owns a BM x BN output tile.  Its waves are arranged WM x WN x WK: WM*WN waves split
+// the tile, WK waves split the k range of each sub-tile (k steps interleaved).  Every wave feeds
+// v_mfma_f32_16x16x32_f16 directly from global memory: a lane's operand is 8 consecutive halves of
+// one row, i.e. one 16-byte load, and because the weight matrix is only ever read by the waves
+// that own its columns there is nothing to share through LDS in the main loop.  Partial sums of
+// the WK waves meet in LDS once, after the loop.
+//
+// The MFMA is issued with the Bt fragment as first operand so that a lane ends up with four
+// consecutive n of one row m (n = n0 + 4*(lane/16) + r, m = m0 + lane%16): the epilogue then
+// stores 8 contiguous bytes per lane.
+//
+// Epilogue functor:  void operator()(int batch, int m, int n, const float (&v)[4])   (n % 4 == 0)
+// Rows/cols beyond M / N are clamped on load and skipped on store, so M and N need not divide.
+template <int BM, int BN, int WM, int WN, int WK, int K, class Epi>
+__device__ __forceinline__ void gemm_tile_kcontig(const half_t* A, const half_t* Bt,
+                                                  int M, int N, int lda, int ldb, int batch, int tile_m,
+                                                  int tile_n, Epi& epi, char* smem) {
+  constexpr int TM = BM / WM / 16;
+  constexpr int TN = BN / WN / 16;
+  constexpr int KSTEPS = K / 32;
+  static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
+  static_assert(K % 32 == 0, "K must be a multiple of 32");
+  const int lane = lane_id();
+  const int wave = wave_id();
+  const int wk = wave % WK;
+  const int wn = (wave / WK) % WN;
+  const int wm = wave / (WK * WN);
+  const int m_base = tile_m * BM + wm * (TM * 16);
+  const int n_base = tile_n * BN + wn * (TN * 16);
+  const int r16 = lane & 15;
+  const int kq = (lane >> 4) * 8;
+
+  const half_t* a_ptr[TM];
+  const half_t* b_ptr[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int m = m_base + i * 16 + r16;
+    m = m < M ? m : M - 1;
+    a_ptr[i] = A + (long)m * lda + kq;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int n = n_base + j * 16 + r16;
+    n = n < N ? n : N - 1;
+    b_ptr[j] = Bt + (long)n * ldb + kq;
+  }
+  float4_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
+#pragma unroll 4
+  for (int s = 0; s < MY_STEPS; ++s) {
+    const int ks = s * WK + wk;
+    if (KSTEPS % WK != 0 && ks >= KSTEPS) break;
+    half8_t a[TM], b[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + ks * 32);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+  }
+
+  if (WK > 1) {
+    // [wk][wm*wn][frag][lane] float4 : each wave writes its own slab, then every wave finalises the
+    // fragments f with f % WK == wk.
+    float4_t* red = reinterpret_cast<float4_t*>(smem);
+    const int mn = wave / WK;
+    __syncthreads();   // smem may still be in use by the previous tile's readers
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        red[((wk * (WM * WN) + mn) * (TM * TN) + (i * TN + j)) * kWaveSize + lane] = acc[i][j];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int f = i * TN + j;
+        if (f % WK != wk) continue;
+        float4_t s = red[((0 * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
+#pragma unroll
+        for (int w = 1; w < WK; ++w) s += red[((w * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
+        const int m = m_base + i * 16 + r16;
+        const int n = n_base + j * 16 + (lane >> 4) * 4;
+        if (m < M && n < N) {
+          float v[4] = {s[0], s[1], s[2], s[3]};
+          epi(batch, m, n, v);
+        }
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int m = m_base + i * 16 + r16;
+        const int n = n_base + j * 16 + (lane >> 4) * 4;
+        if (m < M && n < N) {
+          float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+          epi(batch, m, n, v);
+        }
+      }
+  }
+}
+
+// Correctness fallback for operand layouts / sizes the MFMA path does not take (A or B not
+// contiguous along k, K not a multiple of 32): one thread per output element, fp32 accumulation.
+// Strides are in elements.  Epilogue functor as above but with a single value:
+//   void operator()(int batch, int m, int n, float v)
+template <class Epi>
+__device__ __forceinline__ void gemm_naive_element(const half_t* A, const half_t* B, int K, long a_sm, long a_sk,
+                                                   long b_sk, long b_sn, int batch, int m, int n, Epi& epi) {
+  float acc = 0.f;
+  const half_t* a = A + m * a_sm;
+  const half_t* b = B + n * b_sn;
+  for (int k = 0; k < K; ++k) acc += (float)a[k * a_sk] * (float)b[k * b_sk];
+  epi(batch, m, n, acc);
+}
+
+}  // namespace mononn_dev

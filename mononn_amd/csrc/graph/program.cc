@@ -1,0 +1,436 @@
+#include "graph/program.h"
+
+#include <algorithm>
+#include <functional>
+#include <sstream>
+
+#include "codegen/cluster_codegen.h"
+#include "common/status.h"
+
+namespace mononn {
+namespace graph {
+
+using hlo::Instr;
+
+bool is_alias_op(const Instr* ins) { return ins->opcode == "bitcast" || ins->opcode == "reshape"; }
+
+const Instr* Program::storage_root(const Instr* v) const {
+  while (is_alias_op(v)) v = v->operands[0];
+  return v;
+}
+
+const Node* Program::node_of(const Instr* member) const {
+  for (auto& n : nodes)
+    for (auto* m : n.members)
+      if (m == member) return &n;
+  return nullptr;
+}
+
+std::string GemmDesc::problem_hash() const {
+  std::ostringstream os;
+  os << "f16_b" << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_k_contig ? "_bk" : "_bn");
+  return os.str();
+}
+
+std::string Program::summary() const {
+  std::ostringstream os;
+  os << "stages=" << num_stages << " nodes=" << nodes.size() << " temp_bytes=" << temp_bytes << "\n";
+  for (auto& n : nodes) {
+    os << "  stage " << n.stage << "  " << (n.kind == NodeKind::kGemm ? "gemm   " : (n.row_program ? "rowred " : "elewise")) << " " << n.name;
+    if (n.kind == NodeKind::kGemm) os << "  [" << n.gemm.problem_hash() << "] members=" << n.members.size();
+    else os << "  members=" << n.members.size() << (n.row_program ? " rows=" + std::to_string(n.rows) + " len=" + std::to_string(n.row_len) : "");
+    os << "\n";
+  }
+  return os.str();
+}
+
+namespace {
+
+struct Builder {
+  Program& p;
+  const BuildOptions& opt;
+  std::vector<Node> nodes;
+  std::map<const Instr*, int> node_of_member;   // entry instr -> index in nodes (alive)
+
+  bool enabled(const char* pass) const { return !opt.disabled_passes.count(pass); }
+
+  // value defined by a member of node `n`?  (a fusion member defines its get-tuple-elements too)
+  const Instr* defining_member(const Instr* root) const {
+    if (root->opcode == "get-tuple-element") return root->operands[0];
+    return root;
+  }
+
+  GemmDesc describe_gemm(const Instr* g) {
+    // dimension bookkeeping of GemmImpl::setup (gemm_impl.cc:233-499)
+    MONONN_CHECK(g->operands.size() == 2 || g->operands.size() == 3, kUnsupported) << g->hlo_name << ": GEMM takes 2 or 3 operands";
+    const hlo::Shape &A = g->operands[0]->shape, &B = g->operands[1]->shape, &D = g->shape;
+    MONONN_CHECK(A.rank() == B.rank() && A.rank() == D.rank() && A.rank() >= 2, kUnsupported) << g->hlo_name << ": A, B and D must have equal rank >= 2";
+    MONONN_CHECK(A.dtype == hlo::DType::kF16 && B.dtype == hlo::DType::kF16 && D.dtype == hlo::DType::kF16, kUnsupported)
+        << g->hlo_name << ": only f16 GEMMs are supported";
+    const int r = A.rank();
+    const hlo::GemmConfig& c = g->gemm;
+    GemmDesc d;
+    MONONN_CHECK(c.lhs_contracting == r - 1 || c.lhs_contracting == r - 2, kUnsupported) << g->hlo_name << ": lhs contracting dim must be one of the two minor dims";
+    MONONN_CHECK(c.rhs_contracting == r - 1 || c.rhs_contracting == r - 2, kUnsupported) << g->hlo_name << ": rhs contracting dim must be one of the two minor dims";
+    d.a_k_contig = c.lhs_contracting == r - 1;
+    d.b_k_contig = c.rhs_contracting == r - 1;
+    d.K = A.dims[c.lhs_contracting];
+    d.M = A.dims[d.a_k_contig ? r - 2 : r - 1];
+    d.N = B.dims[d.b_k_contig ? r - 2 : r - 1];
+    MONONN_CHECK(B.dims[c.rhs_contracting] == d.K, kInvalidArgument) << g->hlo_name << ": contracting extents differ";
+    MONONN_CHECK(D.dims[r - 2] == d.M && D.dims[r - 1] == d.N, kInvalidArgument) << g->hlo_name << ": result shape does not match operands";
+    d.batch = 1;
+    for (int i = 0; i < r - 2; ++i) {
+      MONONN_CHECK(A.dims[i] == B.dims[i] && A.dims[i] == D.dims[i], kUnsupported) << g->hlo_name << ": batch dims must agree";
+      d.batch *= A.dims[i];
+    }
+    MONONN_CHECK(d.batch == c.batch_size, kInvalidArgument) << g->hlo_name << ": batch_size " << c.batch_size << " does not match the shapes (" << d.batch << ")";
+    d.a_batch_stride = d.M * d.K;
+    d.b_batch_stride = d.N * d.K;
+    d.d_batch_stride = d.M * d.N;
+    // cross-check against XLA's strides as the reference does (gemm_impl.cc:380-393)
+    if (d.batch > 1) {
+      MONONN_CHECK(c.lhs_stride == 0 || c.lhs_stride == d.a_batch_stride, kInvalidArgument) << g->hlo_name << ": lhs_stride mismatch";
+      MONONN_CHECK(c.rhs_stride == 0 || c.rhs_stride == d.b_batch_stride, kInvalidArgument) << g->hlo_name << ": rhs_stride mismatch";
+    }
+    MONONN_CHECK(c.alpha_imag == 0, kUnsupported) << g->hlo_name << ": complex alpha";
+    d.alpha = c.alpha_real;
+    d.beta = c.beta;
+    d.has_addend = g->operands.size() == 3 && c.beta != 0;
+    return d;
+  }
+
+  void make_nodes() {
+    const hlo::Computation* e = p.module->entry;
+    for (auto& up : e->instrs) {
+      const Instr* ins = up.get();
+      const std::string& op = ins->opcode;
+      if (op == "parameter") continue;
+      if (op == "constant") continue;
+      if (is_alias_op(ins) || op == "get-tuple-element" || op == "tuple") continue;
+      Node n;
+      n.name = ins->name;
+      n.members.push_back(ins);
+      if (op == "custom-call") {
+        MONONN_CHECK(ins->custom_call_target == "__cublas$gemm", kUnsupported) << ins->hlo_name << ": custom-call target '" << ins->custom_call_target << "' has no lowering yet";
+        n.kind = NodeKind::kGemm;
+        n.gemm = describe_gemm(ins);
+      } else {
+        n.kind = NodeKind::kCluster;
+      }
+      node_of_member[ins] = static_cast<int>(nodes.size());
+      nodes.push_back(std::move(n));
+    }
+  }
+
+  // storage roots read by a set of members from outside the set
+  std::vector<const Instr*> external_inputs(const std::vector<const Instr*>& members) const {
+    std::set<const Instr*> in_set(members.begin(), members.end());
+    std::vector<const Instr*> out;
+    std::set<const Instr*> seen;
+    for (auto* m : members)
+      for (auto* o : m->operands) {
+        const Instr* r = p.storage_root(o);
+        if (in_set.count(defining_member(r))) continue;
+        if (r->opcode == "constant" && r->is_scalar_constant()) continue;
+        if (seen.insert(r).second) out.push_back(r);
+      }
+    return out;
+  }
+
+  // node indices a member set depends on (producers of its external inputs)
+  std::set<int> producer_nodes(const std::vector<const Instr*>& members) const {
+    std::set<int> s;
+    for (auto* r : external_inputs(members)) {
+      auto it = node_of_member.find(defining_member(r));
+      if (it != node_of_member.end()) s.insert(it->second);
+    }
+    return s;
+  }
+
+  // does node `from` reach node `to` through a path that leaves the set {from}?
+  bool reaches_via_outside(int from, int to, const std::vector<std::vector<int>>& succ) const {
+    std::vector<int> stack;
+    std::set<int> seen;
+    for (int s : succ[from])
+      if (s != to) stack.push_back(s);
+    while (!stack.empty()) {
+      int x = stack.back();
+      stack.pop_back();
+      if (!seen.insert(x).second) continue;
+      if (x == to) return true;
+      for (int s : succ[x]) stack.push_back(s);
+    }
+    return false;
+  }
+
+  std::vector<std::vector<int>> successors() const {
+    std::vector<std::vector<int>> succ(nodes.size());
+    for (size_t i = 0; i < nodes.size(); ++i) {
+      if (nodes[i].members.empty()) continue;
+      for (int pn : producer_nodes(nodes[i].members)) succ[pn].push_back(static_cast<int>(i));
+    }
+    return succ;
+  }
+
+  // MergeDependentPass counterpart: glue a cluster onto the cluster that feeds it when the merged
+  // body can still be generated as one loop nest (same row space).  Feasibility is decided by the
+  // code generator itself on a dry run.
+  void merge_dependent() {
+    bool changed = true;
+    while (changed) {
+      changed = false;
+      auto succ = successors();
+      for (size_t ci = 0; ci < nodes.size() && !changed; ++ci) {
+        Node& c = nodes[ci];
+        if (c.members.empty() || c.kind != NodeKind::kCluster) continue;
+        for (int pi : producer_nodes(c.members)) {
+          Node& pr = nodes[pi];
+          if (pr.kind != NodeKind::kCluster) continue;
+          if (reaches_via_outside(pi, static_cast<int>(ci), succ)) continue;
+          std::vector<const Instr*> merged = pr.members;
+          merged.insert(merged.end(), c.members.begin(), c.members.end());
+          std::sort(merged.begin(), merged.end(), [](const Instr* a, const Instr* b) { return a->index_in_comp < b->index_in_comp; });
+          if (!codegen::can_merge_clusters(p, pr.members, c.members, merged)) continue;
+          pr.members = merged;
+          pr.name += "_" + c.name;
+          for (auto* m : c.members) node_of_member[m] = pi;
+          c.members.clear();
+          changed = true;
+          break;
+        }
+      }
+    }
+  }
+
+  // A GEMM absorbs element-wise clusters that consume its result element for element; they run in
+  // the epilogue on the fp32 accumulator tile (bias, GELU, residual, head split/merge transposes).
+  void fuse_gemm_epilogues() {
+    bool changed = true;
+    while (changed) {
+      changed = false;
+      auto succ = successors();
+      for (size_t gi = 0; gi < nodes.size() && !changed; ++gi) {
+        Node& g = nodes[gi];
+        if (g.members.empty() || g.kind != NodeKind::kGemm) continue;
+        for (int ci : succ[gi]) {
+          Node& c = nodes[ci];
+          if (c.members.empty() || c.kind != NodeKind::kCluster) continue;
+          if (reaches_via_outside(static_cast<int>(gi), ci, succ)) continue;
+          std::vector<const Instr*> merged = g.members;
+          merged.insert(merged.end(), c.members.begin(), c.members.end());
+          if (!codegen::can_fuse_epilogue(p, g.members, c.members)) continue;
+          g.members = merged;
+          g.name += "_" + c.name;
+          for (auto* m : c.members) node_of_member[m] = static_cast<int>(gi);
+          c.members.clear();
+          changed = true;
+          break;
+        }
+      }
+    }
+  }
+
+  void finalize() {
+    // compact, compute inputs/outputs, stages, order
+    std::vector<Node> alive;
+    std::map<int, int> remap;
+    for (size_t i = 0; i < nodes.size(); ++i)
+      if (!nodes[i].members.empty()) {
+        remap[static_cast<int>(i)] = static_cast<int>(alive.size());
+        alive.push_back(nodes[i]);
+      }
+    for (auto& kv : node_of_member) kv.second = remap.at(kv.second);
+    nodes = alive;
+
+    // module outputs
+    const Instr* root = p.module->entry->root;
+    std::vector<const Instr*> outs;
+    if (root->opcode == "tuple") outs.assign(root->operands.begin(), root->operands.end());
+    else outs.push_back(root);
+    std::set<const Instr*> live_set;
+    for (auto* o : outs) {
+      const Instr* r = p.storage_root(o);
+      MONONN_CHECK(!r->shape.is_tuple(), kUnsupported) << "nested tuple output " << o->hlo_name;
+      MONONN_CHECK(r->opcode != "parameter" && r->opcode != "constant", kUnsupported) << "module output " << o->hlo_name << " is a pass-through of an input";
+      MONONN_CHECK(live_set.insert(r).second, kUnsupported) << "module output " << o->hlo_name << " appears twice in the root tuple";
+      p.live_outs.push_back(r);
+    }
+
+    // users per storage root (entry level)
+    std::map<const Instr*, std::set<int>> readers;
+    for (size_t i = 0; i < nodes.size(); ++i) {
+      nodes[i].inputs = external_inputs(nodes[i].members);
+      for (auto* r : nodes[i].inputs) readers[r].insert(static_cast<int>(i));
+    }
+    // outputs: values defined by a member and read by another node or live-out
+    for (size_t i = 0; i < nodes.size(); ++i) {
+      Node& n = nodes[i];
+      std::set<const Instr*> mem(n.members.begin(), n.members.end());
+      std::vector<const Instr*> cands;
+      for (auto& up : p.module->entry->instrs) {
+        const Instr* v = up.get();
+        if (mem.count(v) && !v->shape.is_tuple()) cands.push_back(v);
+        if (v->opcode == "get-tuple-element" && mem.count(v->operands[0])) cands.push_back(v);
+      }
+      for (auto* v : cands)
+        if (readers.count(v) || live_set.count(v)) n.outputs.push_back(v);
+      MONONN_CHECK(!n.outputs.empty(), kUnsupported) << "node " << n.name << " has no consumer (dead code in the entry computation)";
+      for (auto* v : n.outputs) p.producer[v] = static_cast<int>(i);
+    }
+    // stages: longest path from the sources (BFS-depth rule of the reference's barrier elimination)
+    std::vector<int> depth(nodes.size(), 0);
+    std::vector<int> order;
+    {
+      std::vector<int> state(nodes.size(), 0);
+      std::function<void(int)> visit = [&](int i) {
+        if (state[i] == 2) return;
+        MONONN_CHECK(state[i] == 0, kInternal) << "cycle through node " << nodes[i].name;
+        state[i] = 1;
+        int d = 1;
+        for (auto* r : nodes[i].inputs) {
+          auto it = p.producer.find(r);
+          if (it == p.producer.end()) continue;
+          visit(it->second);
+          d = std::max(d, depth[it->second] + 1);
+        }
+        depth[i] = d;
+        state[i] = 2;
+        order.push_back(i);
+      };
+      for (size_t i = 0; i < nodes.size(); ++i) visit(static_cast<int>(i));
+    }
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return depth[a] < depth[b]; });
+    std::vector<Node> sorted;
+    std::map<int, int> pos;
+    for (int i : order) {
+      pos[i] = static_cast<int>(sorted.size());
+      nodes[i].stage = depth[i];
+      nodes[i].id = static_cast<int>(sorted.size());
+      sorted.push_back(nodes[i]);
+    }
+    for (auto& kv : p.producer) kv.second = pos.at(kv.second);
+    p.nodes = sorted;
+    p.num_stages = 0;
+    for (auto& n : p.nodes) p.num_stages = std::max(p.num_stages, n.stage);
+  }
+
+  void decide_constant_layouts() {
+    if (!opt.transpose_constant_b || !enabled("ConstantLayoutPass")) return;
+    // a constant [K,N] matrix used only as the right operand of GEMMs is stored [N,K] by the host
+    std::map<const Instr*, bool> ok;
+    for (auto& up : p.module->entry->instrs) {
+      const Instr* c = up.get();
+      if (c->opcode != "constant" || c->is_scalar_constant() || c->shape.rank() != 2) continue;
+      bool all = !c->users.empty();
+      for (auto* u : c->users) {
+        bool good = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands.size() >= 2 &&
+                    u->operands[1] == c && u->operands[0] != c && u->gemm.rhs_contracting == 0 && (u->operands.size() < 3 || u->operands[2] != c);
+        if (!good) all = false;
+      }
+      if (all) ok[c] = true;
+    }
+    for (auto& n : p.nodes) {
+      if (n.kind != NodeKind::kGemm) continue;
+      const Instr* b = n.members[0]->operands[1];
+      if (ok.count(b)) {
+        n.gemm.b_k_contig = true;
+        n.gemm.b_transposed_upload = true;
+        p.constant_transform[b] = ConstantTransform::kTranspose2D;
+      }
+    }
+  }
+
+  void assign_buffers() {
+    const hlo::Computation* e = p.module->entry;
+    for (auto* prm : e->params) {
+      MONONN_CHECK(!prm->shape.is_tuple(), kUnsupported) << "tuple-shaped entry parameter " << prm->hlo_name;
+      p.parameters.push_back(prm);
+      Buffer b;
+      b.kind = Buffer::kParameter;
+      b.index = static_cast<int>(prm->parameter_number);
+      b.bytes = prm->shape.byte_size();
+      p.buffers[prm] = b;
+    }
+    for (auto& up : e->instrs) {
+      const Instr* c = up.get();
+      if (c->opcode != "constant" || c->is_scalar_constant()) continue;
+      if (c->users.empty()) continue;
+      Buffer b;
+      b.kind = Buffer::kConstant;
+      b.index = static_cast<int>(p.constants.size());
+      b.bytes = c->shape.byte_size();
+      p.constants.push_back(c);
+      p.buffers[c] = b;
+    }
+    std::map<const Instr*, int> live_index;
+    for (size_t i = 0; i < p.live_outs.size(); ++i) live_index[p.live_outs[i]] = static_cast<int>(i);
+    // temp intervals
+    std::vector<const Instr*> temps;
+    for (auto& n : p.nodes)
+      for (auto* v : n.outputs) {
+        Buffer b;
+        b.bytes = v->shape.byte_size();
+        b.def_stage = b.last_use_stage = n.stage;
+        auto li = live_index.find(v);
+        if (li != live_index.end()) {
+          b.kind = Buffer::kLiveOut;
+          b.index = li->second;
+        } else {
+          b.kind = Buffer::kTemp;
+          temps.push_back(v);
+        }
+        p.buffers[v] = b;
+      }
+    for (auto& n : p.nodes)
+      for (auto* r : n.inputs) {
+        auto it = p.buffers.find(r);
+        MONONN_CHECK(it != p.buffers.end(), kInternal) << "input " << r->hlo_name << " of node " << n.name << " has no buffer";
+        it->second.last_use_stage = std::max(it->second.last_use_stage, n.stage);
+      }
+    // interval colouring over stages; a slot is reusable from the stage after its last reader
+    struct Slot {
+      int64_t offset, bytes;
+      int free_from;
+    };
+    std::vector<Slot> slots;
+    int64_t top = 0;
+    std::stable_sort(temps.begin(), temps.end(), [&](const Instr* a, const Instr* b) { return p.buffers[a].def_stage < p.buffers[b].def_stage; });
+    for (auto* v : temps) {
+      Buffer& b = p.buffers[v];
+      int64_t need = (b.bytes + 255) / 256 * 256;
+      int best = -1;
+      for (size_t s = 0; s < slots.size(); ++s)
+        if (slots[s].free_from <= b.def_stage && slots[s].bytes >= need && (best < 0 || slots[s].bytes < slots[best].bytes)) best = static_cast<int>(s);
+      if (best >= 0) {
+        b.offset = slots[best].offset;
+        slots[best].free_from = b.last_use_stage + 1;
+      } else {
+        b.offset = top;
+        slots.push_back({top, need, b.last_use_stage + 1});
+        top += need;
+      }
+    }
+    p.temp_bytes = top;
+  }
+};
+
+}  // namespace
+
+std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, const BuildOptions& opt) {
+  auto prog = std::make_unique<Program>();
+  prog->module = std::move(module);
+  Builder b{*prog, opt};
+  b.make_nodes();
+  if (opt.merge_dependent && b.enabled("MergeDependentPass")) b.merge_dependent();
+  if (opt.fuse_gemm_epilogue && b.enabled("GemmEpilogueFusionPass")) b.fuse_gemm_epilogues();
+  b.finalize();
+  b.decide_constant_layouts();
+  for (auto& n : prog->nodes)
+    if (n.kind == NodeKind::kCluster) codegen::classify_cluster(*prog, n);
+  b.assign_buffers();
+  return prog;
+}
+
+}  // namespace graph
+}  // namespace mononn

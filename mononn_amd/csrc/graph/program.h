@@ -1,0 +1,98 @@
+// Stage-level program: the HLO entry computation regrouped into work nodes (fused memory-bound
+// clusters and GEMMs), layered into barrier-separated stages, with buffers assigned.
+//
+// Reference counterparts: Graph of Op/ClusterOp built by IRParserFused
+// (mononn_engine/parser/ir_parser_fused.cc:319-385, :490-539), ClusteringSingleNodePass,
+// MergeDependentPass (merge_dependent_pass.cc:37-191), the BFS-depth barrier placement of
+// GlobalSynchronizationEliminationPass (global_synchronization_elimination_pass.cc:32-147) and
+// BufferAssignmentPass (:34-98).  The reference inherits buffer offsets from XLA's buffer
+// assignment; here they are computed (stage-interval colouring of one temp arena).
+#pragma once
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "hlo/hlo.h"
+
+namespace mononn {
+namespace graph {
+
+enum class NodeKind { kCluster, kGemm };
+
+struct GemmDesc {
+  int64_t batch = 1, M = 0, N = 0, K = 0;
+  bool a_k_contig = true;    // A stored [.., M, K]; false: [.., K, M]
+  bool b_k_contig = false;   // B stored [.., N, K]; false: [.., K, N]
+  bool b_transposed_upload = false;   // B is a constant that the host stores as [N, K] at upload
+  int64_t a_batch_stride = 0, b_batch_stride = 0, d_batch_stride = 0;
+  double alpha = 1.0, beta = 0.0;
+  bool has_addend = false;
+  std::string problem_hash() const;   // dtype+shape key, cf. mononn_module_tuner.cc:386-408
+};
+
+struct Node {
+  int id = -1;
+  std::string name;
+  NodeKind kind = NodeKind::kCluster;
+  // entry-level instructions realised by this node, in definition order.  For a GEMM node the
+  // first member is the custom-call; further members are element-wise clusters fused behind it.
+  std::vector<const hlo::Instr*> members;
+  std::vector<const hlo::Instr*> inputs;    // storage roots read from memory
+  std::vector<const hlo::Instr*> outputs;   // entry-level values written to memory (storage roots)
+  int stage = 0;
+  // clusters
+  bool has_reduce = false;
+  bool row_program = false;       // reduces over the minor-most dim, rows handled by a wave / workgroup
+  int64_t rows = 0, row_len = 0;
+  // GEMM
+  GemmDesc gemm;
+  const hlo::Instr* gemm_instr() const { return kind == NodeKind::kGemm ? members[0] : nullptr; }
+};
+
+struct Buffer {
+  enum Kind { kParameter, kConstant, kLiveOut, kTemp };
+  Kind kind = kTemp;
+  int index = 0;          // parameter number / live-out index / constant ordinal
+  int64_t offset = 0;     // within the temp arena
+  int64_t bytes = 0;
+  int def_stage = 0, last_use_stage = 0;
+};
+
+enum class ConstantTransform { kNone, kTranspose2D };
+
+struct Program {
+  std::unique_ptr<hlo::Module> module;
+  std::vector<Node> nodes;                                         // topological, grouped by stage
+  std::map<const hlo::Instr*, Buffer> buffers;                     // storage root -> buffer
+  std::vector<const hlo::Instr*> parameters;                       // entry parameters in order
+  std::vector<const hlo::Instr*> constants;                        // non-scalar entry constants (device buffers)
+  std::map<const hlo::Instr*, ConstantTransform> constant_transform;
+  std::vector<const hlo::Instr*> live_outs;                        // storage roots, root-tuple order
+  std::map<const hlo::Instr*, int> producer;                       // storage root -> node id
+  int num_stages = 0;
+  int64_t temp_bytes = 0;
+
+  // value -> the entry-level instruction whose buffer holds it (follows bitcast / reshape)
+  const hlo::Instr* storage_root(const hlo::Instr* v) const;
+  const Node* node_of(const hlo::Instr* member) const;
+  std::string summary() const;
+};
+
+struct BuildOptions {
+  bool merge_dependent = true;          // glue producer/consumer clusters that share a row space
+  bool fuse_gemm_epilogue = true;       // element-wise consumers of a GEMM run in its epilogue
+  bool transpose_constant_b = true;     // store constant [K,N] GEMM operands as [N,K]
+  std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)
+};
+
+// Takes ownership of the module.  Throws Error(kUnsupported) for graphs outside the dialect.
+std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, const BuildOptions& opt);
+
+// true for entry-level instructions that only rename storage (no code): bitcast, reshape
+bool is_alias_op(const hlo::Instr* ins);
+
+}  // namespace graph
+}  // namespace mononn

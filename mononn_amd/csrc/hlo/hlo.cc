@@ -1,0 +1,536 @@
+#include "hlo/hlo.h"
+
+#include <algorithm>
+#include <cctype>
+#include <cstdlib>
+#include <set>
+
+#include "common/json.h"
+#include "common/status.h"
+
+namespace mononn {
+namespace hlo {
+
+namespace {
+struct DTypeInfo {
+  DType t;
+  const char* name;
+  int bytes;
+  const char* ctype;
+};
+const DTypeInfo kDTypes[] = {
+    {DType::kPred, "pred", 1, "bool"},       {DType::kS8, "s8", 1, "int8_t"},
+    {DType::kS16, "s16", 2, "int16_t"},      {DType::kS32, "s32", 4, "int32_t"},
+    {DType::kS64, "s64", 8, "int64_t"},      {DType::kU8, "u8", 1, "uint8_t"},
+    {DType::kU16, "u16", 2, "uint16_t"},     {DType::kU32, "u32", 4, "uint32_t"},
+    {DType::kU64, "u64", 8, "uint64_t"},     {DType::kF16, "f16", 2, "_Float16"},
+    {DType::kF32, "f32", 4, "float"},        {DType::kF64, "f64", 8, "double"},
+};
+
+// Opcode set of mononn_engine/core/op/op_type.h:20-58 plus `fusion`; everything else is rejected
+// the way ir_parser_fused.cc:311 does.  A few harmless extras XLA prints in the same position
+// (`sqrt`, `power`, `and`, `or`, `not`) are accepted because the emitter handles them.
+const std::set<std::string>& known_opcodes() {
+  static const std::set<std::string> s = {
+      "abs", "add", "bitcast", "broadcast", "clamp", "compare", "concatenate", "constant", "convert",
+      "convolution", "copy", "custom-call", "divide", "dynamic-slice", "dynamic-update-slice",
+      "exponential", "gather", "get-tuple-element", "iota", "log", "maximum", "minimum", "multiply",
+      "negate", "pad", "parameter", "reduce", "reduce-window", "reshape", "rsqrt", "select", "sign",
+      "slice", "subtract", "tanh", "transpose", "tuple", "fusion", "sqrt", "power", "and", "or", "not"};
+  return s;
+}
+}  // namespace
+
+const char* dtype_name(DType t) {
+  for (auto& d : kDTypes)
+    if (d.t == t) return d.name;
+  return t == DType::kTuple ? "tuple" : "invalid";
+}
+int dtype_bytes(DType t) {
+  for (auto& d : kDTypes)
+    if (d.t == t) return d.bytes;
+  return 0;
+}
+const char* dtype_ctype(DType t) {
+  for (auto& d : kDTypes)
+    if (d.t == t) return d.ctype;
+  return "void";
+}
+DType dtype_from_name(const std::string& s) {
+  for (auto& d : kDTypes)
+    if (s == d.name) return d.t;
+  return DType::kInvalid;
+}
+
+std::string Shape::to_string() const {
+  if (is_tuple()) {
+    std::string s = "(";
+    for (size_t i = 0; i < tuple.size(); ++i) s += (i ? ", " : "") + tuple[i].to_string();
+    return s + ")";
+  }
+  std::string s = std::string(dtype_name(dtype)) + "[";
+  for (size_t i = 0; i < dims.size(); ++i) s += (i ? "," : "") + std::to_string(dims[i]);
+  return s + "]";
+}
+
+std::string canonical_name(const std::string& n) {
+  std::string s = n;
+  if (!s.empty() && s[0] == '%') s.erase(0, 1);
+  for (auto& c : s)
+    if (c == '.' || c == '-') c = '_';
+  return s;
+}
+
+std::string module_short_name(const std::string& module_name) {
+  const std::string prefix = "cluster_";
+  MONONN_CHECK(module_name.compare(0, prefix.size(), prefix) == 0, kInvalidArgument)
+      << "module name '" << module_name << "' does not start with cluster_<id>";
+  size_t i = prefix.size();
+  while (i < module_name.size() && isdigit(static_cast<unsigned char>(module_name[i]))) ++i;
+  MONONN_CHECK(i > prefix.size(), kInvalidArgument) << "module name '" << module_name << "' has no cluster id";
+  return module_name.substr(0, i);
+}
+
+// ------------------------------------------------------------------------------------------
+namespace {
+
+class Lexer {
+ public:
+  explicit Lexer(const std::string& s) : s_(s) {}
+  size_t pos = 0;
+  int line = 1;
+
+  bool eof() {
+    skip_ws();
+    return pos >= s_.size();
+  }
+  void skip_ws() {
+    while (pos < s_.size()) {
+      char c = s_[pos];
+      if (c == '\n') {
+        ++line;
+        ++pos;
+      } else if (c == ' ' || c == '\t' || c == '\r') {
+        ++pos;
+      } else if (c == '/' && pos + 1 < s_.size() && s_[pos + 1] == '/') {
+        while (pos < s_.size() && s_[pos] != '\n') ++pos;
+      } else if (c == '/' && pos + 1 < s_.size() && s_[pos + 1] == '*') {
+        size_t e = s_.find("*/", pos + 2);
+        if (e == std::string::npos) fail("unterminated comment");
+        for (size_t i = pos; i < e; ++i)
+          if (s_[i] == '\n') ++line;
+        pos = e + 2;
+      } else {
+        break;
+      }
+    }
+  }
+  char peek() {
+    skip_ws();
+    return pos < s_.size() ? s_[pos] : '\0';
+  }
+  bool consume(char c) {
+    if (peek() == c) {
+      ++pos;
+      return true;
+    }
+    return false;
+  }
+  void expect(char c) {
+    if (!consume(c)) fail(std::string("expected '") + c + "'");
+  }
+  bool consume_word(const std::string& w) {
+    skip_ws();
+    if (s_.compare(pos, w.size(), w) == 0) {
+      size_t e = pos + w.size();
+      if (e >= s_.size() || !(isalnum(static_cast<unsigned char>(s_[e])) || s_[e] == '_')) {
+        pos = e;
+        return true;
+      }
+    }
+    return false;
+  }
+  // identifier characters used by HLO names and opcodes
+  std::string ident() {
+    skip_ws();
+    size_t st = pos;
+    if (pos < s_.size() && s_[pos] == '%') ++pos;
+    while (pos < s_.size()) {
+      char c = s_[pos];
+      if (isalnum(static_cast<unsigned char>(c)) || c == '_' || c == '.' || c == '-' || c == '$') ++pos;
+      else break;
+    }
+    if (st == pos) fail("expected identifier");
+    return s_.substr(st, pos - st);
+  }
+  // balanced blob starting at an opening bracket, returned including the brackets
+  std::string balanced() {
+    skip_ws();
+    size_t st = pos;
+    int depth = 0;
+    bool in_q = false;
+    while (pos < s_.size()) {
+      char c = s_[pos];
+      if (in_q) {
+        if (c == '\\') ++pos;
+        else if (c == '"') in_q = false;
+      } else if (c == '"') {
+        in_q = true;
+      } else if (c == '(' || c == '{' || c == '[') {
+        ++depth;
+      } else if (c == ')' || c == '}' || c == ']') {
+        --depth;
+        if (depth == 0) {
+          ++pos;
+          return s_.substr(st, pos - st);
+        }
+      } else if (c == '\n') {
+        ++line;
+      }
+      ++pos;
+    }
+    fail("unbalanced brackets");
+  }
+  std::string quoted() {
+    skip_ws();
+    if (pos >= s_.size() || s_[pos] != '"') fail("expected string");
+    ++pos;
+    std::string out;
+    while (pos < s_.size() && s_[pos] != '"') {
+      if (s_[pos] == '\\' && pos + 1 < s_.size()) {
+        ++pos;
+        out.push_back(s_[pos]);
+      } else {
+        out.push_back(s_[pos]);
+      }
+      ++pos;
+    }
+    if (pos >= s_.size()) fail("unterminated string");
+    ++pos;
+    return out;
+  }
+  // attribute value: balanced blob, quoted string, or bare token up to a top-level ',' / newline
+  std::string attr_value() {
+    char c = peek();
+    if (c == '{' || c == '(' || c == '[') return balanced();
+    if (c == '"') return quoted();
+    size_t st = pos;
+    while (pos < s_.size() && s_[pos] != ',' && s_[pos] != '\n' && s_[pos] != ' ' && s_[pos] != '}') ++pos;
+    return s_.substr(st, pos - st);
+  }
+  [[noreturn]] void fail(const std::string& what) {
+    MONONN_FAIL(kParseError) << "HLO text line " << line << ": " << what;
+  }
+  const std::string& text() const { return s_; }
+
+ private:
+  const std::string& s_;
+};
+
+std::vector<int64_t> ints_of(const std::string& s) {
+  std::vector<int64_t> v;
+  size_t i = 0;
+  while (i < s.size()) {
+    if (isdigit(static_cast<unsigned char>(s[i])) || (s[i] == '-' && i + 1 < s.size() && isdigit(static_cast<unsigned char>(s[i + 1])))) {
+      size_t st = i++;
+      while (i < s.size() && isdigit(static_cast<unsigned char>(s[i]))) ++i;
+      v.push_back(std::strtoll(s.substr(st, i - st).c_str(), nullptr, 10));
+    } else {
+      ++i;
+    }
+  }
+  return v;
+}
+
+Shape parse_shape(Lexer& lx) {
+  Shape sh;
+  if (lx.peek() == '(') {
+    lx.expect('(');
+    sh.dtype = DType::kTuple;
+    if (lx.peek() != ')') {
+      do {
+        sh.tuple.push_back(parse_shape(lx));
+        if (sh.tuple.back().is_tuple()) MONONN_FAIL(kUnsupported) << "nested tuple shapes are not supported";
+      } while (lx.consume(','));
+    }
+    lx.expect(')');
+    return sh;
+  }
+  std::string t = lx.ident();
+  sh.dtype = dtype_from_name(t);
+  if (sh.dtype == DType::kInvalid) MONONN_FAIL(kUnsupported) << "line " << lx.line << ": unsupported element type '" << t << "'";
+  lx.expect('[');
+  while (lx.peek() != ']') {
+    lx.skip_ws();
+    if (lx.peek() == '<' || lx.peek() == '?') MONONN_FAIL(kUnsupported) << "line " << lx.line << ": dynamic dimensions are not supported";
+    std::string num;
+    while (isdigit(static_cast<unsigned char>(lx.text()[lx.pos]))) num.push_back(lx.text()[lx.pos++]);
+    if (num.empty()) lx.fail("expected dimension");
+    sh.dims.push_back(std::strtoll(num.c_str(), nullptr, 10));
+    lx.consume(',');
+  }
+  lx.expect(']');
+  // optional layout directly attached: {1,0} ; tiling / element size / memory space annotations rejected
+  if (lx.pos < lx.text().size() && lx.text()[lx.pos] == '{') {
+    std::string lay = lx.balanced();
+    if (lay.find(':') != std::string::npos) MONONN_FAIL(kUnsupported) << "line " << lx.line << ": tiled or annotated layouts are not supported: " << lay;
+    for (auto v : ints_of(lay)) sh.minor_to_major.push_back(static_cast<int>(v));
+    MONONN_CHECK(sh.minor_to_major.size() == sh.dims.size(), kParseError) << "layout rank mismatch in " << lay;
+    for (size_t i = 0; i < sh.dims.size(); ++i)
+      if (sh.minor_to_major[i] != static_cast<int>(sh.dims.size() - 1 - i))
+        MONONN_FAIL(kUnsupported) << "line " << lx.line << ": only descending minor-to-major layouts are supported, got " << lay;
+  } else {
+    for (int i = static_cast<int>(sh.dims.size()) - 1; i >= 0; --i) sh.minor_to_major.push_back(i);
+  }
+  return sh;
+}
+
+void decode_gemm_config(Instr* ins) {
+  auto it = ins->attrs.find("backend_config");
+  MONONN_CHECK(it != ins->attrs.end(), kParseError) << ins->hlo_name << ": __cublas$gemm without backend_config";
+  Json j = Json::parse(it->second);
+  GemmConfig& g = ins->gemm;
+  g.alpha_real = j.at("alpha_real").as_double();
+  if (j.contains("alpha_imag")) g.alpha_imag = j.at("alpha_imag").as_double();
+  g.beta = j.at("beta").as_double();
+  const Json& dn = j.at("dot_dimension_numbers");
+  const Json& lc = dn.at("lhs_contracting_dimensions");
+  const Json& rc = dn.at("rhs_contracting_dimensions");
+  MONONN_CHECK(lc.size() == 1 && rc.size() == 1, kUnsupported) << ins->hlo_name << ": exactly one contracting dimension per operand is supported";
+  g.lhs_contracting = static_cast<int>(lc.at(size_t(0)).as_int());
+  g.rhs_contracting = static_cast<int>(rc.at(size_t(0)).as_int());
+  g.batch_size = j.contains("batch_size") ? j.at("batch_size").as_int() : 1;
+  if (dn.contains("lhs_batch_dimensions"))
+    for (auto& v : dn.at("lhs_batch_dimensions").items()) g.lhs_batch.push_back(static_cast<int>(v.as_int()));
+  if (dn.contains("rhs_batch_dimensions"))
+    for (auto& v : dn.at("rhs_batch_dimensions").items()) g.rhs_batch.push_back(static_cast<int>(v.as_int()));
+  if (j.contains("lhs_stride")) g.lhs_stride = j.at("lhs_stride").as_int();
+  if (j.contains("rhs_stride")) g.rhs_stride = j.at("rhs_stride").as_int();
+  if (j.contains("selected_algorithm")) {
+    const Json& a = j.at("selected_algorithm");
+    g.selected_algorithm = a.is_string() ? a.as_string() : std::to_string(a.as_int());
+  }
+}
+
+void decode_attrs(Instr* ins, Module* mod) {
+  auto has = [&](const char* k) { return ins->attrs.count(k) > 0; };
+  auto get = [&](const char* k) -> const std::string& { return ins->attrs.at(k); };
+  auto need = [&](const char* k) -> const std::string& {
+    MONONN_CHECK(has(k), kParseError) << ins->hlo_name << " (" << ins->opcode << "): missing attribute " << k;
+    return get(k);
+  };
+  auto comp_ref = [&](const std::string& raw) -> Computation* {
+    auto it = mod->by_name.find(canonical_name(raw));
+    MONONN_CHECK(it != mod->by_name.end(), kParseError) << ins->hlo_name << ": unknown computation " << raw;
+    return it->second;
+  };
+  const std::string& op = ins->opcode;
+  if (op == "broadcast" || op == "transpose" || op == "reduce" || op == "concatenate") {
+    if (op != "broadcast" || has("dimensions")) ins->dimensions = ints_of(need("dimensions"));
+  }
+  if (op == "fusion") {
+    ins->called = comp_ref(need("calls"));
+    ins->fusion_kind = need("kind");
+    MONONN_CHECK(ins->fusion_kind == "kLoop" || ins->fusion_kind == "kInput", kUnsupported)
+        << ins->hlo_name << ": fusion kind " << ins->fusion_kind << " is not supported";
+  }
+  if (op == "reduce" || op == "reduce-window") ins->called = comp_ref(need("to_apply"));
+  if (op == "compare") ins->comparison = need("direction");
+  if (op == "get-tuple-element") ins->tuple_index = std::strtoll(need("index").c_str(), nullptr, 10);
+  if (op == "iota") ins->iota_dimension = std::strtoll(need("iota_dimension").c_str(), nullptr, 10);
+  if (op == "slice") {
+    // slice={[0:8192], [2:4:1]}
+    const std::string& s = need("slice");
+    size_t i = 0;
+    while ((i = s.find('[', i)) != std::string::npos) {
+      size_t e = s.find(']', i);
+      MONONN_CHECK(e != std::string::npos, kParseError) << ins->hlo_name << ": bad slice attribute";
+      auto v = ints_of(s.substr(i, e - i));
+      MONONN_CHECK(v.size() == 2 || v.size() == 3, kParseError) << ins->hlo_name << ": bad slice attribute";
+      ins->slice_starts.push_back(v[0]);
+      ins->slice_limits.push_back(v[1]);
+      ins->slice_strides.push_back(v.size() == 3 ? v[2] : 1);
+      // stride-1 slices only (ir_parser_fused.cc:1321-1327)
+      MONONN_CHECK(ins->slice_strides.back() == 1, kUnsupported) << ins->hlo_name << ": strided slice is not supported";
+      i = e;
+    }
+  }
+  if (op == "pad") {
+    // padding=0_0x1_2 or with interior 0_0_0 ; no interior, non-negative edges (ir_parser_fused.cc:1143-1147)
+    const std::string& s = need("padding");
+    size_t st = 0;
+    while (st <= s.size()) {
+      size_t e = s.find('x', st);
+      std::string part = s.substr(st, e == std::string::npos ? std::string::npos : e - st);
+      std::vector<int64_t> v;
+      size_t p = 0;
+      while (p <= part.size()) {
+        size_t q = part.find('_', p);
+        v.push_back(std::strtoll(part.substr(p, q == std::string::npos ? std::string::npos : q - p).c_str(), nullptr, 10));
+        if (q == std::string::npos) break;
+        p = q + 1;
+      }
+      MONONN_CHECK(v.size() >= 2, kParseError) << ins->hlo_name << ": bad padding attribute";
+      MONONN_CHECK(v[0] >= 0 && v[1] >= 0 && (v.size() < 3 || v[2] == 0), kUnsupported)
+          << ins->hlo_name << ": negative or interior padding is not supported";
+      ins->pad_low.push_back(v[0]);
+      ins->pad_high.push_back(v[1]);
+      ins->pad_interior.push_back(0);
+      if (e == std::string::npos) break;
+      st = e + 1;
+    }
+  }
+  if (op == "dynamic-slice") ins->dynamic_slice_sizes = ints_of(need("dynamic_slice_sizes"));
+  if (op == "gather") {
+    ins->offset_dims = ints_of(need("offset_dims"));
+    ins->collapsed_slice_dims = ints_of(need("collapsed_slice_dims"));
+    ins->start_index_map = ints_of(need("start_index_map"));
+    ins->index_vector_dim = std::strtoll(need("index_vector_dim").c_str(), nullptr, 10);
+    ins->slice_sizes = ints_of(need("slice_sizes"));
+  }
+  if (op == "custom-call") {
+    ins->custom_call_target = need("custom_call_target");
+    if (ins->custom_call_target == "__cublas$gemm") {
+      decode_gemm_config(ins);
+    } else if (ins->custom_call_target == "__cudnn$convForward") {
+      // decoded by the convolution lowering from attrs (window, dim_labels)
+    } else {
+      // any other target aborts in the reference (core/op/custom_call.cc:96-100)
+      MONONN_FAIL(kUnsupported) << ins->hlo_name << ": custom-call target '" << ins->custom_call_target << "' is not supported";
+    }
+  }
+  if (op == "convolution") {
+    // a bare convolution aborts in the reference as well (ir_parser_fused.cc:728-732)
+    MONONN_FAIL(kUnsupported) << ins->hlo_name << ": bare convolution is not supported; expected custom-call __cudnn$convForward";
+  }
+}
+
+}  // namespace
+
+std::unique_ptr<Module> parse_module(const std::string& text) {
+  auto mod = std::make_unique<Module>();
+  Lexer lx(text);
+  if (!lx.consume_word("HloModule")) lx.fail("expected 'HloModule'");
+  {
+    std::string n = lx.ident();
+    mod->name = n;
+    // skip the rest of the header line (module attributes)
+    while (lx.pos < text.size() && text[lx.pos] != '\n') ++lx.pos;
+  }
+  struct Pending {
+    Instr* ins;
+    std::vector<std::string> operand_names;
+    int line;
+  };
+  while (!lx.eof()) {
+    auto comp = std::make_unique<Computation>();
+    comp->is_entry = lx.consume_word("ENTRY");
+    comp->hlo_name = lx.ident();
+    comp->name = canonical_name(comp->hlo_name);
+    // optional signature "(p: f32[..]) -> f32[..]"
+    if (lx.peek() == '(') {
+      lx.balanced();
+      lx.skip_ws();
+      if (text.compare(lx.pos, 2, "->") == 0) {
+        lx.pos += 2;
+        parse_shape(lx);
+      }
+    }
+    lx.expect('{');
+    std::map<std::string, Instr*> local;
+    std::vector<Pending> pend;
+    while (lx.peek() != '}') {
+      if (lx.eof()) lx.fail("unterminated computation");
+      auto ins = std::make_unique<Instr>();
+      ins->parent = comp.get();
+      ins->is_root = lx.consume_word("ROOT");
+      ins->hlo_name = lx.ident();
+      ins->name = canonical_name(ins->hlo_name);
+      lx.expect('=');
+      ins->shape = parse_shape(lx);
+      ins->opcode = lx.ident();
+      int line = lx.line;
+      if (!known_opcodes().count(ins->opcode))
+        MONONN_FAIL(kUnsupported) << "line " << line << ": opcode '" << ins->opcode << "' is not supported";
+      std::string body = lx.balanced();
+      body = body.substr(1, body.size() - 2);
+      Pending p{ins.get(), {}, line};
+      if (ins->opcode == "parameter") {
+        ins->parameter_number = std::strtoll(body.c_str(), nullptr, 10);
+      } else if (ins->opcode == "constant") {
+        ins->literal = body;
+        std::string squeezed;
+        for (char c : body)
+          if (!isspace(static_cast<unsigned char>(c))) squeezed.push_back(c);
+        ins->literal_elided = squeezed == "{...}";
+      } else {
+        // operands: "[shape] %name" separated by top-level commas
+        Lexer ol(body);
+        while (!ol.eof()) {
+          // skip an optional shape prefix: anything before the final identifier of this operand
+          size_t start = ol.pos;
+          int depth = 0;
+          size_t i = start;
+          for (; i < body.size(); ++i) {
+            char c = body[i];
+            if (c == '(' || c == '{' || c == '[') ++depth;
+            else if (c == ')' || c == '}' || c == ']') --depth;
+            else if (c == ',' && depth == 0) break;
+          }
+          std::string piece = body.substr(start, i - start);
+          while (!piece.empty() && isspace(static_cast<unsigned char>(piece.back()))) piece.pop_back();
+          size_t sp = piece.find_last_of(" \t");
+          std::string nm = sp == std::string::npos ? piece : piece.substr(sp + 1);
+          size_t lead = nm.find_first_not_of(" \t\n");
+          nm = lead == std::string::npos ? "" : nm.substr(lead);
+          if (nm.empty()) MONONN_FAIL(kParseError) << "line " << line << ": empty operand";
+          p.operand_names.push_back(canonical_name(nm));
+          ol.pos = i < body.size() ? i + 1 : body.size();
+        }
+      }
+      // attributes
+      while (lx.consume(',')) {
+        std::string key = lx.ident();
+        lx.expect('=');
+        ins->attrs[key] = lx.attr_value();
+      }
+      ins->index_in_comp = static_cast<int>(comp->instrs.size());
+      MONONN_CHECK(!local.count(ins->name), kParseError) << "line " << line << ": duplicate instruction name " << ins->hlo_name;
+      local[ins->name] = ins.get();
+      if (ins->is_root) comp->root = ins.get();
+      pend.push_back(std::move(p));
+      comp->instrs.push_back(std::move(ins));
+    }
+    lx.expect('}');
+    MONONN_CHECK(!comp->instrs.empty(), kParseError) << "computation " << comp->hlo_name << " is empty";
+    if (!comp->root) comp->root = comp->instrs.back().get();
+    for (auto& p : pend) {
+      for (auto& on : p.operand_names) {
+        auto it = local.find(on);
+        MONONN_CHECK(it != local.end(), kParseError) << "line " << p.line << ": operand '" << on << "' of " << p.ins->hlo_name << " is not defined";
+        MONONN_CHECK(it->second->index_in_comp < p.ins->index_in_comp, kParseError) << "line " << p.line << ": operand '" << on << "' is used before its definition";
+        p.ins->operands.push_back(it->second);
+        it->second->users.push_back(p.ins);
+      }
+      decode_attrs(p.ins, mod.get());
+      if (p.ins->opcode == "parameter") {
+        MONONN_CHECK(p.ins->parameter_number >= 0, kParseError) << "bad parameter number for " << p.ins->hlo_name;
+        if (comp->params.size() <= static_cast<size_t>(p.ins->parameter_number)) comp->params.resize(p.ins->parameter_number + 1, nullptr);
+        comp->params[p.ins->parameter_number] = p.ins;
+      }
+    }
+    for (auto* pp : comp->params) MONONN_CHECK(pp != nullptr, kParseError) << "computation " << comp->hlo_name << " has a gap in its parameter numbers";
+    MONONN_CHECK(!mod->by_name.count(comp->name), kParseError) << "duplicate computation " << comp->hlo_name;
+    mod->by_name[comp->name] = comp.get();
+    if (comp->is_entry) {
+      MONONN_CHECK(mod->entry == nullptr, kParseError) << "more than one ENTRY computation";
+      mod->entry = comp.get();
+    }
+    mod->computations.push_back(std::move(comp));
+  }
+  MONONN_CHECK(mod->entry != nullptr, kParseError) << "module has no ENTRY computation";
+  return mod;
+}
+
+}  // namespace hlo
+}  // namespace mononn

@@ -1,0 +1,260 @@
+#include "module/mononn_module.h"
+
+#include <sys/stat.h>
+
+#include <cstring>
+#include <fstream>
+#include <sstream>
+
+#include "common/env.h"
+#include "common/status.h"
+#include "hlo/hlo.h"
+#include "runtime/rtc.h"
+
+namespace mononn {
+namespace module {
+
+void make_dirs(const std::string& path) {
+  std::string cur;
+  for (size_t i = 0; i <= path.size(); ++i) {
+    if (i == path.size() || path[i] == '/') {
+      if (!cur.empty()) {
+        if (::mkdir(cur.c_str(), 0755) != 0 && errno != EEXIST) MONONN_FAIL(kRuntimeError) << "cannot create directory " << cur;
+      }
+    }
+    if (i < path.size()) cur.push_back(path[i]);
+  }
+}
+void write_file(const std::string& path, const std::string& data) {
+  std::ofstream f(path, std::ios::binary);
+  MONONN_CHECK(f.good(), kRuntimeError) << "cannot write " << path;
+  f.write(data.data(), static_cast<std::streamsize>(data.size()));
+}
+void write_file(const std::string& path, const std::vector<char>& data) {
+  std::ofstream f(path, std::ios::binary);
+  MONONN_CHECK(f.good(), kRuntimeError) << "cannot write " << path;
+  f.write(data.data(), static_cast<std::streamsize>(data.size()));
+}
+bool read_file(const std::string& path, std::string* out) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f.good()) return false;
+  std::ostringstream ss;
+  ss << f.rdbuf();
+  *out = ss.str();
+  return true;
+}
+
+MonoNNModule::MonoNNModule(const std::string& hlo_text, const std::string& spec_json, const std::string& kernel_name)
+    : hlo_text_(hlo_text), kernel_name_(kernel_name) {
+  if (!spec_json.empty()) {
+    spec_ = spec::GraphSpecification::from_json(Json::parse(spec_json));
+    spec_given_ = true;
+  } else {
+    spec_.runtime.grid_dim.x = spec_.device.sm_count;
+    spec_.runtime.block_dim.x = 256;
+  }
+}
+
+void MonoNNModule::generate_code() {
+  auto mod = hlo::parse_module(hlo_text_);
+  module_name_ = mod->name;
+  if (kernel_name_.empty()) {
+    // kernel naming convention mononn_cluster_<id> (README.md:186)
+    std::string shortn = "cluster_0";
+    try {
+      shortn = hlo::module_short_name(hlo::canonical_name(module_name_));
+    } catch (const Error&) {
+    }
+    kernel_name_ = "mononn_" + shortn;
+  }
+  // MONONN_CODEGEN_ALLOW_LIST_OVERRIDE (mononn_module.cc:62-89)
+  auto override_list = env::allow_list_override();
+  if (!override_list.empty()) spec_.codegen_allow_list = override_list;
+  program_ = graph::build_program(std::move(mod), codegen::build_options_from(spec_));
+  hip_ = codegen::generate_program(*program_, spec_, kernel_name_);
+  grid_ = hip_.grid;
+  code_object_.clear();
+}
+
+void MonoNNModule::build_assembly() {
+  MONONN_CHECK(program_ != nullptr, kInvalidArgument) << "build_assembly called before generate_code";
+  auto res = runtime::compile_hip(hip_.files, "main.hip", spec_.device.cuda_arch);
+  code_object_ = std::move(res.code_object);
+  compile_log_ = res.log;
+}
+
+std::string MonoNNModule::summary() const {
+  std::ostringstream os;
+  os << "module " << module_name_ << " kernel " << kernel_name_ << "\n";
+  if (program_) os << program_->summary();
+  os << "grid=" << hip_.grid << " block=" << hip_.block << " smem=" << hip_.smem << " barriers=" << hip_.num_barriers << "\n";
+  for (size_t i = 0; i < hip_.param_bytes.size(); ++i) os << "Parameter " << i << ": " << hip_.param_bytes[i] << " bytes.\n";
+  for (size_t i = 0; i < hip_.liveout_bytes.size(); ++i) os << "Liveout(output) buffer " << i << " size: " << hip_.liveout_bytes[i] << " bytes.\n";
+  os << "Temporary buffer size: " << hip_.temp_bytes << " bytes.\n";
+  return os.str();
+}
+
+// ---------------------------------------------------------------------------------------------
+static const codegen::ConstantInfo* find_constant(const codegen::HipProgram& hp, const std::string& name) {
+  std::string canon = hlo::canonical_name(name);
+  for (auto& c : hp.constants)
+    if (c.name == canon || c.hlo_name == name || c.symbol == name) return &c;
+  return nullptr;
+}
+
+void MonoNNModule::set_constant(const std::string& name, const void* host_data, size_t bytes) {
+  MONONN_CHECK(program_ != nullptr, kInvalidArgument) << "set_constant called before generate_code";
+  const codegen::ConstantInfo* ci = find_constant(hip_, name);
+  MONONN_CHECK(ci != nullptr, kNotFound) << "the module has no constant named '" << name << "'";
+  MONONN_CHECK(static_cast<int64_t>(bytes) == ci->bytes, kInvalidArgument)
+      << "constant '" << name << "' needs " << ci->bytes << " bytes, got " << bytes;
+  std::vector<char> payload(static_cast<const char*>(host_data), static_cast<const char*>(host_data) + bytes);
+  if (dev_.loaded()) {
+    upload_constant(*ci, payload);
+  } else {
+    host_constants_[ci->name] = std::move(payload);
+  }
+}
+
+void MonoNNModule::upload_constant(const codegen::ConstantInfo& ci, const std::vector<char>& payload) {
+  size_t n = 0;
+  void* dst = dev_.global(ci.symbol, &n);
+  MONONN_CHECK(static_cast<int64_t>(n) >= ci.bytes, kRuntimeError) << "global " << ci.symbol << " is smaller than its constant";
+  if (ci.transform == graph::ConstantTransform::kTranspose2D) {
+    const int es = hlo::dtype_bytes(ci.dtype);
+    const int64_t rows = ci.dims[0], cols = ci.dims[1];
+    std::vector<char> t(payload.size());
+    for (int64_t r = 0; r < rows; ++r)
+      for (int64_t c = 0; c < cols; ++c) std::memcpy(&t[(c * rows + r) * es], &payload[(r * cols + c) * es], es);
+    dev_.upload(dst, t.data(), t.size());
+  } else {
+    dev_.upload(dst, payload.data(), payload.size());
+  }
+  uploaded_[ci.name] = true;
+}
+
+std::vector<std::string> MonoNNModule::missing_constants() const {
+  std::vector<std::string> out;
+  for (auto& c : hip_.constants)
+    if (c.literal.empty() && !uploaded_.count(c.name) && !host_constants_.count(c.name)) out.push_back(c.hlo_name);
+  return out;
+}
+
+static std::vector<char> literal_payload(const codegen::ConstantInfo& ci) {
+  // parse "{ {1, 2}, {3, 4} }" into the constant's element type
+  std::vector<char> out(static_cast<size_t>(ci.bytes));
+  std::string tok;
+  int64_t i = 0;
+  const int es = hlo::dtype_bytes(ci.dtype);
+  auto flush = [&]() {
+    if (tok.empty()) return;
+    MONONN_CHECK(i * es < ci.bytes, kParseError) << "constant " << ci.hlo_name << ": literal has too many elements";
+    double d = 0;
+    long long ll = 0;
+    if (tok == "true") d = 1, ll = 1;
+    else if (tok == "false") d = 0, ll = 0;
+    else if (tok == "inf") d = __builtin_inf();
+    else if (tok == "-inf") d = -__builtin_inf();
+    else if (tok == "nan") d = __builtin_nan("");
+    else {
+      d = std::strtod(tok.c_str(), nullptr);
+      ll = std::strtoll(tok.c_str(), nullptr, 10);
+    }
+    char* p = &out[static_cast<size_t>(i * es)];
+    switch (ci.dtype) {
+      case hlo::DType::kF16: { _Float16 v = static_cast<_Float16>(d); std::memcpy(p, &v, 2); break; }
+      case hlo::DType::kF32: { float v = static_cast<float>(d); std::memcpy(p, &v, 4); break; }
+      case hlo::DType::kF64: std::memcpy(p, &d, 8); break;
+      case hlo::DType::kPred: case hlo::DType::kS8: case hlo::DType::kU8: { int8_t v = static_cast<int8_t>(ll); std::memcpy(p, &v, 1); break; }
+      case hlo::DType::kS16: case hlo::DType::kU16: { int16_t v = static_cast<int16_t>(ll); std::memcpy(p, &v, 2); break; }
+      case hlo::DType::kS32: case hlo::DType::kU32: { int32_t v = static_cast<int32_t>(ll); std::memcpy(p, &v, 4); break; }
+      default: { int64_t v = ll; std::memcpy(p, &v, 8); }
+    }
+    ++i;
+    tok.clear();
+  };
+  for (char ch : ci.literal) {
+    if (ch == '{' || ch == '}' || ch == ',' || isspace(static_cast<unsigned char>(ch))) flush();
+    else tok.push_back(ch);
+  }
+  flush();
+  MONONN_CHECK(i * es == ci.bytes, kParseError) << "constant " << ci.hlo_name << ": literal has " << i << " elements, expected " << ci.bytes / es;
+  return out;
+}
+
+void MonoNNModule::load(int device) {
+  MONONN_CHECK(has_code_object(), kInvalidArgument) << "load called before build_assembly";
+  runtime::DeviceProperties props = runtime::query_device(device);
+  MONONN_CHECK(props.arch == spec_.device.cuda_arch, kRuntimeError)
+      << "code object was built for " << spec_.device.cuda_arch << " but device " << device << " is " << props.arch;
+  dev_.load(device, code_object_, kernel_name_);
+  dev_.set_dynamic_smem(hip_.smem);
+  // The grid barrier needs every workgroup resident at once.  The reference's barrier would
+  // deadlock on an over-sized grid; here it is rejected from the occupancy query before launch.
+  int capacity = dev_.max_coresident_blocks(hip_.block, hip_.smem);
+  MONONN_CHECK(capacity >= hip_.grid, kResourceExhausted)
+      << "grid of " << hip_.grid << " workgroups x " << hip_.block << " threads exceeds the co-resident capacity of device " << device << " ("
+      << capacity << ")";
+  grid_ = hip_.grid;
+  size_t flag_bytes = 0;
+  void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
+  dev_.zero(flags, flag_bytes);
+  uploaded_.clear();
+  for (auto& ci : hip_.constants) {
+    if (!ci.literal.empty()) {
+      upload_constant(ci, literal_payload(ci));
+      continue;
+    }
+    auto it = host_constants_.find(ci.name);
+    if (it != host_constants_.end()) upload_constant(ci, it->second);
+  }
+  host_constants_.clear();
+}
+
+void MonoNNModule::launch(void* const* device_ptrs, size_t n, void* stream) {
+  MONONN_CHECK(dev_.loaded(), kInvalidArgument) << "launch called before load";
+  MONONN_CHECK(n == num_args(), kInvalidArgument) << "kernel takes " << num_args() << " buffers (parameters, live-outs, temp), got " << n;
+  auto missing = missing_constants();
+  MONONN_CHECK(missing.empty(), kInvalidArgument) << missing.size() << " constants have no payload yet, first: " << missing[0];
+  std::vector<void*> vals(device_ptrs, device_ptrs + n);
+  std::vector<void*> args(n);
+  for (size_t i = 0; i < n; ++i) {
+    MONONN_CHECK(vals[i] != nullptr || (i + 1 == n && hip_.temp_bytes == 0), kInvalidArgument) << "buffer " << i << " is null";
+    args[i] = &vals[i];
+  }
+  dev_.launch(grid_, hip_.block, hip_.smem, args.data(), stream);
+}
+
+float MonoNNModule::time_kernel(void* const* device_ptrs, size_t n, void* stream, int warmup, int iters, std::vector<float>* each) {
+  MONONN_CHECK(dev_.loaded(), kInvalidArgument) << "time_kernel called before load";
+  MONONN_CHECK(n == num_args(), kInvalidArgument) << "kernel takes " << num_args() << " buffers, got " << n;
+  std::vector<void*> vals(device_ptrs, device_ptrs + n);
+  std::vector<void*> args(n);
+  for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
+  return dev_.time_launches(grid_, hip_.block, hip_.smem, args.data(), stream, warmup, iters, each);
+}
+
+// ---------------------------------------------------------------------------------------------
+std::string MonoNNModule::cluster_dir(const std::string& dump_dir) const {
+  std::string shortn = hlo::module_short_name(hlo::canonical_name(module_name_));
+  return dump_dir + "/" + shortn;
+}
+
+void MonoNNModule::dump_candidate(const std::string& dump_dir) const {
+  std::string dir = cluster_dir(dump_dir);
+  std::string ctx = spec_.context_string();
+  make_dirs(dir + "/" + ctx + "_src");
+  write_file(dir + "/" + ctx + ".json", tuning_spec_json());
+  if (has_code_object()) write_file(dir + "/" + ctx + ".hsaco", code_object_);
+  for (auto& kv : hip_.files) write_file(dir + "/" + ctx + "_src/" + kv.first, kv.second);
+}
+
+void MonoNNModule::dump_best(const std::string& dump_dir) const {
+  std::string dir = cluster_dir(dump_dir);
+  make_dirs(dir);
+  write_file(dir + "/best_tuning_spec.json", tuning_spec_json());
+  if (has_code_object()) write_file(dir + "/best_tuning_spec.hsaco", code_object_);
+}
+
+}  // namespace module
+}  // namespace mononn

@@ -1,0 +1,94 @@
+// Tuning specification ("GraphSpecification") and its JSON form.
+//
+// The reference keeps this as a protobuf whose schema lives in its absent TensorFlow fork; the
+// field names below are reconstructed from the accessors used in-tree
+// (mononn_engine/core/context/cuda_context.cc:59-77, cuda_runtime_context.cc:32-55,
+// cuda_device_context.cc:117-150, core/gpu/dim3.cc:26-42, core/gpu/cutlass/cutlass_config.cc:32-59,
+// gemm_backend_config.cc:36-87, tuning/tuning_space_generator.cc:151-160,184-194,255-269,318-335,
+// 405-414) and printed the way helpers/protobuf.cc:32-46 prints them (original field names,
+// primitive fields always present).  gfx950-specific choices (wave arrangement of a GEMM tile,
+// fusion decisions, barrier flavour) live in the same per-node maps / a `mononn_hip` section.
+#pragma once
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common/json.h"
+
+namespace mononn {
+namespace spec {
+
+struct Dim3 {
+  int x = 1, y = 1, z = 1;
+};
+
+struct DeviceContext {      // cuda_device_context
+  int device_count = 1;
+  int sm_count = 256;                        // compute units
+  int static_smem_size = 65536;              // LDS a workgroup may use without opting in
+  int max_configurable_smem_size = 163840;   // 160 KiB LDS per CU
+  std::string cuda_arch = "gfx950";
+  int register_per_block = 131072;           // 512 VGPRs x 64 lanes x 4 SIMDs
+  int warp_size = 64;
+  int reserved_smem_per_block = 0;
+};
+
+struct RuntimeContext {     // cuda_runtime_context
+  Dim3 grid_dim, block_dim;
+  int smem_size = 0;
+  std::string stream = "0";
+};
+
+struct ClusterElewiseSpec {
+  std::string name;
+  int ilp_factor = 1;
+};
+
+struct ClusterReduceSpec {
+  std::string name;
+  int ilp_factor = 1;
+  int locality_tier = 1;          // 1 = wave per row, 2 = workgroup per row (reference: warp / block)
+  int reduce_implementation = 0;
+};
+
+struct GemmSpec {
+  // cutlass_config fields re-used with their gfx950 meaning
+  int tb_m = 32, tb_n = 32, tb_k = 32;       // threadblockshape: workgroup tile (k = one MFMA step)
+  int warp_m = 32, warp_n = 32, warp_k = 32; // warpshape: per-wave tile
+  int inst_m = 16, inst_n = 16, inst_k = 32; // instructionshape: v_mfma_f32_16x16x32_f16
+  std::string operator_class = "MFMA";
+  std::string arch_tag = "gfx950";
+  int stages = 1;
+  int wave_m = 1, wave_n = 1, wave_k = 4;    // arrangement of the workgroup's waves over the tile
+  Json backend_config;                       // gemm_backend_config as carried by the HLO
+};
+
+struct HipOptions {       // "mononn_hip" section
+  bool merge_dependent = true;
+  bool gemm_epilogue_fusion = true;
+  bool transpose_constant_b = true;
+  std::string barrier = "flags";
+};
+
+struct GraphSpecification {
+  RuntimeContext runtime;
+  DeviceContext device;
+  std::string hlo_module_proto_file;
+  std::vector<std::string> feeds, input_data_files, fetches;
+  std::map<std::string, ClusterElewiseSpec> cluster_elewise_spec;
+  std::map<std::string, ClusterReduceSpec> cluster_reduce_spec;
+  std::map<std::string, GemmSpec> gemm_spec_list;
+  std::map<std::string, Json> conv_spec_list;
+  std::vector<std::string> codegen_allow_list, codegen_reject_list;
+  HipOptions hip;
+
+  Json to_json() const;
+  // unknown keys are rejected like the reference's loader does (helpers/protobuf.cc:48-65)
+  static GraphSpecification from_json(const Json& j);
+  // "<gx>_<gy>_<gz>__<bx>_<by>_<bz>" (mononn_module_tuner.cc:374-383)
+  std::string context_string() const;
+};
+
+}  // namespace spec
+}  // namespace mononn

@@ -1,0 +1,416 @@
+"""CPU oracle: a NumPy evaluator for the fused-HLO dialect MonoNN consumes.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product (`mononn_amd/`, the C-ABI library) may import
+this file; it is the checker used by `tests/`, `__graft_entry__.smoke()` and the `cpu_baseline`
+leg of `bench.py`.
+
+The reference has no CPU execution path of its own and cannot be built here (it needs its
+TensorFlow and CUTLASS forks, both absent), so this is a restatement of the *semantics* the
+reference attaches to each instruction when it lowers it:
+
+  * opcode set ......................... mononn_engine/core/op/op_type.h:20-65
+  * dtype / layout rules ............... mononn_engine/parser/ir_parser_fused.cc:68-152
+  * fusion -> called computation ....... ir_parser_fused.cc:490-539, :866-1019
+  * reduce (one reduced dim, constant
+    init, reducer = called computation)  ir_parser_fused.cc:1169-1213,
+                                          mononn_engine/codegen/reduction_functor_generator.cc:224-294
+  * broadcast/transpose/slice/pad/
+    concatenate/gather/dynamic-slice
+    index maps ......................... mononn_engine/core/context/index_tracer.cc:67-456
+  * row gather ......................... index_tracer.cc:235-280
+  * element-wise op -> functor ......... mononn_engine/core/gpu/functor.cc:42-88, :145-168
+  * __cublas$gemm backend_config ....... mononn_engine/core/op_impl/gemm_impl.cc:182-231, :233-499
+    (D = alpha * A.B + beta * C, fp32 accumulation, batch = leading dims)
+
+The parser below is written independently of the product's C++ parser so that a parsing bug is
+not shared between the thing under test and its checker.
+
+Pinning (what fixes these functions besides the formulae above): tests/test_oracle_pinning.py
+checks the evaluator against closed forms and library routines -- fp64 triple-loop GEMM on tiny
+shapes, the two worked backend_config examples of gemm_impl.cc:290-316 against numpy einsum,
+torch.nn.functional soft-max / layer_norm / gelu(tanh), brute-force gather, and a whole BERT
+layer against an independent torch restatement.  Bit-level results of the CUDA build (CUTLASS
+accumulation order, -use_fast_math intrinsics) are not reproducible offline: parity unpinned at
+that level; the north-star tolerance is defined against fp32 evaluation, which this is.
+
+precision="as_written": every f16-typed instruction result is rounded to IEEE half (what the
+HLO says).  precision="fp32": f16 is carried as float32 without rounding (the "fp32 reference"
+the tolerance max-abs-err <= 2e-2 / cosine >= 0.9999 is stated against).
+"""
+from __future__ import annotations
+
+import json
+import re
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+_NP = {"pred": np.bool_, "s8": np.int8, "u8": np.uint8, "s16": np.int16, "u16": np.uint16,
+       "s32": np.int32, "u32": np.uint32, "s64": np.int64, "u64": np.uint64,
+       "f16": np.float16, "f32": np.float32, "f64": np.float64}
+
+
+class Shape:
+    __slots__ = ("dtype", "dims", "tuple_shapes")
+
+    def __init__(self, dtype=None, dims=(), tuple_shapes=None):
+        self.dtype, self.dims, self.tuple_shapes = dtype, tuple(dims), tuple_shapes
+
+
+class Instr:
+    __slots__ = ("name", "shape", "opcode", "operands", "attrs", "literal", "is_root")
+
+
+class Comp:
+    def __init__(self, name):
+        self.name = name
+        self.instrs: List[Instr] = []
+        self.root: Optional[Instr] = None
+
+
+# ------------------------------------------------------------------------------------------
+# text -> structures
+# ------------------------------------------------------------------------------------------
+def _split_top(s: str, sep: str = ",") -> List[str]:
+    """Split on `sep` outside (), {}, [] and double-quoted strings."""
+    out, depth, cur, i, in_q = [], 0, [], 0, False
+    while i < len(s):
+        c = s[i]
+        if in_q:
+            cur.append(c)
+            if c == "\\" and i + 1 < len(s):
+                cur.append(s[i + 1])
+                i += 1
+            elif c == '"':
+                in_q = False
+        elif c == '"':
+            in_q = True
+            cur.append(c)
+        elif c in "({[":
+            depth += 1
+            cur.append(c)
+        elif c in ")}]":
+            depth -= 1
+            cur.append(c)
+        elif c == sep and depth == 0:
+            out.append("".join(cur).strip())
+            cur = []
+        else:
+            cur.append(c)
+        i += 1
+    tail = "".join(cur).strip()
+    if tail:
+        out.append(tail)
+    return out
+
+
+def _parse_shape(s: str) -> Shape:
+    s = s.strip()
+    if s.startswith("("):
+        inner = s[1:s.rindex(")")]
+        return Shape(tuple_shapes=[_parse_shape(p) for p in _split_top(inner)])
+    m = re.match(r"([a-z]+\d*)\[([^\]]*)\](\{[^}]*\})?", s)
+    if not m:
+        raise ValueError(f"bad shape: {s!r}")
+    dims = [int(d) for d in m.group(2).split(",") if d.strip()]
+    if m.group(3):
+        lay = [int(x) for x in m.group(3)[1:-1].split(",") if x.strip()]
+        if lay != list(reversed(range(len(dims)))):
+            raise ValueError(f"only descending minor-to-major layouts are supported: {s}")
+    return Shape(m.group(1), dims)
+
+
+def _match_paren(s: str, start: int) -> int:
+    depth, i, in_q = 0, start, False
+    while i < len(s):
+        c = s[i]
+        if in_q:
+            if c == "\\":
+                i += 1
+            elif c == '"':
+                in_q = False
+        elif c == '"':
+            in_q = True
+        elif c in "({[":
+            depth += 1
+        elif c in ")}]":
+            depth -= 1
+            if depth == 0:
+                return i
+        i += 1
+    raise ValueError("unbalanced parentheses")
+
+
+def _parse_instr(line: str) -> Instr:
+    ins = Instr()
+    line = line.strip()
+    ins.is_root = line.startswith("ROOT ")
+    if ins.is_root:
+        line = line[5:].strip()
+    name, rest = line.split("=", 1)
+    ins.name = name.strip().lstrip("%")
+    rest = rest.strip()
+    # shape: either a tuple "(...)" or token up to the first space
+    if rest.startswith("("):
+        end = _match_paren(rest, 0)
+        shape_s, rest = rest[:end + 1], rest[end + 1:].strip()
+    else:
+        shape_s, rest = rest.split(" ", 1)
+    ins.shape = _parse_shape(shape_s)
+    p = rest.index("(")
+    ins.opcode = rest[:p].strip()
+    end = _match_paren(rest, p)
+    body = rest[p + 1:end]
+    tail = rest[end + 1:].strip()
+    ins.literal = None
+    ins.operands = []
+    if ins.opcode in ("constant", "parameter"):
+        ins.literal = body.strip()
+    else:
+        for o in _split_top(body):
+            ins.operands.append(o.split()[-1].lstrip("%"))
+    ins.attrs = {}
+    if tail.startswith(","):
+        for a in _split_top(tail[1:]):
+            if "=" in a:
+                k, v = a.split("=", 1)
+                ins.attrs[k.strip()] = v.strip()
+    return ins
+
+
+def parse_module(text: str) -> Dict[str, object]:
+    comps: Dict[str, Comp] = {}
+    entry = None
+    cur = None
+    mod_name = None
+    for raw in text.splitlines():
+        line = raw.strip()
+        if not line or line.startswith("//"):
+            continue
+        if line.startswith("HloModule"):
+            mod_name = line.split()[1].rstrip(",")
+            continue
+        if cur is None:
+            if line.endswith("{"):
+                is_entry = line.startswith("ENTRY")
+                head = line[5:].strip() if is_entry else line
+                cname = re.split(r"[\s({]", head.lstrip("%"), 1)[0]
+                cur = Comp(cname)
+                if is_entry:
+                    entry = cur
+            continue
+        if line == "}":
+            if cur.root is None and cur.instrs:
+                cur.root = cur.instrs[-1]
+            comps[cur.name] = cur
+            cur = None
+            continue
+        ins = _parse_instr(line)
+        cur.instrs.append(ins)
+        if ins.is_root:
+            cur.root = ins
+    if entry is None:
+        raise ValueError("no ENTRY computation")
+    return {"name": mod_name, "comps": comps, "entry": entry}
+
+
+# ------------------------------------------------------------------------------------------
+# evaluation
+# ------------------------------------------------------------------------------------------
+def _ints(attr: str) -> List[int]:
+    return [int(x) for x in re.findall(r"-?\d+", attr)]
+
+
+def _parse_literal(lit: str, dtype, dims):
+    body = lit.replace("{", " ").replace("}", " ").replace(",", " ").split()
+    conv = {"true": 1, "false": 0, "inf": np.inf, "-inf": -np.inf, "nan": np.nan}
+    vals = [conv[t] if t in conv else float(t) if np.issubdtype(dtype, np.floating) else int(t)
+            for t in body]
+    with np.errstate(over="ignore"):
+        return np.array(vals, dtype=np.float64 if np.issubdtype(dtype, np.floating) else np.int64
+                        ).astype(dtype).reshape(dims)
+
+
+_UNARY = {
+    "abs": np.abs, "negate": np.negative, "exponential": np.exp, "log": np.log, "tanh": np.tanh,
+    "sqrt": np.sqrt, "sign": np.sign, "not": np.logical_not, "copy": lambda x: x,
+    "rsqrt": lambda x: (1.0 / np.sqrt(x)).astype(x.dtype),
+}
+_BINARY = {
+    "add": np.add, "subtract": np.subtract, "multiply": np.multiply, "maximum": np.maximum,
+    "minimum": np.minimum, "and": np.logical_and, "or": np.logical_or,
+}
+_CMP = {"EQ": np.equal, "NE": np.not_equal, "LT": np.less, "LE": np.less_equal,
+        "GT": np.greater, "GE": np.greater_equal}
+_REDUCERS = {"add": np.add, "maximum": np.maximum, "minimum": np.minimum, "multiply": np.multiply,
+             "and": np.logical_and, "or": np.logical_or}
+
+
+class Evaluator:
+    def __init__(self, text: str, constants: Optional[Dict[str, np.ndarray]] = None,
+                 precision: str = "as_written"):
+        assert precision in ("as_written", "fp32")
+        self.mod = parse_module(text)
+        self.constants = constants or {}
+        self.fp32 = precision == "fp32"
+        self.trace: Dict[str, np.ndarray] = {}
+
+    def np_dtype(self, hlo_dtype: str):
+        if self.fp32 and hlo_dtype == "f16":
+            return np.float32
+        return _NP[hlo_dtype]
+
+    def run(self, params: Sequence[np.ndarray], keep_trace: bool = False):
+        self._keep = keep_trace
+        res = self._run_comp(self.mod["entry"], list(params), top=True)
+        return list(res) if isinstance(res, tuple) else [res]
+
+    def _cast_in(self, a: np.ndarray, shape: Shape) -> np.ndarray:
+        a = np.asarray(a)
+        if tuple(a.shape) != tuple(shape.dims):
+            raise ValueError(f"shape mismatch: got {a.shape}, HLO says {shape.dims}")
+        return a.astype(self.np_dtype(shape.dtype), copy=False)
+
+    def _run_comp(self, comp: Comp, args: List[np.ndarray], top: bool = False):
+        env: Dict[str, object] = {}
+        for ins in comp.instrs:
+            env[ins.name] = self._eval(ins, env, args)
+            if top and self._keep and isinstance(env[ins.name], np.ndarray):
+                self.trace[ins.name] = env[ins.name]
+        return env[comp.root.name]
+
+    def _eval(self, ins: Instr, env, args):
+        op = ins.opcode
+        x = [env[o] for o in ins.operands]
+        sh = ins.shape
+        dt = self.np_dtype(sh.dtype) if sh.tuple_shapes is None else None
+        if op == "parameter":
+            return self._cast_in(args[int(ins.literal)], sh)
+        if op == "constant":
+            if ins.literal.replace(" ", "") == "{...}":
+                if ins.name not in self.constants:
+                    raise KeyError(f"payload for elided constant {ins.name} not supplied")
+                return self._cast_in(self.constants[ins.name], sh)
+            return _parse_literal(ins.literal, dt, sh.dims)
+        if op in ("tuple",):
+            return tuple(x)
+        if op == "get-tuple-element":
+            return x[0][int(ins.attrs["index"])]
+        if op in ("bitcast", "reshape"):
+            return np.ascontiguousarray(x[0]).reshape(sh.dims)
+        if op == "fusion" or op == "call":
+            key = "calls" if "calls" in ins.attrs else "to_apply"
+            return self._run_comp(self.mod["comps"][ins.attrs[key].lstrip("%")], x)
+        if op == "convert":
+            src = x[0]
+            if np.issubdtype(dt, np.integer) and np.issubdtype(src.dtype, np.floating):
+                src = np.trunc(src)
+            with np.errstate(over="ignore"):
+                return src.astype(dt)
+        if op in _UNARY:
+            with np.errstate(all="ignore"):
+                return _UNARY[op](x[0]).astype(dt, copy=False)
+        if op in _BINARY:
+            with np.errstate(all="ignore"):
+                return _BINARY[op](x[0], x[1]).astype(dt, copy=False)
+        if op == "divide":
+            with np.errstate(all="ignore"):
+                if np.issubdtype(dt, np.integer):
+                    q = np.trunc(x[0].astype(np.float64) / x[1].astype(np.float64))
+                    return q.astype(dt)
+                return np.divide(x[0], x[1]).astype(dt, copy=False)
+        if op == "power":
+            return np.power(x[0], x[1]).astype(dt, copy=False)
+        if op == "compare":
+            return _CMP[ins.attrs["direction"]](x[0], x[1])
+        if op == "select":
+            return np.where(x[0], x[1], x[2]).astype(dt, copy=False)
+        if op == "clamp":
+            return np.minimum(np.maximum(x[1], x[0]), x[2]).astype(dt, copy=False)
+        if op == "broadcast":
+            mapping = _ints(ins.attrs.get("dimensions", "{}"))
+            shape1 = [1] * len(sh.dims)
+            for i, m in enumerate(mapping):
+                shape1[m] = x[0].shape[i]
+            return np.broadcast_to(x[0].reshape(shape1), sh.dims)
+        if op == "transpose":
+            return np.transpose(x[0], _ints(ins.attrs["dimensions"]))
+        if op == "iota":
+            d = int(ins.attrs["iota_dimension"])
+            shape1 = [1] * len(sh.dims)
+            shape1[d] = sh.dims[d]
+            return np.broadcast_to(np.arange(sh.dims[d], dtype=dt).reshape(shape1), sh.dims)
+        if op == "slice":
+            parts = re.findall(r"\[(\d+):(\d+)(?::(\d+))?\]", ins.attrs["slice"])
+            idx = tuple(slice(int(a), int(b), int(c) if c else 1) for a, b, c in parts)
+            return x[0][idx]
+        if op == "concatenate":
+            return np.concatenate(x, axis=_ints(ins.attrs["dimensions"])[0])
+        if op == "pad":
+            cfg = [tuple(int(v) for v in p.split("_")[:2]) for p in ins.attrs["padding"].split("x")]
+            out = np.empty(sh.dims, dt)
+            out[...] = x[1]
+            idx = tuple(slice(lo, lo + n) for (lo, _), n in zip(cfg, x[0].shape))
+            out[idx] = x[0]
+            return out
+        if op == "reduce":
+            return self._reduce(ins, x, dt)
+        if op == "gather":
+            return self._gather(ins, x)
+        if op == "dynamic-slice":
+            sizes = _ints(ins.attrs["dynamic_slice_sizes"])
+            starts = [int(np.clip(int(s), 0, x[0].shape[i] - sizes[i])) for i, s in enumerate(x[1:])]
+            return x[0][tuple(slice(s, s + n) for s, n in zip(starts, sizes))]
+        if op == "custom-call":
+            target = ins.attrs["custom_call_target"].strip('"')
+            if target == "__cublas$gemm":
+                return self._gemm(ins, x, dt)
+            raise NotImplementedError(f"custom-call target {target}")
+        raise NotImplementedError(f"opcode {op}")
+
+    def _reduce(self, ins: Instr, x, dt):
+        dims = _ints(ins.attrs["dimensions"])
+        if len(dims) != 1 or len(x) != 2:
+            raise NotImplementedError("only single-dimension, single-operand reduce")
+        red = self.mod["comps"][ins.attrs["to_apply"].lstrip("%")]
+        fn = _REDUCERS[red.root.opcode]
+        init = x[1]
+        with np.errstate(all="ignore"):
+            r = fn.reduce(x[0], axis=dims[0], dtype=x[0].dtype if x[0].dtype != np.bool_ else None)
+            return fn(r, init).astype(dt, copy=False)
+
+    def _gather(self, ins: Instr, x):
+        table, idx = x
+        a = ins.attrs
+        if (_ints(a["collapsed_slice_dims"]) != [0] or _ints(a["start_index_map"]) != [0]
+                or int(a["index_vector_dim"]) != idx.ndim):
+            raise NotImplementedError("only row gather")
+        sizes = _ints(a["slice_sizes"])
+        if sizes[0] != 1 or list(sizes[1:]) != list(table.shape[1:]):
+            raise NotImplementedError("only whole-row slices")
+        safe = np.clip(idx.astype(np.int64), 0, table.shape[0] - 1)   # XLA clamps start indices
+        return table[safe]
+
+    def _gemm(self, ins: Instr, x, dt):
+        cfg = json.loads(ins.attrs["backend_config"][1:-1].replace('\\"', '"'))
+        dn = cfg["dot_dimension_numbers"]
+        lc = int(dn["lhs_contracting_dimensions"][0])
+        rc = int(dn["rhs_contracting_dimensions"][0])
+        A = x[0].astype(np.float32)
+        B = x[1].astype(np.float32)
+        r = A.ndim
+        if lc == r - 2:
+            A = np.swapaxes(A, -1, -2)
+        if rc == r - 1:
+            B = np.swapaxes(B, -1, -2)
+        D = np.matmul(A, B) * np.float32(cfg["alpha_real"])
+        if len(x) > 2 and float(cfg["beta"]) != 0.0:
+            D = D + np.float32(cfg["beta"]) * x[2].astype(np.float32)
+        with np.errstate(over="ignore"):
+            return D.astype(dt)
+
+
+def evaluate(text: str, params: Sequence[np.ndarray], constants: Optional[Dict[str, np.ndarray]] = None,
+             precision: str = "as_written") -> List[np.ndarray]:
+    """Evaluate the ENTRY computation; returns the list of outputs (root tuple flattened)."""
+    return Evaluator(text, constants, precision).run(params)

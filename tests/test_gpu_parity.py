@@ -1,0 +1,94 @@
+"""GPU parity: the generated monolithic kernel against the NumPy oracle on the same seeded inputs.
+Tolerance (stated by the north star): max-abs-err <= 2e-2 and cosine >= 0.9999 against the fp32
+evaluation of the HLO; integer / gather work bit-exact."""
+import numpy as np
+import pytest
+
+from mononn_amd import MonoNNModule
+from mononn_amd.hlo import models
+from mononn_amd.hlo.builder import HloModuleBuilder
+from oracle import hlo_interp
+
+pytestmark = pytest.mark.gpu
+
+
+def run_module(hlo_text, inputs, constants, outputs, spec_json=None):
+    m = MonoNNModule.compile(hlo_text, spec_json)
+    m.set_constants(constants)
+    m.load(0)
+    return m.run(inputs, outputs), m
+
+
+def check_close(got, want32, atol=2e-2, cos_min=0.9999):
+    g = got.astype(np.float64).ravel()
+    w = want32.astype(np.float64).ravel()
+    assert np.all(np.isfinite(g))
+    err = np.abs(g - w).max()
+    cos = float(g @ w / (np.linalg.norm(g) * np.linalg.norm(w) + 1e-30))
+    assert err <= atol, f"max abs err {err}"
+    assert cos >= cos_min, f"cosine {cos}"
+    return err, cos
+
+
+def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=False):
+    mb = HloModuleBuilder("cluster_7__gemm_test.1")
+    e = mb.entry
+    r = len(batch) + 2
+    lhs_c = r - 1 if lhs_c is None else lhs_c
+    rhs_c = r - 2 if rhs_c is None else rhs_c
+    a_dims = list(batch) + ([M, K] if lhs_c == r - 1 else [K, M])
+    b_dims = list(batch) + ([K, N] if rhs_c == r - 2 else [N, K])
+    a = e.parameter("f16", a_dims, "a")
+    b = e.elided_constant("f16", b_dims, "w/kernel") if b_const else e.parameter("f16", b_dims, "b")
+    d = e.gemm(a, b, lhs_c, rhs_c, batch_dims=tuple(range(len(batch))), alpha=alpha)
+    e.set_tuple_root([d])
+    return mb, a_dims, b_dims, list(batch) + [M, N]
+
+
+@pytest.mark.parametrize("case", [
+    dict(M=128, N=768, K=768, b_const=True),                      # weight GEMM, constant transposed at upload
+    dict(M=128, N=96, K=64),                                      # [K,N] parameter operand -> fallback path
+    dict(M=128, N=128, K=64, batch=(1, 12), rhs_c=3, alpha=0.125),  # scores: both operands k-contiguous
+    dict(M=128, N=64, K=128, batch=(2, 3)),                       # context: B stored [K,N]
+    dict(M=100, N=52, K=96, rhs_c=1),                             # ragged M / N on the MFMA path
+    dict(M=64, N=48, K=40, rhs_c=1),                              # K not a multiple of 32
+    dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                     # A stored [K,M]
+])
+def test_gemm_cases(gpu_device, case):
+    mb, a_dims, b_dims, d_dims = gemm_module(**case)
+    rng = np.random.default_rng(3)
+    a = rng.normal(0, 1, a_dims).astype(np.float16)
+    b = rng.normal(0, 1, b_dims).astype(np.float16)
+    text = mb.text()
+    consts = {n: b for n in mb.constants}
+    inputs = [a] if case.get("b_const") else [a, b]
+    (got,), _ = run_module(text, inputs, consts, [{"dtype": "f16", "dims": d_dims}])
+    want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
+    # fp16 output rounding of values up to ~sqrt(K): relative tolerance
+    scale = np.abs(want).max()
+    assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * scale + 1e-3
+
+
+def test_bert_layer_parity(gpu_device):
+    fx = models.bert_layer()
+    consts = fx.make_constants(1234, "random")
+    inputs = fx.make_inputs(1234)
+    (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs)
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    err, cos = check_close(got, want)
+    print(f"bert_layer: max_abs_err={err:.3e} cosine={cos:.6f} dims={m.launch_dims()}")
+
+
+def test_gather_bit_exact(gpu_device):
+    mb = HloModuleBuilder("cluster_3__gather_test.1")
+    e = mb.entry
+    ids = e.parameter("s32", (2, 37), "ids")
+    table = e.elided_constant("f16", (1000, 96), "table")
+    g = e.gather_rows(table, ids)
+    e.set_tuple_root([g])
+    rng = np.random.default_rng(5)
+    t = rng.normal(0, 1, (1000, 96)).astype(np.float16)
+    i = rng.integers(0, 1000, (2, 37), dtype=np.int32)
+    consts = {n: t for n in mb.constants}
+    (got,), _ = run_module(mb.text(), [i], consts, [{"dtype": "f16", "dims": [2, 37, 96]}])
+    assert np.array_equal(got.view(np.uint16), t[i].view(np.uint16))
