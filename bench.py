@@ -1,0 +1,163 @@
+"""Headline benchmark: full BERT-base encoder (12 layers + embeddings, batch 1, seq 128, fp16) as ONE
+monolithic cooperative kernel launch on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one forward pass = one launch of the generated kernel, inputs and weights resident in
+HBM.  Prints one JSON line: throughput (seq/s) as `value`, latency in `ms_per_step` / `latency_us`,
+the HBM roofline of the kernel (algorithmic bytes = weights + gathered rows + ids + output, read or
+written once) with the launch duration measured by HIP events on the launch stream, and the NumPy
+oracle timed on the host cores as `cpu_baseline`.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
+SPEC_DIR = os.path.join(ROOT, "mononn_amd", "specs", "bert_base_b1_s128")
+
+
+def algorithmic_bytes(fx) -> int:
+    """Bytes a perfect fusion must move: every weight / bias / LayerNorm constant once, except the
+    embedding tables of which only the gathered rows are read; ids in; hidden states out."""
+    cfg = fx.config
+    total = 0
+    for meta in fx.constants.values():
+        n = int(np.prod(meta["dims"])) * 2
+        if meta["role"].endswith("word_embeddings") or meta["role"].endswith("token_type_embeddings"):
+            n = cfg["B"] * cfg["S"] * cfg["H"] * 2          # gathered rows
+        elif meta["role"].endswith("position_embeddings"):
+            n = cfg["S"] * cfg["H"] * 2                      # first S rows
+        total += n
+    total += 3 * cfg["B"] * cfg["S"] * 4                     # three int32 id tensors
+    total += cfg["B"] * cfg["S"] * cfg["H"] * 2              # output
+    return total
+
+
+def gemm_flops(cfg) -> int:
+    B, S, H, NH, F, L = cfg["B"], cfg["S"], cfg["H"], cfg["NH"], cfg["F"], cfg["L"]
+    M, d = B * S, H // NH
+    per_layer = 2 * M * H * 3 * H + 2 * M * H * H + 4 * M * H * F + 4 * B * NH * S * S * d
+    return per_layer * L
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--spec-dir", default=SPEC_DIR)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the monolithic kernel's grid barrier cannot span "
+              "devices); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from mononn_amd import MonoNNModule, device_info
+    from mononn_amd.hlo import models
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    fx = models.bert_base(B=1, S=128)
+    consts = fx.make_constants(1235, "baseline")
+    inputs = fx.make_inputs(1235)
+
+    used_spec = "default"
+    module = None
+    if os.path.isdir(args.spec_dir):
+        try:
+            module = MonoNNModule.from_spec_dir(fx.hlo_text, args.spec_dir)
+            used_spec = os.path.relpath(args.spec_dir, ROOT)
+        except Exception as e:  # a stale spec must not silently change what is measured
+            print(f"bench.py: spec dir unusable ({e}); compiling with the default specification", file=sys.stderr)
+            module = None
+    if module is None:
+        module = MonoNNModule.compile(fx.hlo_text)
+    module.set_constants(consts)
+    module.load(0)
+    dims = module.launch_dims()
+
+    # parity of this very configuration against the oracle (also the CPU baseline's subject)
+    got = module.run(inputs, fx.outputs)[0].astype(np.float32)
+
+    ptrs = module.buffer_pointers()
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(args.warmup):
+        module.launch_raw(ptrs, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        module.launch_raw(ptrs, stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    # kernel duration by HIP events on the same stream (what rocprof's kernel trace reports)
+    avg_ms, each = module.time_raw(ptrs, stream, warmup=10, iters=max(50, min(args.steps, 500)))
+    each_us = np.sort(each.astype(np.float64) * 1e3)
+    kern_us = float(avg_ms * 1e3)
+
+    abytes = algorithmic_bytes(fx)
+    flops = gemm_flops(fx.config)
+    achieved_gbs = abytes / (kern_us * 1e-6) / 1e9
+    achieved_tflops = flops / (kern_us * 1e-6) / 1e12
+
+    result = {
+        "metric": "per-forward latency (us) & seq/s, BERT-base b1 s128 fp16, 1 MI355X",
+        "value": round(fx.config["B"] * 1e3 / ms_per_step, 2),
+        "unit": "seq/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "BERT-base encoder, 12 layers + embedding gather, batch 1, seq 128, fp16 weights "
+                               "N(0,0.02), one monolithic cooperative kernel launch per forward",
+                   "tuning_spec": used_spec, "grid": dims["grid"], "block": dims["block"], "lds_bytes": dims["smem"],
+                   "grid_barriers": dims["barriers"]},
+        "latency_us": {"kernel_avg": round(kern_us, 2), "kernel_p10": round(float(each_us[len(each_us) // 10]), 2),
+                       "kernel_median": round(float(each_us[len(each_us) // 2]), 2),
+                       "kernel_p90": round(float(each_us[(len(each_us) * 9) // 10]), 2),
+                       "end_to_end_per_step": round(ms_per_step * 1e3, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 5), "traffic": None,
+                     "algorithmic_bytes": abytes, "kernel": module.kernel_name},
+        "mfma": {"achieved_tflops": round(achieved_tflops, 2), "peak_tflops": MFMA_F16_PEAK_TFLOPS,
+                 "frac": round(achieved_tflops / MFMA_F16_PEAK_TFLOPS, 5), "gemm_flops": flops},
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import hlo_interp
+        ev = hlo_interp.Evaluator(fx.hlo_text, consts, "fp32")
+        want = ev.run(inputs)[0].astype(np.float32)   # also warms the BLAS threads
+        n, t0 = 0, time.perf_counter()
+        while n < 3 or (time.perf_counter() - t0 < 12.0 and n < 50):
+            ev.run(inputs)
+            n += 1
+        cpu_s = (time.perf_counter() - t0) / n
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            cores = os.cpu_count() or 1
+        g, w = got.ravel().astype(np.float64), want.ravel().astype(np.float64)
+        result["cpu_baseline"] = {"value": round(fx.config["B"] / cpu_s, 3), "unit": "seq/s", "cores": cores,
+                                  "kind": "port",
+                                  "sample": f"{n} fp32 forwards of the same HLO and inputs by the NumPy oracle "
+                                            f"(multi-threaded BLAS), {cpu_s * 1e3:.1f} ms each"}
+        result["parity"] = {"max_abs_err": float(np.abs(g - w).max()),
+                            "cosine": float(g @ w / (np.linalg.norm(g) * np.linalg.norm(w)))}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

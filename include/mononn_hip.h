@@ -77,6 +77,10 @@ int mononn_module_buffer_info(const mononn_module* m, int* n_params, const int64
                               int* n_liveouts, const int64_t** liveout_bytes, int64_t* temp_bytes);
 /* grid / block / dynamic LDS of the launch (best_tuning_spec.json keys grid_dim, block_dim, smem_size;
  * README.md:199-200) and the number of grid-wide barriers in the kernel. */
+/* 1 when the kernel hands data between stages through a module-owned coherent (uncached) temp arena:
+ * the caller then passes NULL in the temp slot of mononn_launch.  0: the caller brings the temp buffer
+ * (the reference's contract), at the price of cache maintenance in every grid barrier. */
+int mononn_module_owns_temp(const mononn_module* m);
 int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int* smem, int* barriers);
 
 /* Non-scalar constants of the module ("buffer_for_<node>" globals that the host fills before
@@ -103,6 +107,15 @@ int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, voi
  *           (mononn_engine/module/mononn_module_tuner.cc:250-372, tuning/profiler/cupti_profiling_session.h:20-78). */
 int mononn_time_kernel(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream, int warmup,
                        int iters, float* avg_ms, float* each_ms);
+
+/* Per-stage wall-clock stamps of the last launch, for kernels compiled from a specification with
+ * mononn_hip.profile_stages = true: ticks[(stage * grid + workgroup) * 2 + {0: stage begin, 1: work done}].
+ * Copies at most `capacity` values; n_stages / grid / ticks_per_us describe the layout.  Stage names
+ * (node names joined by '+') come from mononn_module_stage_name.
+ * Replaces: the per-node report of dump_performance_report (mononn_engine/module/mononn_module_tuner.cc:422-448). */
+int mononn_module_stage_clock(mononn_module* m, uint64_t* ticks, size_t capacity, int* n_stages, int* grid,
+                              double* ticks_per_us);
+const char* mononn_module_stage_name(mononn_module* m, int stage);
 
 /* Write <dump_dir>/<cluster_N>/{<ctx>.json,<ctx>.hsaco,<ctx>_src/*,best_tuning_spec.{json,hsaco}}.
  * Replaces: the dump half of final_tuning (mononn_engine/module/mononn_module_tuner.cc:457-603). */

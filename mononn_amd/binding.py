@@ -53,6 +53,7 @@ def _load_library() -> ctypes.CDLL:
     lib.mononn_module_buffer_info.argtypes = [c.c_void_p, P(c.c_int), P(P(c.c_int64)), P(c.c_int), P(P(c.c_int64)),
                                               P(c.c_int64)]
     lib.mononn_module_launch_dims.argtypes = [c.c_void_p, P(c.c_int), P(c.c_int), P(c.c_int), P(c.c_int)]
+    lib.mononn_module_owns_temp.argtypes = [c.c_void_p]
     lib.mononn_module_num_constants.argtypes = [c.c_void_p]
     lib.mononn_module_constant_info.argtypes = [c.c_void_p, c.c_int, P(c.c_char_p), P(c.c_char_p), P(c.c_int64), P(c.c_int)]
     lib.mononn_module_set_constant.argtypes = [c.c_void_p, c.c_char_p, c.c_void_p, c.c_size_t]
@@ -60,6 +61,9 @@ def _load_library() -> ctypes.CDLL:
     lib.mononn_launch.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p]
     lib.mononn_time_kernel.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p, c.c_int, c.c_int,
                                        P(c.c_float), P(c.c_float)]
+    lib.mononn_module_stage_clock.argtypes = [c.c_void_p, P(c.c_uint64), c.c_size_t, P(c.c_int), P(c.c_int), P(c.c_double)]
+    lib.mononn_module_stage_name.argtypes = [c.c_void_p, c.c_int]
+    lib.mononn_module_stage_name.restype = c.c_char_p
     lib.mononn_module_dump.argtypes = [c.c_void_p, c.c_char_p]
     lib.mononn_device_count.restype = c.c_int
     lib.mononn_device_info.argtypes = [c.c_int, P(c.c_int), P(c.c_int), P(c.c_int), c.c_char_p, c.c_size_t]
@@ -71,9 +75,9 @@ _lib = _load_library()
 EXPORTED_SYMBOLS = [
     "mononn_last_error", "mononn_version", "mononn_compile", "mononn_tune", "mononn_compile_from_spec_dir",
     "mononn_module_destroy", "mononn_module_kernel_name", "mononn_module_spec_json", "mononn_module_source",
-    "mononn_module_code_object", "mononn_module_summary", "mononn_module_buffer_info", "mononn_module_launch_dims",
+    "mononn_module_code_object", "mononn_module_summary", "mononn_module_buffer_info", "mononn_module_launch_dims", "mononn_module_owns_temp",
     "mononn_module_num_constants", "mononn_module_constant_info", "mononn_module_set_constant", "mononn_module_load",
-    "mononn_launch", "mononn_time_kernel", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
+    "mononn_launch", "mononn_time_kernel", "mononn_module_stage_clock", "mononn_module_stage_name", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
 
 
 def _check(rc: int):
@@ -122,7 +126,7 @@ class MonoNNModule:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
+        if h and _lib is not None:
             _lib.mononn_module_destroy(h)
 
     # ---- introspection -----------------------------------------------------------------------
@@ -172,6 +176,10 @@ class MonoNNModule:
                         "needs_payload": bool(need.value)})
         return out
 
+    @property
+    def owns_temp(self) -> bool:
+        return bool(_lib.mononn_module_owns_temp(self._h))
+
     def dump(self, dump_dir: str):
         _check(_lib.mononn_module_dump(self._h, dump_dir.encode()))
 
@@ -200,6 +208,25 @@ class MonoNNModule:
                                        ctypes.byref(avg), each))
         return float(avg.value), np.array(each[:], dtype=np.float32)
 
+    def stage_profile(self) -> List[dict]:
+        """Per-stage timing of the last launch (kernel compiled with mononn_hip.profile_stages):
+        `busy_us` = first workgroup in to last workgroup done, `barrier_us` = last workgroup done to the
+        first workgroup entering the next stage, `mean_wg_us` = average per-workgroup work time."""
+        ns, grid, tpu = ctypes.c_int(), ctypes.c_int(), ctypes.c_double()
+        _check(_lib.mononn_module_stage_clock(self._h, None, 0, ctypes.byref(ns), ctypes.byref(grid), ctypes.byref(tpu)))
+        n = ns.value * grid.value * 2
+        buf = (ctypes.c_uint64 * n)()
+        _check(_lib.mononn_module_stage_clock(self._h, buf, n, ctypes.byref(ns), ctypes.byref(grid), ctypes.byref(tpu)))
+        t = np.frombuffer(buf, dtype=np.uint64).astype(np.float64).reshape(ns.value, grid.value, 2) / tpu.value
+        out = []
+        for s in range(ns.value):
+            begin, done = t[s, :, 0].min(), t[s, :, 1].max()
+            nxt = t[s + 1, :, 0].min() if s + 1 < ns.value else done
+            out.append({"stage": s, "nodes": _lib.mononn_module_stage_name(self._h, s).decode(),
+                        "busy_us": done - begin, "barrier_us": nxt - done,
+                        "mean_wg_us": float((t[s, :, 1] - t[s, :, 0]).mean())})
+        return out
+
     # torch is used for device memory and streams only
     def make_buffers(self, device: int = 0):
         import torch
@@ -207,13 +234,14 @@ class MonoNNModule:
         dev = torch.device("cuda", device)
         bufs = {"params": [torch.zeros(max(n, 1), dtype=torch.uint8, device=dev) for n in info["parameters"]],
                 "liveouts": [torch.zeros(max(n, 1), dtype=torch.uint8, device=dev) for n in info["liveouts"]],
-                "temp": torch.zeros(max(info["temp"], 256), dtype=torch.uint8, device=dev)}
+                "temp": None if self.owns_temp else torch.zeros(max(info["temp"], 256), dtype=torch.uint8, device=dev)}
         self._bufs = bufs
         return bufs
 
     def buffer_pointers(self) -> List[int]:
         b = self._bufs
-        return [t.data_ptr() for t in b["params"]] + [t.data_ptr() for t in b["liveouts"]] + [b["temp"].data_ptr()]
+        temp = 0 if b["temp"] is None else b["temp"].data_ptr()
+        return [t.data_ptr() for t in b["params"]] + [t.data_ptr() for t in b["liveouts"]] + [temp]
 
     def run(self, inputs: Sequence[np.ndarray], out_dtypes_dims: Sequence[dict]) -> List[np.ndarray]:
         """Copy `inputs` to the GPU, launch once on torch's current stream, return live-outs as NumPy."""

@@ -160,6 +160,8 @@ int mononn_module_buffer_info(const mononn_module* m, int* n_params, const int64
   });
 }
 
+int mononn_module_owns_temp(const mononn_module* m) { return (m && m->impl->owns_temp()) ? 1 : 0; }
+
 int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int* smem, int* barriers) {
   return guarded([&] {
     require(m != nullptr, "NULL module");
@@ -215,6 +217,27 @@ int mononn_time_kernel(mononn_module* m, void* const* device_ptrs, size_t n_ptrs
     *avg_ms = m->impl->time_kernel(device_ptrs, n_ptrs, stream, warmup, iters, each_ms ? &each : nullptr);
     if (each_ms) std::memcpy(each_ms, each.data(), each.size() * sizeof(float));
   });
+}
+
+int mononn_module_stage_clock(mononn_module* m, uint64_t* ticks, size_t capacity, int* n_stages, int* grid, double* ticks_per_us) {
+  return guarded([&] {
+    require(m && n_stages && grid && ticks_per_us, "NULL argument");
+    std::vector<unsigned long long> t;
+    *ticks_per_us = m->impl->read_stage_clock(&t, n_stages, grid);
+    if (ticks)
+      for (size_t i = 0; i < t.size() && i < capacity; ++i) ticks[i] = t[i];
+  });
+}
+
+const char* mononn_module_stage_name(mononn_module* m, int stage) {
+  if (!m) return "";
+  auto& sn = m->impl->hip_program().stage_nodes;
+  if (stage < 0 || stage >= static_cast<int>(sn.size())) return "";
+  m->names.resize(sn.size());
+  std::string& s = m->names[stage];
+  s.clear();
+  for (auto& n : sn[stage]) s += (s.empty() ? "" : "+") + n;
+  return s.c_str();
 }
 
 int mononn_module_dump(mononn_module* m, const char* dump_dir) {

@@ -78,14 +78,35 @@ void store(CodeBuffer& cb, PointerTable& ptrs, const VarTable& vars, const Instr
   cb.line(ptrs.output(out) + "[" + linearize(idx, out->shape.dims).str(vars) + "] = " + v + ";");
 }
 
+std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs);
+
 NodeFunction finish(const std::string& body, PointerTable& ptrs, Emitter& em, int64_t units, int smem, const std::string& pre = "") {
   NodeFunction f;
   f.pointers = ptrs.entries;
   f.num_units = units;
   f.smem_bytes = smem;
   for (auto& kv : em.literal_tables()) f.globals.push_back(kv.second);
-  f.text = pre + "__device__ __noinline__ void @NAME@(" + signature(ptrs.entries) + ") {\n" + body + "}\n";
+  f.text = pre + "__device__ __noinline__ void @NAME@(" + signature(ptrs.entries) + ") {\n" + align_prologue(ptrs.entries) + body + "}\n";
   return f;
+}
+
+int pick_vector_width(int64_t len, int64_t lanes) {
+  // largest of 8/4/2 elements per thread that divides the row and still keeps every lane busy
+  for (int v : {8, 4, 2})
+    if (len % v == 0 && len / v >= lanes) return v;
+  return 1;
+}
+
+std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs) {
+  // every buffer handed to the kernel is at least 16-byte aligned (temp offsets are multiples of 256,
+  // module globals are aligned(256), caller buffers are checked at launch); telling the compiler
+  // lets it merge the per-element accesses of one thread into 64/128-bit loads and stores
+  std::string out;
+  for (auto& e : ptrs) {
+    std::string T = std::string(e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "*";
+    out += "  " + e.name + " = (" + T + ")__builtin_assume_aligned(" + e.name + ", 16);\n";
+  }
+  return out;
 }
 
 NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
@@ -103,36 +124,6 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     const bool block_tier = t.locality_tier == 2;
     const int stride = block_tier ? ls.block_size : 64;
     int row = vars.add("row", ROWS);
-    int col = vars.add("col", R);
-    const std::string start = block_tier ? "(int)threadIdx.x" : "lane";
-    cb.line("const int lane = mononn_dev::lane_id();");
-    if (block_tier) {
-      cb.line("const int row = unit;");
-      cb.open("");
-    } else {
-      cb.line("const int row = unit * " + S(NW) + " + mononn_dev::wave_id();");
-      cb.open("if (row < " + S(ROWS) + ")");
-    }
-    const std::string col_loop = "for (int col = " + start + "; col < " + S(R) + "; col += " + S(stride) + ")";
-    for (auto* r : em.collect_reduces()) {
-      const Instr* x = r->operands[0];
-      std::string T = hlo::dtype_ctype(r->shape.dtype);
-      std::string acc = em.fresh("red");
-      cb.line(T + " " + acc + " = " + em.value(r->operands[1], {}) + ";");
-      cb.open(col_loop);
-      em.push_scope();
-      std::vector<int64_t> lead(x->shape.dims.begin(), x->shape.dims.end() - 1);
-      Index xi = leading_index(row, ROWS, lead, vars);
-      xi.push_back(LinExpr::variable(col, R));
-      std::string v = em.value(x, xi);
-      cb.line(acc + " = (" + T + ")" + Emitter::reducer_expr(r, acc, v) + ";");
-      em.pop_scope();
-      cb.close();
-      if (block_tier) cb.line(acc + " = mononn_dev::block_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ", reinterpret_cast<" + T + "*>(smem));");
-      else cb.line(acc + " = mononn_dev::wave_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
-      em.bind(r, leading_index(row, ROWS, r->shape.dims, vars), acc);
-    }
-    // row-shaped outputs
     std::vector<const Instr*> row_outs, full_outs;
     for (auto* o : outputs) {
       int64_t n = o->shape.num_elements();
@@ -140,36 +131,124 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       else if (n == ROWS) row_outs.push_back(o);
       else MONONN_FAIL(kUnsupported) << o->hlo_name << ": output with " << n << " elements does not fit a " << ROWS << " x " << R << " row space";
     }
-    if (!row_outs.empty()) {
+    cb.line("const int lane = mononn_dev::lane_id();");
+    cb.line(std::string("const int tid = ") + (block_tier ? "(int)threadIdx.x;" : "lane;"));
+    if (block_tier) {
+      cb.line("const int row = unit;");
+      cb.open("");
+    } else {
+      cb.line("const int row = unit * " + S(NW) + " + mononn_dev::wave_id();");
+      cb.open("if (row < " + S(ROWS) + ")");
+    }
+    auto all_reduce = [&](const Instr* r, const std::string& acc) {
+      std::string T = hlo::dtype_ctype(r->shape.dtype);
+      if (block_tier) cb.line(acc + " = mononn_dev::block_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ", reinterpret_cast<" + T + "*>(smem));");
+      else cb.line(acc + " = mononn_dev::wave_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
+    };
+    auto operand_index = [&](const Instr* x, const LinExpr& col) {
+      std::vector<int64_t> lead(x->shape.dims.begin(), x->shape.dims.end() - 1);
+      Index xi = leading_index(row, ROWS, lead, vars);
+      xi.push_back(col);
+      return xi;
+    };
+    auto emit_row_outputs = [&]() {
+      if (row_outs.empty()) return;
       em.push_scope();
       std::vector<std::pair<const Instr*, std::string>> vals;
-      Index ri;
-      for (auto* o : row_outs) {
-        ri = leading_index(row, ROWS, o->shape.dims, vars);
-        vals.emplace_back(o, em.value(em.resolve_output(o), ri));
-      }
-      cb.open(block_tier ? "if (threadIdx.x == 0)" : "if (lane == 0)");
+      for (auto* o : row_outs) vals.emplace_back(o, em.value(em.resolve_output(o), leading_index(row, ROWS, o->shape.dims, vars)));
+      cb.open("if (tid == 0)");
       for (auto& kv : vals) store(cb, ptrs, vars, kv.first, leading_index(row, ROWS, kv.first->shape.dims, vars), kv.second);
       cb.close();
       em.pop_scope();
-    }
-    if (!full_outs.empty()) {
-      cb.open(col_loop);
-      em.push_scope();
-      for (auto* o : full_outs) {
-        LinExpr lin = LinExpr::variable(row, ROWS).scaled(R).plus(LinExpr::variable(col, R));
-        Index oi = delinearize(lin, o->shape.dims, vars);
-        store(cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
+    };
+
+    // Register-resident form: a thread owns T chunks of V consecutive columns, the whole row program
+    // is straight-line code, so a value loaded for the first reduction is still in a register when
+    // the later phases need it (one trip to memory per row instead of one per phase).
+    const int V = t.ilp_factor > 1 && R % t.ilp_factor == 0 ? t.ilp_factor : pick_vector_width(R, stride);
+    const int64_t NQ = R / V;
+    const int64_t T = (NQ + stride - 1) / stride;
+    if (T * V <= 32) {
+      std::vector<int> qvar(T);
+      std::vector<bool> partial(T);
+      for (int64_t k = 0; k < T; ++k) {
+        partial[k] = (k + 1) * stride > NQ;
+        std::string q = "q" + S(k);
+        if (partial[k]) {
+          cb.line("const bool act" + S(k) + " = tid + " + S(k * stride) + " < " + S(NQ) + ";");
+          cb.line("const int " + q + " = act" + S(k) + " ? tid + " + S(k * stride) + " : " + S(NQ - 1) + ";");
+        } else {
+          cb.line("const int " + q + " = tid + " + S(k * stride) + ";");
+        }
+        qvar[k] = vars.add(q, NQ);
       }
-      em.pop_scope();
-      cb.close();
+      auto col_of = [&](int64_t k, int v) { return LinExpr::variable(qvar[k], NQ).scaled(V).plus_const(v); };
+      for (auto* r : em.collect_reduces()) {
+        std::string Tn = hlo::dtype_ctype(r->shape.dtype);
+        std::string acc = em.fresh("red");
+        cb.line(Tn + " " + acc + " = " + em.value(r->operands[1], {}) + ";");
+        for (int64_t k = 0; k < T; ++k)
+          for (int v = 0; v < V; ++v) {
+            std::string val = em.value(r->operands[0], operand_index(r->operands[0], col_of(k, v)));
+            std::string upd = "(" + Tn + ")" + Emitter::reducer_expr(r, acc, val);
+            if (partial[k]) cb.line(acc + " = act" + S(k) + " ? " + upd + " : " + acc + ";");
+            else cb.line(acc + " = " + upd + ";");
+          }
+        all_reduce(r, acc);
+        em.bind(r, leading_index(row, ROWS, r->shape.dims, vars), acc);
+      }
+      emit_row_outputs();
+      for (int64_t k = 0; k < T; ++k) {
+        std::vector<std::string> lines;
+        for (int v = 0; v < V; ++v)
+          for (auto* o : full_outs) {
+            LinExpr lin = LinExpr::variable(row, ROWS).scaled(R).plus(col_of(k, v));
+            Index oi = delinearize(lin, o->shape.dims, vars);
+            std::string val = em.value(em.resolve_output(o), oi);
+            lines.push_back(ptrs.output(o) + "[" + linearize(oi, o->shape.dims).str(vars) + "] = " + val + ";");
+          }
+        if (lines.empty()) continue;
+        if (partial[k]) cb.open("if (act" + S(k) + ")");
+        for (auto& l : lines) cb.line(l);
+        if (partial[k]) cb.close();
+      }
+    } else {
+      // long rows: loops over the columns, operands re-read per phase
+      int col = vars.add("col", R);
+      const std::string col_loop = "for (int col = tid; col < " + S(R) + "; col += " + S(stride) + ")";
+      for (auto* r : em.collect_reduces()) {
+        std::string Tn = hlo::dtype_ctype(r->shape.dtype);
+        std::string acc = em.fresh("red");
+        cb.line(Tn + " " + acc + " = " + em.value(r->operands[1], {}) + ";");
+        cb.open(col_loop);
+        em.push_scope();
+        std::string v = em.value(r->operands[0], operand_index(r->operands[0], LinExpr::variable(col, R)));
+        cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(r, acc, v) + ";");
+        em.pop_scope();
+        cb.close();
+        all_reduce(r, acc);
+        em.bind(r, leading_index(row, ROWS, r->shape.dims, vars), acc);
+      }
+      emit_row_outputs();
+      if (!full_outs.empty()) {
+        cb.open(col_loop);
+        em.push_scope();
+        for (auto* o : full_outs) {
+          LinExpr lin = LinExpr::variable(row, ROWS).scaled(R).plus(LinExpr::variable(col, R));
+          Index oi = delinearize(lin, o->shape.dims, vars);
+          store(cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
+        }
+        em.pop_scope();
+        cb.close();
+      }
     }
     cb.close();
     int64_t units = block_tier ? ROWS : (ROWS + NW - 1) / NW;
     return finish(cb.text(), ptrs, em, units, block_tier ? NW * 8 : 0);
   }
 
-  // element-wise loop(s); outputs of equal element count share one loop
+  // element-wise loop(s); outputs of equal element count share one loop.  A thread owns V consecutive
+  // elements (V = ilp_factor when it divides the element count) so its accesses can be merged.
   std::vector<std::pair<int64_t, std::vector<const Instr*>>> groups;
   for (auto* o : outputs) {
     int64_t n = o->shape.num_elements();
@@ -181,30 +260,29 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       }
     if (!placed) groups.push_back({n, {o}});
   }
-  const int ILP = std::max(1, t.ilp_factor);
-  const int64_t per_unit = static_cast<int64_t>(ls.block_size) * ILP;
   int64_t unit_base = 0;
   for (size_t gi = 0; gi < groups.size(); ++gi) {
     const int64_t N = groups[gi].first;
-    const int64_t units = (N + per_unit - 1) / per_unit;
+    const int V = (t.ilp_factor > 1 && N % t.ilp_factor == 0 && t.ilp_factor <= 16) ? t.ilp_factor : 1;
+    const int64_t NQ = N / V;
+    const int64_t units = (NQ + ls.block_size - 1) / ls.block_size;
     std::string u = "unit";
     if (groups.size() > 1) {
       cb.open(std::string(gi ? "else " : "") + "if (unit < " + S(unit_base + units) + ")");
       u = "(unit - " + S(unit_base) + ")";
     }
-    std::string iv = "i" + S(gi);
-    int var = vars.add(iv, N);
-    cb.line("#pragma unroll");
-    cb.open("for (int j = 0; j < " + S(ILP) + "; ++j)");
-    cb.line("const int " + iv + " = " + u + " * " + S(per_unit) + " + j * " + S(ls.block_size) + " + (int)threadIdx.x;");
-    cb.open("if (" + iv + " < " + S(N) + ")");
+    std::string qv = "q" + S(gi);
+    int var = vars.add(qv, NQ);
+    cb.line("const int " + qv + " = " + u + " * " + S(ls.block_size) + " + (int)threadIdx.x;");
+    cb.open("if (" + qv + " < " + S(NQ) + ")");
     em.push_scope();
-    for (auto* o : groups[gi].second) {
-      Index oi = leading_index(var, N, o->shape.dims, vars);
-      store(cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
-    }
+    for (int v = 0; v < V; ++v)
+      for (auto* o : groups[gi].second) {
+        LinExpr lin = LinExpr::variable(var, NQ).scaled(V).plus_const(v);
+        Index oi = delinearize(lin, o->shape.dims, vars);
+        store(cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
+      }
     em.pop_scope();
-    cb.close();
     cb.close();
     if (groups.size() > 1) cb.close();
     unit_base += units;
@@ -279,7 +357,7 @@ bool can_merge_clusters(const Program& prog, const std::vector<const Instr*>& pr
 // ------------------------------------------------------------------------------------------
 // GEMM
 // ------------------------------------------------------------------------------------------
-bool gemm_uses_mfma(const graph::GemmDesc& g) { return g.a_k_contig && g.b_k_contig && g.K % 32 == 0; }
+bool gemm_uses_mfma(const graph::GemmDesc& g) { return g.a_k_contig && (g.b_k_contig || g.b_packed) && g.K % 32 == 0; }
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus) {
   (void)num_cus;
@@ -481,6 +559,16 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     auto& e = ptrs.entries[i];
     pre += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
   }
+  if (mfma) {
+    // touch the epilogue's operands ahead of the main loop
+    pre += "  __device__ __forceinline__ void prefetch(int bidx, int m, int n0) const {\n";
+    if (vec4 && !em.simple_loads().empty()) {
+      pre += "    const int n4 = n0 >> 2;\n    #pragma unroll\n    for (int r = 0; r < 4; ++r) {\n";
+      for (auto& l : em.simple_loads()) pre += "      mononn_dev::touch(" + l + ");\n";
+      pre += "    }\n";
+    }
+    pre += "  }\n";
+  }
   if (vec4) pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4]) const {\n";
   else if (mfma) {
     pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&accv)[4]) const {\n";
@@ -504,16 +592,22 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   int64_t units = 0;
   int smem = 0;
   if (mfma) {
+    // Unit order: the workgroups that read the same columns of B (same tile_n, all tile_m) differ by
+    // multiples of 8 in their unit index; with units dealt round-robin over the 8 XCDs they land on
+    // one XCD and share its L2.  tile_n = 8 * (q / tiles_m) + u % 8, tile_m = q % tiles_m, q = u / 8.
     const int64_t tiles_m = (g.M + t.bm - 1) / t.bm, tiles_n = (g.N + t.bn - 1) / t.bn;
-    units = g.batch * tiles_m * tiles_n;
-    fb.line("const int bidx = unit / " + S(tiles_m * tiles_n) + ";");
-    fb.line("const int rem = unit % " + S(tiles_m * tiles_n) + ";");
-    fb.line("const int tile_n = rem / " + S(tiles_m) + ";");
-    fb.line("const int tile_m = rem % " + S(tiles_m) + ";");
+    const int64_t tn_groups = (tiles_n + 7) / 8;
+    const int64_t per_batch = tn_groups * tiles_m * 8;
+    units = g.batch * per_batch;
+    fb.line("const int bidx = unit / " + S(per_batch) + ";");
+    fb.line("const int rem = unit % " + S(per_batch) + ";");
+    fb.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
+    fb.line("const int tile_m = (rem >> 3) % " + S(tiles_m) + ";");
+    if (tiles_n % 8 != 0) fb.line("if (tile_n >= " + S(tiles_n) + ") return;");
     std::ostringstream call;
-    call << "mononn_dev::gemm_tile_kcontig<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << g.K << ">("
-         << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * " << g.b_batch_stride << ", " << g.M << ", " << g.N
-         << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem);";
+    call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << g.K << ", "
+         << (g.b_packed ? "true" : "false") << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * "
+         << g.b_batch_stride << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem);";
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
   } else {

@@ -194,7 +194,9 @@ std::string Emitter::value(const Instr* ins, const Index& idx) {
 
 std::string Emitter::load(const Instr* root, const Index& idx) {
   LinExpr lin = linearize(idx, root->shape.dims);
-  return def(root->shape.dtype, ptrs_.input(root) + "[" + lin.str(vars_) + "]");
+  std::string ref = ptrs_.input(root) + "[" + lin.str(vars_) + "]";
+  if (lin.opaques().empty()) simple_loads_.push_back(ref);
+  return def(root->shape.dtype, ref);
 }
 
 std::string Emitter::serial_reduce(const Instr* ins, const Index& idx) {

@@ -78,6 +78,8 @@ class Emitter {
   static std::string reducer_functor(const hlo::Instr* reduce);       // C++ lambda text
   // device-global arrays for non-scalar literal constants met inside fused computations
   const std::map<std::string, std::string>& literal_tables() const { return literal_tables_; }
+  // "ptr[index]" of every plain load emitted so far whose index only involves loop variables
+  const std::vector<std::string>& simple_loads() const { return simple_loads_; }
 
  private:
   std::string emit(const hlo::Instr* ins, const Index& idx);
@@ -101,6 +103,7 @@ class Emitter {
   };
   std::map<const hlo::Instr*, Bound> bound_;
   std::map<std::string, std::string> literal_tables_;
+  std::vector<std::string> simple_loads_;
   int counter_ = 0;
 };
 

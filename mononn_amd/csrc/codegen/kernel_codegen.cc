@@ -76,6 +76,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     ci.dims = c->shape.dims;
     auto tr = prog.constant_transform.find(c);
     if (tr != prog.constant_transform.end()) ci.transform = tr->second;
+    ci.device_bytes = ci.bytes;
+    if (ci.transform == graph::ConstantTransform::kPackMfmaB) ci.device_bytes = (ci.dims[1] + 15) / 16 * 16 * ci.dims[0] * hlo::dtype_bytes(ci.dtype);
     if (!c->literal_elided) ci.literal = c->literal;
     auto md = c->attrs.find("metadata");
     if (md != c->attrs.end()) {
@@ -195,10 +197,17 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
 
   std::ostringstream src;
   src << "// generated by mononn-hip for " << spec.device.cuda_arch << "; kernel " << kernel_name << "\n";
+  if (spec.hip.barrier == "flags_allfence") src << "#define MONONN_BARRIER_FENCE 1\n";
+  else if (spec.hip.barrier == "flags_coherent") src << "#define MONONN_BARRIER_FENCE 2\n";
+  else MONONN_CHECK(spec.hip.barrier == "flags", kSpecError) << "unknown barrier flavour '" << spec.hip.barrier << "'";
   src << "#include \"headers.h\"\n\n";
   for (auto& c : hp.constants)
-    src << "__device__ __attribute__((aligned(256))) unsigned char " << c.symbol << "[" << std::max<int64_t>(c.bytes, 1) << "];\n";
-  src << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];\n\n";
+    src << "__device__ __attribute__((aligned(256))) unsigned char " << c.symbol << "[" << std::max<int64_t>(c.device_bytes, 1) << "];\n";
+  src << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];\n";
+  hp.profiled = spec.hip.profile_stages;
+  hp.num_stages = static_cast<int>(by_stage.size());
+  if (hp.profiled) src << "__device__ unsigned long long mononn_stage_clock[" << std::max<size_t>(by_stage.size(), 1) * hp.grid * 2 << "];\n";
+  src << "\n";
   for (auto& g : globals) src << g << "\n";
   for (auto& d : fn_defs) src << d << "\n";
 
@@ -209,12 +218,17 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
   src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags);\n";
   bool first = true;
+  int stage_ordinal = 0;
   for (auto& st : by_stage) {
     if (!first) {
       src << "  barrier.sync();\n";
       ++hp.num_barriers;
     }
     first = false;
+    hp.stage_nodes.emplace_back();
+    for (auto& c : st.second) hp.stage_nodes.back().push_back(c.node->name);
+    if (hp.profiled)
+      src << "  if (threadIdx.x == 0) mononn_stage_clock[(" << stage_ordinal << " * " << hp.grid << " + blockIdx.x) * 2] = wall_clock64();\n";
     int64_t total = 0;
     for (auto& c : st.second) total += c.units;
     src << "  // stage " << st.first << "\n";
@@ -228,6 +242,11 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       base += c.units;
     }
     src << "  }\n";
+    if (hp.profiled) {
+      src << "  __syncthreads();\n";
+      src << "  if (threadIdx.x == 0) mononn_stage_clock[(" << stage_ordinal << " * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
+    }
+    ++stage_ordinal;
   }
   src << "}\n";
   hp.files["headers.h"] = device::kPreludeText;

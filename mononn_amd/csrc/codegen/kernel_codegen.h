@@ -25,7 +25,8 @@ struct ConstantInfo {
   std::string hlo_name;
   std::string symbol;      // buffer_for_<name>
   std::string role;        // metadata op_name when present
-  int64_t bytes = 0;
+  int64_t bytes = 0;          // payload size in the HLO layout (what the host passes in)
+  int64_t device_bytes = 0;   // size of the module global (padded when re-laid out)
   hlo::DType dtype = hlo::DType::kInvalid;
   std::vector<int64_t> dims;
   graph::ConstantTransform transform = graph::ConstantTransform::kNone;
@@ -48,6 +49,9 @@ struct HipProgram {
   int num_barriers = 0;
   int grid = 0, block = 0, smem = 0;
   int max_grid = 4096;       // barrier flag capacity
+  int num_stages = 0;        // stages that were emitted
+  bool profiled = false;     // kernel writes mononn_stage_clock[stage][workgroup][2]
+  std::vector<std::vector<std::string>> stage_nodes;   // node names per emitted stage
 };
 
 // Fills `spec` with defaults for nodes it does not mention, validates the rest (a spec naming a

@@ -31,6 +31,10 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef int int4_t __attribute__((ext_vector_type(4)));
 
+#ifndef MONONN_BARRIER_FENCE
+#define MONONN_BARRIER_FENCE 0
+#endif
+
 namespace mononn_dev {
 
 constexpr int kWaveSize = 64;
@@ -52,18 +56,39 @@ struct GridBarrier {
     epoch = __hip_atomic_load(&flags[blockIdx.x * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
+  // MONONN_BARRIER_FENCE: 0 = one thread per workgroup performs the release / acquire cache
+  // maintenance (an agent-scope acquire invalidates the XCD's whole L2, so issuing it from every
+  // wave multiplies that cost by the number of resident waves); 1 = every thread fences;
+  // 2 = no cache maintenance at all (only valid when inter-stage data bypasses the caches).
   __device__ __forceinline__ void sync() {
     __syncthreads();
     epoch += 1;
     if (threadIdx.x == 0) {
+#if MONONN_BARRIER_FENCE == 2
+      __hip_atomic_store(&flags[blockIdx.x * kFlagStride], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#else
       __hip_atomic_store(&flags[blockIdx.x * kFlagStride], epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+#endif
     }
+#if MONONN_BARRIER_FENCE == 0
+    if (threadIdx.x < kWaveSize) {
+      for (int b = threadIdx.x; b < (int)gridDim.x; b += kWaveSize) {
+        while ((int)(__hip_atomic_load(&flags[b * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);   // agent scope: drop stale lines before the next stage reads
+    }
+#else
     for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
       while ((int)(__hip_atomic_load(&flags[b * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
         __builtin_amdgcn_s_sleep(1);
       }
     }
-    __atomic_thread_fence(__ATOMIC_ACQUIRE);   // agent scope: drop stale lines before the next stage reads
+#if MONONN_BARRIER_FENCE == 1
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+#endif
+#endif
     __syncthreads();
   }
 };
@@ -99,34 +124,56 @@ __device__ __forceinline__ float fast_tanh(float x) {
   float e = __expf(2.0f * x);
   return 1.0f - 2.0f / (e + 1.0f);
 }
+// keep a value (and the load that produced it) alive without using it
+template <class T>
+__device__ __forceinline__ void touch(T v) {
+  float f = (float)v;
+  asm volatile("" ::"v"(f));
+}
 template <class T>
 __device__ __forceinline__ T sign_of(T x) {
   return (T)((x > (T)0) - (x < (T)0));
 }
 
 // ---------------------------------------------------------------------------------------------
-// GEMM:  D[m][n] = sum_k A[m][k] * Bt[n][k]      (both operands contiguous along k)
+// GEMM:  D[m][n] = sum_k A[m][k] * B[k][n]      A contiguous along k
 // ---------------------------------------------------------------------------------------------
 // One workgroup owns a BM x BN output tile.  Its waves are arranged WM x WN x WK: WM*WN waves split
 // the tile, WK waves split the k range of each sub-tile (k steps interleaved).  Every wave feeds
-// v_mfma_f32_16x16x32_f16 directly from global memory: a lane's operand is 8 consecutive halves of
-// one row, i.e. one 16-byte load, and because the weight matrix is only ever read by the waves
-// that own its columns there is nothing to share through LDS in the main loop.  Partial sums of
-// the WK waves meet in LDS once, after the loop.
+// v_mfma_f32_16x16x32_f16 directly from global memory: a lane's operand is 8 consecutive halves
+// along k, i.e. one 16-byte load, and because a weight element is only ever needed by the waves that
+// own its columns there is nothing to share through LDS in the main loop.  Partial sums of the WK
+// waves meet in LDS once, after the loop.
 //
-// The MFMA is issued with the Bt fragment as first operand so that a lane ends up with four
+// At batch 1 a stage is bound by memory latency, not by bandwidth or MFMA rate, so the loop is
+// organised around round trips: the k steps of a wave are cut into chunks of CH steps, all loads of
+// a chunk are issued back to back (and the next chunk's before the current chunk's MFMAs), which
+// leaves one exposed memory latency per tile instead of one per k step.
+//
+// B comes in one of two layouts:
+//   PACKED_B = false : Bt[n][k], k contiguous (activation operands such as K in Q.K^T)
+//   PACKED_B = true  : fragment order [n/16][k/32][lane][8] written by the host at upload for
+//                      constant weights: one MFMA operand = one contiguous 1 KiB block, a wave
+//                      walks its k range through consecutive memory.
+//
+// The MFMA is issued with the B fragment as first operand so that a lane ends up with four
 // consecutive n of one row m (n = n0 + 4*(lane/16) + r, m = m0 + lane%16): the epilogue then
 // stores 8 contiguous bytes per lane.
 //
-// Epilogue functor:  void operator()(int batch, int m, int n, const float (&v)[4])   (n % 4 == 0)
+// Epilogue functor:  void prefetch(int batch, int m, int n) const   (touch what operator() will read)
+//                    void operator()(int batch, int m, int n, const float (&v)[4])   (n % 4 == 0)
 // Rows/cols beyond M / N are clamped on load and skipped on store, so M and N need not divide.
-template <int BM, int BN, int WM, int WN, int WK, int K, class Epi>
-__device__ __forceinline__ void gemm_tile_kcontig(const half_t* A, const half_t* Bt,
-                                                  int M, int N, int lda, int ldb, int batch, int tile_m,
-                                                  int tile_n, Epi& epi, char* smem) {
+template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, class Epi>
+__device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
+                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem) {
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int KSTEPS = K / 32;
+  constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
+  // chunk size: keep (TM + TN) * 4 * CH * 2 (double buffer) within ~256 VGPRs
+  constexpr int CH_MAX = 32 / (TM + TN) > 0 ? 32 / (TM + TN) : 1;
+  constexpr int CH = MY_STEPS < CH_MAX ? MY_STEPS : CH_MAX;
+  constexpr int NCHUNK = (MY_STEPS + CH - 1) / CH;
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
   static_assert(K % 32 == 0, "K must be a multiple of 32");
   const int lane = lane_id();
@@ -149,31 +196,64 @@ __device__ __forceinline__ void gemm_tile_kcontig(const half_t* A, const half_t*
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    int n = n_base + j * 16 + r16;
-    n = n < N ? n : N - 1;
-    b_ptr[j] = Bt + (long)n * ldb + kq;
+    if (PACKED_B) {
+      int nt = (n_base >> 4) + j;
+      const int nt_max = (N + 15) / 16 - 1;
+      nt = nt < nt_max ? nt : nt_max;
+      b_ptr[j] = B + ((long)nt * KSTEPS * 64 + lane) * 8;
+    } else {
+      int n = n_base + j * 16 + r16;
+      n = n < N ? n : N - 1;
+      b_ptr[j] = B + (long)n * ldb + kq;
+    }
   }
+  constexpr int B_STEP = PACKED_B ? 64 * 8 : 32;   // halves between consecutive k steps
+
+  half8_t a[2][CH][TM], b[2][CH][TN];
+  auto load_chunk = [&](int c, int buf) {
+#pragma unroll
+    for (int s = 0; s < CH; ++s) {
+      int ks = (c * CH + s) * WK + wk;
+      ks = ks < KSTEPS ? ks : KSTEPS - 1;   // surplus steps re-read a valid block and are not accumulated
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);
+    }
+  };
+
   float4_t acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
-#pragma unroll 4
-  for (int s = 0; s < MY_STEPS; ++s) {
-    const int ks = s * WK + wk;
-    if (KSTEPS % WK != 0 && ks >= KSTEPS) break;
-    half8_t a[TM], b[TN];
+  load_chunk(0, 0);
+  // touch the epilogue's operands (bias, residual) now so that their latency overlaps the main loop
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + ks * 32);
+    for (int j = 0; j < TN; ++j) {
+      if (WK > 1 && (i * TN + j) % WK != wk) continue;
+      const int m = m_base + i * 16 + r16;
+      const int n = n_base + j * 16 + (lane >> 4) * 4;
+      if (m < M && n < N) epi.prefetch(batch, m, n);
+    }
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+  for (int c = 0; c < NCHUNK; ++c) {
+    if (c + 1 < NCHUNK) load_chunk(c + 1, (c + 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+    for (int s = 0; s < CH; ++s) {
+      const int ks = (c * CH + s) * WK + wk;
+      if (ks < KSTEPS) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[c & 1][s][j], a[c & 1][s][i], acc[i][j], 0, 0, 0);
+      }
+    }
   }
 
   if (WK > 1) {
@@ -186,7 +266,7 @@ __device__ __forceinline__ void gemm_tile_kcontig(const half_t* A, const half_t*
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        red[((wk * (WM * WN) + mn) * (TM * TN) + (i * TN + j)) * kWaveSize + lane] = acc[i][j];
+        if ((i * TN + j) % WK != wk) red[((wk * (WM * WN) + mn) * (TM * TN) + (i * TN + j)) * kWaveSize + lane] = acc[i][j];
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -194,9 +274,10 @@ __device__ __forceinline__ void gemm_tile_kcontig(const half_t* A, const half_t*
       for (int j = 0; j < TN; ++j) {
         const int f = i * TN + j;
         if (f % WK != wk) continue;
-        float4_t s = red[((0 * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
+        float4_t s = acc[i][j];
 #pragma unroll
-        for (int w = 1; w < WK; ++w) s += red[((w * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
+        for (int w = 0; w < WK; ++w)
+          if (w != wk) s += red[((w * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
         const int m = m_base + i * 16 + r16;
         const int n = n_base + j * 16 + (lane >> 4) * 4;
         if (m < M && n < N) {

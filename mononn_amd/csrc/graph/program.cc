@@ -28,7 +28,7 @@ const Node* Program::node_of(const Instr* member) const {
 
 std::string GemmDesc::problem_hash() const {
   std::ostringstream os;
-  os << "f16_b" << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_k_contig ? "_bk" : "_bn");
+  os << "f16_b" << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_packed ? "_bp" : (b_k_contig ? "_bk" : "_bn"));
   return os.str();
 }
 
@@ -317,7 +317,7 @@ struct Builder {
 
   void decide_constant_layouts() {
     if (!opt.transpose_constant_b || !enabled("ConstantLayoutPass")) return;
-    // a constant [K,N] matrix used only as the right operand of GEMMs is stored [N,K] by the host
+    // a constant [K,N] matrix used only as the right operand of GEMMs is stored in fragment order by the host
     std::map<const Instr*, bool> ok;
     for (auto& up : p.module->entry->instrs) {
       const Instr* c = up.get();
@@ -325,7 +325,8 @@ struct Builder {
       bool all = !c->users.empty();
       for (auto* u : c->users) {
         bool good = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands.size() >= 2 &&
-                    u->operands[1] == c && u->operands[0] != c && u->gemm.rhs_contracting == 0 && (u->operands.size() < 3 || u->operands[2] != c);
+                    u->operands[1] == c && u->operands[0] != c && u->gemm.rhs_contracting == 0 && c->shape.dims[0] % 32 == 0 &&
+                    u->gemm.lhs_contracting == u->operands[0]->shape.rank() - 1 && (u->operands.size() < 3 || u->operands[2] != c);
         if (!good) all = false;
       }
       if (all) ok[c] = true;
@@ -334,9 +335,8 @@ struct Builder {
       if (n.kind != NodeKind::kGemm) continue;
       const Instr* b = n.members[0]->operands[1];
       if (ok.count(b)) {
-        n.gemm.b_k_contig = true;
-        n.gemm.b_transposed_upload = true;
-        p.constant_transform[b] = ConstantTransform::kTranspose2D;
+        n.gemm.b_packed = true;
+        p.constant_transform[b] = ConstantTransform::kPackMfmaB;
       }
     }
   }

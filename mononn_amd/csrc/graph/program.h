@@ -26,7 +26,7 @@ struct GemmDesc {
   int64_t batch = 1, M = 0, N = 0, K = 0;
   bool a_k_contig = true;    // A stored [.., M, K]; false: [.., K, M]
   bool b_k_contig = false;   // B stored [.., N, K]; false: [.., K, N]
-  bool b_transposed_upload = false;   // B is a constant that the host stores as [N, K] at upload
+  bool b_packed = false;     // B is a constant that the host stores in MFMA fragment order at upload
   int64_t a_batch_stride = 0, b_batch_stride = 0, d_batch_stride = 0;
   double alpha = 1.0, beta = 0.0;
   bool has_addend = false;
@@ -61,7 +61,9 @@ struct Buffer {
   int def_stage = 0, last_use_stage = 0;
 };
 
-enum class ConstantTransform { kNone, kTranspose2D };
+// kPackMfmaB: a [K,N] matrix stored as [ceil(N/16)][K/32][64 lanes][8 halves], lane l holding
+// W[k = 32*ks + 8*(l/16) + j][n = 16*nt + l%16], columns beyond N zero-filled.
+enum class ConstantTransform { kNone, kPackMfmaB };
 
 struct Program {
   std::unique_ptr<hlo::Module> module;
@@ -84,7 +86,7 @@ struct Program {
 struct BuildOptions {
   bool merge_dependent = true;          // glue producer/consumer clusters that share a row space
   bool fuse_gemm_epilogue = true;       // element-wise consumers of a GEMM run in its epilogue
-  bool transpose_constant_b = true;     // store constant [K,N] GEMM operands as [N,K]
+  bool transpose_constant_b = true;     // store constant [K,N] GEMM operands in MFMA fragment order
   std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)
 };
 

@@ -55,6 +55,10 @@ MonoNNModule::MonoNNModule(const std::string& hlo_text, const std::string& spec_
   }
 }
 
+MonoNNModule::~MonoNNModule() {
+  if (own_temp_) runtime::coherent_release(dev_.device(), own_temp_);
+}
+
 void MonoNNModule::generate_code() {
   auto mod = hlo::parse_module(hlo_text_);
   module_name_ = mod->name;
@@ -120,12 +124,25 @@ void MonoNNModule::upload_constant(const codegen::ConstantInfo& ci, const std::v
   size_t n = 0;
   void* dst = dev_.global(ci.symbol, &n);
   MONONN_CHECK(static_cast<int64_t>(n) >= ci.bytes, kRuntimeError) << "global " << ci.symbol << " is smaller than its constant";
-  if (ci.transform == graph::ConstantTransform::kTranspose2D) {
+  if (ci.transform == graph::ConstantTransform::kPackMfmaB) {
+    // [K,N] row-major -> [ceil(N/16)][K/32][64][8]: one MFMA B operand per contiguous KiB
     const int es = hlo::dtype_bytes(ci.dtype);
-    const int64_t rows = ci.dims[0], cols = ci.dims[1];
-    std::vector<char> t(payload.size());
-    for (int64_t r = 0; r < rows; ++r)
-      for (int64_t c = 0; c < cols; ++c) std::memcpy(&t[(c * rows + r) * es], &payload[(r * cols + c) * es], es);
+    const int64_t K = ci.dims[0], N = ci.dims[1];
+    const int64_t nt_count = (N + 15) / 16, ksteps = K / 32;
+    MONONN_CHECK(es == 2 && K % 32 == 0, kInternal) << "constant " << ci.hlo_name << " cannot be packed";
+    std::vector<char> t(static_cast<size_t>(ci.device_bytes), 0);
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(payload.data());
+    uint16_t* dstp = reinterpret_cast<uint16_t*>(t.data());
+    for (int64_t nt = 0; nt < nt_count; ++nt)
+      for (int64_t ks = 0; ks < ksteps; ++ks)
+        for (int l = 0; l < 64; ++l) {
+          const int64_t n = nt * 16 + (l & 15);
+          if (n >= N) continue;
+          const int64_t k0 = ks * 32 + (l >> 4) * 8;
+          uint16_t* o = dstp + ((nt * ksteps + ks) * 64 + l) * 8;
+          for (int j = 0; j < 8; ++j) o[j] = src[(k0 + j) * N + n];
+        }
+    MONONN_CHECK(static_cast<int64_t>(n) >= ci.device_bytes, kRuntimeError) << "global " << ci.symbol << " is smaller than its packed constant";
     dev_.upload(dst, t.data(), t.size());
   } else {
     dev_.upload(dst, payload.data(), payload.size());
@@ -199,6 +216,11 @@ void MonoNNModule::load(int device) {
   size_t flag_bytes = 0;
   void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
   dev_.zero(flags, flag_bytes);
+  if (own_temp_) {
+    runtime::coherent_release(device, own_temp_);
+    own_temp_ = nullptr;
+  }
+  if (owns_temp()) own_temp_ = runtime::coherent_alloc(device, static_cast<size_t>(std::max<int64_t>(hip_.temp_bytes, 256)));
   uploaded_.clear();
   for (auto& ci : hip_.constants) {
     if (!ci.literal.empty()) {
@@ -218,11 +240,37 @@ void MonoNNModule::launch(void* const* device_ptrs, size_t n, void* stream) {
   MONONN_CHECK(missing.empty(), kInvalidArgument) << missing.size() << " constants have no payload yet, first: " << missing[0];
   std::vector<void*> vals(device_ptrs, device_ptrs + n);
   std::vector<void*> args(n);
+  prepare_args(vals);
+  for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
+  dev_.launch(grid_, hip_.block, hip_.smem, args.data(), stream);
+}
+
+double MonoNNModule::read_stage_clock(std::vector<unsigned long long>* ticks, int* n_stages, int* grid) {
+  MONONN_CHECK(dev_.loaded(), kInvalidArgument) << "read_stage_clock called before load";
+  MONONN_CHECK(hip_.profiled, kInvalidArgument) << "kernel was built without mononn_hip.profile_stages";
+  size_t bytes = 0;
+  void* src = dev_.global("mononn_stage_clock", &bytes);
+  ticks->resize(bytes / sizeof(unsigned long long));
+  dev_.download(ticks->data(), src, bytes);
+  *n_stages = hip_.num_stages;
+  *grid = hip_.grid;
+  return dev_.wall_clock_ticks_per_us();
+}
+
+void MonoNNModule::prepare_args(std::vector<void*>& vals) const {
+  const size_t n = vals.size();
+  if (owns_temp()) {
+    // Stages hand data to each other through the temp arena without cache maintenance; that only
+    // works in memory no cache keeps, which the module allocates itself.
+    MONONN_CHECK(vals[n - 1] == nullptr, kInvalidArgument)
+        << "this kernel was built with barrier=flags_coherent and uses the module's own coherent temp arena: pass NULL as temp buffer "
+           "(or compile with barrier=flags to bring your own)";
+    vals[n - 1] = own_temp_;
+  }
   for (size_t i = 0; i < n; ++i) {
     MONONN_CHECK(vals[i] != nullptr || (i + 1 == n && hip_.temp_bytes == 0), kInvalidArgument) << "buffer " << i << " is null";
-    args[i] = &vals[i];
+    MONONN_CHECK(reinterpret_cast<uintptr_t>(vals[i]) % 16 == 0, kInvalidArgument) << "buffer " << i << " is not 16-byte aligned";
   }
-  dev_.launch(grid_, hip_.block, hip_.smem, args.data(), stream);
 }
 
 float MonoNNModule::time_kernel(void* const* device_ptrs, size_t n, void* stream, int warmup, int iters, std::vector<float>* each) {
@@ -230,6 +278,7 @@ float MonoNNModule::time_kernel(void* const* device_ptrs, size_t n, void* stream
   MONONN_CHECK(n == num_args(), kInvalidArgument) << "kernel takes " << num_args() << " buffers, got " << n;
   std::vector<void*> vals(device_ptrs, device_ptrs + n);
   std::vector<void*> args(n);
+  prepare_args(vals);
   for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
   return dev_.time_launches(grid_, hip_.block, hip_.smem, args.data(), stream, warmup, iters, each);
 }

@@ -25,6 +25,9 @@ class MonoNNModule {
  public:
   // spec_json may be empty: defaults are derived for every node
   MonoNNModule(const std::string& hlo_text, const std::string& spec_json, const std::string& kernel_name = "");
+  ~MonoNNModule();
+  // true when the kernel relies on the module-owned coherent temp arena (barrier "flags_coherent")
+  bool owns_temp() const { return spec_.hip.barrier == "flags_coherent"; }
 
   void generate_code();                       // parse, run the passes, emit HIP source
   void build_assembly();                      // hipRTC -> code object (needs generate_code)
@@ -56,6 +59,9 @@ class MonoNNModule {
   int smem() const { return hip_.smem; }
   size_t num_args() const { return hip_.param_bytes.size() + hip_.liveout_bytes.size() + 1; }
   std::vector<std::string> missing_constants() const;
+  // Stage clocks of the last launch of a kernel built with mononn_hip.profile_stages: for every
+  // emitted stage and workgroup, [begin, end-of-work] wall-clock ticks.  Returns ticks per microsecond.
+  double read_stage_clock(std::vector<unsigned long long>* ticks, int* n_stages, int* grid);
 
   // ---- dump (TF_MONONN_DUMP_DIR layout, mononn_module_tuner.cc:457-603) ------------------------
   // writes <dir>/<cluster_N>/<context>.json, <context>.hsaco, <context>_src/{headers.h,main.hip}
@@ -65,6 +71,7 @@ class MonoNNModule {
   std::string cluster_dir(const std::string& dump_dir) const;
 
  private:
+  void prepare_args(std::vector<void*>& vals) const;
   void upload_constant(const codegen::ConstantInfo& ci, const std::vector<char>& payload);
   std::string hlo_text_;
   std::string module_name_;
@@ -77,6 +84,7 @@ class MonoNNModule {
   std::string compile_log_;
   runtime::DeviceModule dev_;
   int grid_ = 0;
+  void* own_temp_ = nullptr;     // coherent arena used when the kernel's barrier does no cache maintenance
   std::map<std::string, std::vector<char>> host_constants_;   // canonical name -> payload as given
   std::map<std::string, bool> uploaded_;
 };

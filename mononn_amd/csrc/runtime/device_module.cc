@@ -2,6 +2,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <mutex>
+
 #include "common/status.h"
 
 #define HIP_OK(expr)                                                                                         \
@@ -38,6 +41,42 @@ DeviceProperties query_device(int device) {
   if (colon != std::string::npos) d.arch = d.arch.substr(0, colon);
   d.name = p.name;
   return d;
+}
+
+namespace {
+struct Arena {
+  int device;
+  void* ptr;
+  size_t bytes;
+  bool in_use;
+};
+std::mutex g_arena_mu;
+std::vector<Arena> g_arenas;
+}  // namespace
+
+void* coherent_alloc(int device, size_t bytes) {
+  std::lock_guard<std::mutex> lock(g_arena_mu);
+  bytes = std::max<size_t>((bytes + 4095) / 4096 * 4096, 4096);
+  Arena* best = nullptr;
+  for (auto& a : g_arenas)
+    if (a.device == device && !a.in_use && a.bytes >= bytes && (!best || a.bytes < best->bytes)) best = &a;
+  if (best) {
+    best->in_use = true;
+    return best->ptr;
+  }
+  HIP_OK(hipSetDevice(device));
+  void* p = nullptr;
+  HIP_OK(hipExtMallocWithFlags(&p, bytes, hipDeviceMallocUncached));
+  HIP_OK(hipMemset(p, 0, bytes));
+  HIP_OK(hipDeviceSynchronize());
+  g_arenas.push_back({device, p, bytes, true});
+  return p;
+}
+
+void coherent_release(int device, void* ptr) {
+  std::lock_guard<std::mutex> lock(g_arena_mu);
+  for (auto& a : g_arenas)
+    if (a.device == device && a.ptr == ptr) a.in_use = false;
 }
 
 DeviceModule::~DeviceModule() {
@@ -91,6 +130,18 @@ void DeviceModule::zero(void* dst, size_t bytes) const {
   HIP_OK(hipSetDevice(device_));
   HIP_OK(hipMemset(dst, 0, bytes));
   HIP_OK(hipDeviceSynchronize());
+}
+
+void DeviceModule::download(void* host_dst, const void* src, size_t bytes) const {
+  HIP_OK(hipSetDevice(device_));
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(host_dst, src, bytes, hipMemcpyDeviceToHost));
+}
+
+double DeviceModule::wall_clock_ticks_per_us() const {
+  int khz = 0;
+  HIP_OK(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device_));
+  return khz / 1000.0;
 }
 
 int DeviceModule::max_coresident_blocks(int block, int smem) const {

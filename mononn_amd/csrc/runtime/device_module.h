@@ -26,6 +26,12 @@ struct DeviceProperties {
   std::string name;
 };
 
+// Device memory that no cache level keeps (every access goes to the memory side, so it is coherent
+// across the XCDs of one GPU without cache maintenance).  Arenas are pooled per device and handed
+// back with coherent_release; they are never returned to the driver before the process ends.
+void* coherent_alloc(int device, size_t bytes);
+void coherent_release(int device, void* ptr);
+
 int device_count();                           // 0 when no GPU is visible (never throws)
 DeviceProperties query_device(int device);    // throws Error(kRuntimeError) without a GPU
 
@@ -44,6 +50,8 @@ class DeviceModule {
   void* global(const std::string& symbol, size_t* bytes) const;
   void upload(void* dst, const void* host_src, size_t bytes) const;
   void zero(void* dst, size_t bytes) const;
+  void download(void* host_dst, const void* src, size_t bytes) const;   // synchronises the device first
+  double wall_clock_ticks_per_us() const;
 
   // workgroups of `block` threads and `smem` bytes of LDS that can be resident on the whole device
   int max_coresident_blocks(int block, int smem) const;

@@ -130,6 +130,7 @@ Json GraphSpecification::to_json() const {
   h["gemm_epilogue_fusion"] = hip.gemm_epilogue_fusion;
   h["transpose_constant_b"] = hip.transpose_constant_b;
   h["barrier"] = hip.barrier;
+  h["profile_stages"] = hip.profile_stages;
   j["mononn_hip"] = h;
   return j;
 }
@@ -214,11 +215,12 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
   s.codegen_reject_list = strings_from(j, "codegen_reject_list");
   if (j.contains("mononn_hip")) {
     const Json& h = j.at("mononn_hip");
-    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "barrier"}, "mononn_hip");
+    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "barrier", "profile_stages"}, "mononn_hip");
     s.hip.merge_dependent = getb(h, "merge_dependent", true);
     s.hip.gemm_epilogue_fusion = getb(h, "gemm_epilogue_fusion", true);
     s.hip.transpose_constant_b = getb(h, "transpose_constant_b", true);
-    s.hip.barrier = gets(h, "barrier", "flags");
+    s.hip.barrier = gets(h, "barrier", "flags_coherent");
+    s.hip.profile_stages = getb(h, "profile_stages", false);
   }
   MONONN_CHECK(s.runtime.grid_dim.x >= 1 && s.runtime.grid_dim.y == 1 && s.runtime.grid_dim.z == 1, kSpecError) << "grid must be 1-D";
   MONONN_CHECK(s.runtime.block_dim.x >= 64 && s.runtime.block_dim.x % 64 == 0 && s.runtime.block_dim.x <= 1024 && s.runtime.block_dim.y == 1 && s.runtime.block_dim.z == 1,
