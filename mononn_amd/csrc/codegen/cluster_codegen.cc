@@ -74,8 +74,8 @@ Index leading_index(int var, int64_t extent, const std::vector<int64_t>& dims, c
   return delinearize(LinExpr::variable(var, extent), dims, vars);
 }
 
-void store(CodeBuffer& cb, PointerTable& ptrs, const VarTable& vars, const Instr* out, const Index& idx, const std::string& v) {
-  cb.line(ptrs.output(out) + "[" + linearize(idx, out->shape.dims).str(vars) + "] = " + v + ";");
+void store(const Program& prog, CodeBuffer& cb, PointerTable& ptrs, const VarTable& vars, const Instr* out, const Index& idx, const std::string& v) {
+  cb.line("mononn_dev::st1(" + ptrs.output(out) + " + " + physical_offset(prog, out, idx).str(vars) + ", " + v + ");");
 }
 
 std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs);
@@ -157,7 +157,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       std::vector<std::pair<const Instr*, std::string>> vals;
       for (auto* o : row_outs) vals.emplace_back(o, em.value(em.resolve_output(o), leading_index(row, ROWS, o->shape.dims, vars)));
       cb.open("if (tid == 0)");
-      for (auto& kv : vals) store(cb, ptrs, vars, kv.first, leading_index(row, ROWS, kv.first->shape.dims, vars), kv.second);
+      for (auto& kv : vals) store(prog, cb, ptrs, vars, kv.first, leading_index(row, ROWS, kv.first->shape.dims, vars), kv.second);
       cb.close();
       em.pop_scope();
     };
@@ -200,13 +200,30 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       emit_row_outputs();
       for (int64_t k = 0; k < T; ++k) {
         std::vector<std::string> lines;
-        for (int v = 0; v < V; ++v)
-          for (auto* o : full_outs) {
+        for (auto* o : full_outs) {
+          std::vector<std::string> vals;
+          std::vector<LinExpr> offs;
+          for (int v = 0; v < V; ++v) {
             LinExpr lin = LinExpr::variable(row, ROWS).scaled(R).plus(col_of(k, v));
             Index oi = delinearize(lin, o->shape.dims, vars);
-            std::string val = em.value(em.resolve_output(o), oi);
-            lines.push_back(ptrs.output(o) + "[" + linearize(oi, o->shape.dims).str(vars) + "] = " + val + ";");
+            vals.push_back(em.value(em.resolve_output(o), oi));
+            offs.push_back(physical_offset(prog, o, oi));
           }
+          // one packed store when the V elements are adjacent in memory and the pack is 4/8/16 bytes
+          const int bytes = V * hlo::dtype_bytes(o->shape.dtype);
+          bool adjacent = V > 1 && (bytes == 4 || bytes == 8 || bytes == 16);
+          for (int v = 1; adjacent && v < V; ++v) adjacent = offs[v].equals(offs[0].plus_const(v));
+          if (adjacent) {
+            std::string T = hlo::dtype_ctype(o->shape.dtype);
+            std::string arr = em.fresh("pk");
+            std::string init;
+            for (int v = 0; v < V; ++v) init += (v ? ", " : "") + vals[v];
+            lines.push_back("const " + T + " " + arr + "[" + S(V) + "] = {" + init + "};");
+            lines.push_back("mononn_dev::stN<" + T + ", " + S(V) + ">(" + ptrs.output(o) + " + " + offs[0].str(vars) + ", " + arr + ");");
+          } else {
+            for (int v = 0; v < V; ++v) lines.push_back("mononn_dev::st1(" + ptrs.output(o) + " + " + offs[v].str(vars) + ", " + vals[v] + ");");
+          }
+        }
         if (lines.empty()) continue;
         if (partial[k]) cb.open("if (act" + S(k) + ")");
         for (auto& l : lines) cb.line(l);
@@ -236,7 +253,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
         for (auto* o : full_outs) {
           LinExpr lin = LinExpr::variable(row, ROWS).scaled(R).plus(LinExpr::variable(col, R));
           Index oi = delinearize(lin, o->shape.dims, vars);
-          store(cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
+          store(prog, cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
         }
         em.pop_scope();
         cb.close();
@@ -280,7 +297,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       for (auto* o : groups[gi].second) {
         LinExpr lin = LinExpr::variable(var, NQ).scaled(V).plus_const(v);
         Index oi = delinearize(lin, o->shape.dims, vars);
-        store(cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
+        store(prog, cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
       }
     em.pop_scope();
     cb.close();
@@ -532,13 +549,13 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
       }
       std::string v = em.value(em.resolve_output(out.o), out.idx);
       if (vec4) {
-        LinExpr full = linearize(out.idx, out.o->shape.dims);
-        LinExpr base = linearize(out.idx_base, out.o->shape.dims);
+        LinExpr full = physical_offset(prog, out.o, out.idx);
+        LinExpr base = physical_offset(prog, out.o, out.idx_base);
         out.vector_store = full.equals(base.plus(LinExpr::variable(vr, 4))) && out.o->shape.dtype == DType::kF16;
         if (out.vector_store) cb.line(out.stage + "[r] = " + v + ";");
-        else store(cb, ptrs, vars, out.o, out.idx, v);
+        else store(prog, cb, ptrs, vars, out.o, out.idx, v);
       } else {
-        store(cb, ptrs, vars, out.o, out.idx, v);
+        store(prog, cb, ptrs, vars, out.o, out.idx, v);
       }
     }
   }
@@ -547,9 +564,8 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   if (vec4) {
     for (auto& out : outs)
       if (out.vector_store) {
-        std::string lin = linearize(out.idx_base, out.o->shape.dims).str(vars);
-        cb.line("*reinterpret_cast<half4_t*>(" + ptrs.output(out.o) + " + " + lin + ") = half4_t{" + out.stage + "[0], " + out.stage + "[1], " +
-                out.stage + "[2], " + out.stage + "[3]};");
+        std::string lin = physical_offset(prog, out.o, out.idx_base).str(vars);
+        cb.line("mononn_dev::stN<_Float16, 4>(" + ptrs.output(out.o) + " + " + lin + ", " + out.stage + ");");
       }
   }
 
@@ -596,14 +612,21 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     // multiples of 8 in their unit index; with units dealt round-robin over the 8 XCDs they land on
     // one XCD and share its L2.  tile_n = 8 * (q / tiles_m) + u % 8, tile_m = q % tiles_m, q = u / 8.
     const int64_t tiles_m = (g.M + t.bm - 1) / t.bm, tiles_n = (g.N + t.bn - 1) / t.bn;
-    const int64_t tn_groups = (tiles_n + 7) / 8;
-    const int64_t per_batch = tn_groups * tiles_m * 8;
-    units = g.batch * per_batch;
-    fb.line("const int bidx = unit / " + S(per_batch) + ";");
-    fb.line("const int rem = unit % " + S(per_batch) + ";");
-    fb.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
-    fb.line("const int tile_m = (rem >> 3) % " + S(tiles_m) + ";");
-    if (tiles_n % 8 != 0) fb.line("if (tile_n >= " + S(tiles_n) + ") return;");
+    if (tiles_n % 8 == 0) {
+      const int64_t per_batch = tiles_n * tiles_m;
+      units = g.batch * per_batch;
+      fb.line("const int bidx = unit / " + S(per_batch) + ";");
+      fb.line("const int rem = unit % " + S(per_batch) + ";");
+      fb.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
+      fb.line("const int tile_m = (rem >> 3) % " + S(tiles_m) + ";");
+    } else {
+      const int64_t per_batch = tiles_n * tiles_m;
+      units = g.batch * per_batch;
+      fb.line("const int bidx = unit / " + S(per_batch) + ";");
+      fb.line("const int rem = unit % " + S(per_batch) + ";");
+      fb.line("const int tile_n = rem / " + S(tiles_m) + ";");
+      fb.line("const int tile_m = rem % " + S(tiles_m) + ";");
+    }
     std::ostringstream call;
     call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << g.K << ", "
          << (g.b_packed ? "true" : "false") << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * "

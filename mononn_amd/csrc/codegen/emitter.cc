@@ -45,6 +45,18 @@ std::string PointerTable::output(const Instr* root) {
   return entries.back().name;
 }
 
+LinExpr physical_offset(const graph::Program& prog, const Instr* root, const Index& idx) {
+  auto it = prog.physical_perm.find(root);
+  if (it == prog.physical_perm.end()) return linearize(idx, root->shape.dims);
+  Index pi;
+  std::vector<int64_t> pd;
+  for (int d : it->second) {
+    pi.push_back(idx[d]);
+    pd.push_back(root->shape.dims[d]);
+  }
+  return linearize(pi, pd);
+}
+
 // ------------------------------------------------------------------------------------------
 Emitter::Emitter(const graph::Program& prog, const std::vector<const Instr*>& members, CodeBuffer& out,
                  VarTable& vars, PointerTable& ptrs)
@@ -193,7 +205,7 @@ std::string Emitter::value(const Instr* ins, const Index& idx) {
 }
 
 std::string Emitter::load(const Instr* root, const Index& idx) {
-  LinExpr lin = linearize(idx, root->shape.dims);
+  LinExpr lin = physical_offset(prog_, root, idx);
   std::string ref = ptrs_.input(root) + "[" + lin.str(vars_) + "]";
   if (lin.opaques().empty()) simple_loads_.push_back(ref);
   return def(root->shape.dtype, ref);

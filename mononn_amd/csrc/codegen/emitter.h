@@ -51,6 +51,9 @@ struct PointerTable {
   std::string output(const hlo::Instr* root);
 };
 
+// element offset of `idx` inside the buffer of storage root `root`, honouring a permuted physical layout
+LinExpr physical_offset(const graph::Program& prog, const hlo::Instr* root, const Index& idx);
+
 class Emitter {
  public:
   Emitter(const graph::Program& prog, const std::vector<const hlo::Instr*>& members, CodeBuffer& out,

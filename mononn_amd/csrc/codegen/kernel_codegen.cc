@@ -21,6 +21,8 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.merge_dependent = s.hip.merge_dependent;
   o.fuse_gemm_epilogue = s.hip.gemm_epilogue_fusion;
   o.transpose_constant_b = s.hip.transpose_constant_b;
+  o.assign_operand_layouts = s.hip.assign_operand_layouts;
+  o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
   for (auto& p : env::disabled_passes()) o.disabled_passes.insert(p);
   return o;
 }
@@ -195,20 +197,36 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   MONONN_CHECK(smem <= spec.device.max_configurable_smem_size, kResourceExhausted)
       << "kernel needs " << smem << " bytes of LDS, device offers " << spec.device.max_configurable_smem_size;
 
-  std::ostringstream src;
-  src << "// generated by mononn-hip for " << spec.device.cuda_arch << "; kernel " << kernel_name << "\n";
-  if (spec.hip.barrier == "flags_allfence") src << "#define MONONN_BARRIER_FENCE 1\n";
-  else if (spec.hip.barrier == "flags_coherent") src << "#define MONONN_BARRIER_FENCE 2\n";
+  // The translation unit is kept in three parts so that the tuner can put many candidate kernels of
+  // one node class into a single hipRTC compilation: preamble (defines + include), global
+  // declarations (shared by all candidates), body (node functions + kernel).
+  std::ostringstream pre, glob, src;
+  pre << "// generated by mononn-hip for " << spec.device.cuda_arch << "\n";
+  if (spec.hip.barrier == "flags_allfence") pre << "#define MONONN_BARRIER_FENCE 1\n";
+  else if (spec.hip.barrier == "flags_coherent") pre << "#define MONONN_BARRIER_FENCE 2\n#define MONONN_COHERENT_STORES 1\n";
   else MONONN_CHECK(spec.hip.barrier == "flags", kSpecError) << "unknown barrier flavour '" << spec.hip.barrier << "'";
-  src << "#include \"headers.h\"\n\n";
-  for (auto& c : hp.constants)
-    src << "__device__ __attribute__((aligned(256))) unsigned char " << c.symbol << "[" << std::max<int64_t>(c.device_bytes, 1) << "];\n";
-  src << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];\n";
+  pre << "#include \"headers.h\"\n\n";
+  for (auto& c : hp.constants) {
+    std::ostringstream d;
+    d << "__device__ __attribute__((aligned(256))) unsigned char " << c.symbol << "[" << std::max<int64_t>(c.device_bytes, 1) << "];";
+    hp.global_decls.push_back(d.str());
+  }
+  {
+    std::ostringstream d;
+    d << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];";
+    hp.global_decls.push_back(d.str());
+  }
   hp.profiled = spec.hip.profile_stages;
   hp.num_stages = static_cast<int>(by_stage.size());
-  if (hp.profiled) src << "__device__ unsigned long long mononn_stage_clock[" << std::max<size_t>(by_stage.size(), 1) * hp.grid * 2 << "];\n";
-  src << "\n";
-  for (auto& g : globals) src << g << "\n";
+  if (hp.profiled) {
+    // sized for the deepest kernel the barrier supports so that candidates of one class can share it
+    std::ostringstream d;
+    d << "__device__ unsigned long long mononn_stage_clock[" << std::max<size_t>(by_stage.size(), 1) * hp.grid * 2 << "];";
+    hp.global_decls.push_back(d.str());
+  }
+  for (auto& g : globals) hp.global_decls.push_back(g);
+  for (auto& g : hp.global_decls) glob << g << "\n";
+  glob << "\n";
   for (auto& d : fn_defs) src << d << "\n";
 
   src << "extern \"C\" __launch_bounds__(" << ls.block_size << ") __global__ void " << kernel_name << "(";
@@ -249,8 +267,10 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     ++stage_ordinal;
   }
   src << "}\n";
+  hp.preamble = pre.str();
+  hp.body = src.str();
   hp.files["headers.h"] = device::kPreludeText;
-  hp.files["main.hip"] = src.str();
+  hp.files["main.hip"] = hp.preamble + glob.str() + hp.body;
   return hp;
 }
 

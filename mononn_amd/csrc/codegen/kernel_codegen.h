@@ -42,6 +42,9 @@ struct NodeReport {
 struct HipProgram {
   std::string kernel_name;
   std::map<std::string, std::string> files;   // "headers.h" (device runtime) and "main.hip"
+  // main.hip = preamble + global_decls + body; kept apart for multi-candidate translation units
+  std::string preamble, body;
+  std::vector<std::string> global_decls;
   std::vector<int64_t> param_bytes, liveout_bytes;
   int64_t temp_bytes = 0;
   std::vector<ConstantInfo> constants;

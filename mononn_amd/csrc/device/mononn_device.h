@@ -14,6 +14,7 @@
 #pragma once
 
 // hipRTC provides no <cstdint>; generated code uses these names for HLO integer types
+#if defined(__HIPCC_RTC__)
 typedef signed char int8_t;
 typedef unsigned char uint8_t;
 typedef short int16_t;
@@ -22,6 +23,9 @@ typedef int int32_t;
 typedef unsigned int uint32_t;
 typedef long long int64_t;
 typedef unsigned long long uint64_t;
+#else
+#include <cstdint>
+#endif
 
 typedef _Float16 half_t;
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -33,6 +37,9 @@ typedef int int4_t __attribute__((ext_vector_type(4)));
 
 #ifndef MONONN_BARRIER_FENCE
 #define MONONN_BARRIER_FENCE 0
+#endif
+#ifndef MONONN_COHERENT_STORES
+#define MONONN_COHERENT_STORES 0
 #endif
 
 namespace mononn_dev {
@@ -59,7 +66,7 @@ struct GridBarrier {
   // MONONN_BARRIER_FENCE: 0 = one thread per workgroup performs the release / acquire cache
   // maintenance (an agent-scope acquire invalidates the XCD's whole L2, so issuing it from every
   // wave multiplies that cost by the number of resident waves); 1 = every thread fences;
-  // 2 = no cache maintenance at all (only valid when inter-stage data bypasses the caches).
+  // 2 = no cache maintenance at all (valid with MONONN_COHERENT_STORES and a write-once temp arena).
   __device__ __forceinline__ void sync() {
     __syncthreads();
     epoch += 1;
@@ -92,6 +99,61 @@ struct GridBarrier {
     __syncthreads();
   }
 };
+
+// ---------------------------------------------------------------------------------------------
+// stores of data that another workgroup reads in a later stage
+// ---------------------------------------------------------------------------------------------
+// The XCDs of one GPU do not keep their L2s coherent with each other.  Instead of flushing and
+// invalidating caches at every grid barrier, stage outputs are written with agent-scope (write-
+// through) stores: the data is at the memory side when the store retires, no L2 keeps a dirty copy.
+// Together with the rule that an address of the temp arena is written at most once per launch, a
+// reader can never find a stale line: nothing can have cached the line before its only write, and
+// the launch boundary invalidates what earlier launches left behind.  Readers use plain cached loads.
+#if MONONN_COHERENT_STORES
+template <class T>
+__device__ __forceinline__ void st1(T* p, T v) {
+  if constexpr (sizeof(T) == 1) {
+    unsigned char b;
+    __builtin_memcpy(&b, &v, 1);
+    __hip_atomic_store(reinterpret_cast<unsigned char*>(p), b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else if constexpr (sizeof(T) == 2) {
+    unsigned short b;
+    __builtin_memcpy(&b, &v, 2);
+    __hip_atomic_store(reinterpret_cast<unsigned short*>(p), b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else if constexpr (sizeof(T) == 4) {
+    unsigned b;
+    __builtin_memcpy(&b, &v, 4);
+    __hip_atomic_store(reinterpret_cast<unsigned*>(p), b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    unsigned long long b;
+    __builtin_memcpy(&b, &v, 8);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+#else
+template <class T>
+__device__ __forceinline__ void st1(T* p, T v) { *p = v; }
+#endif
+// N consecutive elements starting at an address aligned to N * sizeof(T) (N * sizeof(T) in {4, 8, 16})
+template <class T, int N>
+__device__ __forceinline__ void stN(T* p, const T (&v)[N]) {
+  constexpr int BYTES = N * (int)sizeof(T);
+  static_assert(BYTES == 4 || BYTES == 8 || BYTES == 16, "unsupported packed store");
+  if constexpr (BYTES == 4) {
+    unsigned b;
+    __builtin_memcpy(&b, v, 4);
+    st1(reinterpret_cast<unsigned*>(p), b);
+  } else if constexpr (BYTES == 8) {
+    unsigned long long b;
+    __builtin_memcpy(&b, v, 8);
+    st1(reinterpret_cast<unsigned long long*>(p), b);
+  } else {
+    unsigned long long b[2];
+    __builtin_memcpy(b, v, 16);
+    st1(reinterpret_cast<unsigned long long*>(p), b[0]);
+    st1(reinterpret_cast<unsigned long long*>(p) + 1, b[1]);
+  }
+}
 
 // ---------------------------------------------------------------------------------------------
 // reductions (all lanes / all threads receive the result)

@@ -341,6 +341,42 @@ struct Builder {
     }
   }
 
+  // LayoutAssignment: a right-hand GEMM operand [.., K, N] that this kernel produces itself (and that
+  // nothing but such GEMMs reads) is stored [.., N, K]; its producer writes through the permutation.
+  void assign_operand_layouts() {
+    if (!opt.assign_operand_layouts || !enabled("OperandLayoutPass")) return;
+    for (auto& n : p.nodes) {
+      if (n.kind != NodeKind::kGemm || n.gemm.b_k_contig || n.gemm.b_packed || !n.gemm.a_k_contig || n.gemm.K % 32 != 0) continue;
+      const Instr* g = n.members[0];
+      const Instr* root = p.storage_root(g->operands[1]);
+      if (!p.producer.count(root)) continue;                         // parameter / constant
+      if (root->shape.dims != g->operands[1]->shape.dims) continue;   // reached through a reshaping alias
+      bool ok = true;
+      std::function<void(const Instr*)> scan = [&](const Instr* v) {
+        for (auto* u : v->users) {
+          if (is_alias_op(u)) { ok = false; continue; }
+          bool as_b = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands[1] == v && u->operands[0] != v &&
+                      (u->operands.size() < 3 || u->operands[2] != v) && u->gemm.rhs_contracting == g->gemm.rhs_contracting;
+          if (!as_b) ok = false;
+        }
+      };
+      scan(root);
+      for (auto* lo : p.live_outs)
+        if (lo == root) ok = false;
+      if (!ok) continue;
+      int r = root->shape.rank();
+      std::vector<int> perm(r);
+      for (int i = 0; i < r; ++i) perm[i] = i;
+      std::swap(perm[r - 1], perm[r - 2]);
+      p.physical_perm[root] = perm;
+    }
+    for (auto& n : p.nodes) {
+      if (n.kind != NodeKind::kGemm) continue;
+      const Instr* root = p.storage_root(n.members[0]->operands[1]);
+      if (p.physical_perm.count(root)) n.gemm.b_k_contig = true;
+    }
+  }
+
   void assign_buffers() {
     const hlo::Computation* e = p.module->entry;
     for (auto* prm : e->params) {
@@ -400,7 +436,7 @@ struct Builder {
       Buffer& b = p.buffers[v];
       int64_t need = (b.bytes + 255) / 256 * 256;
       int best = -1;
-      for (size_t s = 0; s < slots.size(); ++s)
+      for (size_t s = 0; opt.reuse_temp_slots && s < slots.size(); ++s)
         if (slots[s].free_from <= b.def_stage && slots[s].bytes >= need && (best < 0 || slots[s].bytes < slots[best].bytes)) best = static_cast<int>(s);
       if (best >= 0) {
         b.offset = slots[best].offset;
@@ -426,6 +462,7 @@ std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, cons
   if (opt.fuse_gemm_epilogue && b.enabled("GemmEpilogueFusionPass")) b.fuse_gemm_epilogues();
   b.finalize();
   b.decide_constant_layouts();
+  b.assign_operand_layouts();
   for (auto& n : prog->nodes)
     if (n.kind == NodeKind::kCluster) codegen::classify_cluster(*prog, n);
   b.assign_buffers();

@@ -72,6 +72,9 @@ struct Program {
   std::vector<const hlo::Instr*> parameters;                       // entry parameters in order
   std::vector<const hlo::Instr*> constants;                        // non-scalar entry constants (device buffers)
   std::map<const hlo::Instr*, ConstantTransform> constant_transform;
+  // storage roots kept in a permuted physical order: physical dim i = logical dim perm[i]
+  // (right-hand GEMM operands produced inside the kernel are stored with k minor-most)
+  std::map<const hlo::Instr*, std::vector<int>> physical_perm;
   std::vector<const hlo::Instr*> live_outs;                        // storage roots, root-tuple order
   std::map<const hlo::Instr*, int> producer;                       // storage root -> node id
   int num_stages = 0;
@@ -87,6 +90,8 @@ struct BuildOptions {
   bool merge_dependent = true;          // glue producer/consumer clusters that share a row space
   bool fuse_gemm_epilogue = true;       // element-wise consumers of a GEMM run in its epilogue
   bool transpose_constant_b = true;     // store constant [K,N] GEMM operands in MFMA fragment order
+  bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
+  bool reuse_temp_slots = true;         // false: every temp value gets its own address (written once per launch)
   std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)
 };
 

@@ -259,14 +259,6 @@ double MonoNNModule::read_stage_clock(std::vector<unsigned long long>* ticks, in
 
 void MonoNNModule::prepare_args(std::vector<void*>& vals) const {
   const size_t n = vals.size();
-  if (owns_temp()) {
-    // Stages hand data to each other through the temp arena without cache maintenance; that only
-    // works in memory no cache keeps, which the module allocates itself.
-    MONONN_CHECK(vals[n - 1] == nullptr, kInvalidArgument)
-        << "this kernel was built with barrier=flags_coherent and uses the module's own coherent temp arena: pass NULL as temp buffer "
-           "(or compile with barrier=flags to bring your own)";
-    vals[n - 1] = own_temp_;
-  }
   for (size_t i = 0; i < n; ++i) {
     MONONN_CHECK(vals[i] != nullptr || (i + 1 == n && hip_.temp_bytes == 0), kInvalidArgument) << "buffer " << i << " is null";
     MONONN_CHECK(reinterpret_cast<uintptr_t>(vals[i]) % 16 == 0, kInvalidArgument) << "buffer " << i << " is not 16-byte aligned";

@@ -26,8 +26,7 @@ class MonoNNModule {
   // spec_json may be empty: defaults are derived for every node
   MonoNNModule(const std::string& hlo_text, const std::string& spec_json, const std::string& kernel_name = "");
   ~MonoNNModule();
-  // true when the kernel relies on the module-owned coherent temp arena (barrier "flags_coherent")
-  bool owns_temp() const { return spec_.hip.barrier == "flags_coherent"; }
+  bool owns_temp() const { return false; }   // the caller always brings the temp buffer (reference contract)
 
   void generate_code();                       // parse, run the passes, emit HIP source
   void build_assembly();                      // hipRTC -> code object (needs generate_code)

@@ -111,6 +111,14 @@ void DeviceModule::load(int device, const std::vector<char>& code_object, const 
   compute_units_ = props.compute_units;
 }
 
+void DeviceModule::use_kernel(const std::string& kernel_name) {
+  MONONN_CHECK(module_ != nullptr, kRuntimeError) << "module is not loaded";
+  hipFunction_t f;
+  hipError_t e = hipModuleGetFunction(&f, module_, kernel_name.c_str());
+  if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "kernel '" << kernel_name << "' not found in the code object: " << hipGetErrorString(e);
+  function_ = f;
+}
+
 void* DeviceModule::global(const std::string& symbol, size_t* bytes) const {
   MONONN_CHECK(module_ != nullptr, kRuntimeError) << "module is not loaded";
   hipDeviceptr_t p = nullptr;

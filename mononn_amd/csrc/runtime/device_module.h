@@ -44,6 +44,7 @@ class DeviceModule {
 
   void load(int device, const std::vector<char>& code_object, const std::string& kernel_name);
   bool loaded() const { return module_ != nullptr; }
+  void use_kernel(const std::string& kernel_name);   // switch to another kernel of the loaded code object
   int device() const { return device_; }
 
   // address and size of a module global

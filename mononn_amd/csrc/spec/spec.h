@@ -68,9 +68,11 @@ struct HipOptions {       // "mononn_hip" section
   bool merge_dependent = true;
   bool gemm_epilogue_fusion = true;
   bool transpose_constant_b = true;
-  // "flags_coherent": fence-free flag barrier, stages exchange data through a module-owned uncached
-  // arena; "flags": same barrier with agent-scope release/acquire, caller-provided temp buffer;
-  // "flags_allfence": every thread fences (measurement only)
+  bool assign_operand_layouts = true;
+  // "flags_coherent": fence-free flag barrier; stage outputs are written with agent-scope write-through
+  // stores to temp addresses that are used once per launch, readers use cached loads.
+  // "flags": the same barrier with agent-scope release/acquire (L2 write-back + invalidate) around it,
+  // plain stores, temp slots re-used.  "flags_allfence": every thread fences (measurement only).
   std::string barrier = "flags_coherent";
   bool profile_stages = false;   // per-stage wall-clock stamps (performance_report.csv equivalent)
 };

@@ -1,13 +1,405 @@
 #include "tuner/tuner.h"
 
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <set>
+#include <sstream>
+#include <thread>
+
+#include "codegen/cluster_codegen.h"
+#include "common/env.h"
 #include "common/status.h"
+#include "runtime/device_module.h"
+#include "runtime/rtc.h"
 
 namespace mononn {
 namespace tuner {
 
-std::unique_ptr<module::MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) {
-  (void)params;
-  MONONN_FAIL(kUnsupported) << "tuner not built yet";
+using module::MonoNNModule;
+using spec::GraphSpecification;
+
+namespace {
+
+// Worker pool for candidate compilation (reference: CompilationThreadpool, size from
+// TF_MONONN_THREADPOOL_SIZE or the hardware concurrency, compilation_threadpool.cc:35-39).
+template <class F>
+void parallel_for(size_t n, int threads, F&& f) {
+  std::atomic<size_t> next{0};
+  std::vector<std::thread> pool;
+  threads = std::max(1, std::min<int>(threads, static_cast<int>(n)));
+  for (int t = 0; t < threads; ++t)
+    pool.emplace_back([&] {
+      for (;;) {
+        size_t i = next.fetch_add(1);
+        if (i >= n) return;
+        f(i);
+      }
+    });
+  for (auto& th : pool) th.join();
+}
+
+struct DeviceBuffers {
+  int device;
+  std::vector<void*> ptrs;   // params, live-outs, temp (may be null)
+  ~DeviceBuffers() {
+    for (auto* p : ptrs)
+      if (p) (void)hipFree(p);
+  }
+};
+
+void alloc_zero(void** p, size_t bytes) {
+  bytes = std::max<size_t>(bytes, 256);
+  hipError_t e = hipMalloc(p, bytes);
+  if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipMalloc(" << bytes << "): " << hipGetErrorString(e);
+  e = hipMemset(*p, 0, bytes);
+  if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipMemset: " << hipGetErrorString(e);
+}
+
+struct GemmCandidate {
+  codegen::GemmTuning t;
+};
+
+// Every wave arrangement x per-wave fragment tile that the code generator accepts for this problem
+// (reference: all CUTLASS tiles that fit, tuning_space_generator.cc:139-307).
+std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int waves, int budget) {
+  std::vector<codegen::GemmTuning> out;
+  if (!codegen::gemm_uses_mfma(g)) return out;
+  const int ksteps = static_cast<int>(g.K / 32);
+  for (int wk = 1; wk <= waves; wk *= 2) {
+    if (wk > ksteps) break;
+    for (int wm = 1; wm * wk <= waves; wm *= 2) {
+      int wn = waves / (wk * wm);
+      if (wm * wn * wk != waves) continue;
+      for (int tm : {1, 2, 3, 4, 6, 8})
+        for (int tn : {1, 2, 3, 4, 6, 8}) {
+          if (tm * tn > 16) continue;
+          codegen::GemmTuning t;
+          t.wm = wm;
+          t.wn = wn;
+          t.wk = wk;
+          t.bm = wm * tm * 16;
+          t.bn = wn * tn * 16;
+          // tiles much larger than the problem only add idle lanes
+          if (t.bm >= 2 * g.M + 16 && tm * wm > 1) continue;
+          if (t.bn >= 2 * g.N + 16 && tn * wn > 1) continue;
+          // LDS for the cross-wave reduction
+          if (wk > 1 && waves * tm * tn * 1024 > 64 * 1024) continue;
+          out.push_back(t);
+        }
+    }
+  }
+  if (budget >= 1) {
+    // faster tuning: keep the shapes with a balanced per-wave tile
+    std::vector<codegen::GemmTuning> kept;
+    for (auto& t : out) {
+      int tm = t.bm / t.wm / 16, tn = t.bn / t.wn / 16;
+      if (tm * tn >= 2 && tm * tn <= 8 && (budget < 2 || (tm <= 2 && tn <= 2))) kept.push_back(t);
+    }
+    out = kept;
+  }
+  return out;
+}
+
+struct ClassInfo {
+  std::string function;                 // de-duplicated device function name under the default spec
+  std::vector<std::string> nodes;       // node names sharing it
+  std::string kind;                     // gemm | cluster_reduce | cluster_elewise
+  const graph::Node* sample = nullptr;
+};
+
+struct Trial {
+  std::string label;
+  GraphSpecification spec;
+  std::unique_ptr<MonoNNModule> mod;
+  std::string error;
+  double us = -1;
+};
+
+void apply_gemm(GraphSpecification& s, const std::string& node, const codegen::GemmTuning& t, int64_t K) {
+  spec::GemmSpec& g = s.gemm_spec_list[node];
+  g.tb_m = t.bm;
+  g.tb_n = t.bn;
+  g.wave_m = t.wm;
+  g.wave_n = t.wn;
+  g.wave_k = t.wk;
+  g.warp_m = t.bm / t.wm;
+  g.warp_n = t.bn / t.wn;
+  g.warp_k = static_cast<int>(K / t.wk);
+}
+
+double time_module(MonoNNModule& m, int device, DeviceBuffers& bufs, int warmup, int iters) {
+  m.load(device);
+  std::vector<void*> ptrs = bufs.ptrs;
+  float ms = m.time_kernel(ptrs.data(), ptrs.size(), nullptr, warmup, iters);
+  return ms * 1000.0;
+}
+
+// Mean time of one stage (first workgroup in -> last workgroup done) of a kernel built with stage
+// clocks, averaged over its stages and over `iters` launches.  Launch overhead and barrier time are
+// not part of the figure, so candidates of one node class compare on the work itself.
+double stage_time(MonoNNModule& m, int device, DeviceBuffers& bufs, int warmup, int iters) {
+  m.load(device);
+  std::vector<void*> ptrs = bufs.ptrs;
+  for (int i = 0; i < warmup; ++i) m.launch(ptrs.data(), ptrs.size(), nullptr);
+  double total = 0;
+  int count = 0;
+  std::vector<unsigned long long> t;
+  for (int i = 0; i < iters; ++i) {
+    m.launch(ptrs.data(), ptrs.size(), nullptr);
+    int ns = 0, grid = 0;
+    double tpu = m.read_stage_clock(&t, &ns, &grid);
+    for (int s = 0; s < ns; ++s) {
+      unsigned long long lo = ~0ull, hi = 0;
+      for (int w = 0; w < grid; ++w) {
+        lo = std::min(lo, t[(static_cast<size_t>(s) * grid + w) * 2]);
+        hi = std::max(hi, t[(static_cast<size_t>(s) * grid + w) * 2 + 1]);
+      }
+      total += static_cast<double>(hi - lo) / tpu;
+      ++count;
+    }
+  }
+  return count ? total / count : -1;
+}
+
+}  // namespace
+
+std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) {
+  runtime::DeviceProperties props = runtime::query_device(params.device);
+  MONONN_CHECK(props.wave_size == 64, kRuntimeError) << "device " << params.device << " does not run 64-wide wavefronts";
+  const int threads = env::threadpool_size();
+  const int budget = std::max(params.budget, env::is_true("MONONN_FASTEST_TUNING") ? 2 : (env::is_true("MONONN_FASTER_TUNING") ? 1 : 0));
+  std::ostringstream log, report;
+  log << "Tuning result for each thread grid setting:\n";
+
+  // launch contexts: workgroups per CU x threads per workgroup
+  // (reference: {1,2,3} blocks per SM x {128,256} threads, tuning_space_generator.cc:65-66)
+  struct Ctx {
+    int per_cu, block;
+  };
+  std::vector<Ctx> contexts = {{1, 256}, {1, 512}};
+  if (budget == 0) contexts.push_back({2, 256});
+  if (budget >= 2) contexts = {{1, 256}};
+
+  std::unique_ptr<MonoNNModule> best;
+  double best_us = -1;
+  DeviceBuffers bufs{params.device, {}};
+
+  for (auto& cx : contexts) {
+    GraphSpecification base;
+    base.device.sm_count = props.compute_units;
+    base.device.cuda_arch = props.arch;
+    base.device.max_configurable_smem_size = std::max(props.max_lds_per_block, 65536);
+    base.runtime.grid_dim.x = props.compute_units * cx.per_cu;
+    base.runtime.block_dim.x = cx.block;
+    const std::string ctx_str = base.context_string();
+
+    // default module of this context: classes of identical node functions
+    MonoNNModule def(params.hlo_text, base.to_json().dump(0), params.kernel_name);
+    def.generate_code();
+    GraphSpecification filled = def.tuning_spec();
+    if (bufs.ptrs.empty()) {
+      hipError_t e = hipSetDevice(params.device);
+      if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipSetDevice: " << hipGetErrorString(e);
+      auto& hp = def.hip_program();
+      for (auto b : hp.param_bytes) {
+        bufs.ptrs.push_back(nullptr);
+        alloc_zero(&bufs.ptrs.back(), static_cast<size_t>(b));
+      }
+      for (auto b : hp.liveout_bytes) {
+        bufs.ptrs.push_back(nullptr);
+        alloc_zero(&bufs.ptrs.back(), static_cast<size_t>(b));
+      }
+      bufs.ptrs.push_back(nullptr);
+      alloc_zero(&bufs.ptrs.back(), static_cast<size_t>(hp.temp_bytes));
+    }
+    std::map<std::string, ClassInfo> classes;
+    for (auto& r : def.hip_program().nodes) {
+      ClassInfo& c = classes[r.function];
+      c.function = r.function;
+      c.kind = r.kind;
+      c.nodes.push_back(r.name);
+    }
+    for (auto& n : def.program().nodes)
+      for (auto& kv : classes)
+        if (!kv.second.sample && kv.second.nodes[0] == n.name) kv.second.sample = &n;
+
+    // ---- candidates of every class ------------------------------------------------------------
+    std::vector<Trial> trials;
+    std::map<std::string, std::vector<size_t>> trials_of_class;
+    for (auto& kv : classes) {
+      ClassInfo& c = kv.second;
+      auto add = [&](const std::string& label, GraphSpecification s) {
+        s.codegen_allow_list = c.nodes;
+        s.hip.profile_stages = true;
+        Trial t;
+        t.label = label;
+        t.spec = std::move(s);
+        trials_of_class[c.function].push_back(trials.size());
+        trials.push_back(std::move(t));
+      };
+      add("default", filled);
+      if (c.kind == "gemm") {
+        for (auto& t : gemm_candidates(c.sample->gemm, cx.block / 64, budget)) {
+          GraphSpecification s = filled;
+          for (auto& n : c.nodes) apply_gemm(s, n, t, c.sample->gemm.K);
+          char lbl[96];
+          std::snprintf(lbl, sizeof lbl, "tile%dx%d_waves%dx%dx%d", t.bm, t.bn, t.wm, t.wn, t.wk);
+          add(lbl, s);
+        }
+      } else if (c.kind == "cluster_reduce") {
+        for (int tier : {1, 2})
+          for (int ilp : {1, 2, 4, 8}) {
+            if (budget >= 2 && ilp > 2) continue;
+            GraphSpecification s = filled;
+            for (auto& n : c.nodes) {
+              s.cluster_reduce_spec[n].locality_tier = tier;
+              s.cluster_reduce_spec[n].ilp_factor = ilp;
+            }
+            add("tier" + std::to_string(tier) + "_ilp" + std::to_string(ilp), s);
+          }
+      } else {
+        for (int ilp : {2, 4, 8}) {
+          GraphSpecification s = filled;
+          for (auto& n : c.nodes) s.cluster_elewise_spec[n].ilp_factor = ilp;
+          add("ilp" + std::to_string(ilp), s);
+        }
+      }
+    }
+    // ---- code generation in the pool; one hipRTC compilation and one module load per class -----------
+    parallel_for(trials.size(), threads, [&](size_t i) {
+      Trial& t = trials[i];
+      try {
+        t.mod = std::make_unique<MonoNNModule>(params.hlo_text, t.spec.to_json().dump(0), "mononn_tune_" + std::to_string(i));
+        t.mod->generate_code();
+      } catch (const Error& e) {
+        t.error = e.what();
+        t.mod.reset();
+      }
+    });
+    GraphSpecification stitched = filled;
+    const bool verbose = env::is_true("TF_MONONN_ENABLE_WORKER_THRAED_LOGGING") || env::is_true("MONONN_TUNER_VERBOSE");
+    for (auto& kv : classes) {
+      ClassInfo& c = kv.second;
+      std::vector<size_t> live;
+      for (size_t i : trials_of_class[c.function])
+        if (trials[i].mod) live.push_back(i);
+      if (live.empty()) continue;
+      // translation unit: shared preamble + union of the global declarations + one namespace per candidate
+      std::map<std::string, std::string> files;
+      std::string tu = trials[live[0]].mod->hip_program().preamble;
+      std::set<std::string> decls;
+      for (size_t i : live)
+        for (auto& d : trials[i].mod->hip_program().global_decls)
+          if (decls.insert(d).second) tu += d + "\n";
+      for (size_t i : live) tu += "namespace cand_" + std::to_string(i) + " {\n" + trials[i].mod->hip_program().body + "}\n";
+      files["headers.h"] = trials[live[0]].mod->hip_program().files.at("headers.h");
+      files["main.hip"] = tu;
+      double best_class = -1;
+      size_t best_i = live[0];
+      try {
+        auto res = runtime::compile_hip(files, "main.hip", props.arch);
+        runtime::DeviceModule dm;
+        dm.load(params.device, res.code_object, trials[live[0]].mod->kernel_name());
+        size_t fb = 0;
+        dm.zero(dm.global("mononn_barrier_flags", &fb), fb);
+        for (size_t i : live) {
+          Trial& t = trials[i];
+          const codegen::HipProgram& hp = t.mod->hip_program();
+          try {
+            dm.use_kernel(t.mod->kernel_name());
+            dm.set_dynamic_smem(hp.smem);
+            if (dm.max_coresident_blocks(hp.block, hp.smem) < hp.grid) {
+              t.error = "grid exceeds the co-resident capacity";
+              continue;
+            }
+            std::vector<void*> vals = bufs.ptrs, args(vals.size());
+            for (size_t a = 0; a < vals.size(); ++a) args[a] = &vals[a];
+            const int warm = 2, iters = budget >= 1 ? 4 : 8;
+            size_t cb = 0;
+            void* clk = dm.global("mononn_stage_clock", &cb);
+            std::vector<unsigned long long> ticks(cb / sizeof(unsigned long long));
+            const double tpu = dm.wall_clock_ticks_per_us();
+            double total = 0;
+            int count = 0;
+            for (int it = 0; it < warm + iters; ++it) {
+              dm.launch(hp.grid, hp.block, hp.smem, args.data(), nullptr);
+              if (it < warm) continue;
+              dm.download(ticks.data(), clk, cb);
+              for (int st = 0; st < hp.num_stages; ++st) {
+                unsigned long long lo = ~0ull, hi = 0;
+                for (int w = 0; w < hp.grid; ++w) {
+                  lo = std::min(lo, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2]);
+                  hi = std::max(hi, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2 + 1]);
+                }
+                total += static_cast<double>(hi - lo) / tpu;
+                ++count;
+              }
+            }
+            t.us = count ? total / count : -1;
+          } catch (const Error& e) {
+            t.error = e.what();
+            t.us = -1;
+          }
+          if (t.us > 0 && (best_class < 0 || t.us < best_class)) {
+            best_class = t.us;
+            best_i = i;
+          }
+        }
+      } catch (const Error& e) {
+        log << "  [" << ctx_str << "] class of " << c.nodes[0] << " failed: " << e.what() << "\n";
+      }
+      for (size_t i : trials_of_class[c.function]) trials[i].mod.reset();
+      if (verbose) std::fprintf(stderr, "[mononn tuner] %s %s x%zu: %zu candidates, best %.2f us\n", ctx_str.c_str(), c.kind.c_str(), c.nodes.size(), live.size(), best_class);
+      if (best_class < 0) continue;
+      const GraphSpecification& w = trials[best_i].spec;
+      for (auto& n : c.nodes) {
+        if (c.kind == "gemm") stitched.gemm_spec_list[n] = w.gemm_spec_list.at(n);
+        else if (c.kind == "cluster_reduce") stitched.cluster_reduce_spec[n] = w.cluster_reduce_spec.at(n);
+        else stitched.cluster_elewise_spec[n] = w.cluster_elewise_spec.at(n);
+        report << ctx_str << "," << n << "," << best_class << "\n";
+      }
+      log << "  [" << ctx_str << "] " << c.kind << " x" << c.nodes.size() << " (" << c.nodes[0] << "): best " << trials[best_i].label << " "
+          << best_class << " us per stage;";
+      for (size_t i : trials_of_class[c.function])
+        if (trials[i].us > 0) log << " " << trials[i].label << "=" << trials[i].us;
+      log << "\n";
+    }
+    // ---- whole kernel of this context --------------------------------------------------------------
+    stitched.codegen_allow_list.clear();
+    stitched.hip.profile_stages = false;
+    auto full = std::make_unique<MonoNNModule>(params.hlo_text, stitched.to_json().dump(0), params.kernel_name);
+    double us = -1;
+    try {
+      full->generate_code();
+      full->build_assembly();
+      us = time_module(*full, params.device, bufs, 5, 30);
+    } catch (const Error& e) {
+      log << ctx_str << " failed: " << e.what() << "\n";
+      continue;
+    }
+    log << ctx_str << " " << us / 1000.0 << " ms\n";
+    if (!params.dump_dir.empty()) full->dump_candidate(params.dump_dir);
+    if (best_us < 0 || us < best_us) {
+      best_us = us;
+      // hand back an unloaded module: the caller uploads constants and loads it where it wants
+      best = std::make_unique<MonoNNModule>(params.hlo_text, stitched.to_json().dump(0), params.kernel_name);
+      best->generate_code();
+      best->set_code_object(full->code_object());
+    }
+  }
+  MONONN_CHECK(best != nullptr, kRuntimeError) << "no launch context could be tuned:\n" << log.str();
+  if (!params.dump_dir.empty()) {
+    best->dump_best(params.dump_dir);
+    std::string dir = best->cluster_dir(params.dump_dir);
+    module::write_file(dir + "/tuning_log.log", log.str());
+    module::write_file(dir + "/performance_report.csv", report.str());
+  }
+  return best;
 }
 
 }  // namespace tuner
