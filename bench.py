@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--spec-dir", default=SPEC_DIR)
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the monolithic kernel's grid barrier cannot span "
@@ -90,6 +92,13 @@ def main():
 
     # parity of this very configuration against the oracle (also the CPU baseline's subject)
     got = module.run(inputs, fx.outputs)[0].astype(np.float32)
+
+    if args.calibration_copy:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
 
     ptrs = module.buffer_pointers()
     stream = torch.cuda.current_stream().cuda_stream

@@ -7,8 +7,10 @@ import fails, and launching without a GPU raises.
 """
 from __future__ import annotations
 
+import atexit
 import ctypes
 import os
+import weakref
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -97,6 +99,16 @@ def device_info(device: int = 0) -> dict:
             "arch": arch.value.decode()}
 
 
+_live_modules: "weakref.WeakSet" = weakref.WeakSet()
+
+
+@atexit.register
+def _destroy_all_modules():
+    # unload code objects while the HIP runtime is still alive (interpreter teardown order is arbitrary)
+    for m in list(_live_modules):
+        m.close()
+
+
 class MonoNNModule:
     """One HLO module compiled into one monolithic kernel."""
 
@@ -104,6 +116,13 @@ class MonoNNModule:
         self._h = ctypes.c_void_p(handle)
         self._bufs = None
         self._ptr_array = None
+        _live_modules.add(self)
+
+    def close(self):
+        h, self._h = getattr(self, "_h", None), None
+        self._bufs = None
+        if h and _lib is not None:
+            _lib.mononn_module_destroy(h)
 
     # ---- construction ------------------------------------------------------------------------
     @classmethod
@@ -125,9 +144,7 @@ class MonoNNModule:
         return cls(h.value)
 
     def __del__(self):
-        h, self._h = getattr(self, "_h", None), None
-        if h and _lib is not None:
-            _lib.mononn_module_destroy(h)
+        self.close()
 
     # ---- introspection -----------------------------------------------------------------------
     @property

@@ -1,0 +1,221 @@
+"""CPU tests of the host compiler and the C ABI: parsing, stage scheduling, specification handling,
+dump tree, error codes.  No kernel is launched here; hipRTC cross-compiles for gfx950 without a GPU."""
+import ctypes
+import json
+import os
+import re
+import subprocess
+
+import pytest
+
+from mononn_amd import MonoNNError, MonoNNModule, binding
+from mononn_amd.hlo import models
+from mononn_amd.hlo.builder import HloModuleBuilder
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def layer():
+    return models.bert_layer(B=1, S=32, H=128, NH=4, F=256)
+
+
+def test_abi_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "mononn_hip.h")).read()
+    declared = set(re.findall(r"\b(mononn_[a-z_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = ctypes.CDLL(binding.LIB_PATH)
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} is declared in include/mononn_hip.h but not exported"
+    assert declared == set(binding.EXPORTED_SYMBOLS)
+
+
+def test_kernel_name_buffers_and_argument_order(layer):
+    m = MonoNNModule.compile(layer.hlo_text, build=False)
+    assert m.kernel_name == "mononn_cluster_0"          # README.md:186 naming convention
+    info = m.buffer_info()
+    assert info["parameters"] == [1 * 32 * 128 * 2, 32 * 4]
+    assert info["liveouts"] == [32 * 128 * 2]
+    src = m.get_source("main.hip")
+    sig = re.search(r'extern "C" .*void mononn_cluster_0\(([^)]*)\)', src).group(1)
+    assert [a.strip() for a in sig.split(",")] == ["void* arg0", "void* arg1", "void* liveout_buffer_0", "void* temp_buffer"]
+    assert "buffer_for_constant_" in src                # constants are module globals filled by the host
+    names = [c["name"] for c in m.constants()]
+    assert len(names) == 16 and all(c["needs_payload"] for c in m.constants())
+
+
+def test_bert_base_parameters_match_reference_log():
+    m = MonoNNModule.compile(models.bert_base().hlo_text, build=False)
+    info = m.buffer_info()
+    assert info["parameters"] == [512, 512, 512]        # README.md:192-194
+    assert info["liveouts"] == [196608]
+
+
+def test_stage_structure_and_function_sharing(layer):
+    m = MonoNNModule.compile(layer.hlo_text, build=False)
+    s = m.summary()
+    stages = [int(x) for x in re.findall(r"^\s+stage (\d+)", s, re.M)]
+    assert stages == sorted(stages)
+    assert max(stages) == 9 and m.launch_dims()["barriers"] == 8
+    # Q, K and V projections share a stage; soft-max and LayerNorm chains were merged into row programs
+    assert stages.count(1) == 3
+    assert len(re.findall(r"rowred", s)) == 3
+    two = MonoNNModule.compile(models.bert_encoder(L=2, B=1, S=32, H=128, NH=4, F=256, vocab=100, max_pos=64).hlo_text, build=False)
+    one = MonoNNModule.compile(models.bert_encoder(L=1, B=1, S=32, H=128, NH=4, F=256, vocab=100, max_pos=64).hlo_text, build=False)
+    n2 = len(re.findall(r"__noinline__ void node_fn_", two.get_source()))
+    n1 = len(re.findall(r"__noinline__ void node_fn_", one.get_source()))
+    assert n2 <= n1 + 1, "a repeated layer must reuse the device functions of the first one"
+
+
+def test_disabled_pass_env(layer, monkeypatch):
+    base = MonoNNModule.compile(layer.hlo_text, build=False).launch_dims()["barriers"]
+    monkeypatch.setenv("MONONN_OPTIMIZATION_DISABLED_PASS", "MergeDependentPass,GemmEpilogueFusionPass")
+    unfused = MonoNNModule.compile(layer.hlo_text, build=False).launch_dims()["barriers"]
+    assert unfused > base
+
+
+def test_spec_round_trip_and_reload(layer, tmp_path):
+    m = MonoNNModule.compile(layer.hlo_text, build=False)
+    spec = json.loads(m.get_tuning_spec())
+    rt = spec["cuda_context"]["cuda_runtime_context"]
+    assert rt["grid_dim"] == {"x": 256, "y": 1, "z": 1} and rt["block_dim"]["x"] == 256 and "smem_size" in rt
+    assert spec["cuda_context"]["cuda_device_context"]["warp_size"] == 64
+    for key in ("cluster_elewise_spec", "cluster_reduce_spec", "gemm_spec_list", "conv_spec_list", "codegen_allow_list",
+                "codegen_reject_list", "feeds", "fetches", "input_data_files", "hlo_module_proto_file"):
+        assert key in spec
+    g = next(iter(spec["gemm_spec_list"].values()))
+    assert set(g["cutlass_config"]) >= {"threadblockshape", "warpshape", "instructionshape", "operatorclass", "archtag", "stages"}
+    assert "alpha_real" in g["gemm_backend_config"]
+    m2 = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
+    assert json.loads(m2.get_tuning_spec()) == spec
+    assert m2.get_source() == m.get_source()
+    # dump tree (README.md:155-177, context string with a double underscore: mononn_module_tuner.cc:374-383)
+    mb = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=True)
+    mb.dump(str(tmp_path))
+    d = tmp_path / "cluster_0"
+    for f in ("256_1_1__256_1_1.json", "256_1_1__256_1_1.hsaco", "256_1_1__256_1_1_src/main.hip", "256_1_1__256_1_1_src/headers.h",
+              "best_tuning_spec.json", "best_tuning_spec.hsaco"):
+        assert (d / f).exists(), f
+    m3 = MonoNNModule.from_spec_dir(layer.hlo_text, str(tmp_path))
+    assert m3.get_code_object() == mb.get_code_object()      # cached code object was picked up
+    os.environ["TF_MONONN_EXISTING_TUNING_SPEC_DIR"] = str(tmp_path)
+    try:
+        m4 = MonoNNModule.from_spec_dir(layer.hlo_text, None)
+        assert json.loads(m4.get_tuning_spec()) == json.loads(mb.get_tuning_spec())
+    finally:
+        del os.environ["TF_MONONN_EXISTING_TUNING_SPEC_DIR"]
+
+
+def test_spec_changes_generated_code(layer):
+    m = MonoNNModule.compile(layer.hlo_text, build=False)
+    spec = json.loads(m.get_tuning_spec())
+    name = next(n for n in spec["gemm_spec_list"] if "fusion" in n)
+    cc = spec["gemm_spec_list"][name]["cutlass_config"]
+    cc["threadblockshape"].update(m=16, n=64)
+    cc["wave_arrangement"].update(m=1, n=2, k=2)
+    src = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False).get_source()
+    assert "gemm_tile<16, 64, 1, 2, 2," in src
+
+
+@pytest.mark.parametrize("mutate,status", [
+    (lambda s: s["gemm_spec_list"].update({"no_such_node": next(iter(s["gemm_spec_list"].values()))}), "SPEC_ERROR"),
+    (lambda s: s.update({"unknown_field": 1}), "SPEC_ERROR"),
+    (lambda s: s["cuda_context"]["cuda_runtime_context"]["block_dim"].update(x=100), "SPEC_ERROR"),
+    (lambda s: s["cuda_context"]["cuda_runtime_context"]["grid_dim"].update(x=5000), "SPEC_ERROR"),
+    (lambda s: s["codegen_allow_list"].append("ghost"), "SPEC_ERROR"),
+    (lambda s: s["mononn_hip"].update(barrier="semaphore"), "SPEC_ERROR"),
+    (lambda s: next(iter(s["gemm_spec_list"].values()))["cutlass_config"]["wave_arrangement"].update(m=3), "SPEC_ERROR"),
+])
+def test_bad_specs_are_rejected(layer, mutate, status):
+    spec = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
+    mutate(spec)
+    with pytest.raises(MonoNNError) as e:
+        MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
+    assert e.value.status == status
+
+
+HEAD = "HloModule cluster_9__t.1\n\n"
+
+
+@pytest.mark.parametrize("text,status", [
+    ("not hlo at all", "PARSE_ERROR"),
+    (HEAD + "ENTRY %main {\n  %p = f32[4]{0} parameter(0)\n  ROOT %r = f32[4]{0} add(f32[4]{0} %p, f32[4]{0} %q)\n}\n", "PARSE_ERROR"),
+    (HEAD + "ENTRY %main {\n  %p = f32[4]{0} parameter(0)\n  ROOT %r = f32[4]{0} cosine(f32[4]{0} %p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f32[<=4]{0} parameter(0)\n  ROOT %r = f32[<=4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f32[4,4]{1,0:T(2,2)} parameter(0)\n  ROOT %r = f32[4,4]{1,0} negate(%p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f32[4,4]{0,1} parameter(0)\n  ROOT %r = f32[4,4]{0,1} negate(%p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = bf16[4]{0} parameter(0)\n  ROOT %r = bf16[4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f32[1,4,4,1]{3,2,1,0} parameter(0)\n  %w = f32[1,1,1,1]{3,2,1,0} parameter(1)\n"
+            "  ROOT %r = f32[1,4,4,1]{3,2,1,0} convolution(%p, %w), window={size=1x1}, dim_labels=b01f_01io->b01f\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f16[4,4]{1,0} parameter(0)\n  ROOT %r = f16[4,4]{1,0} custom-call(%p), custom_call_target=\"__my$thing\"\n}\n",
+     "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f32[4]{0} parameter(0)\n  ROOT %r = f32[4]{0} negate(%p)\n", "PARSE_ERROR"),
+])
+def test_bad_hlo_is_rejected_with_a_status(text, status):
+    with pytest.raises(MonoNNError) as e:
+        MonoNNModule.compile(text, build=False)
+    assert e.value.status == status, str(e.value)
+
+
+def test_gemm_stride_cross_check():
+    # XLA's lhs_stride must agree with the shapes (the reference cross-checks it, gemm_impl.cc:380-393)
+    mb = HloModuleBuilder("cluster_4__t.1")
+    e = mb.entry
+    a = e.parameter("f16", (2, 8, 32), "a")
+    b = e.parameter("f16", (2, 32, 8), "b")
+    e.set_tuple_root([e.gemm(a, b, 2, 1, batch_dims=(0,))])
+    good = mb.text()
+    MonoNNModule.compile(good, build=False)
+    bad = good.replace('\\"lhs_stride\\":\\"256\\"', '\\"lhs_stride\\":\\"999\\"')
+    assert bad != good
+    with pytest.raises(MonoNNError) as ex:
+        MonoNNModule.compile(bad, build=False)
+    assert ex.value.status == "INVALID_ARGUMENT"
+
+
+def test_errors_before_load(layer):
+    m = MonoNNModule.compile(layer.hlo_text, build=False)
+    with pytest.raises(MonoNNError) as e:
+        m.get_code_object()
+    assert e.value.status == "NOT_FOUND"
+    with pytest.raises(MonoNNError) as e:
+        m.set_constant("no_such_constant", __import__("numpy").zeros(4, "float16"))
+    assert e.value.status == "NOT_FOUND"
+    c = m.constants()[0]
+    with pytest.raises(MonoNNError) as e:
+        m.set_constant(c["name"], __import__("numpy").zeros(3, "float16"))
+    assert e.value.status == "INVALID_ARGUMENT"
+    with pytest.raises(MonoNNError) as e:
+        m.launch_raw([0, 0, 0, 0])
+    assert e.value.status == "INVALID_ARGUMENT"      # not loaded
+
+
+def test_compile_error_is_reported_not_fatal(layer):
+    # a kernel name that is not an identifier makes hipRTC fail; the process must survive with the log
+    with pytest.raises(MonoNNError) as e:
+        MonoNNModule.compile(layer.hlo_text, None, "not an identifier", build=True)
+    assert e.value.status == "COMPILE_ERROR" and "error" in str(e.value)
+
+
+def test_cli_compiles_and_dumps(layer, tmp_path):
+    hlo = tmp_path / "m.hlo"
+    hlo.write_text(layer.hlo_text)
+    exe = os.path.join(ROOT, "mononn_amd", "bin", "mononn_hipc")
+    out = subprocess.run([exe, str(hlo), "--dump", str(tmp_path / "dump")], capture_output=True, text=True, check=True).stdout
+    assert "Temporary buffer size:" in out and "Parameter 0:" in out
+    assert (tmp_path / "dump" / "cluster_0" / "best_tuning_spec.json").exists()
+    out2 = subprocess.run([exe, str(hlo), "--spec-dir", str(tmp_path / "dump")], capture_output=True, text=True, check=True).stdout
+    assert "kernel mononn_cluster_0" in out2
+
+
+def test_write_once_temp_addresses(layer):
+    # the fence-free barrier relies on every temp address being written once per launch
+    coherent = MonoNNModule.compile(layer.hlo_text, build=False)
+    spec = json.loads(coherent.get_tuning_spec())
+    assert spec["mononn_hip"]["barrier"] == "flags_coherent"
+    offs = re.findall(r"\(_Float16\*\)\(\(char\*\)temp_buffer \+ (\d+)\)", coherent.get_source())
+    assert len(offs) == len(set(offs)), "a temp slot is written by two nodes"
+    assert "MONONN_COHERENT_STORES 1" in coherent.get_source()
+    spec["mononn_hip"]["barrier"] = "flags"
+    fenced = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
+    assert fenced.buffer_info()["temp"] < coherent.buffer_info()["temp"]     # slots are re-used again

@@ -1,0 +1,216 @@
+"""Pins the NumPy oracle (oracle/hlo_interp.py) against things it did not write itself: closed forms,
+brute force in float64, torch library routines and an independent torch restatement of a whole
+BERT layer.  A dropped term, a transposed operand or a wrong contraction index fails one of these."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from mononn_amd.hlo import models
+from mononn_amd.hlo.builder import HloModuleBuilder
+from oracle import hlo_interp
+
+
+def _gemm_module(a_dims, b_dims, lhs_c, rhs_c, batch_dims=(), alpha=1.0, beta=0.0, with_c=False):
+    mb = HloModuleBuilder("cluster_1__pin.1")
+    e = mb.entry
+    a = e.parameter("f32" if False else "f16", a_dims, "a")
+    b = e.parameter("f16", b_dims, "b")
+    c = None
+    if with_c:
+        r = len(a_dims)
+        m = a_dims[r - 2] if lhs_c == r - 1 else a_dims[r - 1]
+        n = b_dims[r - 1] if rhs_c == r - 2 else b_dims[r - 2]
+        c = e.parameter("f16", list(a_dims[:r - 2]) + [m, n], "c")
+    d = e.gemm(a, b, lhs_c, rhs_c, batch_dims=batch_dims, alpha=alpha, beta=beta, addend=c)
+    e.set_tuple_root([d])
+    return mb.text()
+
+
+def test_gemm_brute_force_fp64_tiny():
+    rng = np.random.default_rng(0)
+    a = rng.normal(size=(5, 7)).astype(np.float16)
+    b = rng.normal(size=(7, 3)).astype(np.float16)
+    want = np.zeros((5, 3))
+    for i in range(5):
+        for j in range(3):
+            for k in range(7):
+                want[i, j] += float(a[i, k]) * float(b[k, j])
+    got = hlo_interp.evaluate(_gemm_module([5, 7], [7, 3], 1, 0), [a, b], precision="fp32")[0]
+    assert np.abs(got - want).max() < 1e-5
+
+
+def test_gemm_row_major_example_shapes():
+    # shapes / strides of the row-major worked example in the reference (gemm_impl.cc:290-303):
+    # f16[512,384] = f16[512,128] x f16[128,384], contracting lhs 1 / rhs 0, lhs_stride 65536, rhs_stride 49152
+    rng = np.random.default_rng(1)
+    a = rng.normal(size=(512, 128)).astype(np.float16)
+    b = rng.normal(size=(128, 384)).astype(np.float16)
+    text = _gemm_module([512, 128], [128, 384], 1, 0)
+    assert '\\"lhs_stride\\":\\"65536\\"' in text and '\\"rhs_stride\\":\\"49152\\"' in text
+    got = hlo_interp.evaluate(text, [a, b], precision="fp32")[0]
+    want = np.einsum("mk,kn->mn", a.astype(np.float64), b.astype(np.float64))
+    assert got.shape == (512, 384) and np.abs(got - want).max() < 1e-3
+
+
+def test_gemm_batched_transposed_example_shapes():
+    # the column-major worked example (gemm_impl.cc:305-316): f16[4,2,128,128] from f16[4,2,64,128] and
+    # f16[4,2,128,64], lhs contracting 2, rhs contracting 3, batch dims {0,1}, batch 8, strides 8192 / 8192
+    rng = np.random.default_rng(2)
+    a = rng.normal(size=(4, 2, 64, 128)).astype(np.float16)
+    b = rng.normal(size=(4, 2, 128, 64)).astype(np.float16)
+    text = _gemm_module([4, 2, 64, 128], [4, 2, 128, 64], 2, 3, batch_dims=(0, 1))
+    assert '\\"batch_size\\":\\"8\\"' in text and '\\"lhs_stride\\":\\"8192\\"' in text
+    got = hlo_interp.evaluate(text, [a, b], precision="fp32")[0]
+    want = np.einsum("xykm,xynk->xymn", a.astype(np.float64), b.astype(np.float64))
+    assert got.shape == (4, 2, 128, 128) and np.abs(got - want).max() < 1e-3
+
+
+def test_gemm_alpha_beta_addend():
+    rng = np.random.default_rng(3)
+    a = rng.normal(size=(6, 8)).astype(np.float16)
+    b = rng.normal(size=(8, 4)).astype(np.float16)
+    c = rng.normal(size=(6, 4)).astype(np.float16)
+    got = hlo_interp.evaluate(_gemm_module([6, 8], [8, 4], 1, 0, alpha=0.5, beta=2.0, with_c=True), [a, b, c],
+                              precision="fp32")[0]
+    want = 0.5 * a.astype(np.float64) @ b.astype(np.float64) + 2.0 * c.astype(np.float64)
+    assert np.abs(got - want).max() < 1e-5
+
+
+def test_as_written_rounds_to_half():
+    rng = np.random.default_rng(4)
+    a = rng.normal(size=(6, 64)).astype(np.float16)
+    b = rng.normal(size=(64, 4)).astype(np.float16)
+    got = hlo_interp.evaluate(_gemm_module([6, 64], [64, 4], 1, 0), [a, b])[0]
+    assert got.dtype == np.float16
+    want = (a.astype(np.float32) @ b.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got, want)
+
+
+def _single_fusion(build, params):
+    mb = HloModuleBuilder("cluster_2__pin.1")
+    e = mb.entry
+    ps = [e.parameter(dt, dims, f"p{i}") for i, (dt, dims) in enumerate(params)]
+    outs = build(e, mb, *ps)
+    e.set_tuple_root(outs if isinstance(outs, list) else [outs])
+    return mb.text()
+
+
+def test_softmax_matches_torch():
+    rng = np.random.default_rng(5)
+    x = rng.normal(size=(2, 3, 8, 16)).astype(np.float32)
+
+    def build(e, mb, px):
+        full = (2, 3, 8, 16)
+        mx = e.fusion("kInput", [px], lambda f, p: f.reduce(p, f.scalar("f32", float("-inf")), 3, mb.reducer("maximum", "f32")))
+        sm = e.fusion("kInput", [px, mx], lambda f, p, m: f.reduce(f.exp(f.sub(p, f.broadcast(m, full, [0, 1, 2]))),
+                                                                  f.scalar("f32", 0.0), 3, mb.reducer("add", "f32")))
+        return e.fusion("kLoop", [px, mx, sm], lambda f, p, m, s: f.div(f.exp(f.sub(p, f.broadcast(m, full, [0, 1, 2]))),
+                                                                         f.broadcast(s, full, [0, 1, 2])))
+    got = hlo_interp.evaluate(_single_fusion(build, [("f32", (2, 3, 8, 16))]), [x])[0]
+    want = torch.softmax(torch.tensor(x), -1).numpy()
+    assert np.abs(got - want).max() < 1e-6
+    assert np.abs(got.sum(-1) - 1).max() < 1e-5
+
+
+def test_layer_norm_and_gelu_match_torch():
+    rng = np.random.default_rng(6)
+    x = rng.normal(size=(8, 32)).astype(np.float16)
+    g = (1 + 0.1 * rng.normal(size=32)).astype(np.float16)
+    b = (0.1 * rng.normal(size=32)).astype(np.float16)
+    text = _single_fusion(lambda e, mb, px, pg, pb: models._layer_norm(e, mb, px, pg, pb, 1e-12),
+                          [("f16", (8, 32)), ("f16", (32,)), ("f16", (32,))])
+    got = hlo_interp.evaluate(text, [x, g, b], precision="fp32")[0]
+    want = F.layer_norm(torch.tensor(x.astype(np.float32)), (32,), torch.tensor(g.astype(np.float32)),
+                        torch.tensor(b.astype(np.float32)), 1e-12).numpy()
+    assert np.abs(got - want).max() < 2e-5
+    xs = rng.normal(size=(4, 16)).astype(np.float32) * 3
+    text = _single_fusion(lambda e, mb, px: e.fusion("kLoop", [px], lambda f, p: models._gelu_tanh(f, p)), [("f32", (4, 16))])
+    got = hlo_interp.evaluate(text, [xs])[0]
+    assert np.abs(got - F.gelu(torch.tensor(xs), approximate="tanh").numpy()).max() < 1e-6
+
+
+def test_gather_brute_force_and_clamp():
+    rng = np.random.default_rng(7)
+    table = rng.normal(size=(11, 5)).astype(np.float16)
+    ids = np.array([[0, 10, 3], [7, 7, 2]], np.int32)
+    text = _single_fusion(lambda e, mb, pt, pi: e.gather_rows(pt, pi), [("f16", (11, 5)), ("s32", (2, 3))])
+    got = hlo_interp.evaluate(text, [table, ids])[0]
+    for i in range(2):
+        for j in range(3):
+            assert np.array_equal(got[i, j], table[ids[i, j]])
+    oob = np.array([[-4, 99, 3], [7, 7, 2]], np.int32)   # XLA clamps out-of-range start indices
+    got = hlo_interp.evaluate(text, [table, oob])[0]
+    assert np.array_equal(got[0, 0], table[0]) and np.array_equal(got[0, 1], table[10])
+
+
+def test_shape_ops_against_numpy():
+    rng = np.random.default_rng(8)
+    x = rng.normal(size=(2, 3, 4)).astype(np.float32)
+
+    def build(e, mb, px):
+        def body(f, p):
+            t = f.transpose(p, (2, 0, 1))                 # [4,2,3]
+            r = f.reshape(t, (8, 3))
+            s = f.slice(r, (2, 1), (6, 3))               # [4,2]
+            c = f.concatenate([s, f.splat("f32", 7.0, (4, 1))], 1)   # [4,3]
+            return f.add(c, f.convert(f.iota("s32", (4, 3), 1), "f32"))
+        return e.fusion("kLoop", [px], body)
+    got = hlo_interp.evaluate(_single_fusion(build, [("f32", (2, 3, 4))]), [x])[0]
+    r = np.transpose(x, (2, 0, 1)).reshape(8, 3)[2:6, 1:3]
+    want = np.concatenate([r, np.full((4, 1), 7.0, np.float32)], 1) + np.arange(3, dtype=np.float32)[None, :]
+    assert np.array_equal(got, want)
+
+
+def test_bert_layer_against_independent_torch_restatement():
+    fx = models.bert_layer(B=1, S=32, H=128, NH=4, F=256)
+    consts = fx.make_constants(11, "random")
+    inputs = fx.make_inputs(11)
+    got = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0][0]
+    R = {m["role"].split("layer_0/")[1]: torch.tensor(consts[n].astype(np.float32)) for n, m in fx.constants.items()}
+    h = torch.tensor(inputs[0].astype(np.float32))[0]
+
+    def lin(x, p):
+        return x @ R[p + "/kernel"] + R[p + "/bias"]
+    S, NH, D = 32, 4, 32
+    q, k, v = (lin(h, "attention/" + n).view(S, NH, D).transpose(0, 1) for n in ("query", "key", "value"))
+    p = torch.softmax(q @ k.transpose(1, 2) / math.sqrt(D), -1)
+    ctx = (p @ v).transpose(0, 1).reshape(S, NH * D)
+    x1 = F.layer_norm(lin(ctx, "attention/output") + h, (128,), R["attention/LayerNorm/gamma"], R["attention/LayerNorm/beta"], 1e-12)
+    a = F.gelu(lin(x1, "intermediate"), approximate="tanh")
+    x2 = F.layer_norm(lin(a, "output") + x1, (128,), R["output/LayerNorm/gamma"], R["output/LayerNorm/beta"], 1e-12)
+    assert np.abs(got - x2.numpy()).max() < 2e-5
+
+
+def test_masked_encoder_against_torch():
+    # padding mask (1/0) -> additive -10000 on padded keys; embeddings gathered by id
+    fx = models.bert_encoder(L=1, B=2, S=16, H=64, NH=2, F=128, vocab=50, max_pos=32, mask_kind="length_mask")
+    consts = fx.make_constants(12, "random")
+    inputs = fx.make_inputs(12)
+    got = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    by_role = {m["role"]: torch.tensor(consts[n].astype(np.float32)) for n, m in fx.constants.items()}
+    ids, mask, tt = (torch.tensor(a.astype(np.int64)) for a in inputs)
+    emb = by_role["bert/embeddings/word_embeddings"][ids] + by_role["bert/embeddings/position_embeddings"][:16][None] + \
+        by_role["bert/embeddings/token_type_embeddings"][tt]
+    h = F.layer_norm(emb, (64,), by_role["bert/embeddings/LayerNorm/gamma"], by_role["bert/embeddings/LayerNorm/beta"], 1e-12)
+    add = (1.0 - mask.float()) * -10000.0
+    P = "bert/encoder/layer_0/"
+
+    def lin(x, p):
+        return x @ by_role[P + p + "/kernel"] + by_role[P + p + "/bias"]
+    q, k, v = (lin(h, "attention/" + n).view(2, 16, 2, 32).transpose(1, 2) for n in ("query", "key", "value"))
+    s = q @ k.transpose(2, 3) / math.sqrt(32) + add[:, None, None, :]
+    ctx = (torch.softmax(s, -1) @ v).transpose(1, 2).reshape(2, 16, 64)
+    x1 = F.layer_norm(lin(ctx, "attention/output") + h, (64,), by_role[P + "attention/LayerNorm/gamma"], by_role[P + "attention/LayerNorm/beta"], 1e-12)
+    a = F.gelu(lin(x1, "intermediate"), approximate="tanh")
+    x2 = F.layer_norm(lin(a, "output") + x1, (64,), by_role[P + "output/LayerNorm/gamma"], by_role[P + "output/LayerNorm/beta"], 1e-12)
+    assert np.abs(got - x2.numpy()).max() < 3e-5
+
+
+def test_reference_example_input_shape():
+    ids, mask, seg = models.reference_example_inputs()
+    assert ids.dtype == np.int32 and ids.shape == (1, 128) and ids.nbytes == 512
+    assert ids[0, 0] == 101 and ids[0, -1] == 102 and (ids[0, 1:-1] == 7592).all()
+    assert mask.all() and not seg.any()
