@@ -80,12 +80,13 @@ void store(const Program& prog, CodeBuffer& cb, PointerTable& ptrs, const VarTab
 
 std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs);
 
-NodeFunction finish(const std::string& body, PointerTable& ptrs, Emitter& em, int64_t units, int smem, const std::string& pre = "") {
+NodeFunction finish(const std::string& body, PointerTable& ptrs, const std::vector<std::string>& globals, int64_t units, int smem,
+                    const std::string& pre = "") {
   NodeFunction f;
   f.pointers = ptrs.entries;
   f.num_units = units;
   f.smem_bytes = smem;
-  for (auto& kv : em.literal_tables()) f.globals.push_back(kv.second);
+  f.globals = globals;
   f.text = pre + "__device__ __noinline__ void @NAME@(" + signature(ptrs.entries) + ") {\n" + align_prologue(ptrs.entries) + body + "}\n";
   return f;
 }
@@ -107,6 +108,12 @@ std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs) {
     out += "  " + e.name + " = (" + T + ")__builtin_assume_aligned(" + e.name + ", 16);\n";
   }
   return out;
+}
+
+std::vector<std::string> tables_of(const Emitter& em) {
+  std::vector<std::string> v;
+  for (auto& kv : em.literal_tables()) v.push_back(kv.second);
+  return v;
 }
 
 NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
@@ -261,7 +268,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     }
     cb.close();
     int64_t units = block_tier ? ROWS : (ROWS + NW - 1) / NW;
-    return finish(cb.text(), ptrs, em, units, block_tier ? NW * 8 : 0);
+    return finish(cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 : 0);
   }
 
   // element-wise loop(s); outputs of equal element count share one loop.  A thread owns V consecutive
@@ -304,7 +311,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     if (groups.size() > 1) cb.close();
     unit_base += units;
   }
-  return finish(cb.text(), ptrs, em, unit_base, 0);
+  return finish(cb.text(), ptrs, tables_of(em), unit_base, 0);
 }
 
 }  // namespace
@@ -407,26 +414,23 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
 
 namespace {
 
-struct EpilogueVars {
-  int b, m, n4, r, nn;
+// Epilogue of an MFMA / fallback GEMM as a functor: the GEMM result (fp32 accumulator, scaled, rounded
+// to the f16 value the HLO defines) is bound to a register and every fused element-wise cluster is
+// emitted on top of it.  Pointers the epilogue needs are appended to `ptrs`; the functor's members
+// are all entries from `first_epi` on.
+struct Epilogue {
+  std::string struct_text;   // struct @NAME@_epi { ... };
+  std::string init_line;     // @NAME@_epi epi{...};
+  std::vector<std::string> globals;
 };
 
-NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
-                      const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t) {
-  const Instr* gi = members[0];
-  const bool mfma = gemm_uses_mfma(g);
+Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<const Instr*>& cluster_members,
+                        const std::vector<const Instr*>& outputs, const graph::GemmDesc& g, bool mfma, PointerTable& ptrs,
+                        size_t first_epi) {
   const bool vec4 = mfma && g.N % 4 == 0;
-  if (mfma) validate_gemm_tuning(g, ls, t);
   CodeBuffer cb;   // epilogue body
   VarTable vars;
-  PointerTable ptrs;
-  // the two operands come first in the pointer list
-  std::string pa = ptrs.input(prog.storage_root(gi->operands[0]));
-  std::string pb = ptrs.input(prog.storage_root(gi->operands[1]));
-  const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
-  std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
   Emitter em(prog, cluster_members, cb, vars, ptrs);
-
   const hlo::Shape& D = gi->shape;
   std::vector<int64_t> batch_dims(D.dims.begin(), D.dims.end() - 2);
   int vb = vars.add("bidx", g.batch);
@@ -600,11 +604,30 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   }
   pre += "  }\n};\n";
 
-  CodeBuffer fb;
+  Epilogue out_e;
+  out_e.struct_text = pre;
   std::string init = "@NAME@_epi epi{";
   for (size_t i = first_epi; i < ptrs.entries.size(); ++i) init += (i > first_epi ? ", " : "") + ptrs.entries[i].name;
   init += "};";
-  fb.line(init);
+  out_e.init_line = init;
+  for (auto& kv : em.literal_tables()) out_e.globals.push_back(kv.second);
+  return out_e;
+}
+
+NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
+                      const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t) {
+  const Instr* gi = members[0];
+  const bool mfma = gemm_uses_mfma(g);
+  if (mfma) validate_gemm_tuning(g, ls, t);
+  PointerTable ptrs;
+  // the two operands come first in the pointer list
+  std::string pa = ptrs.input(prog.storage_root(gi->operands[0]));
+  std::string pb = ptrs.input(prog.storage_root(gi->operands[1]));
+  const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
+  std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
+  Epilogue epi = build_epilogue(prog, gi, cluster_members, outputs, g, mfma, ptrs, first_epi);
+  CodeBuffer fb;
+  fb.line(epi.init_line);
   int64_t units = 0;
   int smem = 0;
   if (mfma) {
@@ -648,13 +671,239 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fb.line(call.str());
     fb.close();
   }
-  return finish(fb.text(), ptrs, em, units, smem, pre);
+  return finish(fb.text(), ptrs, epi.globals, units, smem, epi.struct_text);
+}
+
+// GEMM -> row program -> GEMM with everything between the two contractions on chip.
+//
+// A workgroup owns RW blocks of 16 rows m of one batch element; the KW waves of a block split the
+// N1 columns of the first GEMM (the keys) between them.  S = A1 . B1^T is accumulated with the B1
+// fragment as first MFMA operand, which leaves lane (r16, g) with S[m = r16][n = n_w + 16 j + 4 g + r]:
+// the wave's part of a row lives in the 4 lanes r16, r16+16, r16+32, r16+48.  The row program
+// (soft-max) is generated as straight-line code over those values; a reduction finishes with two
+// butterfly steps across the 4 lanes and, for KW > 1, one exchange through LDS.  The result P feeds
+// the second contraction directly: its k index inside one 32-wide MFMA step is enumerated as
+// k(g, i) = 16 (i / 4) + 4 g + i % 4, i < 8, for both operands (a permutation of the summation order
+// leaves the sum unchanged), which is exactly the order the lane already holds P in.  The right
+// operand of the second GEMM is read through the same enumeration: two 8-byte loads per fragment
+// from its k-contiguous layout.  The KW partial products meet in LDS; wave kw finishes the column
+// tiles t with t % KW == kw and runs the epilogue on them.
+NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,
+                           const Instr* g2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epi_members,
+                           const std::vector<const Instr*>& outputs, const LaunchShape& ls) {
+  const int NW = ls.waves();
+  const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
+  MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
+  MONONN_CHECK(K1 % 32 == 0 && N1 % 32 == 0 && N2 % 16 == 0, kUnsupported) << "attention fusion: extents must be MFMA multiples";
+  int KW = 1;
+  while (KW * 2 <= NW && N1 % (32 * KW * 2) == 0 && N1 / (KW * 2) >= 32) KW *= 2;
+  const int RW = NW / KW;
+  const int64_t NKW = N1 / KW;   // keys per wave
+  const int KS1 = static_cast<int>(K1 / 32), NT1 = static_cast<int>(NKW / 16), KS2 = static_cast<int>(NKW / 32), NT2 = static_cast<int>(N2 / 16);
+  RowInfo info = analyze_rows(row_members);
+  MONONN_CHECK(info.row_program && info.rows == d1.batch * M1 && info.row_len == N1, kUnsupported)
+      << "attention fusion: the cluster between the GEMMs is not a row program over the first GEMM's rows";
+  auto row_outs = external_outputs(prog, row_members);
+  MONONN_CHECK(row_outs.size() == 1 && row_outs[0]->shape.num_elements() == d1.batch * M1 * N1 && row_outs[0]->shape.dtype == DType::kF16, kUnsupported)
+      << "attention fusion: the row program must produce exactly one f16 matrix";
+  const Instr* P = row_outs[0];
+
+  PointerTable ptrs;
+  std::string pq = ptrs.input(prog.storage_root(g1->operands[0]));
+  std::string pk = ptrs.input(prog.storage_root(g1->operands[1]));
+  std::string pv = ptrs.input(prog.storage_root(g2->operands[1]));
+  const size_t first_epi = ptrs.entries.size();
+
+  CodeBuffer cb;
+  VarTable vars;
+  Emitter em(prog, row_members, cb, vars, ptrs);
+  const hlo::Shape& D1 = g1->shape;
+  std::vector<int64_t> batch_dims(D1.dims.begin(), D1.dims.end() - 2);
+  int vb = vars.add("bidx", d1.batch);
+  int vm = vars.add("m", M1);
+  int vg = vars.add("g", 4);
+  int vkw = vars.add("kw", KW);
+  auto elem_index = [&](int j, int r) {
+    Index idx = delinearize(LinExpr::variable(vb, d1.batch), batch_dims, vars);
+    idx.push_back(LinExpr::variable(vm, M1));
+    idx.push_back(LinExpr::variable(vkw, KW).scaled(NKW).plus(LinExpr::variable(vg, 4).scaled(4)).plus_const(j * 16 + r));
+    return idx;
+  };
+  Index row_index = delinearize(LinExpr::variable(vb, d1.batch), batch_dims, vars);
+  row_index.push_back(LinExpr::variable(vm, M1));
+
+  std::ostringstream alpha_s;
+  alpha_s.precision(9);
+  alpha_s << d1.alpha;
+  std::string alpha_lit = alpha_s.str();
+  if (alpha_lit.find_first_of(".e") == std::string::npos) alpha_lit += ".0";
+
+  // LDS: one slot of RW*KW*16 values per reduction, then the partial products
+  auto reduces = em.collect_reduces();
+  int smem = 0;
+  std::vector<int> red_off;
+  if (KW > 1) {
+    for (size_t i = 0; i < reduces.size(); ++i) {
+      red_off.push_back(smem);
+      smem += RW * KW * 16 * 8;
+    }
+  }
+  const int o_off = smem;
+  if (KW > 1) smem += RW * KW * NT2 * 64 * 16;
+
+  cb.line("const int lane = mononn_dev::lane_id();");
+  cb.line("const int r16 = lane & 15, g = lane >> 4;");
+  cb.line("const int kw = mononn_dev::wave_id() % " + S(KW) + ", rw = mononn_dev::wave_id() / " + S(KW) + ";");
+  const int64_t blocks = (M1 + 16 * RW - 1) / (16 * RW);
+  cb.line("const int bidx = unit / " + S(blocks) + ";");
+  cb.line("const int mt = (unit % " + S(blocks) + ") * " + S(RW) + " + rw;");
+  cb.line("const bool m_valid = mt * 16 + r16 < " + S(M1) + ";");
+  cb.line("const int m = m_valid ? mt * 16 + r16 : " + S(M1 - 1) + ";");
+  cb.line("const _Float16* qp = " + pq + " + (long)bidx * " + S(d1.a_batch_stride) + " + m * " + S(K1) + " + g * 8;");
+  cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + (kw * " + S(NKW) + " + r16) * " + S(K1) + " + g * 8;");
+  cb.line("const _Float16* vp = " + pv + " + (long)bidx * " + S(d2.b_batch_stride) + " + r16 * " + S(N1) + " + kw * " + S(NKW) + " + g * 4;");
+  // all operand loads up front: one exposed memory latency for the whole unit
+  cb.line("half8_t qf[" + S(KS1) + "], kf[" + S(NT1) + "][" + S(KS1) + "];");
+  cb.line("half4_t vf[" + S(NT2) + "][" + S(KS2) + "][2];");
+  cb.line("#pragma unroll");
+  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qp + ks * 32);");
+  cb.line("#pragma unroll");
+  cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
+  cb.line("#pragma unroll");
+  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + j * " + S(16 * K1) + " + ks * 32);");
+  cb.close();
+  cb.line("#pragma unroll");
+  cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+  cb.line("#pragma unroll");
+  cb.open("for (int ks = 0; ks < " + S(KS2) + "; ++ks)");
+  cb.line("vf[t][ks][0] = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32);");
+  cb.line("vf[t][ks][1] = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32 + 16);");
+  cb.close();
+  cb.close();
+  cb.line("float4_t sacc[" + S(NT1) + "];");
+  cb.line("#pragma unroll");
+  cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
+  cb.line("sacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};");
+  cb.line("#pragma unroll");
+  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[j][ks], qf[ks], sacc[j], 0, 0, 0);");
+  cb.close();
+  // the first GEMM's result as the HLO defines it: scaled, rounded to f16
+  cb.line("_Float16 sv[" + S(NT1) + "][4], pr[" + S(NT1) + "][4];");
+  cb.line("#pragma unroll");
+  cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
+  cb.line("#pragma unroll");
+  cb.line(std::string("for (int r = 0; r < 4; ++r) sv[j][r] = (_Float16)(sacc[j][r]") + (d1.alpha == 1.0 ? "" : " * " + alpha_lit + "f") + ");");
+  cb.close();
+  // ---- row program on the register-resident rows ------------------------------------------------
+  auto bind_elem = [&](int j, int r) { em.bind(g1, elem_index(j, r), "sv[" + S(j) + "][" + S(r) + "]"); };
+  for (size_t ri = 0; ri < reduces.size(); ++ri) {
+    const Instr* red = reduces[ri];
+    std::string Tn = hlo::dtype_ctype(red->shape.dtype);
+    MONONN_CHECK(hlo::dtype_bytes(red->shape.dtype) <= 8, kUnsupported) << "reduction type too wide";
+    std::string acc = em.fresh("red");
+    cb.line(Tn + " " + acc + " = " + em.value(red->operands[1], {}) + ";");
+    for (int j = 0; j < NT1; ++j)
+      for (int r = 0; r < 4; ++r) {
+        bind_elem(j, r);
+        std::string val = em.value(red->operands[0], elem_index(j, r));
+        cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(red, acc, val) + ";");
+      }
+    for (int off : {16, 32}) {
+      std::string other = "__shfl_xor(" + acc + ", " + S(off) + ", 64)";
+      cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(red, acc, other) + ";");
+    }
+    if (KW > 1) {
+      std::string buf = em.fresh("rb");
+      cb.line(Tn + "* " + buf + " = reinterpret_cast<" + Tn + "*>(smem + " + S(red_off[ri]) + ") + rw * " + S(KW * 16) + ";");
+      cb.line("if (g == 0) " + buf + "[kw * 16 + r16] = " + acc + ";");
+      cb.line("__syncthreads();");
+      cb.line(acc + " = " + buf + "[r16];");
+      for (int w = 1; w < KW; ++w) cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(red, acc, buf + "[" + S(w * 16) + " + r16]") + ";");
+    }
+    em.bind(red, row_index, acc);
+  }
+  for (int j = 0; j < NT1; ++j)
+    for (int r = 0; r < 4; ++r) {
+      bind_elem(j, r);
+      cb.line("pr[" + S(j) + "][" + S(r) + "] = " + em.value(em.resolve_output(P), elem_index(j, r)) + ";");
+    }
+  em.unbind(g1);
+  // ---- second contraction ---------------------------------------------------------------------------
+  cb.line("float4_t oacc[" + S(NT2) + "];");
+  cb.line("#pragma unroll");
+  cb.line("for (int t = 0; t < " + S(NT2) + "; ++t) oacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};");
+  cb.line("#pragma unroll");
+  cb.open("for (int ks = 0; ks < " + S(KS2) + "; ++ks)");
+  cb.line("const half8_t pf = {pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]};");
+  cb.line("#pragma unroll");
+  cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+  cb.line("const half8_t vv = {vf[t][ks][0][0], vf[t][ks][0][1], vf[t][ks][0][2], vf[t][ks][0][3], vf[t][ks][1][0], vf[t][ks][1][1], vf[t][ks][1][2], vf[t][ks][1][3]};");
+  cb.line("oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, pf, oacc[t], 0, 0, 0);");
+  cb.close();
+  cb.close();
+
+  std::vector<std::string> globals = tables_of(em);
+  Epilogue epi = build_epilogue(prog, g2, epi_members, outputs, d2, true, ptrs, first_epi);
+  for (auto& gl : epi.globals) globals.push_back(gl);
+  cb.line(epi.init_line);
+  if (KW > 1) {
+    cb.line("float4_t* ob = reinterpret_cast<float4_t*>(smem + " + S(o_off) + ") + rw * " + S(KW * NT2 * 64) + ";");
+    cb.line("#pragma unroll");
+    cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+    cb.line("if (t % " + S(KW) + " != kw) ob[(kw * " + S(NT2) + " + t) * 64 + lane] = oacc[t];");
+    cb.close();
+    cb.line("__syncthreads();");
+    cb.line("#pragma unroll");
+    cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+    cb.line("if (t % " + S(KW) + " != kw) continue;");
+    cb.line("float4_t o = oacc[t];");
+    cb.line("#pragma unroll");
+    cb.line("for (int w = 0; w < " + S(KW) + "; ++w) if (w != kw) o += ob[(w * " + S(NT2) + " + t) * 64 + lane];");
+    cb.open("if (m_valid)");
+    cb.line("const float v[4] = {o[0], o[1], o[2], o[3]};");
+    cb.line("epi(bidx, m, t * 16 + g * 4, v);");
+    cb.close();
+    cb.close();
+    cb.line("__syncthreads();   // LDS is reused by the next unit");
+  } else {
+    cb.open("if (m_valid)");
+    cb.line("#pragma unroll");
+    cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+    cb.line("const float v[4] = {oacc[t][0], oacc[t][1], oacc[t][2], oacc[t][3]};");
+    cb.line("epi(bidx, m, t * 16 + g * 4, v);");
+    cb.close();
+    cb.close();
+  }
+  return finish(cb.text(), ptrs, globals, d1.batch * blocks, smem, epi.struct_text);
 }
 
 }  // namespace
 
 NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchShape& ls, const GemmTuning& t) {
   return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t);
+}
+
+NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls) {
+  std::vector<const Instr*> row(node.members.begin() + 1, node.members.begin() + node.gemm2_index);
+  std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.end());
+  return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls);
+}
+
+bool can_fuse_attention(const Program& prog, const Instr* gemm1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,
+                        const Instr* gemm2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epilogue_members) {
+  try {
+    std::vector<const Instr*> tail{gemm2};
+    tail.insert(tail.end(), epilogue_members.begin(), epilogue_members.end());
+    auto outs = external_outputs(prog, tail);
+    if (outs.empty()) return false;
+    graph::GemmDesc d2k = d2;
+    d2k.b_k_contig = true;   // the layout pass stores the operand k-contiguous before real generation
+    gen_attention(prog, gemm1, d1, row_members, gemm2, d2k, epilogue_members, outs, LaunchShape{});
+    return true;
+  } catch (const Error& e) {
+    if (e.code() == kUnsupported) return false;
+    throw;
+  }
 }
 
 bool can_fuse_epilogue(const Program& prog, const std::vector<const Instr*>& gemm_members, const std::vector<const Instr*>& cluster_members) {

@@ -48,6 +48,8 @@ NodeFunction generate_cluster(const graph::Program& prog, const graph::Node& nod
 NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls,
                            const GemmTuning& t);
 
+NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls);
+
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus);
 // throws Error(kSpecError) when the tile / wave arrangement cannot be generated for this GEMM
 void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t);
@@ -59,6 +61,10 @@ bool can_merge_clusters(const graph::Program& prog, const std::vector<const hlo:
                         const std::vector<const hlo::Instr*>& merged);
 bool can_fuse_epilogue(const graph::Program& prog, const std::vector<const hlo::Instr*>& gemm_members,
                        const std::vector<const hlo::Instr*>& cluster_members);
+
+bool can_fuse_attention(const graph::Program& prog, const hlo::Instr* gemm1, const graph::GemmDesc& d1,
+                        const std::vector<const hlo::Instr*>& row_members, const hlo::Instr* gemm2, const graph::GemmDesc& d2,
+                        const std::vector<const hlo::Instr*>& epilogue_members);
 
 // entry-level values defined by `members` that somebody outside (another instruction or the
 // module root) reads, in definition order

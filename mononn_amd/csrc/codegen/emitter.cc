@@ -84,8 +84,18 @@ std::string Emitter::key(const Instr* ins, const Index& idx) const {
 }
 
 std::string Emitter::def(DType t, const std::string& rhs) {
+  // Value numbering: every definition is a pure function of the variables named in `rhs` (inputs of
+  // a node are never written by it), so an identical right-hand side already in scope is the same
+  // value.  This merges the copies of a sub-expression that XLA duplicated into several fusions
+  // (the soft-max logits, the centred LayerNorm input) once those fusions share a loop body.
+  std::string k = std::string("=") + hlo::dtype_ctype(t) + "|" + rhs;
+  for (auto it = scopes_.rbegin(); it != scopes_.rend(); ++it) {
+    auto f = it->find(k);
+    if (f != it->end()) return f->second;
+  }
   std::string v = fresh();
   out_.line(std::string("const ") + hlo::dtype_ctype(t) + " " + v + " = " + rhs + ";");
+  scopes_.back()[k] = v;
   return v;
 }
 

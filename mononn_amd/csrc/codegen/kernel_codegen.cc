@@ -22,6 +22,7 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.fuse_gemm_epilogue = s.hip.gemm_epilogue_fusion;
   o.transpose_constant_b = s.hip.transpose_constant_b;
   o.assign_operand_layouts = s.hip.assign_operand_layouts;
+  o.fuse_attention = s.hip.fuse_attention;
   o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
   for (auto& p : env::disabled_passes()) o.disabled_passes.insert(p);
   return o;
@@ -110,7 +111,9 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   int smem = 0;
   for (auto& n : prog.nodes) {
     NodeFunction f;
-    if (n.kind == NodeKind::kGemm) {
+    if (n.kind == NodeKind::kAttention) {
+      f = generate_attention(prog, n, ls);
+    } else if (n.kind == NodeKind::kGemm) {
       auto it = spec.gemm_spec_list.find(n.name);
       GemmTuning t;
       if (it == spec.gemm_spec_list.end()) {
@@ -178,7 +181,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     }
     NodeReport rep;
     rep.name = n.name;
-    rep.kind = n.kind == NodeKind::kGemm ? "gemm" : (n.row_program ? "cluster_reduce" : "cluster_elewise");
+    rep.kind = n.kind == NodeKind::kGemm ? "gemm" : n.kind == NodeKind::kAttention ? "attention" : (n.row_program ? "cluster_reduce" : "cluster_elewise");
     rep.function = fn;
     rep.stage = n.stage;
     rep.units = f.num_units;

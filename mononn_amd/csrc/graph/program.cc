@@ -36,8 +36,9 @@ std::string Program::summary() const {
   std::ostringstream os;
   os << "stages=" << num_stages << " nodes=" << nodes.size() << " temp_bytes=" << temp_bytes << "\n";
   for (auto& n : nodes) {
-    os << "  stage " << n.stage << "  " << (n.kind == NodeKind::kGemm ? "gemm   " : (n.row_program ? "rowred " : "elewise")) << " " << n.name;
+    os << "  stage " << n.stage << "  " << (n.kind == NodeKind::kGemm ? "gemm   " : n.kind == NodeKind::kAttention ? "attn   " : (n.row_program ? "rowred " : "elewise")) << " " << n.name;
     if (n.kind == NodeKind::kGemm) os << "  [" << n.gemm.problem_hash() << "] members=" << n.members.size();
+    else if (n.kind == NodeKind::kAttention) os << "  [" << n.gemm.problem_hash() << " -> " << n.gemm2.problem_hash() << "] members=" << n.members.size();
     else os << "  members=" << n.members.size() << (n.row_program ? " rows=" + std::to_string(n.rows) + " len=" + std::to_string(n.row_len) : "");
     os << "\n";
   }
@@ -231,6 +232,83 @@ struct Builder {
     }
   }
 
+  // may the kernel keep the right-hand GEMM operand `root` ([.., K, N]) transposed in memory?
+  bool can_store_k_contig(const Instr* root, const Instr* operand, int rhs_contracting) const {
+    if (root->opcode == "parameter" || root->opcode == "constant") return false;
+    if (root->shape.dims != operand->shape.dims) return false;   // reached through a reshaping alias
+    for (auto* u : root->users) {
+      if (is_alias_op(u)) return false;
+      bool as_b = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands[1] == root && u->operands[0] != root &&
+                  (u->operands.size() < 3 || u->operands[2] != root) && u->gemm.rhs_contracting == rhs_contracting;
+      if (!as_b) return false;
+    }
+    const Instr* mroot = p.module->entry->root;
+    if (mroot == root) return false;
+    if (mroot->opcode == "tuple")
+      for (auto* o : mroot->operands)
+        if (p.storage_root(o) == root) return false;
+    return true;
+  }
+
+  // GEMM -> row program -> GEMM (attention): the row program's only product feeds the second GEMM as
+  // its left operand, and the first GEMM's result is read by nothing else.
+  void fuse_attention() {
+    bool changed = true;
+    while (changed) {
+      changed = false;
+      auto succ = successors();
+      for (size_t ri = 0; ri < nodes.size() && !changed; ++ri) {
+        Node& r = nodes[ri];
+        if (r.members.empty() || r.kind != NodeKind::kCluster) continue;
+        // producer GEMM
+        int g1i = -1;
+        bool ok = true;
+        for (int pn : producer_nodes(r.members)) {
+          if (nodes[pn].kind == NodeKind::kGemm) {
+            if (g1i >= 0) ok = false;
+            g1i = pn;
+          }
+        }
+        if (!ok || g1i < 0) continue;
+        Node& g1 = nodes[g1i];
+        if (g1.members.size() != 1 || succ[g1i].size() != 1 || succ[g1i][0] != static_cast<int>(ri)) continue;
+        if (succ[ri].size() != 1) continue;
+        int g2i = succ[ri][0];
+        Node& g2 = nodes[g2i];
+        if (g2.kind != NodeKind::kGemm) continue;
+        const Instr* gi1 = g1.members[0];
+        const Instr* gi2 = g2.members[0];
+        auto outs = codegen::external_outputs(p, r.members);
+        if (outs.size() != 1 || p.storage_root(gi2->operands[0]) != outs[0] || p.storage_root(gi2->operands[1]) == outs[0]) continue;
+        if (reaches_via_outside(g1i, static_cast<int>(ri), succ) || reaches_via_outside(static_cast<int>(ri), g2i, succ)) continue;
+        // the other producers of gemm2 (V) must not depend on gemm1 / the row program
+        const GemmDesc &d1 = g1.gemm, &d2 = g2.gemm;
+        if (!d1.a_k_contig || !d1.b_k_contig || !d2.a_k_contig || d2.has_addend || d1.has_addend) continue;
+        if (d2.batch != d1.batch || d2.M != d1.M || d2.K != d1.N) continue;
+        if (d1.K % 32 != 0 || d1.N % 32 != 0 || d2.N % 16 != 0 || d1.N > 512 || d2.N > 256 || d1.K > 256) continue;
+        const Instr* vroot = p.storage_root(gi2->operands[1]);
+        if (!d2.b_k_contig && !(opt.assign_operand_layouts && enabled("OperandLayoutPass") && can_store_k_contig(vroot, gi2->operands[1], gi2->gemm.rhs_contracting)))
+          continue;
+        std::vector<const Instr*> epi(g2.members.begin() + 1, g2.members.end());
+        if (!codegen::can_fuse_attention(p, gi1, d1, r.members, gi2, d2, epi)) continue;
+        Node a;
+        a.kind = NodeKind::kAttention;
+        a.name = g1.name + "_" + r.name + "_" + g2.name;
+        a.gemm = d1;
+        a.gemm2 = d2;
+        a.members.push_back(gi1);
+        a.members.insert(a.members.end(), r.members.begin(), r.members.end());
+        a.gemm2_index = a.members.size();
+        a.members.insert(a.members.end(), g2.members.begin(), g2.members.end());
+        for (auto* m : a.members) node_of_member[m] = g1i;
+        nodes[g1i] = a;
+        nodes[ri].members.clear();
+        nodes[g2i].members.clear();
+        changed = true;
+      }
+    }
+  }
+
   void finalize() {
     // compact, compute inputs/outputs, stages, order
     std::vector<Node> alive;
@@ -345,36 +423,26 @@ struct Builder {
   // nothing but such GEMMs reads) is stored [.., N, K]; its producer writes through the permutation.
   void assign_operand_layouts() {
     if (!opt.assign_operand_layouts || !enabled("OperandLayoutPass")) return;
-    for (auto& n : p.nodes) {
-      if (n.kind != NodeKind::kGemm || n.gemm.b_k_contig || n.gemm.b_packed || !n.gemm.a_k_contig || n.gemm.K % 32 != 0) continue;
-      const Instr* g = n.members[0];
+    auto each_gemm = [&](auto&& fn) {
+      for (auto& n : p.nodes) {
+        if (n.kind == NodeKind::kGemm) fn(n.members[0], n.gemm);
+        else if (n.kind == NodeKind::kAttention) fn(n.members[n.gemm2_index], n.gemm2);
+      }
+    };
+    each_gemm([&](const Instr* g, GemmDesc& d) {
+      if (d.b_k_contig || d.b_packed || !d.a_k_contig || d.K % 32 != 0) return;
       const Instr* root = p.storage_root(g->operands[1]);
-      if (!p.producer.count(root)) continue;                         // parameter / constant
-      if (root->shape.dims != g->operands[1]->shape.dims) continue;   // reached through a reshaping alias
-      bool ok = true;
-      std::function<void(const Instr*)> scan = [&](const Instr* v) {
-        for (auto* u : v->users) {
-          if (is_alias_op(u)) { ok = false; continue; }
-          bool as_b = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands[1] == v && u->operands[0] != v &&
-                      (u->operands.size() < 3 || u->operands[2] != v) && u->gemm.rhs_contracting == g->gemm.rhs_contracting;
-          if (!as_b) ok = false;
-        }
-      };
-      scan(root);
-      for (auto* lo : p.live_outs)
-        if (lo == root) ok = false;
-      if (!ok) continue;
+      if (!p.producer.count(root)) return;   // parameter / constant
+      if (!can_store_k_contig(root, g->operands[1], g->gemm.rhs_contracting)) return;
       int r = root->shape.rank();
       std::vector<int> perm(r);
       for (int i = 0; i < r; ++i) perm[i] = i;
       std::swap(perm[r - 1], perm[r - 2]);
       p.physical_perm[root] = perm;
-    }
-    for (auto& n : p.nodes) {
-      if (n.kind != NodeKind::kGemm) continue;
-      const Instr* root = p.storage_root(n.members[0]->operands[1]);
-      if (p.physical_perm.count(root)) n.gemm.b_k_contig = true;
-    }
+    });
+    each_gemm([&](const Instr* g, GemmDesc& d) {
+      if (p.physical_perm.count(p.storage_root(g->operands[1]))) d.b_k_contig = true;
+    });
   }
 
   void assign_buffers() {
@@ -460,6 +528,7 @@ std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, cons
   b.make_nodes();
   if (opt.merge_dependent && b.enabled("MergeDependentPass")) b.merge_dependent();
   if (opt.fuse_gemm_epilogue && b.enabled("GemmEpilogueFusionPass")) b.fuse_gemm_epilogues();
+  if (opt.fuse_attention && b.enabled("AttentionFusionPass")) b.fuse_attention();
   b.finalize();
   b.decide_constant_layouts();
   b.assign_operand_layouts();

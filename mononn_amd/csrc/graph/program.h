@@ -20,7 +20,9 @@
 namespace mononn {
 namespace graph {
 
-enum class NodeKind { kCluster, kGemm };
+// kAttention: GEMM -> row program over the GEMM's rows -> GEMM, executed by one wave per 16 rows with
+// the intermediate matrices kept in registers (members: [gemm1, row members..., gemm2, epilogue members...])
+enum class NodeKind { kCluster, kGemm, kAttention };
 
 struct GemmDesc {
   int64_t batch = 1, M = 0, N = 0, K = 0;
@@ -47,8 +49,11 @@ struct Node {
   bool has_reduce = false;
   bool row_program = false;       // reduces over the minor-most dim, rows handled by a wave / workgroup
   int64_t rows = 0, row_len = 0;
-  // GEMM
+  // GEMM (for kAttention: the first GEMM)
   GemmDesc gemm;
+  // kAttention: second GEMM and where it sits in `members`
+  GemmDesc gemm2;
+  size_t gemm2_index = 0;
   const hlo::Instr* gemm_instr() const { return kind == NodeKind::kGemm ? members[0] : nullptr; }
 };
 
@@ -90,6 +95,7 @@ struct BuildOptions {
   bool merge_dependent = true;          // glue producer/consumer clusters that share a row space
   bool fuse_gemm_epilogue = true;       // element-wise consumers of a GEMM run in its epilogue
   bool transpose_constant_b = true;     // store constant [K,N] GEMM operands in MFMA fragment order
+  bool fuse_attention = true;           // GEMM -> soft-max style row program -> GEMM in one stage
   bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
   bool reuse_temp_slots = true;         // false: every temp value gets its own address (written once per launch)
   std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)

@@ -69,6 +69,7 @@ struct HipOptions {       // "mononn_hip" section
   bool gemm_epilogue_fusion = true;
   bool transpose_constant_b = true;
   bool assign_operand_layouts = true;
+  bool fuse_attention = true;
   // "flags_coherent": fence-free flag barrier; stage outputs are written with agent-scope write-through
   // stores to temp addresses that are used once per launch, readers use cached loads.
   // "flags": the same barrier with agent-scope release/acquire (L2 write-back + invalidate) around it,

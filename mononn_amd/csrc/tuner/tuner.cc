@@ -262,7 +262,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             }
             add("tier" + std::to_string(tier) + "_ilp" + std::to_string(ilp), s);
           }
-      } else {
+      } else if (c.kind == "cluster_elewise") {
         for (int ilp : {2, 4, 8}) {
           GraphSpecification s = filled;
           for (auto& n : c.nodes) s.cluster_elewise_spec[n].ilp_factor = ilp;
@@ -360,7 +360,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       for (auto& n : c.nodes) {
         if (c.kind == "gemm") stitched.gemm_spec_list[n] = w.gemm_spec_list.at(n);
         else if (c.kind == "cluster_reduce") stitched.cluster_reduce_spec[n] = w.cluster_reduce_spec.at(n);
-        else stitched.cluster_elewise_spec[n] = w.cluster_elewise_spec.at(n);
+        else if (c.kind == "cluster_elewise") stitched.cluster_elewise_spec[n] = w.cluster_elewise_spec.at(n);
         report << ctx_str << "," << n << "," << best_class << "\n";
       }
       log << "  [" << ctx_str << "] " << c.kind << " x" << c.nodes.size() << " (" << c.nodes[0] << "): best " << trials[best_i].label << " "
