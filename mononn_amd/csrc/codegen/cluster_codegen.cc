@@ -1,6 +1,8 @@
 #include "codegen/cluster_codegen.h"
 
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <set>
 #include <sstream>
 
@@ -87,7 +89,7 @@ NodeFunction finish(const std::string& body, PointerTable& ptrs, const std::vect
   f.num_units = units;
   f.smem_bytes = smem;
   f.globals = globals;
-  f.text = pre + "__device__ __noinline__ void @NAME@(" + signature(ptrs.entries) + ") {\n" + align_prologue(ptrs.entries) + body + "}\n";
+  f.text = pre + "__device__ __forceinline__ void @NAME@(" + signature(ptrs.entries) + ") {\n" + align_prologue(ptrs.entries) + body + "}\n";
   return f;
 }
 
@@ -402,8 +404,13 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
   return t;
 }
 
-void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t) {
-  (void)g;
+void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t, bool has_prologue) {
+  if (has_prologue) {
+    const int tm = t.bm / std::max(t.wm, 1) / 16, tn = t.bn / std::max(t.wn, 1) / 16;
+    const int64_t ksteps = g.K / 32;
+    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && ksteps / t.wk <= 32 / (tm + tn), kSpecError)
+        << "GEMM with a row-program prologue: a wave's whole k range (" << ksteps / std::max(t.wk, 1) << " steps) must fit one register chunk";
+  }
   MONONN_CHECK(t.wm >= 1 && t.wn >= 1 && t.wk >= 1 && t.wm * t.wn * t.wk == ls.waves(), kSpecError)
       << "GEMM wave arrangement " << t.wm << "x" << t.wn << "x" << t.wk << " does not use " << ls.waves() << " waves";
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)
@@ -614,20 +621,201 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   return out_e;
 }
 
+// Row program (LayerNorm) on the A fragments of gemm_tile.  Lane (r16, g) of the wave with k slot wk
+// holds, for row fragment i and k step s, the 8 elements of row m_base + 16 i + r16 at columns
+// 32 (s WK + wk) + 8 g + e.  The program is generated as straight-line code over those CH * 8 values
+// per row fragment; a reduction ends with two butterfly steps over the 4 lanes of a row and one LDS
+// exchange between the WK waves.  The results replace the fragments in place.
+struct Prologue {
+  std::string struct_text;   // struct @NAME@_pro { ... };
+  std::string init_line;
+  std::vector<std::string> globals;
+  int smem = 0;
+  const Instr* primary = nullptr;   // the [M,K] input whose rows arrive as MFMA fragments
+};
+
+Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& row_members, const Instr* gi, const graph::GemmDesc& g,
+                        const GemmTuning& t, const LaunchShape& ls, bool stores, PointerTable& ptrs) {
+  (void)ls;
+  RowInfo info = analyze_rows(row_members);
+  MONONN_CHECK(info.row_program && info.rows == g.M && info.row_len == g.K && g.batch == 1, kUnsupported)
+      << "GEMM prologue: the cluster is not a row program over the rows of the left operand";
+  auto outs = external_outputs(prog, row_members);
+  MONONN_CHECK(outs.size() == 1 && prog.storage_root(gi->operands[0]) == outs[0] && outs[0]->shape.dtype == DType::kF16 &&
+                   outs[0]->shape.dims == std::vector<int64_t>({g.M, g.K}),
+               kUnsupported)
+      << "GEMM prologue: the row program must produce exactly the f16 [M,K] left operand";
+  const Instr* H = outs[0];
+  const int TM = t.bm / t.wm / 16, WK = t.wk, CH = static_cast<int>(g.K / 32 / WK);
+  // primary input: a [M,K] f16 value read by the cluster from outside
+  const Instr* primary = nullptr;
+  {
+    std::set<const Instr*> mem(row_members.begin(), row_members.end());
+    for (auto* m : row_members)
+      for (auto* o : m->operands) {
+        const Instr* r = prog.storage_root(o);
+        if (mem.count(r) || (r->opcode == "get-tuple-element" && mem.count(r->operands[0]))) continue;
+        if (!primary && r->shape.dtype == DType::kF16 && r->shape.dims == std::vector<int64_t>({g.M, g.K})) primary = r;
+      }
+  }
+  MONONN_CHECK(primary != nullptr, kUnsupported) << "GEMM prologue: no [M,K] f16 input to take the place of the left operand";
+  Prologue out;
+  out.primary = primary;
+  const size_t first = ptrs.entries.size();
+  CodeBuffer cb;
+  VarTable vars;
+  Emitter em(prog, row_members, cb, vars, ptrs);
+  std::vector<int> vm(TM);
+  for (int i = 0; i < TM; ++i) vm[i] = vars.add("m" + S(i), g.M);
+  int vwk = vars.add("wk", WK);
+  int vg = vars.add("g", 4);
+  auto col_of = [&](int s, int e) {
+    return LinExpr::variable(vwk, WK).scaled(32).plus(LinExpr::variable(vg, 4).scaled(8)).plus_const(static_cast<int64_t>(s) * WK * 32 + e);
+  };
+  auto primary_index = [&](int i, int s, int e) {
+    Index idx;
+    idx.push_back(LinExpr::variable(vm[i], g.M));
+    idx.push_back(col_of(s, e));
+    return idx;
+  };
+  auto operand_index = [&](const Instr* x, int i, int s, int e) {
+    // rows of the operand = leading dims; all leading dims together are the row
+    std::vector<int64_t> lead(x->shape.dims.begin(), x->shape.dims.end() - 1);
+    Index idx = delinearize(LinExpr::variable(vm[i], g.M), lead, vars);
+    idx.push_back(col_of(s, e));
+    return idx;
+  };
+  cb.line("const int lane = mononn_dev::lane_id();");
+  cb.line("const int r16 = lane & 15, g = lane >> 4;");
+  for (int i = 0; i < TM; ++i) {
+    cb.line("const bool mv" + S(i) + " = m_base + " + S(i * 16) + " + r16 < " + S(g.M) + ";");
+    cb.line("const int m" + S(i) + " = mv" + S(i) + " ? m_base + " + S(i * 16) + " + r16 : " + S(g.M - 1) + ";");
+  }
+  auto bind_elem = [&](int i, int s, int e) { em.bind(primary, primary_index(i, s, e), "a[" + S(s) + "][" + S(i) + "][" + S(e) + "]"); };
+  auto reduces = em.collect_reduces();
+  std::vector<std::vector<std::string>> reduce_accs_;   // [reduce][row fragment]
+  int smem = 0;
+  for (size_t ri = 0; ri < reduces.size(); ++ri) {
+    const Instr* red = reduces[ri];
+    std::string Tn = hlo::dtype_ctype(red->shape.dtype);
+    MONONN_CHECK(hlo::dtype_bytes(red->shape.dtype) <= 8, kUnsupported) << "reduction type too wide";
+    std::vector<std::string> accs;
+    for (int i = 0; i < TM; ++i) {
+      // earlier reductions of this row fragment are available to the operand of this one
+      for (size_t pj = 0; pj < ri; ++pj)
+        em.bind(reduces[pj], delinearize(LinExpr::variable(vm[i], g.M), reduces[pj]->shape.dims, vars), reduce_accs_[pj][i]);
+      std::string acc = em.fresh("red");
+      accs.push_back(acc);
+      cb.line(Tn + " " + acc + " = " + em.value(red->operands[1], {}) + ";");
+      for (int s = 0; s < CH; ++s)
+        for (int e = 0; e < 8; ++e) {
+          bind_elem(i, s, e);
+          std::string val = em.value(red->operands[0], operand_index(red->operands[0], i, s, e));
+          cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(red, acc, val) + ";");
+        }
+      for (int off : {16, 32}) {
+        std::string other = "__shfl_xor(" + acc + ", " + S(off) + ", 64)";
+        cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(red, acc, other) + ";");
+      }
+    }
+    if (WK > 1) {
+      // [mn wave][row fragment][wk][16 rows]
+      std::string buf = em.fresh("rb");
+      cb.line(Tn + "* " + buf + " = reinterpret_cast<" + Tn + "*>(smem + " + S(smem) + ") + mn_wave * " + S(TM * WK * 16) + ";");
+      smem += t.wm * t.wn * TM * WK * 16 * 8;
+      for (int i = 0; i < TM; ++i) cb.line("if (g == 0) " + buf + "[" + S(i * WK * 16) + " + wk * 16 + r16] = " + accs[i] + ";");
+      cb.line("__syncthreads();");
+      for (int i = 0; i < TM; ++i) {
+        cb.line(accs[i] + " = " + buf + "[" + S(i * WK * 16) + " + r16];");
+        for (int w = 1; w < WK; ++w)
+          cb.line(accs[i] + " = (" + Tn + ")" + Emitter::reducer_expr(red, accs[i], buf + "[" + S(i * WK * 16 + w * 16) + " + r16]") + ";");
+      }
+    }
+    reduce_accs_.push_back(accs);   // bound per row fragment where the results are consumed
+  }
+  // results replace the fragments
+  for (int i = 0; i < TM; ++i) {
+    for (size_t ri = 0; ri < reduces.size(); ++ri) {
+      Index ridx;
+      const Instr* red = reduces[ri];
+      ridx = delinearize(LinExpr::variable(vm[i], g.M), red->shape.dims, vars);
+      em.bind(red, ridx, reduce_accs_[ri][i]);
+    }
+    for (int s = 0; s < CH; ++s) {
+      std::vector<std::string> vals;
+      for (int e = 0; e < 8; ++e) {
+        bind_elem(i, s, e);
+        vals.push_back(em.value(em.resolve_output(H), primary_index(i, s, e)));
+      }
+      std::string arr = em.fresh("hn");
+      std::string init;
+      for (int e = 0; e < 8; ++e) init += (e ? ", " : "") + vals[e];
+      cb.line("const _Float16 " + arr + "[8] = {" + init + "};");
+      cb.line("a[" + S(s) + "][" + S(i) + "] = half8_t{" + arr + "[0], " + arr + "[1], " + arr + "[2], " + arr + "[3], " + arr + "[4], " + arr + "[5], " + arr + "[6], " + arr + "[7]};");
+      if (stores) {
+        LinExpr off = physical_offset(prog, H, primary_index(i, s, 0));
+        cb.line("if (store && mv" + S(i) + ") mononn_dev::stN<_Float16, 8>(" + ptrs.output(H) + " + " + off.str(vars) + ", " + arr + ");");
+      }
+    }
+  }
+  em.unbind(primary);
+  out.smem = smem;
+  for (auto& kv : em.literal_tables()) out.globals.push_back(kv.second);
+  std::string st = "struct @NAME@_pro {\n  static constexpr bool enabled = true;\n";
+  for (size_t i = first; i < ptrs.entries.size(); ++i) {
+    auto& e = ptrs.entries[i];
+    st += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
+  }
+  st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, char* smem) const {\n";
+  {
+    std::istringstream is(cb.text());
+    std::string l;
+    while (std::getline(is, l)) st += "  " + l + "\n";
+  }
+  st += "  }\n};\n";
+  out.struct_text = st;
+  std::string init = "@NAME@_pro pro{";
+  for (size_t i = first; i < ptrs.entries.size(); ++i) init += (i > first ? ", " : "") + ptrs.entries[i].name;
+  init += "};";
+  out.init_line = init;
+  return out;
+}
+
 NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
-                      const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t) {
+                      const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t,
+                      const std::vector<const Instr*>& prologue = {}, bool prologue_stores = false) {
   const Instr* gi = members[0];
   const bool mfma = gemm_uses_mfma(g);
-  if (mfma) validate_gemm_tuning(g, ls, t);
+  const bool has_pro = !prologue.empty();
+  MONONN_CHECK(!has_pro || mfma, kUnsupported) << gi->hlo_name << ": a row-program prologue needs the MFMA path";
+  if (mfma) validate_gemm_tuning(g, ls, t, has_pro);
   PointerTable ptrs;
-  // the two operands come first in the pointer list
-  std::string pa = ptrs.input(prog.storage_root(gi->operands[0]));
-  std::string pb = ptrs.input(prog.storage_root(gi->operands[1]));
+  // the two operands come first in the pointer list; with a prologue the left operand is the row
+  // program's input, whose rows are normalised on the way into the MFMAs
+  Prologue pro;
+  std::string pa, pb;
+  std::vector<const Instr*> epi_outputs = outputs;
+  if (has_pro) {
+    // find the primary input first (the pointer order must start with the operand the GEMM loads)
+    PointerTable probe_ptrs;
+    Prologue probe = build_prologue(prog, prologue, gi, g, t, ls, false, probe_ptrs);
+    pa = ptrs.input(probe.primary);
+    pb = ptrs.input(prog.storage_root(gi->operands[1]));
+    pro = build_prologue(prog, prologue, gi, g, t, ls, prologue_stores, ptrs);
+    auto pouts = external_outputs(prog, prologue);
+    epi_outputs.clear();
+    for (auto* o : outputs)
+      if (std::find(pouts.begin(), pouts.end(), o) == pouts.end()) epi_outputs.push_back(o);
+  } else {
+    pa = ptrs.input(prog.storage_root(gi->operands[0]));
+    pb = ptrs.input(prog.storage_root(gi->operands[1]));
+  }
   const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
   std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
-  Epilogue epi = build_epilogue(prog, gi, cluster_members, outputs, g, mfma, ptrs, first_epi);
+  Epilogue epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, ptrs, first_epi);
   CodeBuffer fb;
   fb.line(epi.init_line);
+  if (has_pro) fb.line(pro.init_line);
   int64_t units = 0;
   int smem = 0;
   if (mfma) {
@@ -653,9 +841,10 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     std::ostringstream call;
     call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << g.K << ", "
          << (g.b_packed ? "true" : "false") << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * "
-         << g.b_batch_stride << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem);";
+         << g.b_batch_stride << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem" << (has_pro ? ", pro" : "") << ");";
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
+    smem = std::max(smem, pro.smem);
   } else {
     const int64_t total = g.batch * g.M * g.N;
     units = (total + ls.block_size - 1) / ls.block_size;
@@ -671,7 +860,9 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fb.line(call.str());
     fb.close();
   }
-  return finish(fb.text(), ptrs, epi.globals, units, smem, epi.struct_text);
+  std::vector<std::string> globals = epi.globals;
+  for (auto& gl : pro.globals) globals.push_back(gl);
+  return finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text);
 }
 
 // GEMM -> row program -> GEMM with everything between the two contractions on chip.
@@ -880,13 +1071,32 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
 }  // namespace
 
 NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchShape& ls, const GemmTuning& t) {
-  return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t);
+  return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores);
 }
 
 NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls) {
   std::vector<const Instr*> row(node.members.begin() + 1, node.members.begin() + node.gemm2_index);
   std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.end());
   return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls);
+}
+
+bool can_fuse_prologue(const Program& prog, const std::vector<const Instr*>& row_members, const std::vector<const Instr*>& gemm_members,
+                       const graph::GemmDesc& g) {
+  try {
+    graph::GemmDesc d = g;
+    if (!d.a_k_contig || d.batch != 1 || d.K % 32 != 0) return false;
+    d.b_k_contig = true;   // constant weights are packed / activations re-laid out before real generation
+    LaunchShape ls;
+    GemmTuning t = default_gemm_tuning(d, ls, 256);
+    auto outs = external_outputs(prog, gemm_members);
+    if (outs.empty()) return false;
+    gen_gemm(prog, gemm_members, outs, d, ls, t, row_members, true);
+    return true;
+  } catch (const Error& e) {
+    if (getenv("MONONN_DEBUG_PASSES")) fprintf(stderr, "[prologue fusion rejected] %s\n", e.what());
+    if (e.code() == kUnsupported || e.code() == kSpecError) return false;
+    throw;
+  }
 }
 
 bool can_fuse_attention(const Program& prog, const Instr* gemm1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,

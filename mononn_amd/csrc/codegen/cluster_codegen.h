@@ -52,7 +52,7 @@ NodeFunction generate_attention(const graph::Program& prog, const graph::Node& n
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus);
 // throws Error(kSpecError) when the tile / wave arrangement cannot be generated for this GEMM
-void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t);
+void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t, bool has_prologue = false);
 bool gemm_uses_mfma(const graph::GemmDesc& g);
 
 // dry runs used by the merge passes
@@ -61,6 +61,9 @@ bool can_merge_clusters(const graph::Program& prog, const std::vector<const hlo:
                         const std::vector<const hlo::Instr*>& merged);
 bool can_fuse_epilogue(const graph::Program& prog, const std::vector<const hlo::Instr*>& gemm_members,
                        const std::vector<const hlo::Instr*>& cluster_members);
+
+bool can_fuse_prologue(const graph::Program& prog, const std::vector<const hlo::Instr*>& row_members,
+                       const std::vector<const hlo::Instr*>& gemm_members, const graph::GemmDesc& g);
 
 bool can_fuse_attention(const graph::Program& prog, const hlo::Instr* gemm1, const graph::GemmDesc& d1,
                         const std::vector<const hlo::Instr*>& row_members, const hlo::Instr* gemm2, const graph::GemmDesc& d2,

@@ -23,24 +23,38 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.transpose_constant_b = s.hip.transpose_constant_b;
   o.assign_operand_layouts = s.hip.assign_operand_layouts;
   o.fuse_attention = s.hip.fuse_attention;
+  o.fuse_gemm_prologue = s.hip.gemm_prologue_fusion;
   o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
   for (auto& p : env::disabled_passes()) o.disabled_passes.insert(p);
   return o;
 }
 
 namespace {
-std::string pointer_expr(const graph::Program& prog, const hlo::Instr* root, bool is_output, const std::map<const hlo::Instr*, std::string>& const_symbol) {
+// where a pointer argument of a node function comes from
+struct Operand {
+  std::string abs = "nullptr";   // module global (constants)
+  int base = -1;                 // >= 0: kernel argument ordinal (parameters, then live-outs, then temp)
+  int64_t off = 0;
+  std::string ctype;             // pointer type at the call site
+};
+
+Operand make_operand(const graph::Program& prog, const hlo::Instr* root, bool is_output, const std::map<const hlo::Instr*, std::string>& const_symbol,
+                     size_t n_params, size_t n_liveouts) {
   auto it = prog.buffers.find(root);
   MONONN_CHECK(it != prog.buffers.end(), kInternal) << "no buffer for " << root->hlo_name;
   const Buffer& b = it->second;
-  std::string T = std::string(is_output ? "" : "const ") + hlo::dtype_ctype(root->shape.dtype) + "*";
+  Operand o;
+  o.ctype = std::string(is_output ? "" : "const ") + hlo::dtype_ctype(root->shape.dtype) + "*";
   switch (b.kind) {
-    case Buffer::kParameter: return "(" + T + ")arg" + std::to_string(b.index);
-    case Buffer::kConstant: return "(" + T + ")" + const_symbol.at(root);
-    case Buffer::kLiveOut: return "(" + T + ")liveout_buffer_" + std::to_string(b.index);
-    case Buffer::kTemp: return "(" + T + ")((char*)temp_buffer + " + std::to_string(b.offset) + ")";
+    case Buffer::kParameter: o.base = b.index; break;
+    case Buffer::kConstant: o.abs = const_symbol.at(root); break;
+    case Buffer::kLiveOut: o.base = static_cast<int>(n_params) + b.index; break;
+    case Buffer::kTemp:
+      o.base = static_cast<int>(n_params + n_liveouts);
+      o.off = b.offset;
+      break;
   }
-  return "";
+  return o;
 }
 }  // namespace
 
@@ -104,9 +118,12 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   struct Call {
     const Node* node;
     std::string fn;
-    std::vector<std::string> args;
+    int fn_id = 0;
+    std::vector<Operand> args;
     int64_t units;
   };
+  std::map<std::string, int> fn_ids;
+  std::map<int, std::vector<std::string>> fn_arg_types;   // fn id -> pointer types of its arguments
   std::map<int, std::vector<Call>> by_stage;
   int smem = 0;
   for (auto& n : prog.nodes) {
@@ -172,6 +189,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       fn = known->second;
     } else if (emit) {
       fn = "node_fn_" + std::to_string(fn_by_text.size());
+      fn_ids[fn] = static_cast<int>(fn_by_text.size());
       fn_by_text[f.text] = fn;
       std::string def = f.text;
       size_t pos;
@@ -192,7 +210,10 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     c.node = &n;
     c.fn = fn;
     c.units = f.num_units;
-    for (auto& e : f.pointers) c.args.push_back(pointer_expr(prog, e.root, e.is_output, const_symbol));
+    c.fn_id = fn_ids.at(fn);
+    for (auto& e : f.pointers) c.args.push_back(make_operand(prog, e.root, e.is_output, const_symbol, hp.param_bytes.size(), hp.liveout_bytes.size()));
+    if (!fn_arg_types.count(c.fn_id))
+      for (auto& a : c.args) fn_arg_types[c.fn_id].push_back(a.ctype);
     by_stage[n.stage].push_back(c);
   }
   hp.smem = smem;
@@ -232,44 +253,87 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   glob << "\n";
   for (auto& d : fn_defs) src << d << "\n";
 
+  // The kernel is a small interpreter: a constant table lists, stage by stage, which node function
+  // runs on which buffers; every distinct node function is inlined exactly once, in one case of the
+  // dispatch switch.  Calling the functions instead would cost a save / restore of the callee-saved
+  // VGPRs through scratch memory on every stage, and inlining every use would multiply the code of a
+  // layer by the number of layers.
+  size_t max_ptrs = 1;
+  size_t n_calls = 0;
+  for (auto& st : by_stage)
+    for (auto& c : st.second) {
+      max_ptrs = std::max(max_ptrs, c.args.size());
+      ++n_calls;
+    }
+  const size_t n_bases = hp.param_bytes.size() + hp.liveout_bytes.size() + 1;
+  src << "struct MononnOperand { const void* abs; int base; long off; };\n";
+  src << "struct MononnCall { int fn; int units; MononnOperand p[" << max_ptrs << "]; };\n";
+  src << "__constant__ MononnCall mononn_calls[" << std::max<size_t>(n_calls, 1) << "] = {\n";
+  std::vector<int> stage_first, stage_units;
+  int call_index = 0;
+  for (auto& st : by_stage) {
+    stage_first.push_back(call_index);
+    int64_t total = 0;
+    hp.stage_nodes.emplace_back();
+    for (auto& c : st.second) {
+      hp.stage_nodes.back().push_back(c.node->name);
+      src << "  {" << c.fn_id << ", " << c.units << ", {";
+      for (size_t i = 0; i < c.args.size(); ++i)
+        src << (i ? ", " : "") << "{" << c.args[i].abs << ", " << c.args[i].base << ", " << c.args[i].off << "}";
+      src << "}},   // stage " << st.first << " " << c.node->name.substr(0, 60) << "\n";
+      total += c.units;
+      ++call_index;
+    }
+    MONONN_CHECK(total < (int64_t(1) << 31), kResourceExhausted) << "stage has too many work units";
+    stage_units.push_back(static_cast<int>(total));
+  }
+  if (n_calls == 0) src << "  {0, 0, {}}\n";
+  stage_first.push_back(call_index);
+  src << "};\n__constant__ int mononn_stage_first_call[" << stage_first.size() << "] = {";
+  for (size_t i = 0; i < stage_first.size(); ++i) src << (i ? ", " : "") << stage_first[i];
+  src << "};\n__constant__ int mononn_stage_units[" << std::max<size_t>(stage_units.size(), 1) << "] = {";
+  for (size_t i = 0; i < stage_units.size(); ++i) src << (i ? ", " : "") << stage_units[i];
+  if (stage_units.empty()) src << "0";
+  src << "};\n\n";
+  hp.num_barriers = by_stage.empty() ? 0 : static_cast<int>(by_stage.size()) - 1;
+
   src << "extern \"C\" __launch_bounds__(" << ls.block_size << ") __global__ void " << kernel_name << "(";
   for (size_t i = 0; i < hp.param_bytes.size(); ++i) src << "void* arg" << i << ", ";
   for (size_t i = 0; i < hp.liveout_bytes.size(); ++i) src << "void* liveout_buffer_" << i << ", ";
   src << "void* temp_buffer) {\n";
   src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
   src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags);\n";
-  bool first = true;
-  int stage_ordinal = 0;
-  for (auto& st : by_stage) {
-    if (!first) {
-      src << "  barrier.sync();\n";
-      ++hp.num_barriers;
-    }
-    first = false;
-    hp.stage_nodes.emplace_back();
-    for (auto& c : st.second) hp.stage_nodes.back().push_back(c.node->name);
-    if (hp.profiled)
-      src << "  if (threadIdx.x == 0) mononn_stage_clock[(" << stage_ordinal << " * " << hp.grid << " + blockIdx.x) * 2] = wall_clock64();\n";
-    int64_t total = 0;
-    for (auto& c : st.second) total += c.units;
-    src << "  // stage " << st.first << "\n";
-    src << "  for (int u = blockIdx.x; u < " << total << "; u += gridDim.x) {\n";
-    int64_t base = 0;
-    for (size_t i = 0; i < st.second.size(); ++i) {
-      auto& c = st.second[i];
-      src << "    " << (i ? "else " : "") << "if (u < " << base + c.units << ") " << c.fn << "(u - " << base;
-      for (auto& a : c.args) src << ", " << a;
-      src << ", smem);\n";
-      base += c.units;
-    }
-    src << "  }\n";
-    if (hp.profiled) {
-      src << "  __syncthreads();\n";
-      src << "  if (threadIdx.x == 0) mononn_stage_clock[(" << stage_ordinal << " * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
-    }
-    ++stage_ordinal;
+  src << "  auto resolve = [&](const MononnOperand& o) -> char* {\n    char* b = (char*)o.abs;\n    switch (o.base) {\n";
+  {
+    size_t k = 0;
+    for (size_t i = 0; i < hp.param_bytes.size(); ++i, ++k) src << "      case " << k << ": b = (char*)arg" << i << "; break;\n";
+    for (size_t i = 0; i < hp.liveout_bytes.size(); ++i, ++k) src << "      case " << k << ": b = (char*)liveout_buffer_" << i << "; break;\n";
+    src << "      case " << k << ": b = (char*)temp_buffer; break;\n";
+    (void)n_bases;
   }
-  src << "}\n";
+  src << "      default: break;\n    }\n    return b + o.off;\n  };\n";
+  src << "  for (int s = 0; s < " << by_stage.size() << "; ++s) {\n";
+  src << "    if (s) barrier.sync();\n";
+  if (hp.profiled) src << "    if (threadIdx.x == 0) mononn_stage_clock[(s * " << hp.grid << " + blockIdx.x) * 2] = wall_clock64();\n";
+  src << "    const int c_end = mononn_stage_first_call[s + 1];\n";
+  src << "    const int total = mononn_stage_units[s];\n";
+  src << "    for (int u = blockIdx.x; u < total; u += gridDim.x) {\n";
+  src << "      int c = mononn_stage_first_call[s], first = 0;\n";
+  src << "      while (c + 1 < c_end && u >= first + mononn_calls[c].units) first += mononn_calls[c++].units;\n";
+  src << "      const MononnCall& k = mononn_calls[c];\n";
+  src << "      const int unit = u - first;\n";
+  src << "      switch (k.fn) {\n";
+  for (auto& kv : fn_arg_types) {
+    src << "        case " << kv.first << ": node_fn_" << kv.first << "(unit";
+    for (size_t i = 0; i < kv.second.size(); ++i) src << ", (" << kv.second[i] << ")resolve(k.p[" << i << "])";
+    src << ", smem); break;\n";
+  }
+  src << "        default: break;\n      }\n    }\n";
+  if (hp.profiled) {
+    src << "    __syncthreads();\n";
+    src << "    if (threadIdx.x == 0) mononn_stage_clock[(s * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
+  }
+  src << "  }\n}\n";
   hp.preamble = pre.str();
   hp.body = src.str();
   hp.files["headers.h"] = device::kPreludeText;

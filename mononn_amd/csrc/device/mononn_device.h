@@ -225,9 +225,20 @@ __device__ __forceinline__ T sign_of(T x) {
 // Epilogue functor:  void prefetch(int batch, int m, int n) const   (touch what operator() will read)
 //                    void operator()(int batch, int m, int n, const float (&v)[4])   (n % 4 == 0)
 // Rows/cols beyond M / N are clamped on load and skipped on store, so M and N need not divide.
-template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, class Epi>
+//
+// Prologue functor (optional): a row program over the rows of A (LayerNorm) applied to the A
+// fragments in registers before they reach the MFMAs.  It needs a wave's whole k range resident
+// (one chunk).  Interface:  static constexpr bool enabled;
+//   void operator()(half8_t (&a)[CH][TM], int m_base, int wk, int mn_wave, bool store, char* smem)
+// `store` is true for the one wave column (wn == 0 of tile_n == 0) that also writes the transformed
+// rows to memory for later consumers.
+struct NoPrologue {
+  static constexpr bool enabled = false;
+};
+
+template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, class Epi, class Pro = NoPrologue>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
-                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem) {
+                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro()) {
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int KSTEPS = K / 32;
@@ -291,6 +302,10 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     for (int j = 0; j < TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   load_chunk(0, 0);
+  if constexpr (Pro::enabled) {
+    static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
+    pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, smem);
+  }
   // touch the epilogue's operands (bias, residual) now so that their latency overlaps the main loop
 #pragma unroll
   for (int i = 0; i < TM; ++i)

@@ -37,7 +37,7 @@ std::string Program::summary() const {
   os << "stages=" << num_stages << " nodes=" << nodes.size() << " temp_bytes=" << temp_bytes << "\n";
   for (auto& n : nodes) {
     os << "  stage " << n.stage << "  " << (n.kind == NodeKind::kGemm ? "gemm   " : n.kind == NodeKind::kAttention ? "attn   " : (n.row_program ? "rowred " : "elewise")) << " " << n.name;
-    if (n.kind == NodeKind::kGemm) os << "  [" << n.gemm.problem_hash() << "] members=" << n.members.size();
+    if (n.kind == NodeKind::kGemm) os << "  [" << n.gemm.problem_hash() << "] members=" << n.members.size() << (n.prologue.empty() ? "" : (n.prologue_stores ? " +row-prologue(stores)" : " +row-prologue"));
     else if (n.kind == NodeKind::kAttention) os << "  [" << n.gemm.problem_hash() << " -> " << n.gemm2.problem_hash() << "] members=" << n.members.size();
     else os << "  members=" << n.members.size() << (n.row_program ? " rows=" + std::to_string(n.rows) + " len=" + std::to_string(n.row_len) : "");
     os << "\n";
@@ -124,6 +124,12 @@ struct Builder {
     }
   }
 
+  static std::vector<const Instr*> with_prologue(const Node& n) {
+    std::vector<const Instr*> v = n.prologue;
+    v.insert(v.end(), n.members.begin(), n.members.end());
+    return v;
+  }
+
   // storage roots read by a set of members from outside the set
   std::vector<const Instr*> external_inputs(const std::vector<const Instr*>& members) const {
     std::set<const Instr*> in_set(members.begin(), members.end());
@@ -169,7 +175,7 @@ struct Builder {
     std::vector<std::vector<int>> succ(nodes.size());
     for (size_t i = 0; i < nodes.size(); ++i) {
       if (nodes[i].members.empty()) continue;
-      for (int pn : producer_nodes(nodes[i].members)) succ[pn].push_back(static_cast<int>(i));
+      for (int pn : producer_nodes(with_prologue(nodes[i]))) succ[pn].push_back(static_cast<int>(i));
     }
     return succ;
   }
@@ -248,6 +254,56 @@ struct Builder {
       for (auto* o : mroot->operands)
         if (p.storage_root(o) == root) return false;
     return true;
+  }
+
+  // A row program whose single product is the left operand of GEMMs (LayerNorm in front of the QKV /
+  // FFN projections) moves into those GEMMs: every workgroup normalises the rows of its own A panel in
+  // registers, so the stage of the row program and its barrier disappear.  One of the GEMMs keeps
+  // writing the product for consumers in later stages (the residual connection).
+  void fuse_gemm_prologues() {
+    for (size_t ri = 0; ri < nodes.size(); ++ri) {
+      Node& r = nodes[ri];
+      if (r.members.empty() || r.kind != NodeKind::kCluster) continue;
+      auto outs = codegen::external_outputs(p, r.members);
+      if (outs.size() != 1) continue;
+      const Instr* h = outs[0];
+      auto succ = successors();
+      std::vector<int> takers;
+      for (int ci : succ[ri]) {
+        Node& c = nodes[ci];
+        if (c.kind != NodeKind::kGemm || !c.prologue.empty()) continue;
+        const Instr* g = c.members[0];
+        if (p.storage_root(g->operands[0]) != h || p.storage_root(g->operands[1]) == h) continue;
+        if (g->operands.size() > 2 && p.storage_root(g->operands[2]) == h) continue;
+        bool reads_h_elsewhere = false;   // e.g. the epilogue of the same GEMM reading the row program's product
+        for (size_t k = 1; k < c.members.size(); ++k)
+          for (auto* o : c.members[k]->operands)
+            if (p.storage_root(o) == h) reads_h_elsewhere = true;
+        if (reads_h_elsewhere) continue;
+        if (!codegen::can_fuse_prologue(p, r.members, c.members, c.gemm)) continue;
+        takers.push_back(ci);
+      }
+      if (takers.empty()) continue;
+      // consumers that cannot take the row program in must come strictly later, i.e. read the stored copy;
+      // they may not be the GEMMs' own producers
+      bool conflict = false;
+      for (int ci : succ[ri]) {
+        if (std::find(takers.begin(), takers.end(), ci) != takers.end()) continue;
+        for (int t : takers)
+          if (reaches_via_outside(ci, t, succ) || ci == t) conflict = true;
+        for (int pn : producer_nodes(with_prologue(nodes[takers[0]])))
+          if (pn == ci) conflict = true;
+      }
+      if (conflict) continue;
+      for (size_t k = 0; k < takers.size(); ++k) {
+        Node& c = nodes[takers[k]];
+        c.prologue = r.members;
+        c.prologue_stores = k == 0;
+        c.name = r.name + "_" + c.name;
+      }
+      for (auto* m : r.members) node_of_member[m] = takers[0];
+      r.members.clear();
+    }
   }
 
   // GEMM -> row program -> GEMM (attention): the row program's only product feeds the second GEMM as
@@ -338,7 +394,7 @@ struct Builder {
     // users per storage root (entry level)
     std::map<const Instr*, std::set<int>> readers;
     for (size_t i = 0; i < nodes.size(); ++i) {
-      nodes[i].inputs = external_inputs(nodes[i].members);
+      nodes[i].inputs = external_inputs(with_prologue(nodes[i]));
       for (auto* r : nodes[i].inputs) readers[r].insert(static_cast<int>(i));
     }
     // outputs: values defined by a member and read by another node or live-out
@@ -353,6 +409,16 @@ struct Builder {
       }
       for (auto* v : cands)
         if (readers.count(v) || live_set.count(v)) n.outputs.push_back(v);
+      if (n.prologue_stores) {
+        // the absorbing GEMMs compute the row program's product themselves; `readers` holds everyone else
+        bool wanted = false;
+        for (auto* v : codegen::external_outputs(p, n.prologue))
+          if (readers.count(v) || live_set.count(v)) {
+            n.outputs.push_back(v);
+            wanted = true;
+          }
+        n.prologue_stores = wanted;
+      }
       MONONN_CHECK(!n.outputs.empty(), kUnsupported) << "node " << n.name << " has no consumer (dead code in the entry computation)";
       for (auto* v : n.outputs) p.producer[v] = static_cast<int>(i);
     }
@@ -526,9 +592,12 @@ std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, cons
   prog->module = std::move(module);
   Builder b{*prog, opt};
   b.make_nodes();
-  if (opt.merge_dependent && b.enabled("MergeDependentPass")) b.merge_dependent();
+  // epilogues first: a bias + residual fusion behind a GEMM belongs to that GEMM, not to the LayerNorm
+  // row program that follows it
   if (opt.fuse_gemm_epilogue && b.enabled("GemmEpilogueFusionPass")) b.fuse_gemm_epilogues();
+  if (opt.merge_dependent && b.enabled("MergeDependentPass")) b.merge_dependent();
   if (opt.fuse_attention && b.enabled("AttentionFusionPass")) b.fuse_attention();
+  if (opt.fuse_gemm_prologue && b.enabled("GemmPrologueFusionPass")) b.fuse_gemm_prologues();
   b.finalize();
   b.decide_constant_layouts();
   b.assign_operand_layouts();

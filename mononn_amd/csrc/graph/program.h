@@ -51,6 +51,10 @@ struct Node {
   int64_t rows = 0, row_len = 0;
   // GEMM (for kAttention: the first GEMM)
   GemmDesc gemm;
+  // kGemm: row program (LayerNorm) applied to the rows of the left operand inside the GEMM; the node
+  // with prologue_stores also writes the row program's result for consumers in later stages
+  std::vector<const hlo::Instr*> prologue;
+  bool prologue_stores = false;
   // kAttention: second GEMM and where it sits in `members`
   GemmDesc gemm2;
   size_t gemm2_index = 0;
@@ -95,6 +99,7 @@ struct BuildOptions {
   bool merge_dependent = true;          // glue producer/consumer clusters that share a row space
   bool fuse_gemm_epilogue = true;       // element-wise consumers of a GEMM run in its epilogue
   bool transpose_constant_b = true;     // store constant [K,N] GEMM operands in MFMA fragment order
+  bool fuse_gemm_prologue = false;      // row programs feeding a GEMM's left operand run inside that GEMM
   bool fuse_attention = true;           // GEMM -> soft-max style row program -> GEMM in one stage
   bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
   bool reuse_temp_slots = true;         // false: every temp value gets its own address (written once per launch)

@@ -131,6 +131,7 @@ Json GraphSpecification::to_json() const {
   h["transpose_constant_b"] = hip.transpose_constant_b;
   h["assign_operand_layouts"] = hip.assign_operand_layouts;
   h["fuse_attention"] = hip.fuse_attention;
+  h["gemm_prologue_fusion"] = hip.gemm_prologue_fusion;
   h["barrier"] = hip.barrier;
   h["profile_stages"] = hip.profile_stages;
   j["mononn_hip"] = h;
@@ -217,12 +218,13 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
   s.codegen_reject_list = strings_from(j, "codegen_reject_list");
   if (j.contains("mononn_hip")) {
     const Json& h = j.at("mononn_hip");
-    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "barrier", "profile_stages"}, "mononn_hip");
+    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "barrier", "profile_stages"}, "mononn_hip");
     s.hip.merge_dependent = getb(h, "merge_dependent", true);
     s.hip.gemm_epilogue_fusion = getb(h, "gemm_epilogue_fusion", true);
     s.hip.transpose_constant_b = getb(h, "transpose_constant_b", true);
     s.hip.assign_operand_layouts = getb(h, "assign_operand_layouts", true);
     s.hip.fuse_attention = getb(h, "fuse_attention", true);
+    s.hip.gemm_prologue_fusion = getb(h, "gemm_prologue_fusion", false);
     s.hip.barrier = gets(h, "barrier", "flags_coherent");
     s.hip.profile_stages = getb(h, "profile_stages", false);
   }

@@ -70,6 +70,9 @@ struct HipOptions {       // "mononn_hip" section
   bool transpose_constant_b = true;
   bool assign_operand_layouts = true;
   bool fuse_attention = true;
+  // LayerNorm inside the consuming GEMM: removes a stage and a barrier but every column tile repeats the
+  // row program on its rows, which only pays off when a GEMM has few column tiles; off unless tuned on
+  bool gemm_prologue_fusion = false;
   // "flags_coherent": fence-free flag barrier; stage outputs are written with agent-scope write-through
   // stores to temp addresses that are used once per launch, readers use cached loads.
   // "flags": the same barrier with agent-scope release/acquire (L2 write-back + invalidate) around it,

@@ -56,22 +56,39 @@ def test_stage_structure_and_function_sharing(layer):
     s = m.summary()
     stages = [int(x) for x in re.findall(r"^\s+stage (\d+)", s, re.M)]
     assert stages == sorted(stages)
-    assert max(stages) == 9 and m.launch_dims()["barriers"] == 8
-    # Q, K and V projections share a stage; soft-max and LayerNorm chains were merged into row programs
+    # QKV | attention | out-proj(+residual) | LayerNorm | FFN1(+GELU) | FFN2(+residual) | LayerNorm
+    assert max(stages) == 7 and m.launch_dims()["barriers"] == 6
+    # Q, K and V projections share a stage; scores -> soft-max -> context became one attention node;
+    # the LayerNorm chains were merged into row programs
     assert stages.count(1) == 3
-    assert len(re.findall(r"rowred", s)) == 3
+    assert len(re.findall(r"\battn\b", s)) == 1 and len(re.findall(r"rowred", s)) == 2
     two = MonoNNModule.compile(models.bert_encoder(L=2, B=1, S=32, H=128, NH=4, F=256, vocab=100, max_pos=64).hlo_text, build=False)
     one = MonoNNModule.compile(models.bert_encoder(L=1, B=1, S=32, H=128, NH=4, F=256, vocab=100, max_pos=64).hlo_text, build=False)
-    n2 = len(re.findall(r"__noinline__ void node_fn_", two.get_source()))
-    n1 = len(re.findall(r"__noinline__ void node_fn_", one.get_source()))
+    n2 = len(re.findall(r"__forceinline__ void node_fn_", two.get_source()))
+    n1 = len(re.findall(r"__forceinline__ void node_fn_", one.get_source()))
+    assert n1 >= 5
     assert n2 <= n1 + 1, "a repeated layer must reuse the device functions of the first one"
 
 
 def test_disabled_pass_env(layer, monkeypatch):
     base = MonoNNModule.compile(layer.hlo_text, build=False).launch_dims()["barriers"]
-    monkeypatch.setenv("MONONN_OPTIMIZATION_DISABLED_PASS", "MergeDependentPass,GemmEpilogueFusionPass")
+    monkeypatch.setenv("MONONN_OPTIMIZATION_DISABLED_PASS", "AttentionFusionPass")
+    no_attn = MonoNNModule.compile(layer.hlo_text, build=False).launch_dims()["barriers"]
+    assert no_attn == base + 2
+    monkeypatch.setenv("MONONN_OPTIMIZATION_DISABLED_PASS", "AttentionFusionPass,MergeDependentPass,GemmEpilogueFusionPass")
     unfused = MonoNNModule.compile(layer.hlo_text, build=False).launch_dims()["barriers"]
-    assert unfused > base
+    assert unfused > no_attn
+
+
+def test_fusion_decisions_in_spec(layer):
+    spec = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
+    base = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False).launch_dims()["barriers"]
+    spec["mononn_hip"]["gemm_prologue_fusion"] = True      # LayerNorm inside the FFN1 GEMM
+    spec["gemm_spec_list"] = {}
+    spec["cluster_reduce_spec"] = {}
+    fused = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
+    assert fused.launch_dims()["barriers"] == base - 1
+    assert "+row-prologue(stores)" in fused.summary()
 
 
 def test_spec_round_trip_and_reload(layer, tmp_path):
@@ -213,8 +230,21 @@ def test_write_once_temp_addresses(layer):
     coherent = MonoNNModule.compile(layer.hlo_text, build=False)
     spec = json.loads(coherent.get_tuning_spec())
     assert spec["mononn_hip"]["barrier"] == "flags_coherent"
-    offs = re.findall(r"\(_Float16\*\)\(\(char\*\)temp_buffer \+ (\d+)\)", coherent.get_source())
-    assert len(offs) == len(set(offs)), "a temp slot is written by two nodes"
+    src = coherent.get_source()
+    # operands with base == temp (ordinal 3: two parameters, one live-out, then temp) that are outputs: every
+    # output offset appears in exactly one call
+    calls = re.findall(r"^  \{(\d+), \d+, \{(.*)\}\},", src, re.M)
+    assert calls
+    written = []
+    sigs = {int(i): sig for i, sig in re.findall(r"void node_fn_(\d+)\(int unit, ([^)]*)\)", src)}
+    for fn, ops in calls:
+        params = [p.strip() for p in sigs[int(fn)].split(",")][:-1]
+        operands = re.findall(r"\{([^{}]*)\}", ops)
+        for prm, op in zip(params, operands):
+            _abs, base, off = [x.strip() for x in op.split(",")]
+            if not prm.startswith("const") and base == "3":
+                written.append(int(off))
+    assert written and len(written) == len(set(written)), "a temp slot is written by two nodes"
     assert "MONONN_COHERENT_STORES 1" in coherent.get_source()
     spec["mononn_hip"]["barrier"] = "flags"
     fenced = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
