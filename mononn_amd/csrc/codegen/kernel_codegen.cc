@@ -253,49 +253,45 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   glob << "\n";
   for (auto& d : fn_defs) src << d << "\n";
 
-  // The kernel is a small interpreter: a constant table lists, stage by stage, which node function
-  // runs on which buffers; every distinct node function is inlined exactly once, in one case of the
-  // dispatch switch.  Calling the functions instead would cost a save / restore of the callee-saved
-  // VGPRs through scratch memory on every stage, and inlining every use would multiply the code of a
-  // layer by the number of layers.
+  // The kernel is a small interpreter over the list of calls (node function + buffers), stage by stage.
+  // Every distinct node function is inlined exactly once, in one case of the dispatch switch: calling
+  // the functions would cost a save / restore of the callee-saved VGPRs through scratch memory on
+  // every stage, and inlining every use would multiply the code of a layer by the number of layers.
+  // The parameters of a call are set up by a second switch from immediates (kernel argument + offset,
+  // or the address of a module global), so no table has to be fetched from memory on the critical path.
   size_t max_ptrs = 1;
-  size_t n_calls = 0;
   for (auto& st : by_stage)
-    for (auto& c : st.second) {
-      max_ptrs = std::max(max_ptrs, c.args.size());
-      ++n_calls;
-    }
-  const size_t n_bases = hp.param_bytes.size() + hp.liveout_bytes.size() + 1;
-  src << "struct MononnOperand { const void* abs; int base; long off; };\n";
-  src << "struct MononnCall { int fn; int units; MononnOperand p[" << max_ptrs << "]; };\n";
-  src << "__constant__ MononnCall mononn_calls[" << std::max<size_t>(n_calls, 1) << "] = {\n";
-  std::vector<int> stage_first, stage_units;
-  int call_index = 0;
+    for (auto& c : st.second) max_ptrs = std::max(max_ptrs, c.args.size());
+  struct Flat {
+    const Call* call;
+    int first_unit, stage_total;
+    bool new_stage;
+  };
+  std::vector<Flat> flat;
   for (auto& st : by_stage) {
-    stage_first.push_back(call_index);
     int64_t total = 0;
+    for (auto& c : st.second) total += c.units;
+    MONONN_CHECK(total < (int64_t(1) << 31), kResourceExhausted) << "stage has too many work units";
     hp.stage_nodes.emplace_back();
+    int64_t first = 0;
+    bool ns = true;
     for (auto& c : st.second) {
       hp.stage_nodes.back().push_back(c.node->name);
-      src << "  {" << c.fn_id << ", " << c.units << ", {";
-      for (size_t i = 0; i < c.args.size(); ++i)
-        src << (i ? ", " : "") << "{" << c.args[i].abs << ", " << c.args[i].base << ", " << c.args[i].off << "}";
-      src << "}},   // stage " << st.first << " " << c.node->name.substr(0, 60) << "\n";
-      total += c.units;
-      ++call_index;
+      flat.push_back({&c, static_cast<int>(first), static_cast<int>(total), ns});
+      ns = false;
+      first += c.units;
     }
-    MONONN_CHECK(total < (int64_t(1) << 31), kResourceExhausted) << "stage has too many work units";
-    stage_units.push_back(static_cast<int>(total));
   }
-  if (n_calls == 0) src << "  {0, 0, {}}\n";
-  stage_first.push_back(call_index);
-  src << "};\n__constant__ int mononn_stage_first_call[" << stage_first.size() << "] = {";
-  for (size_t i = 0; i < stage_first.size(); ++i) src << (i ? ", " : "") << stage_first[i];
-  src << "};\n__constant__ int mononn_stage_units[" << std::max<size_t>(stage_units.size(), 1) << "] = {";
-  for (size_t i = 0; i < stage_units.size(); ++i) src << (i ? ", " : "") << stage_units[i];
-  if (stage_units.empty()) src << "0";
-  src << "};\n\n";
   hp.num_barriers = by_stage.empty() ? 0 : static_cast<int>(by_stage.size()) - 1;
+  auto base_expr = [&](const Operand& o) -> std::string {
+    if (o.base < 0) return "(char*)" + o.abs;
+    std::string b;
+    size_t np = hp.param_bytes.size(), nl = hp.liveout_bytes.size();
+    if (static_cast<size_t>(o.base) < np) b = "(char*)arg" + std::to_string(o.base);
+    else if (static_cast<size_t>(o.base) < np + nl) b = "(char*)liveout_buffer_" + std::to_string(o.base - np);
+    else b = "(char*)temp_buffer";
+    return o.off ? b + " + " + std::to_string(o.off) : b;
+  };
 
   src << "extern \"C\" __launch_bounds__(" << ls.block_size << ") __global__ void " << kernel_name << "(";
   for (size_t i = 0; i < hp.param_bytes.size(); ++i) src << "void* arg" << i << ", ";
@@ -303,37 +299,44 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   src << "void* temp_buffer) {\n";
   src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
   src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags);\n";
-  src << "  auto resolve = [&](const MononnOperand& o) -> char* {\n    char* b = (char*)o.abs;\n    switch (o.base) {\n";
-  {
-    size_t k = 0;
-    for (size_t i = 0; i < hp.param_bytes.size(); ++i, ++k) src << "      case " << k << ": b = (char*)arg" << i << "; break;\n";
-    for (size_t i = 0; i < hp.liveout_bytes.size(); ++i, ++k) src << "      case " << k << ": b = (char*)liveout_buffer_" << i << "; break;\n";
-    src << "      case " << k << ": b = (char*)temp_buffer; break;\n";
-    (void)n_bases;
+  src << "  int stage = -1;\n";
+  src << "  for (int c = 0; c < " << flat.size() << "; ++c) {\n";
+  src << "    int fn = 0, units = 0, first = 0, total = 0;\n    bool new_stage = false;\n";
+  src << "    char*";
+  for (size_t i = 0; i < max_ptrs; ++i) src << (i ? ", *" : " ") << "p" << i << " = nullptr";
+  src << ";\n";
+  src << "    switch (c) {\n";
+  for (size_t i = 0; i < flat.size(); ++i) {
+    const Flat& f = flat[i];
+    src << "      case " << i << ": fn = " << f.call->fn_id << "; units = " << f.call->units << "; first = " << f.first_unit << "; total = "
+        << f.stage_total << "; new_stage = " << (f.new_stage ? "true" : "false") << ";";
+    for (size_t a = 0; a < f.call->args.size(); ++a) src << " p" << a << " = " << base_expr(f.call->args[a]) << ";";
+    src << " break;   // " << f.call->node->name.substr(0, 50) << "\n";
   }
-  src << "      default: break;\n    }\n    return b + o.off;\n  };\n";
-  src << "  for (int s = 0; s < " << by_stage.size() << "; ++s) {\n";
-  src << "    if (s) barrier.sync();\n";
-  if (hp.profiled) src << "    if (threadIdx.x == 0) mononn_stage_clock[(s * " << hp.grid << " + blockIdx.x) * 2] = wall_clock64();\n";
-  src << "    const int c_end = mononn_stage_first_call[s + 1];\n";
-  src << "    const int total = mononn_stage_units[s];\n";
+  src << "      default: break;\n    }\n";
+  src << "    if (new_stage) {\n";
+  if (hp.profiled) {
+    src << "      if (stage >= 0) {\n        __syncthreads();\n";
+    src << "        if (threadIdx.x == 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n      }\n";
+  }
+  src << "      if (stage >= 0) barrier.sync();\n      ++stage;\n";
+  if (hp.profiled) src << "      if (threadIdx.x == 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2] = wall_clock64();\n";
+  src << "    }\n";
   src << "    for (int u = blockIdx.x; u < total; u += gridDim.x) {\n";
-  src << "      int c = mononn_stage_first_call[s], first = 0;\n";
-  src << "      while (c + 1 < c_end && u >= first + mononn_calls[c].units) first += mononn_calls[c++].units;\n";
-  src << "      const MononnCall& k = mononn_calls[c];\n";
   src << "      const int unit = u - first;\n";
-  src << "      switch (k.fn) {\n";
+  src << "      if (unit < 0 || unit >= units) continue;\n";
+  src << "      switch (fn) {\n";
   for (auto& kv : fn_arg_types) {
     src << "        case " << kv.first << ": node_fn_" << kv.first << "(unit";
-    for (size_t i = 0; i < kv.second.size(); ++i) src << ", (" << kv.second[i] << ")resolve(k.p[" << i << "])";
+    for (size_t i = 0; i < kv.second.size(); ++i) src << ", (" << kv.second[i] << ")p" << i;
     src << ", smem); break;\n";
   }
-  src << "        default: break;\n      }\n    }\n";
+  src << "        default: break;\n      }\n    }\n  }\n";
   if (hp.profiled) {
-    src << "    __syncthreads();\n";
-    src << "    if (threadIdx.x == 0) mononn_stage_clock[(s * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
+    src << "  __syncthreads();\n";
+    src << "  if (threadIdx.x == 0 && stage >= 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
   }
-  src << "  }\n}\n";
+  src << "}\n";
   hp.preamble = pre.str();
   hp.body = src.str();
   hp.files["headers.h"] = device::kPreludeText;

@@ -217,16 +217,40 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       bufs.ptrs.push_back(nullptr);
       alloc_zero(&bufs.ptrs.back(), static_cast<size_t>(hp.temp_bytes));
     }
-    std::map<std::string, ClassInfo> classes;
+    // Node classes: nodes that came out as the same device function.  GEMM classes that solve the same
+    // problem in the same stages (the Q, K and V projections of a layer) are tuned as one class, because
+    // their tiles share the workgroups of that stage.
+    std::map<std::string, ClassInfo> by_fn;
+    std::map<std::string, std::vector<int>> stages_of_fn;
     for (auto& r : def.hip_program().nodes) {
-      ClassInfo& c = classes[r.function];
+      ClassInfo& c = by_fn[r.function];
       c.function = r.function;
       c.kind = r.kind;
       c.nodes.push_back(r.name);
+      stages_of_fn[r.function].push_back(r.stage);
     }
     for (auto& n : def.program().nodes)
-      for (auto& kv : classes)
+      for (auto& kv : by_fn)
         if (!kv.second.sample && kv.second.nodes[0] == n.name) kv.second.sample = &n;
+    std::map<std::string, ClassInfo> classes;
+    for (auto& kv : by_fn) {
+      std::string key = kv.first;
+      if (kv.second.kind == "gemm" && kv.second.sample) {
+        const graph::GemmDesc& g = kv.second.sample->gemm;
+        std::ostringstream k;
+        k << "gemm|" << g.batch << "x" << g.M << "x" << g.N << "x" << g.K << "|" << (kv.second.sample->prologue.empty() ? 0 : 1) << "|";
+        std::set<int> distinct(stages_of_fn[kv.first].begin(), stages_of_fn[kv.first].end());
+        for (int st : distinct) k << st << ",";
+        key = k.str();
+      }
+      ClassInfo& c = classes[key];
+      if (c.nodes.empty()) {
+        c = kv.second;
+        c.function = key;
+      } else {
+        c.nodes.insert(c.nodes.end(), kv.second.nodes.begin(), kv.second.nodes.end());
+      }
+    }
 
     // ---- candidates of every class ------------------------------------------------------------
     std::vector<Trial> trials;

@@ -231,19 +231,13 @@ def test_write_once_temp_addresses(layer):
     spec = json.loads(coherent.get_tuning_spec())
     assert spec["mononn_hip"]["barrier"] == "flags_coherent"
     src = coherent.get_source()
-    # operands with base == temp (ordinal 3: two parameters, one live-out, then temp) that are outputs: every
-    # output offset appears in exactly one call
-    calls = re.findall(r"^  \{(\d+), \d+, \{(.*)\}\},", src, re.M)
-    assert calls
+    sigs = {int(i): [p.strip() for p in sig.split(",")][:-1] for i, sig in re.findall(r"void node_fn_(\d+)\(int unit, ([^)]*)\)", src)}
     written = []
-    sigs = {int(i): sig for i, sig in re.findall(r"void node_fn_(\d+)\(int unit, ([^)]*)\)", src)}
-    for fn, ops in calls:
-        params = [p.strip() for p in sigs[int(fn)].split(",")][:-1]
-        operands = re.findall(r"\{([^{}]*)\}", ops)
-        for prm, op in zip(params, operands):
-            _abs, base, off = [x.strip() for x in op.split(",")]
-            if not prm.startswith("const") and base == "3":
-                written.append(int(off))
+    for fn, rest in re.findall(r"case \d+: fn = (\d+); units = \d+; first = \d+; total = \d+; new_stage = \w+;(.*?) break;", src):
+        ptrs = dict(re.findall(r"p(\d+) = ([^;]*);", rest))
+        for i, prm in enumerate(sigs[int(fn)]):
+            if not prm.startswith("const") and "temp_buffer" in ptrs[str(i)]:
+                written.append(ptrs[str(i)])
     assert written and len(written) == len(set(written)), "a temp slot is written by two nodes"
     assert "MONONN_COHERENT_STORES 1" in coherent.get_source()
     spec["mononn_hip"]["barrier"] = "flags"
