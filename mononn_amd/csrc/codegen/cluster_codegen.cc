@@ -411,6 +411,7 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
     MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && ksteps / t.wk <= 32 / (tm + tn), kSpecError)
         << "GEMM with a row-program prologue: a wave's whole k range (" << ksteps / std::max(t.wk, 1) << " steps) must fit one register chunk";
   }
+  MONONN_CHECK(t.split_k >= 1 && g.K % (32 * t.split_k) == 0, kSpecError) << "split_k " << t.split_k << " does not divide the k steps of the GEMM";
   MONONN_CHECK(t.wm >= 1 && t.wn >= 1 && t.wk >= 1 && t.wm * t.wn * t.wk == ls.waves(), kSpecError)
       << "GEMM wave arrangement " << t.wm << "x" << t.wn << "x" << t.wk << " does not use " << ls.waves() << " waves";
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)
@@ -434,6 +435,26 @@ struct Epilogue {
 Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<const Instr*>& cluster_members,
                         const std::vector<const Instr*>& outputs, const graph::GemmDesc& g, bool mfma, PointerTable& ptrs,
                         size_t first_epi) {
+  if (g.split_k > 1) {
+    // fp32 partial sums [split][batch][M][N]; the consumers add them up and apply the rounding
+    MONONN_CHECK(mfma && g.N % 4 == 0 && cluster_members.empty() && outputs.size() == 1 && outputs[0] == gi && !g.has_addend, kSpecError)
+        << gi->hlo_name << ": split_k needs the MFMA path, N % 4 == 0 and no fused epilogue";
+    std::string po = ptrs.output(gi, DType::kF32);
+    std::ostringstream al;
+    al.precision(9);
+    al << g.alpha;
+    std::string a = al.str();
+    if (a.find_first_of(".e") == std::string::npos) a += ".0";
+    Epilogue e;
+    e.struct_text = "struct @NAME@_epi {\n  float* out;\n  int ksplit;\n"
+                    "  __device__ __forceinline__ void prefetch(int, int, int) const {}\n"
+                    "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4]) const {\n"
+                    "    const float v[4] = {acc[0] * " + a + "f, acc[1] * " + a + "f, acc[2] * " + a + "f, acc[3] * " + a + "f};\n"
+                    "    mononn_dev::stN<float, 4>(out + (long)ksplit * " + S(g.batch * g.M * g.N) + " + (long)bidx * " + S(g.M * g.N) + " + m * " + S(g.N) + " + n0, v);\n"
+                    "  }\n};\n";
+    e.init_line = "@NAME@_epi epi{" + po + ", ksplit};";
+    return e;
+  }
   const bool vec4 = mfma && g.N % 4 == 0;
   CodeBuffer cb;   // epilogue body
   VarTable vars;
@@ -814,7 +835,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
   Epilogue epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, ptrs, first_epi);
   CodeBuffer fb;
-  fb.line(epi.init_line);
+  if (g.split_k <= 1) fb.line(epi.init_line);
   if (has_pro) fb.line(pro.init_line);
   int64_t units = 0;
   int smem = 0;
@@ -823,25 +844,27 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     // multiples of 8 in their unit index; with units dealt round-robin over the 8 XCDs they land on
     // one XCD and share its L2.  tile_n = 8 * (q / tiles_m) + u % 8, tile_m = q % tiles_m, q = u / 8.
     const int64_t tiles_m = (g.M + t.bm - 1) / t.bm, tiles_n = (g.N + t.bn - 1) / t.bn;
-    if (tiles_n % 8 == 0) {
-      const int64_t per_batch = tiles_n * tiles_m;
-      units = g.batch * per_batch;
-      fb.line("const int bidx = unit / " + S(per_batch) + ";");
-      fb.line("const int rem = unit % " + S(per_batch) + ";");
+    const int S_ = std::max(1, g.split_k);
+    const int64_t KS = g.K / S_;   // k extent of one split
+    const int64_t per_batch = tiles_n * tiles_m * S_;
+    units = g.batch * per_batch;
+    fb.line("const int bidx = unit / " + S(per_batch) + ";");
+    fb.line("const int rem0 = unit % " + S(per_batch) + ";");
+    fb.line("const int ksplit = rem0 % " + S(S_) + ";");
+    fb.line("const int rem = rem0 / " + S(S_) + ";");
+    if (g.split_k > 1) fb.line(epi.init_line);
+    if (tiles_n % 8 == 0 && S_ == 1) {
       fb.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
       fb.line("const int tile_m = (rem >> 3) % " + S(tiles_m) + ";");
     } else {
-      const int64_t per_batch = tiles_n * tiles_m;
-      units = g.batch * per_batch;
-      fb.line("const int bidx = unit / " + S(per_batch) + ";");
-      fb.line("const int rem = unit % " + S(per_batch) + ";");
       fb.line("const int tile_n = rem / " + S(tiles_m) + ";");
       fb.line("const int tile_m = rem % " + S(tiles_m) + ";");
     }
     std::ostringstream call;
-    call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << g.K << ", "
-         << (g.b_packed ? "true" : "false") << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * "
-         << g.b_batch_stride << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem" << (has_pro ? ", pro" : "") << ");";
+    call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
+         << (g.b_packed ? "true" : "false") << ", " << g.K << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << KS << ", " << pb
+         << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS) << ", " << g.M << ", " << g.N << ", " << g.K << ", "
+         << g.K << ", bidx, tile_m, tile_n, epi, smem" << (has_pro ? ", pro" : "") << ");";
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
     smem = std::max(smem, pro.smem);

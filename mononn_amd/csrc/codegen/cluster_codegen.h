@@ -30,6 +30,7 @@ struct ClusterTuning {
 struct GemmTuning {
   int bm = 32, bn = 32;      // workgroup tile
   int wm = 1, wn = 1, wk = 4;   // wave arrangement; wm*wn*wk == waves per workgroup
+  int split_k = 1;              // k range also split over workgroups (fp32 partial sums to memory)
 };
 
 struct NodeFunction {

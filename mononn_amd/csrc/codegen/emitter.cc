@@ -28,20 +28,20 @@ void CodeBuffer::close(const std::string& tail) {
   line("}" + tail);
 }
 
-std::string PointerTable::input(const Instr* root) {
+std::string PointerTable::input(const Instr* root, DType as) {
   for (auto& e : entries)
     if (e.root == root && !e.is_output) return e.name;
   int n = 0;
   for (auto& e : entries) n += e.is_output ? 0 : 1;
-  entries.push_back({root, false, "in" + std::to_string(n), root->shape.dtype});
+  entries.push_back({root, false, "in" + std::to_string(n), as == DType::kInvalid ? root->shape.dtype : as});
   return entries.back().name;
 }
-std::string PointerTable::output(const Instr* root) {
+std::string PointerTable::output(const Instr* root, DType as) {
   for (auto& e : entries)
     if (e.root == root && e.is_output) return e.name;
   int n = 0;
   for (auto& e : entries) n += e.is_output ? 1 : 0;
-  entries.push_back({root, true, "out" + std::to_string(n), root->shape.dtype});
+  entries.push_back({root, true, "out" + std::to_string(n), as == DType::kInvalid ? root->shape.dtype : as});
   return entries.back().name;
 }
 
@@ -216,6 +216,20 @@ std::string Emitter::value(const Instr* ins, const Index& idx) {
 
 std::string Emitter::load(const Instr* root, const Index& idx) {
   LinExpr lin = physical_offset(prog_, root, idx);
+  auto sk = prog_.split_k.find(root);
+  if (sk != prog_.split_k.end()) {
+    // split-K GEMM result: S fp32 partial sums, added in a fixed order, then rounded to the f16 value
+    // the HLO defines
+    std::string p = ptrs_.input(root, DType::kF32);
+    const int64_t E = root->shape.num_elements();
+    std::string sum;
+    for (int i = 0; i < sk->second; ++i) {
+      std::string ref = p + "[" + lin.plus_const(i * E).str(vars_) + "]";
+      if (lin.opaques().empty()) simple_loads_.push_back(ref);
+      sum += (i ? " + " : "") + ref;
+    }
+    return def(root->shape.dtype, "(" + std::string(hlo::dtype_ctype(root->shape.dtype)) + ")(" + sum + ")");
+  }
   std::string ref = ptrs_.input(root) + "[" + lin.str(vars_) + "]";
   if (lin.opaques().empty()) simple_loads_.push_back(ref);
   return def(root->shape.dtype, ref);

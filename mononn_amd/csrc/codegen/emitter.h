@@ -47,8 +47,8 @@ struct PointerTable {
     hlo::DType dtype;
   };
   std::vector<Entry> entries;
-  std::string input(const hlo::Instr* root);
-  std::string output(const hlo::Instr* root);
+  std::string input(const hlo::Instr* root, hlo::DType as = hlo::DType::kInvalid);    // `as`: element type override
+  std::string output(const hlo::Instr* root, hlo::DType as = hlo::DType::kInvalid);
 };
 
 // element offset of `idx` inside the buffer of storage root `root`, honouring a permuted physical layout

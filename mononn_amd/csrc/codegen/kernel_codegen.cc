@@ -25,6 +25,8 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.fuse_attention = s.hip.fuse_attention;
   o.fuse_gemm_prologue = s.hip.gemm_prologue_fusion;
   o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
+  for (auto& kv : s.gemm_spec_list)
+    if (kv.second.split_k > 1) o.gemm_split_k[kv.first] = kv.second.split_k;
   for (auto& p : env::disabled_passes()) o.disabled_passes.insert(p);
   return o;
 }
@@ -38,13 +40,13 @@ struct Operand {
   std::string ctype;             // pointer type at the call site
 };
 
-Operand make_operand(const graph::Program& prog, const hlo::Instr* root, bool is_output, const std::map<const hlo::Instr*, std::string>& const_symbol,
-                     size_t n_params, size_t n_liveouts) {
+Operand make_operand(const graph::Program& prog, const hlo::Instr* root, bool is_output, hlo::DType elem,
+                     const std::map<const hlo::Instr*, std::string>& const_symbol, size_t n_params, size_t n_liveouts) {
   auto it = prog.buffers.find(root);
   MONONN_CHECK(it != prog.buffers.end(), kInternal) << "no buffer for " << root->hlo_name;
   const Buffer& b = it->second;
   Operand o;
-  o.ctype = std::string(is_output ? "" : "const ") + hlo::dtype_ctype(root->shape.dtype) + "*";
+  o.ctype = std::string(is_output ? "" : "const ") + hlo::dtype_ctype(elem) + "*";
   switch (b.kind) {
     case Buffer::kParameter: o.base = b.index; break;
     case Buffer::kConstant: o.abs = const_symbol.at(root); break;
@@ -155,6 +157,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         t.wn = it->second.wave_n;
         t.wk = it->second.wave_k;
       }
+      t.split_k = n.gemm.split_k;
       f = generate_gemm(prog, n, ls, t);
     } else {
       ClusterTuning t;
@@ -211,7 +214,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     c.fn = fn;
     c.units = f.num_units;
     c.fn_id = fn_ids.at(fn);
-    for (auto& e : f.pointers) c.args.push_back(make_operand(prog, e.root, e.is_output, const_symbol, hp.param_bytes.size(), hp.liveout_bytes.size()));
+    for (auto& e : f.pointers) c.args.push_back(make_operand(prog, e.root, e.is_output, e.dtype, const_symbol, hp.param_bytes.size(), hp.liveout_bytes.size()));
     if (!fn_arg_types.count(c.fn_id))
       for (auto& a : c.args) fn_arg_types[c.fn_id].push_back(a.ctype);
     by_stage[n.stage].push_back(c);

@@ -236,7 +236,9 @@ struct NoPrologue {
   static constexpr bool enabled = false;
 };
 
-template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, class Epi, class Pro = NoPrologue>
+// K is the k extent this call contracts over; KTOTAL the k extent of the operands in memory (they differ
+// when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
+template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
                                           int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro()) {
   constexpr int TM = BM / WM / 16;
@@ -273,7 +275,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       int nt = (n_base >> 4) + j;
       const int nt_max = (N + 15) / 16 - 1;
       nt = nt < nt_max ? nt : nt_max;
-      b_ptr[j] = B + ((long)nt * KSTEPS * 64 + lane) * 8;
+      b_ptr[j] = B + ((long)nt * (KTOTAL / 32) * 64 + lane) * 8;
     } else {
       int n = n_base + j * 16 + r16;
       n = n < N ? n : N - 1;

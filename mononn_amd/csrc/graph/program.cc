@@ -220,6 +220,7 @@ struct Builder {
       for (size_t gi = 0; gi < nodes.size() && !changed; ++gi) {
         Node& g = nodes[gi];
         if (g.members.empty() || g.kind != NodeKind::kGemm) continue;
+        if (opt.gemm_split_k.count(g.members[0]->name) && opt.gemm_split_k.at(g.members[0]->name) > 1) continue;   // epilogue moves to the consumer
         for (int ci : succ[gi]) {
           Node& c = nodes[ci];
           if (c.members.empty() || c.kind != NodeKind::kCluster) continue;
@@ -511,6 +512,32 @@ struct Builder {
     });
   }
 
+  void apply_split_k() {
+    for (auto& kv : opt.gemm_split_k) {
+      if (kv.second <= 1) continue;
+      Node* node = nullptr;
+      for (auto& n : p.nodes)
+        if (n.kind == NodeKind::kGemm && n.members[0]->name == kv.first) node = &n;
+      MONONN_CHECK(node != nullptr, kSpecError) << "split_k names GEMM '" << kv.first << "' which is not a GEMM node of the graph";
+      const Instr* g = node->members[0];
+      MONONN_CHECK(node->members.size() == 1 && node->prologue.empty() && !node->gemm.has_addend, kSpecError)
+          << "split_k: GEMM " << kv.first << " has a fused epilogue / prologue / addend";
+      MONONN_CHECK(node->gemm.K % (32 * kv.second) == 0, kSpecError) << "split_k: K of " << kv.first << " is not a multiple of 32 * " << kv.second;
+      for (auto* lo : p.live_outs) MONONN_CHECK(lo != g, kSpecError) << "split_k: the result of " << kv.first << " is a module output";
+      for (auto& n : p.nodes)
+        for (auto* r : n.inputs)
+          if (r == g) {
+            bool via_emitter = n.kind == NodeKind::kCluster;
+            if (n.kind == NodeKind::kGemm) {   // allowed inside an epilogue, not as a matrix operand
+              via_emitter = p.storage_root(n.members[0]->operands[0]) != g && p.storage_root(n.members[0]->operands[1]) != g && n.prologue.empty();
+            }
+            MONONN_CHECK(via_emitter, kSpecError) << "split_k: " << kv.first << " is read by " << n.name << " as a matrix operand";
+          }
+      node->gemm.split_k = kv.second;
+      p.split_k[g] = kv.second;
+    }
+  }
+
   void assign_buffers() {
     const hlo::Computation* e = p.module->entry;
     for (auto* prm : e->params) {
@@ -541,6 +568,8 @@ struct Builder {
       for (auto* v : n.outputs) {
         Buffer b;
         b.bytes = v->shape.byte_size();
+        auto sk = p.split_k.find(v);
+        if (sk != p.split_k.end()) b.bytes = v->shape.num_elements() * 4 * sk->second;
         b.def_stage = b.last_use_stage = n.stage;
         auto li = live_index.find(v);
         if (li != live_index.end()) {
@@ -601,6 +630,7 @@ std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, cons
   b.finalize();
   b.decide_constant_layouts();
   b.assign_operand_layouts();
+  b.apply_split_k();
   for (auto& n : prog->nodes)
     if (n.kind == NodeKind::kCluster) codegen::classify_cluster(*prog, n);
   b.assign_buffers();

@@ -29,6 +29,7 @@ struct GemmDesc {
   bool a_k_contig = true;    // A stored [.., M, K]; false: [.., K, M]
   bool b_k_contig = false;   // B stored [.., N, K]; false: [.., K, N]
   bool b_packed = false;     // B is a constant that the host stores in MFMA fragment order at upload
+  int split_k = 1;           // k range split over workgroups, fp32 partial sums as output
   int64_t a_batch_stride = 0, b_batch_stride = 0, d_batch_stride = 0;
   double alpha = 1.0, beta = 0.0;
   bool has_addend = false;
@@ -84,6 +85,8 @@ struct Program {
   // storage roots kept in a permuted physical order: physical dim i = logical dim perm[i]
   // (right-hand GEMM operands produced inside the kernel are stored with k minor-most)
   std::map<const hlo::Instr*, std::vector<int>> physical_perm;
+  // GEMM results kept as S fp32 partial sums [S][elements] (split-K); readers add them up
+  std::map<const hlo::Instr*, int> split_k;
   std::vector<const hlo::Instr*> live_outs;                        // storage roots, root-tuple order
   std::map<const hlo::Instr*, int> producer;                       // storage root -> node id
   int num_stages = 0;
@@ -102,6 +105,7 @@ struct BuildOptions {
   bool fuse_gemm_prologue = false;      // row programs feeding a GEMM's left operand run inside that GEMM
   bool fuse_attention = true;           // GEMM -> soft-max style row program -> GEMM in one stage
   bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
+  std::map<std::string, int> gemm_split_k;   // GEMM instruction (canonical name) -> k split over workgroups
   bool reuse_temp_slots = true;         // false: every temp value gets its own address (written once per launch)
   std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)
 };

@@ -115,6 +115,7 @@ Json GraphSpecification::to_json() const {
     cc["archtag"] = at;
     cc["stages"] = g.stages;
     cc["wave_arrangement"] = shape_json(g.wave_m, g.wave_n, g.wave_k);
+    cc["split_k"] = g.split_k;
     e["cutlass_config"] = cc;
     e["gemm_backend_config"] = g.backend_config.is_null() ? Json::object() : g.backend_config;
     gl[kv.first] = e;
@@ -194,7 +195,7 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
       check_keys(kv.second, {"cutlass_config", "gemm_backend_config"}, "gemm_spec_list entry");
       GemmSpec g;
       const Json& cc = kv.second.at("cutlass_config");
-      check_keys(cc, {"threadblockshape", "warpshape", "instructionshape", "operatorclass", "archtag", "stages", "wave_arrangement"}, "cutlass_config");
+      check_keys(cc, {"threadblockshape", "warpshape", "instructionshape", "operatorclass", "archtag", "stages", "wave_arrangement", "split_k"}, "cutlass_config");
       auto shp = [&](const char* k, int& m, int& n, int& kk) {
         if (!cc.contains(k)) return;
         check_keys(cc.at(k), {"m", "n", "k"}, k);
@@ -209,6 +210,8 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
       if (cc.contains("operatorclass")) g.operator_class = gets(cc.at("operatorclass"), "name", g.operator_class);
       if (cc.contains("archtag")) g.arch_tag = gets(cc.at("archtag"), "name", g.arch_tag);
       g.stages = geti(cc, "stages", 1);
+      g.split_k = geti(cc, "split_k", 1);
+      MONONN_CHECK(g.split_k >= 1 && g.split_k <= 64, kSpecError) << "split_k of " << kv.first << " out of range";
       if (kv.second.contains("gemm_backend_config")) g.backend_config = kv.second.at("gemm_backend_config");
       s.gemm_spec_list[kv.first] = g;
     }

@@ -61,6 +61,9 @@ struct GemmSpec {
   std::string arch_tag = "gfx950";
   int stages = 1;
   int wave_m = 1, wave_n = 1, wave_k = 4;    // arrangement of the workgroup's waves over the tile
+  // > 1: the k range is also split over workgroups; fp32 partial sums go to memory and the consuming
+  // cluster adds them up (only for GEMMs without fused epilogue whose readers are all clusters)
+  int split_k = 1;
   Json backend_config;                       // gemm_backend_config as carried by the HLO
 };
 

@@ -92,3 +92,75 @@ def test_gather_bit_exact(gpu_device):
     consts = {n: t for n in mb.constants}
     (got,), _ = run_module(mb.text(), [i], consts, [{"dtype": "f16", "dims": [2, 37, 96]}])
     assert np.array_equal(got.view(np.uint16), t[i].view(np.uint16))
+
+
+def _spec_with(hlo_text, gemm_overrides=None, hip=None):
+    """Default specification with some entries replaced; per-node maps are cleared so that nodes whose names
+    change with the fusion decisions get fresh defaults."""
+    import json
+    spec = json.loads(MonoNNModule.compile(hlo_text, build=False).get_tuning_spec())
+    template = next(iter(spec["gemm_spec_list"].values()))
+    spec["gemm_spec_list"] = {}
+    spec["cluster_reduce_spec"] = {}
+    spec["cluster_elewise_spec"] = {}
+    for name, cc in (gemm_overrides or {}).items():
+        entry = json.loads(json.dumps(template))
+        entry["cutlass_config"].update(cc)
+        spec["gemm_spec_list"][name] = entry
+    spec["mononn_hip"].update(hip or {})
+    return json.dumps(spec)
+
+
+def _gemm_instr_names(hlo_text):
+    import re
+    return [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", hlo_text)]
+
+
+def test_fusion_variants_agree(gpu_device):
+    """Every stage-fusion decision must leave the result unchanged (bit for bit where the arithmetic is the
+    same, within fp16 rounding where a reduction order changes)."""
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
+    consts = fx.make_constants(21, "random")
+    inputs = fx.make_inputs(21)
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    (base,), m0 = run_module(fx.hlo_text, inputs, consts, fx.outputs)
+    check_close(base, want)
+    gemms = _gemm_instr_names(fx.hlo_text)
+    # out-projection and FFN2 of both layers: k split over workgroups, partial sums added by the LayerNorm stage
+    split = {}
+    for layer in range(2):
+        split[gemms[layer * 6 + 3]] = {"split_k": 2}
+        split[gemms[layer * 6 + 5]] = {"split_k": 4}
+    variants = {
+        "fenced barrier, reused temp slots": _spec_with(fx.hlo_text, hip={"barrier": "flags"}),
+        "no attention fusion": _spec_with(fx.hlo_text, hip={"fuse_attention": False}),
+        "no epilogue fusion": _spec_with(fx.hlo_text, hip={"gemm_epilogue_fusion": False}),
+        "LayerNorm as GEMM prologue": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}),
+        "plain weight layout": _spec_with(fx.hlo_text, hip={"transpose_constant_b": False, "assign_operand_layouts": False}),
+        "split-K": _spec_with(fx.hlo_text, gemm_overrides=split),
+    }
+    for name, spec in variants.items():
+        (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, spec)
+        err, cos = check_close(got, want)
+        diff = np.abs(got.astype(np.float32) - base.astype(np.float32)).max()
+        print(f"{name}: barriers={m.launch_dims()['barriers']} max_abs_err={err:.2e} vs default {diff:.2e}")
+        assert diff <= 8e-3, name
+    (fenced,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants["fenced barrier, reused temp slots"])
+    assert np.array_equal(fenced.view(np.uint16), base.view(np.uint16)), "barrier flavour must not change any bit"
+
+
+def test_repeated_launches_are_bit_identical(gpu_device):
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
+    consts = fx.make_constants(22, "random")
+    inputs = fx.make_inputs(22)
+    m = MonoNNModule.compile(fx.hlo_text)
+    m.set_constants(consts)
+    m.load(0)
+    first = m.run(inputs, fx.outputs)[0]
+    for _ in range(100):
+        again = m.run(inputs, fx.outputs)[0]
+        assert np.array_equal(first.view(np.uint16), again.view(np.uint16))
+    other = fx.make_inputs(23)
+    changed = m.run(other, fx.outputs)[0]
+    want = hlo_interp.evaluate(fx.hlo_text, other, consts, "fp32")[0]
+    check_close(changed, want)
