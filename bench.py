@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
 SPEC_DIR = os.path.join(ROOT, "mononn_amd", "specs", "bert_base_b1_s128")
+# HBM-side bytes of one launch of the kernel built from SPEC_DIR: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of
+# this script, each scaled by what the same counter reads for the 256 MiB --calibration-copy (summary under
+# profiles/).  Counters cannot be read inside a timed run, so the figure is carried here.
+MEASURED_TRAFFIC_BYTES = None
 
 
 def algorithmic_bytes(fx) -> int:
@@ -51,6 +55,40 @@ def gemm_flops(cfg) -> int:
     return per_layer * L
 
 
+def stage_profile(module, fx, consts, inputs, args):
+    """Per-stage clocks of the benchmark's own specification (stamped by every workgroup at stage entry / exit)."""
+    from mononn_amd import MonoNNModule
+    spec = json.loads(module.get_tuning_spec())
+    spec["mononn_hip"]["profile_stages"] = True
+    prof_mod = MonoNNModule.compile(fx.hlo_text, json.dumps(spec))
+    prof_mod.set_constants(consts)
+    prof_mod.load(0)
+    for _ in range(max(args.warmup, 3)):
+        prof_mod.run(inputs, fx.outputs)
+    acc = None
+    n = max(1, min(args.steps, 50))
+    for _ in range(n):
+        prof_mod.run(inputs, fx.outputs)
+        p = prof_mod.stage_profile()
+        if acc is None:
+            acc = p
+        else:
+            for a, b in zip(acc, p):
+                for k in ("busy_us", "barrier_us", "mean_wg_us"):
+                    a[k] += b[k]
+    for a in acc:
+        for k in ("busy_us", "barrier_us", "mean_wg_us"):
+            a[k] /= n
+    print(f"stage clocks, mean of {n} launches; busy = first workgroup in -> last workgroup done, "
+          f"barrier = last workgroup done -> first workgroup in the next stage")
+    print(f"{'stage':>5} {'busy_us':>8} {'mean_wg_us':>10} {'barrier_us':>10}  nodes")
+    for a in acc:
+        print(f"{a['stage']:5d} {a['busy_us']:8.2f} {a['mean_wg_us']:10.2f} {a['barrier_us']:10.2f}  {a['nodes'][:90]}")
+    busy, bar = sum(a["busy_us"] for a in acc), sum(a["barrier_us"] for a in acc)
+    print(f"total: busy {busy:.1f} us in {len(acc)} stages, barriers {bar:.1f} us ({len(acc) - 1} barriers)")
+    prof_mod.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -60,6 +98,9 @@ def main():
     ap.add_argument("--spec-dir", default=SPEC_DIR)
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof counters)")
+    ap.add_argument("--stage-profile", action="store_true",
+                    help="instead of the benchmark: rebuild the same specification with per-stage clocks and print, "
+                         "per stage, busy time / barrier time averaged over --steps launches")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the monolithic kernel's grid barrier cannot span "
@@ -90,6 +131,10 @@ def main():
     module.load(0)
     dims = module.launch_dims()
 
+    if args.stage_profile:
+        stage_profile(module, fx, consts, inputs, args)
+        return
+
     # parity of this very configuration against the oracle (also the CPU baseline's subject)
     got = module.run(inputs, fx.outputs)[0].astype(np.float32)
 
@@ -117,6 +162,18 @@ def main():
     each_us = np.sort(each.astype(np.float64) * 1e3)
     kern_us = float(avg_ms * 1e3)
 
+    # cold caches: a 1 GiB fill between launches evicts L2 and the 256 MiB memory-side cache, so every weight
+    # byte of the timed launch comes from HBM
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    cold = []
+    for i in range(12):
+        flush.fill_(i)
+        torch.cuda.synchronize()
+        _, one = module.time_raw(ptrs, stream, warmup=0, iters=1)
+        cold.append(float(one[0]) * 1e3)
+    del flush
+    cold_us = float(np.median(cold[2:]))
+
     abytes = algorithmic_bytes(fx)
     flops = gemm_flops(fx.config)
     achieved_gbs = abytes / (kern_us * 1e-6) / 1e9
@@ -137,9 +194,11 @@ def main():
         "latency_us": {"kernel_avg": round(kern_us, 2), "kernel_p10": round(float(each_us[len(each_us) // 10]), 2),
                        "kernel_median": round(float(each_us[len(each_us) // 2]), 2),
                        "kernel_p90": round(float(each_us[(len(each_us) * 9) // 10]), 2),
+                       "kernel_cold_caches_median": round(cold_us, 2),
                        "end_to_end_per_step": round(ms_per_step * 1e3, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 5), "traffic": None,
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 5),
+                     "traffic": MEASURED_TRAFFIC_BYTES if used_spec != "default" else None,
                      "algorithmic_bytes": abytes, "kernel": module.kernel_name},
         "mfma": {"achieved_tflops": round(achieved_tflops, 2), "peak_tflops": MFMA_F16_PEAK_TFLOPS,
                  "frac": round(achieved_tflops / MFMA_F16_PEAK_TFLOPS, 5), "gemm_flops": flops},

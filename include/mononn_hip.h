@@ -117,7 +117,7 @@ int mononn_module_stage_clock(mononn_module* m, uint64_t* ticks, size_t capacity
                               double* ticks_per_us);
 const char* mononn_module_stage_name(mononn_module* m, int stage);
 
-/* Write <dump_dir>/<cluster_N>/{<ctx>.json,<ctx>.hsaco,<ctx>_src/*,best_tuning_spec.{json,hsaco}}.
+/* Write <dump_dir>/<cluster_N>/{<ctx>.json,<ctx>.hsaco,<ctx>_src/...,best_tuning_spec.{json,hsaco}}.
  * Replaces: the dump half of final_tuning (mononn_engine/module/mononn_module_tuner.cc:457-603). */
 int mononn_module_dump(mononn_module* m, const char* dump_dir);
 

@@ -46,6 +46,9 @@ void parallel_for(size_t n, int threads, F&& f) {
 struct DeviceBuffers {
   int device;
   std::vector<void*> ptrs;   // params, live-outs, temp (may be null)
+  size_t temp_capacity = 0;
+  // candidates differ in temp size (split-K partial sums, slot re-use): the arena grows to the largest
+  void ensure_temp(size_t bytes);
   ~DeviceBuffers() {
     for (auto* p : ptrs)
       if (p) (void)hipFree(p);
@@ -58,6 +61,16 @@ void alloc_zero(void** p, size_t bytes) {
   if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipMalloc(" << bytes << "): " << hipGetErrorString(e);
   e = hipMemset(*p, 0, bytes);
   if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipMemset: " << hipGetErrorString(e);
+}
+
+void DeviceBuffers::ensure_temp(size_t bytes) {
+  if (bytes <= temp_capacity) return;
+  MONONN_CHECK(!ptrs.empty(), kInternal) << "tuner buffers not allocated";
+  if (ptrs.back()) (void)hipFree(ptrs.back());
+  ptrs.back() = nullptr;
+  temp_capacity = 0;
+  alloc_zero(&ptrs.back(), bytes);
+  temp_capacity = std::max<size_t>(bytes, 256);
 }
 
 struct GemmCandidate {
@@ -117,7 +130,8 @@ struct Trial {
   GraphSpecification spec;
   std::unique_ptr<MonoNNModule> mod;
   std::string error;
-  double us = -1;
+  double us = -1;        // mean time of one profiled stage
+  double total_us = -1;  // all profiled stages of one launch together
 };
 
 void apply_gemm(GraphSpecification& s, const std::string& node, const codegen::GemmTuning& t, int64_t K) {
@@ -137,33 +151,6 @@ double time_module(MonoNNModule& m, int device, DeviceBuffers& bufs, int warmup,
   std::vector<void*> ptrs = bufs.ptrs;
   float ms = m.time_kernel(ptrs.data(), ptrs.size(), nullptr, warmup, iters);
   return ms * 1000.0;
-}
-
-// Mean time of one stage (first workgroup in -> last workgroup done) of a kernel built with stage
-// clocks, averaged over its stages and over `iters` launches.  Launch overhead and barrier time are
-// not part of the figure, so candidates of one node class compare on the work itself.
-double stage_time(MonoNNModule& m, int device, DeviceBuffers& bufs, int warmup, int iters) {
-  m.load(device);
-  std::vector<void*> ptrs = bufs.ptrs;
-  for (int i = 0; i < warmup; ++i) m.launch(ptrs.data(), ptrs.size(), nullptr);
-  double total = 0;
-  int count = 0;
-  std::vector<unsigned long long> t;
-  for (int i = 0; i < iters; ++i) {
-    m.launch(ptrs.data(), ptrs.size(), nullptr);
-    int ns = 0, grid = 0;
-    double tpu = m.read_stage_clock(&t, &ns, &grid);
-    for (int s = 0; s < ns; ++s) {
-      unsigned long long lo = ~0ull, hi = 0;
-      for (int w = 0; w < grid; ++w) {
-        lo = std::min(lo, t[(static_cast<size_t>(s) * grid + w) * 2]);
-        hi = std::max(hi, t[(static_cast<size_t>(s) * grid + w) * 2 + 1]);
-      }
-      total += static_cast<double>(hi - lo) / tpu;
-      ++count;
-    }
-  }
-  return count ? total / count : -1;
 }
 
 }  // namespace
@@ -215,7 +202,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         alloc_zero(&bufs.ptrs.back(), static_cast<size_t>(b));
       }
       bufs.ptrs.push_back(nullptr);
-      alloc_zero(&bufs.ptrs.back(), static_cast<size_t>(hp.temp_bytes));
+      bufs.ensure_temp(static_cast<size_t>(hp.temp_bytes));
     }
     // Node classes: nodes that came out as the same device function.  GEMM classes that solve the same
     // problem in the same stages (the Q, K and V projections of a layer) are tuned as one class, because
@@ -307,13 +294,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     });
     GraphSpecification stitched = filled;
     const bool verbose = env::is_true("TF_MONONN_ENABLE_WORKER_THRAED_LOGGING") || env::is_true("MONONN_TUNER_VERBOSE");
-    for (auto& kv : classes) {
-      ClassInfo& c = kv.second;
-      std::vector<size_t> live;
-      for (size_t i : trials_of_class[c.function])
-        if (trials[i].mod) live.push_back(i);
-      if (live.empty()) continue;
-      // translation unit: shared preamble + union of the global declarations + one namespace per candidate
+    // Compiles the candidates `live` as one translation unit (shared preamble, one namespace per candidate),
+    // loads it once and times the profiled stages of every candidate.
+    auto measure = [&](const std::vector<size_t>& live) {
       std::map<std::string, std::string> files;
       std::string tu = trials[live[0]].mod->hip_program().preamble;
       std::set<std::string> decls;
@@ -323,57 +306,68 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       for (size_t i : live) tu += "namespace cand_" + std::to_string(i) + " {\n" + trials[i].mod->hip_program().body + "}\n";
       files["headers.h"] = trials[live[0]].mod->hip_program().files.at("headers.h");
       files["main.hip"] = tu;
+      auto res = runtime::compile_hip(files, "main.hip", props.arch);
+      runtime::DeviceModule dm;
+      dm.load(params.device, res.code_object, trials[live[0]].mod->kernel_name());
+      size_t fb = 0;
+      dm.zero(dm.global("mononn_barrier_flags", &fb), fb);
+      for (size_t i : live) {
+        Trial& t = trials[i];
+        const codegen::HipProgram& hp = t.mod->hip_program();
+        try {
+          dm.use_kernel(t.mod->kernel_name());
+          dm.set_dynamic_smem(hp.smem);
+          if (dm.max_coresident_blocks(hp.block, hp.smem) < hp.grid) {
+            t.error = "grid exceeds the co-resident capacity";
+            continue;
+          }
+          bufs.ensure_temp(static_cast<size_t>(hp.temp_bytes));
+          std::vector<void*> vals = bufs.ptrs, args(vals.size());
+          for (size_t a = 0; a < vals.size(); ++a) args[a] = &vals[a];
+          const int warm = 2, iters = budget >= 1 ? 4 : 8;
+          size_t cb = 0;
+          void* clk = dm.global("mononn_stage_clock", &cb);
+          std::vector<unsigned long long> ticks(cb / sizeof(unsigned long long));
+          const double tpu = dm.wall_clock_ticks_per_us();
+          double total = 0;
+          int count = 0;
+          for (int it = 0; it < warm + iters; ++it) {
+            dm.launch(hp.grid, hp.block, hp.smem, args.data(), nullptr);
+            if (it < warm) continue;
+            dm.download(ticks.data(), clk, cb);
+            for (int st = 0; st < hp.num_stages; ++st) {
+              unsigned long long lo = ~0ull, hi = 0;
+              for (int w = 0; w < hp.grid; ++w) {
+                lo = std::min(lo, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2]);
+                hi = std::max(hi, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2 + 1]);
+              }
+              total += static_cast<double>(hi - lo) / tpu;
+              ++count;
+            }
+          }
+          t.us = count ? total / count : -1;
+          t.total_us = count ? total / iters : -1;
+        } catch (const Error& e) {
+          t.error = e.what();
+          t.us = -1;
+        }
+      }
+    };
+    for (auto& kv : classes) {
+      ClassInfo& c = kv.second;
+      std::vector<size_t> live;
+      for (size_t i : trials_of_class[c.function])
+        if (trials[i].mod) live.push_back(i);
+      if (live.empty()) continue;
       double best_class = -1;
       size_t best_i = live[0];
       try {
-        auto res = runtime::compile_hip(files, "main.hip", props.arch);
-        runtime::DeviceModule dm;
-        dm.load(params.device, res.code_object, trials[live[0]].mod->kernel_name());
-        size_t fb = 0;
-        dm.zero(dm.global("mononn_barrier_flags", &fb), fb);
-        for (size_t i : live) {
-          Trial& t = trials[i];
-          const codegen::HipProgram& hp = t.mod->hip_program();
-          try {
-            dm.use_kernel(t.mod->kernel_name());
-            dm.set_dynamic_smem(hp.smem);
-            if (dm.max_coresident_blocks(hp.block, hp.smem) < hp.grid) {
-              t.error = "grid exceeds the co-resident capacity";
-              continue;
-            }
-            std::vector<void*> vals = bufs.ptrs, args(vals.size());
-            for (size_t a = 0; a < vals.size(); ++a) args[a] = &vals[a];
-            const int warm = 2, iters = budget >= 1 ? 4 : 8;
-            size_t cb = 0;
-            void* clk = dm.global("mononn_stage_clock", &cb);
-            std::vector<unsigned long long> ticks(cb / sizeof(unsigned long long));
-            const double tpu = dm.wall_clock_ticks_per_us();
-            double total = 0;
-            int count = 0;
-            for (int it = 0; it < warm + iters; ++it) {
-              dm.launch(hp.grid, hp.block, hp.smem, args.data(), nullptr);
-              if (it < warm) continue;
-              dm.download(ticks.data(), clk, cb);
-              for (int st = 0; st < hp.num_stages; ++st) {
-                unsigned long long lo = ~0ull, hi = 0;
-                for (int w = 0; w < hp.grid; ++w) {
-                  lo = std::min(lo, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2]);
-                  hi = std::max(hi, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2 + 1]);
-                }
-                total += static_cast<double>(hi - lo) / tpu;
-                ++count;
-              }
-            }
-            t.us = count ? total / count : -1;
-          } catch (const Error& e) {
-            t.error = e.what();
-            t.us = -1;
-          }
-          if (t.us > 0 && (best_class < 0 || t.us < best_class)) {
-            best_class = t.us;
+        measure(live);
+        for (size_t i : live)
+          if (trials[i].us > 0 && (best_class < 0 || trials[i].us < best_class)) {
+            best_class = trials[i].us;
             best_i = i;
           }
-        }
       } catch (const Error& e) {
         log << "  [" << ctx_str << "] class of " << c.nodes[0] << " failed: " << e.what() << "\n";
       }
@@ -393,6 +387,208 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         if (trials[i].us > 0) log << " " << trials[i].label << "=" << trials[i].us;
       log << "\n";
     }
+
+    // ---- split-K: GEMM classes with a long k range and few output tiles ---------------------------------
+    // A split GEMM writes fp32 partial sums and its fused epilogue moves into the consuming cluster, so the
+    // graph changes shape: the candidates are compared on GEMM stage + consumer stage together, against the
+    // same pair of stages of the unsplit graph.
+    double stitched_us = -1;
+    auto whole_kernel_us = [&](GraphSpecification s) -> double {
+      s.codegen_allow_list.clear();
+      s.hip.profile_stages = false;
+      try {
+        MonoNNModule m(params.hlo_text, s.to_json().dump(0), params.kernel_name);
+        m.generate_code();
+        m.build_assembly();
+        bufs.ensure_temp(static_cast<size_t>(m.hip_program().temp_bytes));
+        return time_module(m, params.device, bufs, 5, 40);
+      } catch (const Error&) {
+        return -1;
+      }
+    };
+    if (!env::is_true("MONONN_TUNER_NO_SPLIT_K")) {
+      for (auto& kv : classes) {
+        ClassInfo& c = kv.second;
+        if (c.kind != "gemm" || !c.sample || !c.sample->prologue.empty()) continue;
+        const graph::GemmDesc g = c.sample->gemm;
+        if (!codegen::gemm_uses_mfma(g) || g.batch != 1 || g.K < 512) continue;
+        // GEMM instruction behind every node of the class (node names differ once an epilogue is fused)
+        std::vector<std::string> instrs;
+        for (auto& n : def.program().nodes)
+          if (n.kind == graph::NodeKind::kGemm && std::find(c.nodes.begin(), c.nodes.end(), n.name) != c.nodes.end())
+            instrs.push_back(n.members[0]->name);
+        if (instrs.size() != c.nodes.size()) continue;
+        // node names in use before this class is touched
+        auto names_and_consumers = [&](const graph::Program& p, const std::set<std::string>& gemm_instrs, std::vector<std::string>* allow,
+                                       std::vector<std::string>* consumers) {
+          std::set<const hlo::Instr*> outs;
+          for (auto& n : p.nodes)
+            if (n.kind == graph::NodeKind::kGemm && gemm_instrs.count(n.members[0]->name)) {
+              allow->push_back(n.name);
+              for (auto* o : n.outputs) outs.insert(o);
+            }
+          for (auto& n : p.nodes) {
+            if (std::find(allow->begin(), allow->end(), n.name) != allow->end()) continue;
+            bool reads = false;
+            for (auto* in : n.inputs) reads = reads || outs.count(in);
+            if (reads) consumers->push_back(n.name);
+          }
+        };
+        auto drop_unknown = [&](GraphSpecification& s, const graph::Program& p) {
+          std::set<std::string> known;
+          for (auto& n : p.nodes) known.insert(n.name);
+          for (auto it = s.gemm_spec_list.begin(); it != s.gemm_spec_list.end();) it = known.count(it->first) ? std::next(it) : s.gemm_spec_list.erase(it);
+          for (auto it = s.cluster_reduce_spec.begin(); it != s.cluster_reduce_spec.end();)
+            it = known.count(it->first) ? std::next(it) : s.cluster_reduce_spec.erase(it);
+          for (auto it = s.cluster_elewise_spec.begin(); it != s.cluster_elewise_spec.end();)
+            it = known.count(it->first) ? std::next(it) : s.cluster_elewise_spec.erase(it);
+        };
+        const std::set<std::string> instr_set(instrs.begin(), instrs.end());
+        std::vector<Trial> cand;
+        // unsplit pair of stages
+        std::vector<std::string> base_consumers;
+        int base_barriers = 0;
+        {
+          GraphSpecification s = stitched;
+          s.hip.profile_stages = true;
+          s.codegen_allow_list.clear();
+          MonoNNModule probe(params.hlo_text, s.to_json().dump(0), "mononn_probe");
+          try {
+            probe.generate_code();
+          } catch (const Error&) {
+            continue;
+          }
+          std::vector<std::string> allow;
+          names_and_consumers(probe.program(), instr_set, &allow, &base_consumers);
+          if (base_consumers.empty()) continue;
+          base_barriers = probe.hip_program().num_barriers;
+          // the consuming clusters must be row programs (they get the partial sums for free in registers)
+          allow.insert(allow.end(), base_consumers.begin(), base_consumers.end());
+          s.codegen_allow_list = allow;
+          Trial t;
+          t.label = "unsplit";
+          t.spec = s;
+          cand.push_back(std::move(t));
+        }
+        // the tuned row-program knobs of the unsplit consumer carry over to the split one
+        spec::ClusterReduceSpec consumer_knobs;
+        bool have_knobs = false;
+        for (auto& n : base_consumers) {
+          auto it = stitched.cluster_reduce_spec.find(n);
+          if (it != stitched.cluster_reduce_spec.end()) {
+            consumer_knobs = it->second;
+            have_knobs = true;
+            break;
+          }
+        }
+        for (int S : {2, 4, 8}) {
+          if (g.K % (32 * S) != 0 || g.K / S < 256) continue;
+          GraphSpecification s0 = stitched;
+          s0.hip.profile_stages = true;
+          s0.codegen_allow_list.clear();
+          for (auto& n : c.nodes) s0.gemm_spec_list.erase(n);
+          for (auto& n : base_consumers) {
+            s0.cluster_reduce_spec.erase(n);
+            s0.cluster_elewise_spec.erase(n);
+          }
+          graph::GemmDesc part = g;
+          part.K = g.K / S;
+          codegen::LaunchShape shape;
+          shape.block_size = cx.block;
+          for (auto& in : instrs) {
+            apply_gemm(s0, in, codegen::default_gemm_tuning(part, shape, props.compute_units), part.K);
+            s0.gemm_spec_list[in].split_k = S;
+          }
+          // first pass without an allow list: learns whether the split is legal here and the new node names
+          std::vector<std::string> allow, consumers;
+          try {
+            GraphSpecification probe_spec = s0;
+            MonoNNModule probe(params.hlo_text, probe_spec.to_json().dump(0), "mononn_probe");
+            probe.generate_code();
+            // an epilogue that cannot move into the consumer becomes a stage of its own: not a candidate
+            if (probe.hip_program().num_barriers > base_barriers) continue;
+            names_and_consumers(probe.program(), instr_set, &allow, &consumers);
+          } catch (const Error& e) {
+            if (verbose) std::fprintf(stderr, "[mononn tuner] split_k=%d not applicable to %s: %s\n", S, instrs[0].c_str(), e.what());
+            continue;
+          }
+          std::vector<std::string> both = allow;
+          both.insert(both.end(), consumers.begin(), consumers.end());
+          for (auto& t : gemm_candidates(part, cx.block / 64, std::max(budget, 1))) {
+            GraphSpecification s = s0;
+            for (auto& in : instrs) {
+              apply_gemm(s, in, t, part.K);
+              s.gemm_spec_list[in].split_k = S;
+            }
+            if (have_knobs)
+              for (auto& n : consumers) {
+                spec::ClusterReduceSpec r = consumer_knobs;
+                r.name = n;
+                s.cluster_reduce_spec[n] = r;
+              }
+            s.codegen_allow_list = both;
+            Trial tr;
+            char lbl[112];
+            std::snprintf(lbl, sizeof lbl, "split%d_tile%dx%d_waves%dx%dx%d", S, t.bm, t.bn, t.wm, t.wn, t.wk);
+            tr.label = lbl;
+            tr.spec = std::move(s);
+            cand.push_back(std::move(tr));
+          }
+        }
+        if (cand.size() < 2) continue;
+        const size_t first = trials.size();
+        for (auto& t : cand) trials.push_back(std::move(t));
+        parallel_for(cand.size(), threads, [&](size_t j) {
+          Trial& t = trials[first + j];
+          try {
+            t.mod = std::make_unique<MonoNNModule>(params.hlo_text, t.spec.to_json().dump(0), "mononn_tune_" + std::to_string(first + j));
+            t.mod->generate_code();
+          } catch (const Error& e) {
+            t.error = e.what();
+            t.mod.reset();
+          }
+        });
+        std::vector<size_t> live;
+        for (size_t i = first; i < trials.size(); ++i)
+          if (trials[i].mod) live.push_back(i);
+        if (live.empty() || live[0] != first) {
+          for (size_t i = first; i < trials.size(); ++i) trials[i].mod.reset();
+          continue;
+        }
+        size_t best_i = first;
+        try {
+          measure(live);
+          for (size_t i : live)
+            if (trials[i].total_us > 0 && trials[first].total_us > 0 && trials[i].total_us < trials[best_i].total_us) best_i = i;
+        } catch (const Error& e) {
+          log << "  [" << ctx_str << "] split-K candidates of " << instrs[0] << " failed: " << e.what() << "\n";
+        }
+        const double per = static_cast<double>(instrs.size());
+        log << "  [" << ctx_str << "] split-K x" << instrs.size() << " (" << instrs[0] << "), GEMM + consumer stages per GEMM: best " << trials[best_i].label
+            << " " << trials[best_i].total_us / per << " us;";
+        for (size_t i : live)
+          if (trials[i].total_us > 0) log << " " << trials[i].label << "=" << trials[i].total_us / per;
+        log << "\n";
+        if (verbose)
+          std::fprintf(stderr, "[mononn tuner] %s split-K x%zu (%s): %zu candidates, unsplit %.2f us, best %s %.2f us\n", ctx_str.c_str(), instrs.size(),
+                       instrs[0].c_str(), live.size(), trials[first].total_us / per, trials[best_i].label.c_str(), trials[best_i].total_us / per);
+        // The stage clocks leave out barrier skew and cache effects between stages, so the winner is adopted
+        // only when the whole kernel with it is faster than the whole kernel without.
+        if (best_i != first && trials[best_i].total_us < 0.97 * trials[first].total_us) {
+          GraphSpecification adopted = trials[best_i].spec;
+          drop_unknown(adopted, trials[best_i].mod->program());
+          if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);
+          const double with_split = whole_kernel_us(adopted);
+          log << "    whole kernel: " << stitched_us << " us without, " << with_split << " us with " << trials[best_i].label << "\n";
+          if (with_split > 0 && stitched_us > 0 && with_split < 0.995 * stitched_us) {
+            for (auto& in : instrs) report << ctx_str << "," << in << "," << trials[best_i].total_us / per << "\n";
+            stitched = std::move(adopted);
+            stitched_us = with_split;
+          }
+        }
+        for (size_t i = first; i < trials.size(); ++i) trials[i].mod.reset();
+      }
+    }
     // ---- whole kernel of this context --------------------------------------------------------------
     stitched.codegen_allow_list.clear();
     stitched.hip.profile_stages = false;
@@ -401,6 +597,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     try {
       full->generate_code();
       full->build_assembly();
+      bufs.ensure_temp(static_cast<size_t>(full->hip_program().temp_bytes));
       us = time_module(*full, params.device, bufs, 5, 30);
     } catch (const Error& e) {
       log << ctx_str << " failed: " << e.what() << "\n";
