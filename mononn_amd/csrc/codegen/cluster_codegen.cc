@@ -447,8 +447,9 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     if (a.find_first_of(".e") == std::string::npos) a += ".0";
     Epilogue e;
     e.struct_text = "struct @NAME@_epi {\n  float* out;\n  int ksplit;\n"
-                    "  __device__ __forceinline__ void prefetch(int, int, int) const {}\n"
-                    "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4]) const {\n"
+                    "  struct Pre {};\n"
+                    "  __device__ __forceinline__ void preload(int, int, int, Pre&) const {}\n"
+                    "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4], const Pre&) const {\n"
                     "    const float v[4] = {acc[0] * " + a + "f, acc[1] * " + a + "f, acc[2] * " + a + "f, acc[3] * " + a + "f};\n"
                     "    mononn_dev::stN<float, 4>(out + (long)ksplit * " + S(g.batch * g.M * g.N) + " + (long)bidx * " + S(g.M * g.N) + " + m * " + S(g.N) + " + n0, v);\n"
                     "  }\n};\n";
@@ -607,26 +608,44 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     auto& e = ptrs.entries[i];
     pre += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
   }
+  // Operands of the epilogue (bias, residual) whose address depends on (bidx, m, n) only are loaded into
+  // registers ahead of the GEMM main loop, so their latency overlaps it; the body then reads the registers.
+  std::vector<std::pair<std::string, std::string>> preloads;
+  std::string body_text = cb.text();
   if (mfma) {
-    // touch the epilogue's operands ahead of the main loop
-    pre += "  __device__ __forceinline__ void prefetch(int bidx, int m, int n0) const {\n";
-    if (vec4 && !em.simple_loads().empty()) {
+    pre += "  struct Pre {\n";
+    if (vec4) {
+      for (auto& l : em.simple_loads()) {
+        bool seen = false;
+        for (auto& q : preloads) seen = seen || q.first == l.first;
+        if (!seen) preloads.push_back(l);
+      }
+      for (size_t i = 0; i < preloads.size(); ++i) pre += "    " + preloads[i].second + " v" + S(i) + "[4];\n";
+    }
+    pre += "  };\n";
+    pre += "  __device__ __forceinline__ void preload(int bidx, int m, int n0, Pre& pre) const {\n";
+    if (!preloads.empty()) {
       pre += "    const int n4 = n0 >> 2;\n    #pragma unroll\n    for (int r = 0; r < 4; ++r) {\n";
-      for (auto& l : em.simple_loads()) pre += "      mononn_dev::touch(" + l + ");\n";
+      for (size_t i = 0; i < preloads.size(); ++i) pre += "      pre.v" + S(i) + "[r] = " + preloads[i].first + ";\n";
       pre += "    }\n";
     }
     pre += "  }\n";
+    for (size_t i = 0; i < preloads.size(); ++i) {
+      const std::string& ref = preloads[i].first;
+      const std::string with = "pre.v" + S(i) + "[r]";
+      for (size_t pos = body_text.find(ref); pos != std::string::npos; pos = body_text.find(ref, pos + with.size())) body_text.replace(pos, ref.size(), with);
+    }
   }
-  if (vec4) pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4]) const {\n";
+  if (vec4) pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4], const Pre& pre) const {\n";
   else if (mfma) {
-    pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&accv)[4]) const {\n";
+    pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&accv)[4], const Pre&) const {\n";
     pre += "    for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") { const float acc = accv[r]; one(bidx, m, nn, acc); } }\n  }\n";
     pre += "  __device__ __forceinline__ void one(int bidx, int m, int nn, float acc) const {\n";
   } else {
     pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int nn, float acc) const {\n";
   }
   {
-    std::istringstream is(cb.text());
+    std::istringstream is(body_text);
     std::string l;
     while (std::getline(is, l)) pre += "  " + l + "\n";
   }
@@ -1075,7 +1094,9 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.line("for (int w = 0; w < " + S(KW) + "; ++w) if (w != kw) o += ob[(w * " + S(NT2) + " + t) * 64 + lane];");
     cb.open("if (m_valid)");
     cb.line("const float v[4] = {o[0], o[1], o[2], o[3]};");
-    cb.line("epi(bidx, m, t * 16 + g * 4, v);");
+    cb.line("decltype(epi)::Pre pre;");
+    cb.line("epi.preload(bidx, m, t * 16 + g * 4, pre);");
+    cb.line("epi(bidx, m, t * 16 + g * 4, v, pre);");
     cb.close();
     cb.close();
     cb.line("__syncthreads();   // LDS is reused by the next unit");
@@ -1084,7 +1105,9 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.line("#pragma unroll");
     cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
     cb.line("const float v[4] = {oacc[t][0], oacc[t][1], oacc[t][2], oacc[t][3]};");
-    cb.line("epi(bidx, m, t * 16 + g * 4, v);");
+    cb.line("decltype(epi)::Pre pre;");
+    cb.line("epi.preload(bidx, m, t * 16 + g * 4, pre);");
+    cb.line("epi(bidx, m, t * 16 + g * 4, v, pre);");
     cb.close();
     cb.close();
   }

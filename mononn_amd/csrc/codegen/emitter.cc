@@ -225,13 +225,13 @@ std::string Emitter::load(const Instr* root, const Index& idx) {
     std::string sum;
     for (int i = 0; i < sk->second; ++i) {
       std::string ref = p + "[" + lin.plus_const(i * E).str(vars_) + "]";
-      if (lin.opaques().empty()) simple_loads_.push_back(ref);
+      if (lin.opaques().empty()) simple_loads_.emplace_back(ref, "float");
       sum += (i ? " + " : "") + ref;
     }
     return def(root->shape.dtype, "(" + std::string(hlo::dtype_ctype(root->shape.dtype)) + ")(" + sum + ")");
   }
   std::string ref = ptrs_.input(root) + "[" + lin.str(vars_) + "]";
-  if (lin.opaques().empty()) simple_loads_.push_back(ref);
+  if (lin.opaques().empty()) simple_loads_.emplace_back(ref, hlo::dtype_ctype(root->shape.dtype));
   return def(root->shape.dtype, ref);
 }
 

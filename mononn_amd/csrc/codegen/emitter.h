@@ -82,7 +82,8 @@ class Emitter {
   // device-global arrays for non-scalar literal constants met inside fused computations
   const std::map<std::string, std::string>& literal_tables() const { return literal_tables_; }
   // "ptr[index]" of every plain load emitted so far whose index only involves loop variables
-  const std::vector<std::string>& simple_loads() const { return simple_loads_; }
+  // loads whose address depends on the loop variables only, as (reference text, C type), in emission order
+  const std::vector<std::pair<std::string, std::string>>& simple_loads() const { return simple_loads_; }
 
  private:
   std::string emit(const hlo::Instr* ins, const Index& idx);
@@ -106,7 +107,7 @@ class Emitter {
   };
   std::map<const hlo::Instr*, Bound> bound_;
   std::map<std::string, std::string> literal_tables_;
-  std::vector<std::string> simple_loads_;
+  std::vector<std::pair<std::string, std::string>> simple_loads_;
   int counter_ = 0;
 };
 

@@ -45,7 +45,7 @@ typedef int int4_t __attribute__((ext_vector_type(4)));
 namespace mononn_dev {
 
 constexpr int kWaveSize = 64;
-constexpr int kFlagStride = 16;   // one 64-byte line per workgroup flag
+constexpr int kFlagStride = 64;   // 256 bytes between workgroup flags: measured fastest among 64 B .. 4 KiB
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWaveSize - 1); }
 __device__ __forceinline__ int wave_id() { return threadIdx.x / kWaveSize; }
@@ -222,7 +222,7 @@ __device__ __forceinline__ T sign_of(T x) {
 // consecutive n of one row m (n = n0 + 4*(lane/16) + r, m = m0 + lane%16): the epilogue then
 // stores 8 contiguous bytes per lane.
 //
-// Epilogue functor:  void prefetch(int batch, int m, int n) const   (touch what operator() will read)
+// Epilogue functor:  struct Pre;  void preload(int batch, int m, int n, Pre&) const   (loads what operator() will read)
 //                    void operator()(int batch, int m, int n, const float (&v)[4])   (n % 4 == 0)
 // Rows/cols beyond M / N are clamped on load and skipped on store, so M and N need not divide.
 //
@@ -308,7 +308,9 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
     pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, smem);
   }
-  // touch the epilogue's operands (bias, residual) now so that their latency overlaps the main loop
+  // the epilogue's operands (bias, residual) of the fragments this wave finalises: issued now, used after
+  // the main loop, so that their latency overlaps it
+  typename Epi::Pre pre[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -316,7 +318,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       if (WK > 1 && (i * TN + j) % WK != wk) continue;
       const int m = m_base + i * 16 + r16;
       const int n = n_base + j * 16 + (lane >> 4) * 4;
-      if (m < M && n < N) epi.prefetch(batch, m, n);
+      if (m < M && n < N) epi.preload(batch, m, n, pre[i][j]);
     }
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
@@ -361,7 +363,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         const int n = n_base + j * 16 + (lane >> 4) * 4;
         if (m < M && n < N) {
           float v[4] = {s[0], s[1], s[2], s[3]};
-          epi(batch, m, n, v);
+          epi(batch, m, n, v, pre[i][j]);
         }
       }
   } else {
@@ -373,7 +375,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         const int n = n_base + j * 16 + (lane >> 4) * 4;
         if (m < M && n < N) {
           float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
-          epi(batch, m, n, v);
+          epi(batch, m, n, v, pre[i][j]);
         }
       }
   }

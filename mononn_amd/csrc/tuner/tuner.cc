@@ -183,6 +183,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     base.device.max_configurable_smem_size = std::max(props.max_lds_per_block, 65536);
     base.runtime.grid_dim.x = props.compute_units * cx.per_cu;
     base.runtime.block_dim.x = cx.block;
+    if (env::is_true("MONONN_TUNER_GEMM_PROLOGUE")) base.hip.gemm_prologue_fusion = true;
     const std::string ctx_str = base.context_string();
 
     // default module of this context: classes of identical node functions
