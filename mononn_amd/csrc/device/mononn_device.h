@@ -308,18 +308,22 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
     pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, smem);
   }
-  // the epilogue's operands (bias, residual) of the fragments this wave finalises: issued now, used after
-  // the main loop, so that their latency overlaps it
-  typename Epi::Pre pre[TM][TN];
+  // The epilogue's operands (bias, residual) of the fragments this wave finalises are requested now and used
+  // after the main loop, so that their latency overlaps it.  Slot q belongs to fragment q * WK + wk; the
+  // addresses are clamped instead of guarded so that the loads stay in this basic block (a load under a
+  // branch gets its wait inside the branch, which would stall on every operand load issued above).
+  constexpr int NSLOT = (TM * TN + WK - 1) / WK;
+  typename Epi::Pre pre[NSLOT];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      if (WK > 1 && (i * TN + j) % WK != wk) continue;
-      const int m = m_base + i * 16 + r16;
-      const int n = n_base + j * 16 + (lane >> 4) * 4;
-      if (m < M && n < N) epi.preload(batch, m, n, pre[i][j]);
-    }
+  for (int q = 0; q < NSLOT; ++q) {
+    int f = q * WK + wk;
+    f = f < TM * TN ? f : TM * TN - 1;
+    int m = m_base + (f / TN) * 16 + r16;
+    int n = n_base + (f % TN) * 16 + (lane >> 4) * 4;
+    m = m < M ? m : M - 1;
+    n = n < N ? n : (N >= 4 ? N - 4 : 0);
+    epi.preload(batch, m, n, pre[q]);
+  }
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     if (c + 1 < NCHUNK) load_chunk(c + 1, (c + 1) & 1);
@@ -363,7 +367,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         const int n = n_base + j * 16 + (lane >> 4) * 4;
         if (m < M && n < N) {
           float v[4] = {s[0], s[1], s[2], s[3]};
-          epi(batch, m, n, v, pre[i][j]);
+          epi(batch, m, n, v, pre[f / WK]);
         }
       }
   } else {
@@ -375,7 +379,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         const int n = n_base + j * 16 + (lane >> 4) * 4;
         if (m < M && n < N) {
           float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
-          epi(batch, m, n, v, pre[i][j]);
+          epi(batch, m, n, v, pre[i * TN + j]);
         }
       }
   }
