@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <set>
+#include <regex>
 #include <sstream>
 
 #include "common/status.h"
@@ -116,6 +117,48 @@ std::vector<std::string> tables_of(const Emitter& em) {
   std::vector<std::string> v;
   for (auto& kv : em.literal_tables()) v.push_back(kv.second);
   return v;
+}
+
+// Row programs are straight-line code in which a load is emitted where its value is first needed.  A load
+// whose address depends on the row and column only (LayerNorm gamma / beta, a residual) and that is first
+// needed after a workgroup reduction would be issued after that reduction's barrier, putting one more trip
+// to memory on the critical path.  Such loads are moved up to the head of the program: definitions of the
+// form `const T vN = <expression of inK[..], row, qK>;` go right behind the last `const int qK = ...;`.
+std::string hoist_row_loads(const std::string& text) {
+  std::vector<std::string> lines;
+  {
+    std::istringstream is(text);
+    std::string l;
+    while (std::getline(is, l)) lines.push_back(l);
+  }
+  static const std::regex q_def(R"(^\s*const int q\d+ = .*;$)");
+  static const std::regex v_def(R"(^\s*const [A-Za-z_][\w ]* v\d+ = (.*);$)");
+  static const std::regex ident(R"((^|[^\w.])([A-Za-z_]\w*))");
+  static const std::regex allowed(R"(^(in\d+|q\d+|row|lane|tid|float|double|_Float16|int|long|unsigned|short|char|bool|int8_t|uint8_t|int16_t|uint16_t|int32_t|uint32_t|int64_t|uint64_t)$)");
+  int anchor = -1;
+  for (size_t i = 0; i < lines.size(); ++i)
+    if (std::regex_match(lines[i], q_def)) anchor = static_cast<int>(i);
+  if (anchor < 0) return text;
+  std::vector<std::string> hoisted, rest;
+  for (size_t i = static_cast<size_t>(anchor) + 1; i < lines.size(); ++i) {
+    std::smatch m;
+    bool hoist = false;
+    if (std::regex_match(lines[i], m, v_def)) {
+      const std::string rhs = m[1].str();
+      hoist = rhs.find('[') != std::string::npos;
+      for (auto it = std::sregex_iterator(rhs.begin(), rhs.end(), ident); hoist && it != std::sregex_iterator(); ++it)
+        hoist = std::regex_match((*it)[2].str(), allowed);
+    }
+    (hoist ? hoisted : rest).push_back(lines[i]);
+  }
+  std::string out;
+  for (int i = 0; i <= anchor; ++i) out += lines[i] + "\n";
+  for (auto& l : hoisted) out += l + "\n";
+  // keeps the instruction scheduler from sinking a load to its first use (it would then wait for each
+  // load in turn instead of having all of them in flight)
+  if (!hoisted.empty()) out += "    __builtin_amdgcn_sched_barrier(0);\n";
+  for (auto& l : rest) out += l + "\n";
+  return out;
 }
 
 NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
@@ -270,7 +313,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     }
     cb.close();
     int64_t units = block_tier ? ROWS : (ROWS + NW - 1) / NW;
-    return finish(cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 : 0);
+    return finish(T * V <= 32 ? hoist_row_loads(cb.text()) : cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 : 0);
   }
 
   // element-wise loop(s); outputs of equal element count share one loop.  A thread owns V consecutive

@@ -222,11 +222,12 @@ std::string Emitter::load(const Instr* root, const Index& idx) {
     // the HLO defines
     std::string p = ptrs_.input(root, DType::kF32);
     const int64_t E = root->shape.num_elements();
+    // every partial sum is a definition of its own, so that all of them can be requested before the first add
     std::string sum;
     for (int i = 0; i < sk->second; ++i) {
       std::string ref = p + "[" + lin.plus_const(i * E).str(vars_) + "]";
       if (lin.opaques().empty()) simple_loads_.emplace_back(ref, "float");
-      sum += (i ? " + " : "") + ref;
+      sum += (i ? " + " : "") + def(DType::kF32, ref);
     }
     return def(root->shape.dtype, "(" + std::string(hlo::dtype_ctype(root->shape.dtype)) + ")(" + sum + ")");
   }

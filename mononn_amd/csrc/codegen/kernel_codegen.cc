@@ -229,6 +229,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   // declarations (shared by all candidates), body (node functions + kernel).
   std::ostringstream pre, glob, src;
   pre << "// generated by mononn-hip for " << spec.device.cuda_arch << "\n";
+  pre << "#define MONONN_BLOCK_SIZE " << hp.block << "\n";
   if (spec.hip.barrier == "flags_allfence") pre << "#define MONONN_BARRIER_FENCE 1\n";
   else if (spec.hip.barrier == "flags_coherent") pre << "#define MONONN_BARRIER_FENCE 2\n#define MONONN_COHERENT_STORES 1\n";
   else MONONN_CHECK(spec.hip.barrier == "flags", kSpecError) << "unknown barrier flavour '" << spec.hip.barrier << "'";

@@ -158,18 +158,46 @@ __device__ __forceinline__ void stN(T* p, const T (&v)[N]) {
 // ---------------------------------------------------------------------------------------------
 // reductions (all lanes / all threads receive the result)
 // ---------------------------------------------------------------------------------------------
+// value of `v` in the lane that the DPP control word names (rows of 16 lanes)
+template <int CTRL, class T>
+__device__ __forceinline__ T dpp_move(T v) {
+  static_assert(sizeof(T) == 4, "DPP moves one dword");
+  int b;
+  __builtin_memcpy(&b, &v, 4);
+  b = __builtin_amdgcn_update_dpp(b, b, CTRL, 0xf, 0xf, false);
+  T r;
+  __builtin_memcpy(&r, &b, 4);
+  return r;
+}
+
 template <class T, class Op>
 __device__ __forceinline__ T wave_all_reduce(T v, Op op) {
+  if constexpr (sizeof(T) == 4) {
+    // inside a row of 16 lanes: data-parallel-primitive moves on the vector ALU (neighbour in the quad, other
+    // pair of the quad, mirrored half row, mirrored row); across the four rows: two LDS-crossbar permutes
+    v = op(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+    v = op(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+    v = op(v, dpp_move<0x141>(v));   // row_half_mirror
+    v = op(v, dpp_move<0x140>(v));   // row_mirror
+    v = op(v, __shfl_xor(v, 16, kWaveSize));
+    v = op(v, __shfl_xor(v, 32, kWaveSize));
+    return v;
+  } else {
 #pragma unroll
-  for (int off = kWaveSize / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWaveSize));
-  return v;
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWaveSize));
+    return v;
+  }
 }
 
 // `scratch` holds at least blockDim.x / 64 elements of T in LDS
 template <class T, class Op>
 __device__ __forceinline__ T block_all_reduce(T v, Op op, T* scratch) {
   v = wave_all_reduce(v, op);
+#if defined(MONONN_BLOCK_SIZE)
+  constexpr int nw = MONONN_BLOCK_SIZE / kWaveSize;   // the kernel is generated for one workgroup size
+#else
   const int nw = blockDim.x / kWaveSize;
+#endif
   if (lane_id() == 0) scratch[wave_id()] = v;
   __syncthreads();
   T r = scratch[0];
