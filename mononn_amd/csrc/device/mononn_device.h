@@ -212,7 +212,7 @@ __device__ __forceinline__ T block_all_reduce(T v, Op op, T* scratch) {
 __device__ __forceinline__ float fast_tanh(float x) {
   // tanh(x) = 1 - 2 / (exp(2x) + 1); exact enough in fp32 and safe for large |x|
   float e = __expf(2.0f * x);
-  return 1.0f - 2.0f / (e + 1.0f);
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 // keep a value (and the load that produced it) alive without using it
 template <class T>
@@ -371,7 +371,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
 
   if (WK > 1) {
     // [wk][wm*wn][frag][lane] float4 : each wave writes its own slab, then every wave finalises the
-    // fragments f with f % WK == wk.
+    // fragments f with f % WK == wk from all WK slabs.
     float4_t* red = reinterpret_cast<float4_t*>(smem);
     const int mn = wave / WK;
     __syncthreads();   // smem may still be in use by the previous tile's readers
@@ -379,7 +379,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        if ((i * TN + j) % WK != wk) red[((wk * (WM * WN) + mn) * (TM * TN) + (i * TN + j)) * kWaveSize + lane] = acc[i][j];
+        red[((wk * (WM * WN) + mn) * (TM * TN) + (i * TN + j)) * kWaveSize + lane] = acc[i][j];
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -387,10 +387,14 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       for (int j = 0; j < TN; ++j) {
         const int f = i * TN + j;
         if (f % WK != wk) continue;
-        float4_t s = acc[i][j];
+        // every slab is read, the wave's own included: no branch on the wave index, so the LDS reads are
+        // issued together, and the k slices are added in one order whatever wave finalises the fragment
+        float4_t part[WK];
 #pragma unroll
-        for (int w = 0; w < WK; ++w)
-          if (w != wk) s += red[((w * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
+        for (int w = 0; w < WK; ++w) part[w] = red[((w * (WM * WN) + mn) * (TM * TN) + f) * kWaveSize + lane];
+        float4_t s = part[0];
+#pragma unroll
+        for (int w = 1; w < WK; ++w) s += part[w];
         const int m = m_base + i * 16 + r16;
         const int n = n_base + j * 16 + (lane >> 4) * 4;
         if (m < M && n < N) {
