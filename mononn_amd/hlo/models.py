@@ -300,6 +300,42 @@ def bert_large(B=16, S=384) -> ModelFixture:
     return bert_encoder(L=24, B=B, S=S, H=1024, NH=16, F=4096, mask_kind="length_mask")
 
 
+def gpt2(L=12, B=4, S=512, H=768, NH=12, F=3072, vocab=50257, max_pos=1024, eps=1e-5) -> ModelFixture:
+    """GPT-2 style decoder prefill: token + learned position embeddings, L pre-LayerNorm layers with causal
+    self-attention and tanh-GELU MLP, final LayerNorm, LM head tied to the token embedding
+    (logits = h . wte^T, a GEMM whose right operand is contracted over its minor dimension)."""
+    mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
+    e = mb.entry
+    ids = e.parameter("s32", (B, S), "input_ids")
+    wte = e.elided_constant("f16", (vocab, H), "gpt2/wte")
+    wpe = e.elided_constant("f16", (max_pos, H), "gpt2/wpe")
+
+    def emb_body(f, pi, pw, pp):
+        w = f.convert(f.gather_rows(pw, pi), "f32")
+        p = f.convert(f.broadcast(f.slice(pp, (0, 0), (S, H)), (B, S, H), [1, 2]), "f32")
+        return f.convert(f.add(w, p), "f16")
+    h = e.bitcast(e.fusion("kLoop", [ids, wte, wpe], emb_body), (B * S, H))
+    D = H // NH
+    for l in range(L):
+        W = _layer_weights(e, f"gpt2/h_{l}", H, F)
+        a = _layer_norm(e, mb, h, W["ln1_g"], W["ln1_b"], eps)
+        ctx = _attention(e, mb, a, None, B, S, NH, D, W, causal=True)
+        h = _residual_f16(e, e.gemm(ctx, W["o_w"], 1, 0), W["o_b"], h)
+        m = _layer_norm(e, mb, h, W["ln2_g"], W["ln2_b"], eps)
+        act = _ffn_act(e, e.gemm(m, W["f1_w"], 1, 0), W["f1_b"])
+        h = _residual_f16(e, e.gemm(act, W["f2_w"], 1, 0), W["f2_b"], h)
+    lnf_g = e.elided_constant("f16", (H,), "gpt2/ln_f/gamma")
+    lnf_b = e.elided_constant("f16", (H,), "gpt2/ln_f/beta")
+    hf = _layer_norm(e, mb, h, lnf_g, lnf_b, eps)
+    logits = e.gemm(hf, wte, 1, 1)
+    e.set_tuple_root([e.bitcast(logits, (B, S, vocab))])
+    return ModelFixture(
+        f"gpt2_L{L}_H{H}", mb.text(),
+        [{"name": "input_ids", "dtype": "s32", "dims": [B, S], "kind": "token_ids", "vocab": vocab}],
+        mb.constants, [{"dtype": "f16", "dims": [B, S, vocab]}],
+        dict(B=B, S=S, H=H, NH=NH, F=F, L=L, vocab=vocab, eps=eps))
+
+
 def reference_example_inputs(S=128) -> List[np.ndarray]:
     """The reference's example feed (examples/data/bert_bs1.npy): ids [101, 7592 x (S-2), 102],
     attention mask all ones, segment ids all zeros, int32 [1,S].  The file itself is a pickled

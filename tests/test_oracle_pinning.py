@@ -214,3 +214,34 @@ def test_reference_example_input_shape():
     assert ids.dtype == np.int32 and ids.shape == (1, 128) and ids.nbytes == 512
     assert ids[0, 0] == 101 and ids[0, -1] == 102 and (ids[0, 1:-1] == 7592).all()
     assert mask.all() and not seg.any()
+
+
+def test_gpt2_decoder_against_torch():
+    # pre-LN decoder, causal mask built from iota/compare/select, LM head tied to the token embedding
+    B, S, H, NH, Fd, V = 2, 24, 64, 4, 128, 97
+    fx = models.gpt2(L=2, B=B, S=S, H=H, NH=NH, F=Fd, vocab=V, max_pos=32)
+    consts = fx.make_constants(21, "random")
+    inputs = fx.make_inputs(21)
+    got = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    R = {m["role"]: torch.tensor(consts[n].astype(np.float32)) for n, m in fx.constants.items()}
+    ids = torch.tensor(inputs[0].astype(np.int64))
+    h = R["gpt2/wte"][ids] + R["gpt2/wpe"][:S][None]
+    D = H // NH
+    causal = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    for l in range(2):
+        P = f"gpt2/h_{l}/"
+
+        def lin(x, p):
+            return x @ R[P + p + "/kernel"] + R[P + p + "/bias"]
+        a = F.layer_norm(h, (H,), R[P + "attention/LayerNorm/gamma"], R[P + "attention/LayerNorm/beta"], 1e-5)
+        q, k, v = (lin(a, "attention/" + n).view(B, S, NH, D).transpose(1, 2) for n in ("query", "key", "value"))
+        s = q @ k.transpose(2, 3) / math.sqrt(D)
+        s = torch.where(causal, s, torch.tensor(-10000.0))
+        ctx = (torch.softmax(s, -1) @ v).transpose(1, 2).reshape(B, S, H)
+        h = h + lin(ctx, "attention/output")
+        m = F.layer_norm(h, (H,), R[P + "output/LayerNorm/gamma"], R[P + "output/LayerNorm/beta"], 1e-5)
+        h = h + lin(F.gelu(lin(m, "intermediate"), approximate="tanh"), "output")
+    hf = F.layer_norm(h, (H,), R["gpt2/ln_f/gamma"], R["gpt2/ln_f/beta"], 1e-5)
+    want = (hf @ R["gpt2/wte"].T).numpy()
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() < 3e-5
