@@ -188,7 +188,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "BERT-base encoder, 12 layers + embedding gather, batch 1, seq 128, fp16 weights "
-                               "N(0,0.02), one monolithic cooperative kernel launch per forward",
+                               "N(0,0.02), one launch of the monolithic persistent kernel per forward",
                    "tuning_spec": used_spec, "grid": dims["grid"], "block": dims["block"], "lds_bytes": dims["smem"],
                    "grid_barriers": dims["barriers"]},
         "latency_us": {"kernel_avg": round(kern_us, 2), "kernel_p10": round(float(each_us[len(each_us) // 10]), 2),

@@ -245,6 +245,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     hp.global_decls.push_back(d.str());
   }
   hp.profiled = spec.hip.profile_stages;
+  hp.cooperative = spec.hip.cooperative_launch;
   hp.num_stages = static_cast<int>(by_stage.size());
   if (hp.profiled) {
     // sized for the deepest kernel the barrier supports so that candidates of one class can share it

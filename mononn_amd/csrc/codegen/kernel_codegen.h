@@ -50,6 +50,7 @@ struct HipProgram {
   std::vector<ConstantInfo> constants;
   std::vector<NodeReport> nodes;
   int num_barriers = 0;
+  bool cooperative = false;   // launch through the cooperative-launch entry point
   int grid = 0, block = 0, smem = 0;
   int max_grid = 4096;       // barrier flag capacity
   int num_stages = 0;        // stages that were emitted

@@ -242,7 +242,7 @@ void MonoNNModule::launch(void* const* device_ptrs, size_t n, void* stream) {
   std::vector<void*> args(n);
   prepare_args(vals);
   for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
-  dev_.launch(grid_, hip_.block, hip_.smem, args.data(), stream);
+  dev_.launch(grid_, hip_.block, hip_.smem, args.data(), stream, hip_.cooperative);
 }
 
 double MonoNNModule::read_stage_clock(std::vector<unsigned long long>* ticks, int* n_stages, int* grid) {
@@ -272,7 +272,7 @@ float MonoNNModule::time_kernel(void* const* device_ptrs, size_t n, void* stream
   std::vector<void*> args(n);
   prepare_args(vals);
   for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
-  return dev_.time_launches(grid_, hip_.block, hip_.smem, args.data(), stream, warmup, iters, each);
+  return dev_.time_launches(grid_, hip_.block, hip_.smem, args.data(), stream, warmup, iters, each, hip_.cooperative);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -2,6 +2,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include <algorithm>
 #include <mutex>
 
@@ -163,21 +165,22 @@ void DeviceModule::set_dynamic_smem(int smem) const {
   if (smem > 48 * 1024) HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(function_), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
 }
 
-void DeviceModule::launch(int grid, int block, int smem, void** args, void* stream) const {
+void DeviceModule::launch(int grid, int block, int smem, void** args, void* stream, bool cooperative) const {
   MONONN_CHECK(module_ != nullptr, kRuntimeError) << "module is not loaded";
-  HIP_OK(hipModuleLaunchCooperativeKernel(function_, grid, 1, 1, block, 1, 1, smem, static_cast<hipStream_t>(stream), args));
+  if (cooperative) HIP_OK(hipModuleLaunchCooperativeKernel(function_, grid, 1, 1, block, 1, 1, smem, static_cast<hipStream_t>(stream), args));
+  else HIP_OK(hipModuleLaunchKernel(function_, grid, 1, 1, block, 1, 1, smem, static_cast<hipStream_t>(stream), args, nullptr));
 }
 
 float DeviceModule::time_launches(int grid, int block, int smem, void** args, void* stream, int warmup, int iters,
-                                  std::vector<float>* per_launch_ms) const {
+                                  std::vector<float>* per_launch_ms, bool cooperative) const {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  for (int i = 0; i < warmup; ++i) launch(grid, block, smem, args, stream);
+  for (int i = 0; i < warmup; ++i) launch(grid, block, smem, args, stream, cooperative);
   HIP_OK(hipStreamSynchronize(s));
   std::vector<hipEvent_t> ev(static_cast<size_t>(iters) + 1);
   for (auto& e : ev) HIP_OK(hipEventCreate(&e));
   HIP_OK(hipEventRecord(ev[0], s));
   for (int i = 0; i < iters; ++i) {
-    launch(grid, block, smem, args, stream);
+    launch(grid, block, smem, args, stream, cooperative);
     HIP_OK(hipEventRecord(ev[i + 1], s));
   }
   HIP_OK(hipEventSynchronize(ev[iters]));

@@ -58,10 +58,10 @@ class DeviceModule {
   int max_coresident_blocks(int block, int smem) const;
   void set_dynamic_smem(int smem) const;
   // one cooperative launch; args = array of pointers to the argument values
-  void launch(int grid, int block, int smem, void** args, void* stream) const;
+  void launch(int grid, int block, int smem, void** args, void* stream, bool cooperative = false) const;
   // average milliseconds per launch over `iters` launches after `warmup`
   float time_launches(int grid, int block, int smem, void** args, void* stream, int warmup, int iters,
-                      std::vector<float>* per_launch_ms = nullptr) const;
+                      std::vector<float>* per_launch_ms = nullptr, bool cooperative = false) const;
   void unload();
 
  private:

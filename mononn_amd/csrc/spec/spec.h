@@ -82,6 +82,11 @@ struct HipOptions {       // "mononn_hip" section
   // plain stores, temp slots re-used.  "flags_allfence": every thread fences (measurement only).
   std::string barrier = "flags_coherent";
   bool profile_stages = false;   // per-stage wall-clock stamps (performance_report.csv equivalent)
+  // false: ordinary kernel launch, as the reference does (mononn_module_tuner.cc:135-139); the grid is checked
+  // against the co-resident capacity at load time, and launches of such kernels must not overlap on the device
+  // (two half-resident grids would wait for each other at their first barrier).  true: cooperative launch, the
+  // runtime keeps such kernels apart at the price of ~20 us more per launch.
+  bool cooperative_launch = false;
 };
 
 struct GraphSpecification {

@@ -138,6 +138,7 @@ def test_fusion_variants_agree(gpu_device):
         "LayerNorm as GEMM prologue": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}),
         "plain weight layout": _spec_with(fx.hlo_text, hip={"transpose_constant_b": False, "assign_operand_layouts": False}),
         "split-K": _spec_with(fx.hlo_text, gemm_overrides=split),
+        "cooperative launch": _spec_with(fx.hlo_text, hip={"cooperative_launch": True}),
     }
     for name, spec in variants.items():
         (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, spec)
@@ -147,6 +148,8 @@ def test_fusion_variants_agree(gpu_device):
         assert diff <= 8e-3, name
     (fenced,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants["fenced barrier, reused temp slots"])
     assert np.array_equal(fenced.view(np.uint16), base.view(np.uint16)), "barrier flavour must not change any bit"
+    (coop,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants["cooperative launch"])
+    assert np.array_equal(coop.view(np.uint16), base.view(np.uint16)), "the launch entry point must not change any bit"
 
 
 def test_repeated_launches_are_bit_identical(gpu_device):
