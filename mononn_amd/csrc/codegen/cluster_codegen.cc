@@ -426,7 +426,10 @@ bool can_merge_clusters(const Program& prog, const std::vector<const Instr*>& pr
 // ------------------------------------------------------------------------------------------
 // GEMM
 // ------------------------------------------------------------------------------------------
-bool gemm_uses_mfma(const graph::GemmDesc& g) { return g.a_k_contig && (g.b_k_contig || g.b_packed) && g.K % 32 == 0; }
+bool gemm_uses_mfma(const graph::GemmDesc& g) {
+  if (g.is_conv && !g.conv_fragment_loads()) return false;
+  return g.a_k_contig && (g.b_k_contig || g.b_packed) && g.K % 32 == 0;
+}
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus) {
   (void)num_cus;
@@ -515,8 +518,14 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     vnn = vars.add("nn", g.N);
   }
   auto gemm_index = [&](bool with_r) {
-    Index idx = delinearize(LinExpr::variable(vb, g.batch), batch_dims, vars);
-    idx.push_back(LinExpr::variable(vm, g.M));
+    Index idx;
+    if (g.is_conv) {
+      // the GEMM row m enumerates the output pixels (n, p, q) in row-major order
+      idx = delinearize(LinExpr::variable(vm, g.M), std::vector<int64_t>(D.dims.begin(), D.dims.end() - 1), vars);
+    } else {
+      idx = delinearize(LinExpr::variable(vb, g.batch), batch_dims, vars);
+      idx.push_back(LinExpr::variable(vm, g.M));
+    }
     if (vec4) {
       LinExpr n = LinExpr::variable(vn4, g.N / 4).scaled(4);
       if (with_r) n = n.plus(LinExpr::variable(vr, 4));
@@ -897,6 +906,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
   Epilogue epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, ptrs, first_epi);
   CodeBuffer fb;
+  std::string conv_struct;
   if (g.split_k <= 1) fb.line(epi.init_line);
   if (has_pro) fb.line(pro.init_line);
   int64_t units = 0;
@@ -923,10 +933,26 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
       fb.line("const int tile_m = rem % " + S(tiles_m) + ";");
     }
     std::ostringstream call;
-    call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
-         << (g.b_packed ? "true" : "false") << ", " << g.K << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << KS << ", " << pb
-         << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS) << ", " << g.M << ", " << g.N << ", " << g.K << ", "
-         << g.K << ", bidx, tile_m, tile_n, epi, smem" << (has_pro ? ", pro" : "") << ");";
+    if (g.is_conv) {
+      MONONN_CHECK(!has_pro && S_ == 1, kUnsupported) << gi->hlo_name << ": a convolution takes neither a row-program prologue nor split-K";
+      const hlo::ConvConfig& c = g.conv;
+      std::ostringstream am;
+      am << "struct @NAME@_amap {\n  static constexpr bool kRowMajor = false;\n"
+         << "  __device__ __forceinline__ const half_t* operator()(const half_t* in, int m, int k, int) const {\n"
+         << "    const int n = m / " << c.P * c.Q << ", pq = m % " << c.P * c.Q << ", p = pq / " << c.Q << ", q = pq % " << c.Q << ";\n"
+         << "    const int r = k / " << c.S * c.C << ", sc = k % " << c.S * c.C << ";\n"
+         << "    return in + (((long)n * " << c.H << " + p * " << c.stride_h << " + r) * " << c.W << " + q * " << c.stride_w << ") * " << c.C << " + sc;\n"
+         << "  }\n};\n";
+      conv_struct = am.str();
+      call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", false, " << g.K
+           << ", @NAME@_epi, mononn_dev::NoPrologue, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
+           << ", bidx, tile_m, tile_n, epi, smem, mononn_dev::NoPrologue(), @NAME@_amap());";
+    } else {
+      call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
+           << (g.b_packed ? "true" : "false") << ", " << g.K << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << KS << ", " << pb
+           << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS) << ", " << g.M << ", " << g.N << ", " << g.K << ", "
+           << g.K << ", bidx, tile_m, tile_n, epi, smem" << (has_pro ? ", pro" : "") << ");";
+    }
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
     smem = std::max(smem, pro.smem);
@@ -939,15 +965,21 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fb.line("const int m = (int)((e / " + S(g.N) + ") % " + S(g.M) + ");");
     fb.line("const int n = (int)(e % " + S(g.N) + ");");
     std::ostringstream call;
-    call << "mononn_dev::gemm_naive_element(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * "
-         << g.b_batch_stride << ", " << g.K << ", " << (g.a_k_contig ? g.K : 1) << ", " << (g.a_k_contig ? 1 : g.M) << ", "
-         << (g.b_k_contig ? 1 : g.N) << ", " << (g.b_k_contig ? g.K : 1) << ", bidx, m, n, epi);";
+    if (g.is_conv) {
+      const hlo::ConvConfig& c = g.conv;
+      call << "mononn_dev::conv_naive_element(" << pa << ", " << pb << ", " << c.H << ", " << c.W << ", " << c.C << ", " << c.R << ", " << c.S << ", "
+           << c.P << ", " << c.Q << ", " << c.stride_h << ", " << c.stride_w << ", " << c.pad_h << ", " << c.pad_w << ", m, n, epi);";
+    } else {
+      call << "mononn_dev::gemm_naive_element(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * "
+           << g.b_batch_stride << ", " << g.K << ", " << (g.a_k_contig ? g.K : 1) << ", " << (g.a_k_contig ? 1 : g.M) << ", "
+           << (g.b_k_contig ? 1 : g.N) << ", " << (g.b_k_contig ? g.K : 1) << ", bidx, m, n, epi);";
+    }
     fb.line(call.str());
     fb.close();
   }
   std::vector<std::string> globals = epi.globals;
   for (auto& gl : pro.globals) globals.push_back(gl);
-  return finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text);
+  return finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text + conv_struct);
 }
 
 // GEMM -> row program -> GEMM with everything between the two contractions on chip.

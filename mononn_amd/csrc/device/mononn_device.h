@@ -264,11 +264,20 @@ struct NoPrologue {
   static constexpr bool enabled = false;
 };
 
+// Where row m, column k of the left operand lives.  The default is a row-major [M, lda] matrix; an implicit-GEMM
+// convolution supplies a map that gathers the row from the input image.  k is a multiple of 8 and the 8 elements
+// from there on are contiguous and 16-byte aligned.
+struct RowMajorA {
+  static constexpr bool kRowMajor = true;
+  __device__ __forceinline__ const half_t* operator()(const half_t* A, int m, int k, int lda) const { return A + (long)m * lda + k; }
+};
+
 // K is the k extent this call contracts over; KTOTAL the k extent of the operands in memory (they differ
 // when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
-template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue>
+template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
-                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro()) {
+                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
+                                          const AMap& amap = AMap()) {
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int KSTEPS = K / 32;
@@ -291,10 +300,12 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
 
   const half_t* a_ptr[TM];
   const half_t* b_ptr[TN];
+  int a_row[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     int m = m_base + i * 16 + r16;
     m = m < M ? m : M - 1;
+    a_row[i] = m;
     a_ptr[i] = A + (long)m * lda + kq;
   }
 #pragma unroll
@@ -321,7 +332,10 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
 #pragma unroll
       for (int j = 0; j < TN; ++j) b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);
+      for (int i = 0; i < TM; ++i) {
+        if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);
+        else a[buf][s][i] = *reinterpret_cast<const half8_t*>(amap(A, a_row[i], ks * 32 + kq, lda));
+      }
     }
   };
 
@@ -429,6 +443,27 @@ __device__ __forceinline__ void gemm_naive_element(const half_t* A, const half_t
   const half_t* b = B + n * b_sn;
   for (int k = 0; k < K; ++k) acc += (float)a[k * a_sk] * (float)b[k * b_sk];
   epi(batch, m, n, acc);
+}
+
+// Correctness fallback for convolutions the fragment loads do not cover (padding, channel counts that break the
+// 16-byte pieces): one thread per output element.  Input N,H,W,C, filter K,R,S,C, output N,P,Q,K.
+template <class Epi>
+__device__ __forceinline__ void conv_naive_element(const half_t* in, const half_t* flt, int H, int W, int C, int R, int S, int P, int Q,
+                                                   int stride_h, int stride_w, int pad_h, int pad_w, int m, int k_out, Epi& epi) {
+  const int n = m / (P * Q), pq = m % (P * Q), p = pq / Q, q = pq % Q;
+  float acc = 0.f;
+  for (int r = 0; r < R; ++r) {
+    const int h = p * stride_h + r - pad_h;
+    if (h < 0 || h >= H) continue;
+    for (int s = 0; s < S; ++s) {
+      const int w = q * stride_w + s - pad_w;
+      if (w < 0 || w >= W) continue;
+      const half_t* x = in + (((long)n * H + h) * W + w) * C;
+      const half_t* f = flt + (((long)k_out * R + r) * S + s) * C;
+      for (int c = 0; c < C; ++c) acc += (float)x[c] * (float)f[c];
+    }
+  }
+  epi(0, m, k_out, acc);
 }
 
 }  // namespace mononn_dev

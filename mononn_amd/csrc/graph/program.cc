@@ -29,6 +29,7 @@ const Node* Program::node_of(const Instr* member) const {
 std::string GemmDesc::problem_hash() const {
   std::ostringstream os;
   os << "f16_b" << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_packed ? "_bp" : (b_k_contig ? "_bk" : "_bn"));
+  if (is_conv) os << "_conv" << conv.R << "x" << conv.S << "s" << conv.stride_h << "x" << conv.stride_w << "p" << conv.pad_h << "x" << conv.pad_w;
   return os.str();
 }
 
@@ -101,6 +102,22 @@ struct Builder {
     return d;
   }
 
+  GemmDesc describe_conv(const Instr* g) {
+    const hlo::ConvConfig& c = g->conv;
+    GemmDesc d;
+    d.is_conv = true;
+    d.conv = c;
+    d.batch = 1;
+    d.M = c.N * c.P * c.Q;
+    d.N = c.K;
+    d.K = c.R * c.S * c.C;
+    d.a_k_contig = true;
+    d.b_k_contig = true;
+    d.alpha = c.result_scale;
+    d.a_batch_stride = d.b_batch_stride = d.d_batch_stride = 0;
+    return d;
+  }
+
   void make_nodes() {
     const hlo::Computation* e = p.module->entry;
     for (auto& up : e->instrs) {
@@ -113,9 +130,8 @@ struct Builder {
       n.name = ins->name;
       n.members.push_back(ins);
       if (op == "custom-call") {
-        MONONN_CHECK(ins->custom_call_target == "__cublas$gemm", kUnsupported) << ins->hlo_name << ": custom-call target '" << ins->custom_call_target << "' has no lowering yet";
         n.kind = NodeKind::kGemm;
-        n.gemm = describe_gemm(ins);
+        n.gemm = ins->is_conv() ? describe_conv(ins) : describe_gemm(ins);
       } else {
         n.kind = NodeKind::kCluster;
       }
@@ -272,7 +288,7 @@ struct Builder {
       std::vector<int> takers;
       for (int ci : succ[ri]) {
         Node& c = nodes[ci];
-        if (c.kind != NodeKind::kGemm || !c.prologue.empty()) continue;
+        if (c.kind != NodeKind::kGemm || !c.prologue.empty() || c.gemm.is_conv) continue;
         const Instr* g = c.members[0];
         if (p.storage_root(g->operands[0]) != h || p.storage_root(g->operands[1]) == h) continue;
         if (g->operands.size() > 2 && p.storage_root(g->operands[2]) == h) continue;
@@ -340,7 +356,7 @@ struct Builder {
         if (reaches_via_outside(g1i, static_cast<int>(ri), succ) || reaches_via_outside(static_cast<int>(ri), g2i, succ)) continue;
         // the other producers of gemm2 (V) must not depend on gemm1 / the row program
         const GemmDesc &d1 = g1.gemm, &d2 = g2.gemm;
-        if (!d1.a_k_contig || !d1.b_k_contig || !d2.a_k_contig || d2.has_addend || d1.has_addend) continue;
+        if (!d1.a_k_contig || !d1.b_k_contig || !d2.a_k_contig || d2.has_addend || d1.has_addend || d1.is_conv || d2.is_conv) continue;
         if (d2.batch != d1.batch || d2.M != d1.M || d2.K != d1.N) continue;
         if (d1.K % 32 != 0 || d1.N % 32 != 0 || d2.N % 16 != 0 || d1.N > 512 || d2.N > 256 || d1.K > 256) continue;
         const Instr* vroot = p.storage_root(gi2->operands[1]);
@@ -520,8 +536,8 @@ struct Builder {
         if (n.kind == NodeKind::kGemm && n.members[0]->name == kv.first) node = &n;
       MONONN_CHECK(node != nullptr, kSpecError) << "split_k names GEMM '" << kv.first << "' which is not a GEMM node of the graph";
       const Instr* g = node->members[0];
-      MONONN_CHECK(node->members.size() == 1 && node->prologue.empty() && !node->gemm.has_addend, kSpecError)
-          << "split_k: GEMM " << kv.first << " has a fused epilogue / prologue / addend";
+      MONONN_CHECK(node->members.size() == 1 && node->prologue.empty() && !node->gemm.has_addend && !node->gemm.is_conv, kSpecError)
+          << "split_k: GEMM " << kv.first << " has a fused epilogue / prologue / addend or is a convolution";
       MONONN_CHECK(node->gemm.K % (32 * kv.second) == 0, kSpecError) << "split_k: K of " << kv.first << " is not a multiple of 32 * " << kv.second;
       for (auto* lo : p.live_outs) MONONN_CHECK(lo != g, kSpecError) << "split_k: the result of " << kv.first << " is a module output";
       for (auto& n : p.nodes)

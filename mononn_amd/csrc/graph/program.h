@@ -33,6 +33,17 @@ struct GemmDesc {
   int64_t a_batch_stride = 0, b_batch_stride = 0, d_batch_stride = 0;
   double alpha = 1.0, beta = 0.0;
   bool has_addend = false;
+  // Forward convolution seen as a GEMM (implicit GEMM, conv_impl.cc:51): M = N*P*Q output pixels, N = K output
+  // channels, K = R*S*C; row m of the left operand is gathered from the N,H,W,C input, the filter K,R,S,C is the
+  // k-contiguous right operand, the result N,P,Q,K is row-major [M, N].
+  bool is_conv = false;
+  hlo::ConvConfig conv;
+  // left-operand fragments can be loaded 8 halves at a time: no padding, and every 8-element piece of a row
+  // lies inside one contiguous run of S*C input elements at a 16-byte aligned address
+  bool conv_fragment_loads() const {
+    return is_conv && conv.pad_h == 0 && conv.pad_w == 0 && (conv.S * conv.C) % 8 == 0 && (conv.W * conv.C) % 8 == 0 &&
+           (conv.stride_w * conv.C) % 8 == 0 && (conv.N == 1 || (conv.H * conv.W * conv.C) % 8 == 0);
+  }
   std::string problem_hash() const;   // dtype+shape key, cf. mononn_module_tuner.cc:386-408
 };
 

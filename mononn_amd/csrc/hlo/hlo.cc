@@ -4,6 +4,7 @@
 #include <cctype>
 #include <cstdlib>
 #include <set>
+#include <sstream>
 
 #include "common/json.h"
 #include "common/status.h"
@@ -312,6 +313,109 @@ void decode_gemm_config(Instr* ins) {
   }
 }
 
+// window={size=16x16 stride=16x16 pad=1_1x1_1}: fields separated by blanks, dimensions by 'x'
+std::map<std::string, std::vector<std::string>> window_fields(const std::string& raw) {
+  std::map<std::string, std::vector<std::string>> out;
+  std::string s = raw;
+  for (char& c : s)
+    if (c == '{' || c == '}') c = ' ';
+  std::istringstream is(s);
+  std::string field;
+  while (is >> field) {
+    size_t eq = field.find('=');
+    if (eq == std::string::npos) continue;
+    std::vector<std::string> dims;
+    std::string v = field.substr(eq + 1);
+    size_t st = 0;
+    while (st <= v.size()) {
+      size_t e = v.find('x', st);
+      dims.push_back(v.substr(st, e == std::string::npos ? std::string::npos : e - st));
+      if (e == std::string::npos) break;
+      st = e + 1;
+    }
+    out[field.substr(0, eq)] = dims;
+  }
+  return out;
+}
+
+void decode_conv_config(Instr* ins) {
+  auto attr = [&](const char* k) -> std::string {
+    auto it = ins->attrs.find(k);
+    return it == ins->attrs.end() ? std::string() : it->second;
+  };
+  MONONN_CHECK(ins->operands.size() == 2, kUnsupported) << ins->hlo_name << ": convolution with a side input / bias operand is not supported";
+  MONONN_CHECK(ins->shape.is_tuple() && ins->shape.tuple.size() == 2, kParseError) << ins->hlo_name << ": __cudnn$convForward yields (output, scratch)";
+  std::string labels = attr("dim_labels");
+  labels.erase(std::remove_if(labels.begin(), labels.end(), [](char c) { return isspace(static_cast<unsigned char>(c)); }), labels.end());
+  // the lowering assumes N,H,W,C / K,R,S,C / N,P,Q,K in memory (conv_impl.cc:295-298); with the row-major layouts
+  // this parser accepts, that is exactly this labelling
+  MONONN_CHECK(labels == "b01f_o01i->b01f", kUnsupported) << ins->hlo_name << ": dim_labels '" << labels << "' (only b01f_o01i->b01f is supported)";
+  const std::string fg = attr("feature_group_count");
+  MONONN_CHECK(fg.empty() || std::strtoll(fg.c_str(), nullptr, 10) == 1, kUnsupported) << ins->hlo_name << ": grouped convolution is not supported";
+  const hlo::Shape &in = ins->operands[0]->shape, &flt = ins->operands[1]->shape, &out = ins->shape.tuple[0];
+  MONONN_CHECK(in.rank() == 4 && flt.rank() == 4 && out.rank() == 4, kUnsupported) << ins->hlo_name << ": only 2-d convolutions are supported";
+  MONONN_CHECK(in.dtype == DType::kF16 && flt.dtype == DType::kF16 && out.dtype == DType::kF16, kUnsupported) << ins->hlo_name << ": only f16 convolutions are supported";
+  ConvConfig& c = ins->conv;
+  c.N = in.dims[0], c.H = in.dims[1], c.W = in.dims[2], c.C = in.dims[3];
+  c.K = flt.dims[0], c.R = flt.dims[1], c.S = flt.dims[2];
+  c.P = out.dims[1], c.Q = out.dims[2];
+  MONONN_CHECK(flt.dims[3] == c.C, kInvalidArgument) << ins->hlo_name << ": channel extents of input and filter differ";
+  MONONN_CHECK(out.dims[0] == c.N && out.dims[3] == c.K, kInvalidArgument) << ins->hlo_name << ": output shape does not match the operands";
+  auto w = window_fields(attr("window"));
+  auto two = [&](const char* key, int64_t dflt, int64_t* a, int64_t* b) {
+    auto it = w.find(key);
+    if (it == w.end()) {
+      *a = *b = dflt;
+      return;
+    }
+    MONONN_CHECK(it->second.size() == 2, kUnsupported) << ins->hlo_name << ": window field " << key << " must have two dimensions";
+    *a = std::strtoll(it->second[0].c_str(), nullptr, 10);
+    *b = std::strtoll(it->second[1].c_str(), nullptr, 10);
+  };
+  int64_t sr = 0, ss = 0, d0 = 1, d1 = 1;
+  two("size", 0, &sr, &ss);
+  MONONN_CHECK(sr == c.R && ss == c.S, kInvalidArgument) << ins->hlo_name << ": window size does not match the filter";
+  two("stride", 1, &c.stride_h, &c.stride_w);
+  two("lhs_dilate", 1, &d0, &d1);
+  MONONN_CHECK(d0 == 1 && d1 == 1, kUnsupported) << ins->hlo_name << ": dilated convolution is not supported";
+  two("rhs_dilate", 1, &d0, &d1);
+  MONONN_CHECK(d0 == 1 && d1 == 1, kUnsupported) << ins->hlo_name << ": dilated convolution is not supported";
+  auto pit = w.find("pad");
+  if (pit != w.end()) {
+    MONONN_CHECK(pit->second.size() == 2, kUnsupported) << ins->hlo_name << ": pad must have two dimensions";
+    int64_t lo[2], hi[2];
+    for (int i = 0; i < 2; ++i) {
+      const std::string& v = pit->second[i];
+      size_t us = v.find('_');
+      MONONN_CHECK(us != std::string::npos, kParseError) << ins->hlo_name << ": bad pad field";
+      lo[i] = std::strtoll(v.substr(0, us).c_str(), nullptr, 10);
+      hi[i] = std::strtoll(v.substr(us + 1).c_str(), nullptr, 10);
+      // only symmetric padding (ir_parser_fused.cc:782-798)
+      MONONN_CHECK(lo[i] == hi[i] && lo[i] >= 0, kUnsupported) << ins->hlo_name << ": only symmetric, non-negative padding is supported";
+    }
+    c.pad_h = lo[0];
+    c.pad_w = lo[1];
+  }
+  MONONN_CHECK(c.stride_h >= 1 && c.stride_w >= 1, kInvalidArgument) << ins->hlo_name << ": bad stride";
+  MONONN_CHECK((c.H + 2 * c.pad_h - c.R) / c.stride_h + 1 == c.P && (c.W + 2 * c.pad_w - c.S) / c.stride_w + 1 == c.Q, kInvalidArgument)
+      << ins->hlo_name << ": output extents do not follow from input, window, stride and padding";
+  auto bc = ins->attrs.find("backend_config");
+  if (bc != ins->attrs.end()) {
+    Json j = Json::parse(bc->second);
+    if (j.contains("conv_result_scale")) c.result_scale = j.at("conv_result_scale").as_double();
+    if (j.contains("side_input_scale")) MONONN_CHECK(j.at("side_input_scale").as_double() == 0, kUnsupported) << ins->hlo_name << ": side input is not supported";
+    if (j.contains("activation_mode")) {
+      const Json& a = j.at("activation_mode");
+      const std::string mode = a.is_string() ? a.as_string() : std::to_string(a.as_int());
+      // conv_impl.cc:245-247 aborts on any other mode
+      MONONN_CHECK(mode == "0", kUnsupported) << ins->hlo_name << ": activation mode " << mode << " inside the convolution call is not supported";
+    }
+  }
+  // from here on the call is an array-valued instruction; its get-tuple-element index 0 is an alias of it
+  Shape arr = out;
+  ins->shape = arr;
+}
+
 void decode_attrs(Instr* ins, Module* mod) {
   auto has = [&](const char* k) { return ins->attrs.count(k) > 0; };
   auto get = [&](const char* k) -> const std::string& { return ins->attrs.at(k); };
@@ -336,7 +440,15 @@ void decode_attrs(Instr* ins, Module* mod) {
   }
   if (op == "reduce" || op == "reduce-window") ins->called = comp_ref(need("to_apply"));
   if (op == "compare") ins->comparison = need("direction");
-  if (op == "get-tuple-element") ins->tuple_index = std::strtoll(need("index").c_str(), nullptr, 10);
+  if (op == "get-tuple-element") {
+    ins->tuple_index = std::strtoll(need("index").c_str(), nullptr, 10);
+    if (!ins->operands.empty() && ins->operands[0]->is_conv()) {
+      // (output, scratch) of the convolution call: element 0 aliases the call (which has been given the array
+      // shape), the scratch buffer is never read (the reference wires only element 0, ir_parser_fused.cc:802-821)
+      MONONN_CHECK(ins->tuple_index == 0, kUnsupported) << ins->hlo_name << ": the scratch result of a convolution call cannot be used";
+      ins->opcode = "bitcast";
+    }
+  }
   if (op == "iota") ins->iota_dimension = std::strtoll(need("iota_dimension").c_str(), nullptr, 10);
   if (op == "slice") {
     // slice={[0:8192], [2:4:1]}
@@ -393,7 +505,7 @@ void decode_attrs(Instr* ins, Module* mod) {
     if (ins->custom_call_target == "__cublas$gemm") {
       decode_gemm_config(ins);
     } else if (ins->custom_call_target == "__cudnn$convForward") {
-      // decoded by the convolution lowering from attrs (window, dim_labels)
+      decode_conv_config(ins);
     } else {
       // any other target aborts in the reference (core/op/custom_call.cc:96-100)
       MONONN_FAIL(kUnsupported) << ins->hlo_name << ": custom-call target '" << ins->custom_call_target << "' is not supported";

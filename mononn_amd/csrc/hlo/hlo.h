@@ -52,6 +52,14 @@ struct GemmConfig {   // backend_config of __cublas$gemm (gemm_impl.cc:182-231)
   std::string selected_algorithm;
 };
 
+// __cudnn$convForward (attributes read by ir_parser_fused.cc:749-823, lowering conv_impl.cc:252-324):
+// input N,H,W,C, filter K,R,S,C, output N,P,Q,K, symmetric padding, no dilation, one feature group
+struct ConvConfig {
+  int64_t N = 0, H = 0, W = 0, C = 0, K = 0, R = 0, S = 0, P = 0, Q = 0;
+  int64_t stride_h = 1, stride_w = 1, pad_h = 0, pad_w = 0;
+  double result_scale = 1;
+};
+
 struct Instr {
   std::string name;            // canonical: '.' and '-' replaced by '_' (string_helpers.cc:22-32)
   std::string hlo_name;        // as written in the text
@@ -82,6 +90,8 @@ struct Instr {
   // custom-call
   std::string custom_call_target;
   GemmConfig gemm;
+  ConvConfig conv;
+  bool is_conv() const { return opcode == "custom-call" && custom_call_target == "__cudnn$convForward"; }
 
   std::vector<Instr*> users;           // within the same computation
   bool is_scalar_constant() const { return opcode == "constant" && shape.num_elements() == 1 && !literal_elided; }

@@ -262,6 +262,36 @@ class Computation:
                           attrs=f'custom_call_target="__cublas$gemm", backend_config="{cfg_s}"',
                           name_hint="cublas-batch-gemm" if batch > 1 else "cublas-gemm")
 
+    def conv_forward(self, x: Value, filt: Value, stride: Sequence[int] = (1, 1), pad: Sequence[int] = (0, 0),
+                     result_scale: float = 1.0) -> Value:
+        """`__cudnn$convForward` custom call on an N,H,W,C input and a K,R,S,C filter (dim_labels
+        b01f_o01i->b01f), symmetric padding, no dilation, one feature group -- the form the reference accepts
+        (ir_parser_fused.cc:749-823).  The call yields (output, scratch); the output is taken with
+        get-tuple-element index 0, as XLA does."""
+        n, h, w, c = x.dims
+        k, r, s, c2 = filt.dims
+        assert c == c2
+        p = (h + 2 * pad[0] - r) // stride[0] + 1
+        q = (w + 2 * pad[1] - s) // stride[1] + 1
+        out = Value("", x.dtype, (n, p, q, k))
+        window = f"size={r}x{s}"
+        if tuple(stride) != (1, 1):
+            window += f" stride={stride[0]}x{stride[1]}"
+        if tuple(pad) != (0, 0):
+            window += f" pad={pad[0]}_{pad[0]}x{pad[1]}_{pad[1]}"
+        cfg = json.dumps({"conv_result_scale": result_scale, "activation_mode": "0", "side_input_scale": 0},
+                         separators=(",", ":")).replace('"', '\\"')
+        name = self.module.fresh("cudnn-conv")
+        tshape = f"({out.shape_str}, u8[0]{{0}})"
+        self.lines.append(f"%{name} = {tshape} custom-call({x.operand_str}, {filt.operand_str}), window={{{window}}}, "
+                          f"dim_labels=b01f_o01i->b01f, custom_call_target=\"__cudnn$convForward\", backend_config=\"{cfg}\"")
+        gte = self.module.fresh("get-tuple-element")
+        v = Value(gte, x.dtype, out.dims)
+        self.lines.append(f"%{gte} = {v.shape_str} get-tuple-element({tshape} %{name}), index=0")
+        self.root = v
+        self.root_is_tuple = False
+        return v
+
     def set_tuple_root(self, values: Sequence[Value]):
         name = self.module.fresh("tuple")
         tshape = "(" + ", ".join(v.shape_str for v in values) + ")"

@@ -336,6 +336,52 @@ def gpt2(L=12, B=4, S=512, H=768, NH=12, F=3072, vocab=50257, max_pos=1024, eps=
         dict(B=B, S=S, H=H, NH=NH, F=F, L=L, vocab=vocab, eps=eps))
 
 
+def vit(L=12, B=8, image=224, patch=16, H=768, NH=12, F=3072, eps=1e-6) -> ModelFixture:
+    """ViT-B/16 style encoder: NCHW pixels -> NHWC, patch embedding as a strided forward convolution
+    (`__cudnn$convForward`, window = stride = patch), class token + learned positions, L pre-LayerNorm layers
+    without masking, final LayerNorm.  Output f16[B, 1 + (image/patch)^2, H]."""
+    mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
+    e = mb.entry
+    G = image // patch
+    S = G * G + 1
+    pixels = e.parameter("f16", (B, 3, image, image), "pixel_values")
+    filt = e.elided_constant("f16", (H, patch, patch, 3), "vit/embeddings/patch_embeddings/kernel")
+    pbias = e.elided_constant("f16", (H,), "vit/embeddings/patch_embeddings/bias")
+    cls = e.elided_constant("f16", (1, 1, H), "vit/embeddings/cls_token")
+    pos = e.elided_constant("f16", (S, H), "vit/embeddings/position_embeddings")
+    nhwc = e.fusion("kLoop", [pixels], lambda f, px: f.transpose(px, (0, 2, 3, 1)))
+    conv = e.conv_forward(nhwc, filt, stride=(patch, patch))
+
+    def bias_body(f, pc, pb):
+        x = f.add(f.convert(pc, "f32"), f.broadcast(f.convert(pb, "f32"), pc.dims, [3]))
+        return f.convert(x, "f16")
+    patches = e.fusion("kLoop", [conv, pbias], bias_body)
+
+    def emb_body(f, pp, pc, ppos):
+        tok = f.concatenate([f.broadcast(f.reshape(pc, (H,)), (B, 1, H), [2]), f.reshape(pp, (B, G * G, H))], 1)
+        x = f.add(f.convert(tok, "f32"), f.broadcast(f.convert(ppos, "f32"), (B, S, H), [1, 2]))
+        return f.convert(x, "f16")
+    h = e.bitcast(e.fusion("kLoop", [patches, cls, pos], emb_body), (B * S, H))
+    D = H // NH
+    for l in range(L):
+        W = _layer_weights(e, f"vit/encoder/layer_{l}", H, F)
+        a = _layer_norm(e, mb, h, W["ln1_g"], W["ln1_b"], eps)
+        ctx = _attention(e, mb, a, None, B, S, NH, D, W, causal=False)
+        h = _residual_f16(e, e.gemm(ctx, W["o_w"], 1, 0), W["o_b"], h)
+        m = _layer_norm(e, mb, h, W["ln2_g"], W["ln2_b"], eps)
+        act = _ffn_act(e, e.gemm(m, W["f1_w"], 1, 0), W["f1_b"])
+        h = _residual_f16(e, e.gemm(act, W["f2_w"], 1, 0), W["f2_b"], h)
+    lnf_g = e.elided_constant("f16", (H,), "vit/layernorm/gamma")
+    lnf_b = e.elided_constant("f16", (H,), "vit/layernorm/beta")
+    out = _layer_norm(e, mb, h, lnf_g, lnf_b, eps)
+    e.set_tuple_root([e.bitcast(out, (B, S, H))])
+    return ModelFixture(
+        f"vit_L{L}_H{H}", mb.text(),
+        [{"name": "pixel_values", "dtype": "f16", "dims": [B, 3, image, image], "kind": "uniform_pm1"}],
+        mb.constants, [{"dtype": "f16", "dims": [B, S, H]}],
+        dict(B=B, S=S, H=H, NH=NH, F=F, L=L, image=image, patch=patch, eps=eps))
+
+
 def reference_example_inputs(S=128) -> List[np.ndarray]:
     """The reference's example feed (examples/data/bert_bs1.npy): ids [101, 7592 x (S-2), 102],
     attention mask all ones, segment ids all zeros, int32 [1,S].  The file itself is a pickled

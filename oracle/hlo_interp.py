@@ -365,6 +365,8 @@ class Evaluator:
             target = ins.attrs["custom_call_target"].strip('"')
             if target == "__cublas$gemm":
                 return self._gemm(ins, x, dt)
+            if target == "__cudnn$convForward":
+                return self._conv_forward(ins, x)
             raise NotImplementedError(f"custom-call target {target}")
         raise NotImplementedError(f"opcode {op}")
 
@@ -408,6 +410,48 @@ class Evaluator:
             D = D + np.float32(cfg["beta"]) * x[2].astype(np.float32)
         with np.errstate(over="ignore"):
             return D.astype(dt)
+
+
+    def _conv_forward(self, ins: Instr, x):
+        """cuDNN forward convolution custom call as the reference lowers it (conv_impl.cc:252-324, attributes
+        from ir_parser_fused.cc:749-823): input N,H,W,C; filter K,R,S,C; output N,P,Q,K;
+        out[n,p,q,k] = scale * sum_{r,s,c} in[n, p*sh + r - ph, q*sw + s - pw, c] * filt[k,r,s,c], zero outside.
+        Result is the tuple (output, scratch)."""
+        a = ins.attrs
+        if a.get("dim_labels", "").strip() != "b01f_o01i->b01f":
+            raise NotImplementedError("only dim_labels=b01f_o01i->b01f")
+        if int(a.get("feature_group_count", "1")) != 1:
+            raise NotImplementedError("grouped convolution")
+        win = a["window"].strip("{} ")
+        fields = dict(f.split("=") for f in win.split())
+        size = [int(v) for v in fields["size"].split("x")]
+        stride = [int(v) for v in fields.get("stride", "1x1").split("x")]
+        pad = [[int(t) for t in v.split("_")] for v in fields.get("pad", "0_0x0_0").split("x")]
+        for key in ("lhs_dilate", "rhs_dilate"):
+            if key in fields and any(int(v) != 1 for v in fields[key].split("x")):
+                raise NotImplementedError("dilated convolution")
+        cfg = json.loads(a["backend_config"][1:-1].replace('\\"', '"'))
+        if float(cfg.get("side_input_scale", 0)) != 0.0 or str(cfg.get("activation_mode", "0")) != "0":
+            raise NotImplementedError("side input / activation in the convolution call")
+        inp = x[0].astype(np.float32)
+        flt = x[1].astype(np.float32)
+        N, H, W, C = inp.shape
+        K, R, S, C2 = flt.shape
+        assert C == C2 and [R, S] == size
+        out_sh = ins.shape.tuple_shapes[0]
+        P, Q = out_sh.dims[1], out_sh.dims[2]
+        padded = np.zeros((N, H + pad[0][0] + pad[0][1], W + pad[1][0] + pad[1][1], C), np.float32)
+        padded[:, pad[0][0]:pad[0][0] + H, pad[1][0]:pad[1][0] + W, :] = inp
+        out = np.zeros((N, P, Q, K), np.float32)
+        for r in range(R):
+            for s_ in range(S):
+                patch = padded[:, r:r + (P - 1) * stride[0] + 1:stride[0], s_:s_ + (Q - 1) * stride[1] + 1:stride[1], :]
+                out += np.einsum("npqc,kc->npqk", patch, flt[:, r, s_, :], optimize=True)
+        out *= np.float32(cfg.get("conv_result_scale", 1))
+        with np.errstate(over="ignore"):
+            res = out.astype(self.np_dtype(out_sh.dtype))
+        scratch = np.zeros(ins.shape.tuple_shapes[1].dims, np.uint8)
+        return (res, scratch)
 
 
 def evaluate(text: str, params: Sequence[np.ndarray], constants: Optional[Dict[str, np.ndarray]] = None,

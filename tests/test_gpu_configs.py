@@ -105,3 +105,68 @@ def test_gpt2_full_size_properties(gpu_device):
     out4 = m.run(inputs, fx.outputs)[0]
     assert np.array_equal(out4[..., 7], out4[..., 11])
     m.close()
+
+
+def _conv_module(xd, fd, stride, pad, bias):
+    from mononn_amd.hlo.builder import HloModuleBuilder
+    mb = HloModuleBuilder("cluster_9__conv.1")
+    e = mb.entry
+    x = e.parameter("f16", xd, "x")
+    f = e.parameter("f16", fd, "f")
+    y = e.conv_forward(x, f, stride=stride, pad=pad)
+    if bias:
+        b = e.parameter("f16", (fd[0],), "b")
+
+        def body(fz, py, pb):
+            return fz.convert(fz.add(fz.convert(py, "f32"), fz.broadcast(fz.convert(pb, "f32"), py.dims, [3])), "f16")
+        y = e.fusion("kLoop", [y, b], body)
+    e.set_tuple_root([y])
+    return mb.text(), y.dims
+
+
+@pytest.mark.parametrize("xd,fd,stride,pad,bias", [
+    ((2, 64, 64, 8), (64, 16, 16, 8), (16, 16), (0, 0), True),      # patch embedding: MFMA tiles, gathered rows
+    ((3, 48, 32, 16), (40, 4, 2, 16), (4, 2), (0, 0), False),       # ragged N (40), rectangular window
+    ((8, 224, 224, 3), (768, 16, 16, 3), (16, 16), (0, 0), True),   # the ViT-B/16 patch GEMM [1568,768]x[768,768]
+    ((2, 9, 10, 4), (6, 3, 3, 4), (2, 1), (1, 1), True),            # padding + overlapping windows: per-element path
+    ((1, 12, 12, 3), (5, 4, 4, 3), (4, 4), (0, 0), False),          # 3 channels, 4x4 window: pieces not 16-byte aligned
+])
+def test_convolution_parity(gpu_device, xd, fd, stride, pad, bias):
+    from mononn_amd import MonoNNModule
+    text, out_dims = _conv_module(xd, fd, stride, pad, bias)
+    rng = np.random.default_rng(41)
+    args = [rng.normal(0, 1, xd).astype(np.float16), rng.normal(0, 0.05, fd).astype(np.float16)]
+    if bias:
+        args.append(rng.normal(0, 0.5, (fd[0],)).astype(np.float16))
+    m = MonoNNModule.compile(text)
+    m.load(gpu_device)
+    got = m.run(args, [{"dtype": "f16", "dims": list(out_dims)}])[0]
+    m.close()
+    want = hlo_interp.evaluate(text, args, {}, "fp32")[0]
+    _check(got, want, f"conv {xd} * {fd} stride {stride} pad {pad}")
+
+
+def test_vit_encoder_parity(gpu_device):
+    fx = models.vit(L=2, B=2, image=64, patch=16, H=256, NH=4, F=512)
+    consts = fx.make_constants(1238, "random")
+    inputs = fx.make_inputs(1238)
+    m, got = _run(fx, consts, inputs, gpu_device)
+    m.close()
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _check(got, want, "vit L=2 B=2 64x64/16")
+
+
+def test_vit_full_size_properties(gpu_device):
+    """ViT-B/16, 12 layers, batch 8, 224x224 pixels, 197 tokens per image."""
+    fx = models.vit()
+    consts = fx.make_constants(1238, "baseline")
+    inputs = fx.make_inputs(1238)
+    m, out = _run(fx, consts, inputs, gpu_device)
+    x = out.astype(np.float64)
+    assert out.shape == (8, 197, 768) and np.isfinite(x).all()
+    assert np.abs(x.mean(-1)).max() < 5e-3 and np.abs(x.var(-1) - 1.0).max() < 2e-2   # final LayerNorm, gamma 1 / beta 0
+    # images are independent: reversing the batch reverses the output, value for value
+    out_rev = m.run([np.ascontiguousarray(inputs[0][::-1])], fx.outputs)[0]
+    assert np.array_equal(out_rev[::-1], out)
+    assert np.array_equal(m.run(inputs, fx.outputs)[0], out)
+    m.close()

@@ -243,3 +243,41 @@ def test_write_once_temp_addresses(layer):
     spec["mononn_hip"]["barrier"] = "flags"
     fenced = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
     assert fenced.buffer_info()["temp"] < coherent.buffer_info()["temp"]     # slots are re-used again
+
+
+def _conv_text(xd=(2, 64, 64, 8), fd=(64, 16, 16, 8), stride=(16, 16), pad=(0, 0)):
+    mb = HloModuleBuilder("cluster_9__conv.1")
+    e = mb.entry
+    x = e.parameter("f16", xd, "x")
+    f = e.parameter("f16", fd, "f")
+    e.set_tuple_root([e.conv_forward(x, f, stride=stride, pad=pad)])
+    return mb.text()
+
+
+def test_convolution_call_is_lowered_as_implicit_gemm():
+    # conv_impl.cc:51: forward convolution = GEMM over (output pixels) x (output channels) x (R*S*C)
+    m = MonoNNModule.compile(_conv_text(), build=False)
+    assert "f16_b1_m32_n64_k2048_ak_bk_conv16x16s16x16p0x0" in m.summary()
+    src = m.get_source("main.hip")
+    assert "_amap" in src and "gemm_tile<" in src          # patch convolution: MFMA tiles with gathered rows
+    # padding breaks the fragment loads: per-element fallback, still one stage
+    m2 = MonoNNModule.compile(_conv_text((2, 9, 10, 4), (6, 3, 3, 4), (2, 1), (1, 1)), build=False)
+    assert "conv_naive_element" in m2.get_source("main.hip")
+    assert m2.buffer_info()["liveouts"] == [2 * 5 * 10 * 6 * 2]
+
+
+@pytest.mark.parametrize("edit,fragment", [
+    (lambda t: t.replace("window={size=16x16 stride=16x16}", "window={size=16x16 stride=16x16 rhs_dilate=2x2}"), "dilated"),
+    (lambda t: t.replace("window={size=16x16 stride=16x16}", "window={size=16x16 stride=16x16 pad=0_1x0_0}"), "symmetric"),
+    (lambda t: t.replace("b01f_o01i->b01f", "bf01_oi01->bf01"), "dim_labels"),
+    (lambda t: t.replace("dim_labels=", "feature_group_count=2, dim_labels="), "grouped"),
+    (lambda t: t.replace("index=0", "index=1").replace("f16[2,4,4,64]{3,2,1,0} get-tuple-element", "u8[0]{0} get-tuple-element", 1), "scratch"),
+])
+def test_unsupported_convolutions_are_rejected(edit, fragment):
+    # the reference aborts on the same constructs (ir_parser_fused.cc:749-798)
+    text = edit(_conv_text())
+    assert text != _conv_text()
+    with pytest.raises(MonoNNError) as e:
+        MonoNNModule.compile(text, build=False)
+    assert e.value.status == "UNSUPPORTED", str(e.value)
+    assert fragment in str(e.value)

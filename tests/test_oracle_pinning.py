@@ -245,3 +245,57 @@ def test_gpt2_decoder_against_torch():
     want = (hf @ R["gpt2/wte"].T).numpy()
     assert got.shape == want.shape
     assert np.abs(got - want).max() < 3e-5
+
+
+def _conv_module(xd, fd, stride, pad):
+    mb = HloModuleBuilder("cluster_9__conv.1")
+    e = mb.entry
+    x = e.parameter("f16", xd, "x")
+    f = e.parameter("f16", fd, "f")
+    e.set_tuple_root([e.conv_forward(x, f, stride=stride, pad=pad)])
+    return mb.text()
+
+
+@pytest.mark.parametrize("xd,fd,stride,pad", [((2, 9, 10, 4), (6, 3, 3, 4), (2, 1), (1, 1)),
+                                              ((1, 12, 12, 3), (5, 4, 4, 3), (4, 4), (0, 0)),
+                                              ((3, 7, 5, 2), (4, 1, 1, 2), (1, 1), (0, 0)),
+                                              ((2, 8, 8, 8), (16, 5, 3, 8), (1, 2), (2, 1))])
+def test_conv_forward_matches_torch_conv2d(xd, fd, stride, pad):
+    # N,H,W,C input, K,R,S,C filter, N,P,Q,K output against the library routine on NCHW / OIHW
+    rng = np.random.default_rng(31)
+    x = rng.normal(0, 1, xd).astype(np.float16)
+    w = rng.normal(0, 1, fd).astype(np.float16)
+    got = hlo_interp.evaluate(_conv_module(xd, fd, stride, pad), [x, w], {}, "fp32")[0]
+    want = F.conv2d(torch.tensor(x.astype(np.float32)).permute(0, 3, 1, 2), torch.tensor(w.astype(np.float32)).permute(0, 3, 1, 2),
+                    stride=stride, padding=pad).permute(0, 2, 3, 1).numpy()
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() < 2e-5
+
+
+def test_vit_encoder_against_torch():
+    B, image, patch, H, NH, Fd = 2, 32, 8, 64, 4, 128
+    fx = models.vit(L=2, B=B, image=image, patch=patch, H=H, NH=NH, F=Fd)
+    consts = fx.make_constants(23, "random")
+    inputs = fx.make_inputs(23)
+    got = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    R = {m["role"]: torch.tensor(consts[n].astype(np.float32)) for n, m in fx.constants.items()}
+    px = torch.tensor(inputs[0].astype(np.float32))
+    S, D = (image // patch) ** 2 + 1, H // NH
+    emb = F.conv2d(px, R["vit/embeddings/patch_embeddings/kernel"].permute(0, 3, 1, 2), R["vit/embeddings/patch_embeddings/bias"], stride=patch)
+    # the patch embedding is rounded to fp16 where the HLO says so only in "as_written" mode; fp32 mode keeps it wide
+    tok = torch.cat([R["vit/embeddings/cls_token"].expand(B, 1, H), emb.flatten(2).transpose(1, 2)], 1)
+    h = tok + R["vit/embeddings/position_embeddings"][None]
+    for l in range(2):
+        P = f"vit/encoder/layer_{l}/"
+
+        def lin(x, p):
+            return x @ R[P + p + "/kernel"] + R[P + p + "/bias"]
+        a = F.layer_norm(h, (H,), R[P + "attention/LayerNorm/gamma"], R[P + "attention/LayerNorm/beta"], 1e-6)
+        q, k, v = (lin(a, "attention/" + n).view(B, S, NH, D).transpose(1, 2) for n in ("query", "key", "value"))
+        ctx = (torch.softmax(q @ k.transpose(2, 3) / math.sqrt(D), -1) @ v).transpose(1, 2).reshape(B, S, H)
+        h = h + lin(ctx, "attention/output")
+        m = F.layer_norm(h, (H,), R[P + "output/LayerNorm/gamma"], R[P + "output/LayerNorm/beta"], 1e-6)
+        h = h + lin(F.gelu(lin(m, "intermediate"), approximate="tanh"), "output")
+    want = F.layer_norm(h, (H,), R["vit/layernorm/gamma"], R["vit/layernorm/beta"], 1e-6).numpy()
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() < 5e-5
