@@ -55,6 +55,70 @@ def gemm_flops(cfg) -> int:
     return per_layer * L
 
 
+def torch_baseline(fx, consts, inputs, got):
+    """The same encoder as plain PyTorch-ROCm fp16 (rocBLAS / MIOpen kernels), for scale: eager launches and the same
+    launches replayed from a captured HIP graph.  Not part of the measured path."""
+    import math
+    import torch
+    import torch.nn.functional as F
+    cfg = fx.config
+    dev = torch.device("cuda", 0)
+    R = {m["role"]: torch.from_numpy(consts[n]).to(dev) for n, m in fx.constants.items()}
+    B, S, H, NH, L = cfg["B"], cfg["S"], cfg["H"], cfg["NH"], cfg["L"]
+    D = H // NH
+    ids, mask, tt = (torch.from_numpy(a.astype(np.int64)).to(dev) for a in inputs)
+    Wt = {k: v.t().contiguous() for k, v in R.items() if k.endswith("/kernel")}   # F.linear takes [out, in]
+
+    def forward():
+        emb = R["bert/embeddings/word_embeddings"][ids] + R["bert/embeddings/position_embeddings"][:S][None] + \
+            R["bert/embeddings/token_type_embeddings"][tt]
+        h = F.layer_norm(emb, (H,), R["bert/embeddings/LayerNorm/gamma"], R["bert/embeddings/LayerNorm/beta"], 1e-12)
+        add = ((1.0 - mask.to(torch.float16)) * -10000.0)[:, None, None, :]
+        for l in range(L):
+            P = f"bert/encoder/layer_{l}/"
+
+            def lin(x, p):
+                return F.linear(x, Wt[P + p + "/kernel"], R[P + p + "/bias"])
+            q, k, v = (lin(h, "attention/" + n).view(B, S, NH, D).transpose(1, 2) for n in ("query", "key", "value"))
+            p = torch.softmax(q @ k.transpose(2, 3) / math.sqrt(D) + add, -1)
+            ctx = (p @ v).transpose(1, 2).reshape(B, S, H)
+            x1 = F.layer_norm(lin(ctx, "attention/output") + h, (H,), R[P + "attention/LayerNorm/gamma"], R[P + "attention/LayerNorm/beta"], 1e-12)
+            a = F.gelu(lin(x1, "intermediate"), approximate="tanh")
+            h = F.layer_norm(lin(a, "output") + x1, (H,), R[P + "output/LayerNorm/gamma"], R[P + "output/LayerNorm/beta"], 1e-12)
+        return h
+
+    def time_it(fn, n):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    with torch.no_grad():
+        out = forward()
+        eager_us = time_it(forward, 100)
+        graph_us = None
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    forward()
+            torch.cuda.current_stream().wait_stream(side)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                forward()
+            graph_us = time_it(g.replay, 200)
+        except Exception as e:   # graph capture is a convenience here, not a requirement
+            print(f"bench.py: HIP graph capture of the torch model failed: {e}", file=sys.stderr)
+    diff = float(np.abs(out.float().cpu().numpy() - got).max())
+    return {"eager_us_per_forward": round(eager_us, 1), "hip_graph_us_per_forward": None if graph_us is None else round(graph_us, 1),
+            "max_abs_diff_vs_kernel": diff, "note": "torch.nn.functional fp16 on the same GPU; scale only"}
+
+
 def stage_profile(module, fx, consts, inputs, args):
     """Per-stage clocks of the benchmark's own specification (stamped by every workgroup at stage entry / exit)."""
     from mononn_amd import MonoNNModule
@@ -98,6 +162,9 @@ def main():
     ap.add_argument("--spec-dir", default=SPEC_DIR)
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof counters)")
+    ap.add_argument("--torch-baseline", action="store_true",
+                    help="also time the same model written with torch.nn.functional in fp16 on this GPU (eager and "
+                         "captured in a HIP graph), reported under \"torch_baseline\"")
     ap.add_argument("--stage-profile", action="store_true",
                     help="instead of the benchmark: rebuild the same specification with per-stage clocks and print, "
                          "per stage, busy time / barrier time averaged over --steps launches")
@@ -203,6 +270,9 @@ def main():
         "mfma": {"achieved_tflops": round(achieved_tflops, 2), "peak_tflops": MFMA_F16_PEAK_TFLOPS,
                  "frac": round(achieved_tflops / MFMA_F16_PEAK_TFLOPS, 5), "gemm_flops": flops},
     }
+
+    if args.torch_baseline:
+        result["torch_baseline"] = torch_baseline(fx, consts, inputs, got)
 
     if not args.no_cpu_baseline:
         from oracle import hlo_interp

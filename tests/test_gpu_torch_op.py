@@ -1,0 +1,40 @@
+"""The PyTorch front end (mononn_amd/torch_op.py): same kernel, torch tensors as buffers, torch's current stream."""
+import numpy as np
+import pytest
+
+from mononn_amd.hlo import models
+
+pytestmark = pytest.mark.gpu
+
+
+def test_custom_op_matches_the_ctypes_path_bit_for_bit(gpu_device):
+    import torch
+    from mononn_amd import MonoNNModule
+    from mononn_amd import torch_op
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
+    consts = fx.make_constants(31, "random")
+    inputs = fx.make_inputs(31)
+    m = MonoNNModule.compile(fx.hlo_text)
+    m.set_constants(consts)
+    m.load(gpu_device)
+    want = m.run(inputs, fx.outputs)[0]
+    fn = torch_op.MonoNNFunction(m, fx.outputs, gpu_device)
+    dev = torch.device("cuda", gpu_device)
+    tin = [torch.from_numpy(a).to(dev) for a in inputs]
+    (got,) = torch_op.forward(fn, *tin)
+    assert got.dtype == torch.float16 and tuple(got.shape) == tuple(fx.outputs[0]["dims"])
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # on a side stream, ordered after work that torch queued there
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        ids2 = (tin[0] + 1) % 300
+        (got2,) = torch.ops.mononn.forward(fn.handle, [ids2, tin[1], tin[2]])
+        back = (ids2 - 1) % 300
+        (got3,) = torch.ops.mononn.forward(fn.handle, [back, tin[1], tin[2]])
+    side.synchronize()
+    assert not np.array_equal(got2.cpu().numpy(), want)
+    assert np.array_equal(got3.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    with pytest.raises(AssertionError):
+        fn(tin[0][:, :32], tin[1], tin[2])          # wrong size is refused before anything is launched
+    fn.close()
+    m.close()
