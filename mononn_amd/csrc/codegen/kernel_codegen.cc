@@ -1,5 +1,7 @@
 #include "codegen/kernel_codegen.h"
 
+#include "codegen/host_codegen.h"
+
 #include <algorithm>
 #include <set>
 #include <sstream>
@@ -346,6 +348,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   hp.body = src.str();
   hp.files["headers.h"] = device::kPreludeText;
   hp.files["main.hip"] = hp.preamble + glob.str() + hp.body;
+  hp.files["host_main.cpp"] = generate_host_driver(hp);
   return hp;
 }
 

@@ -129,7 +129,7 @@ struct Builder {
       Node n;
       n.name = ins->name;
       n.members.push_back(ins);
-      if (op == "custom-call") {
+      if (op == "custom-call" || op == "dot") {
         n.kind = NodeKind::kGemm;
         n.gemm = ins->is_conv() ? describe_conv(ins) : describe_gemm(ins);
       } else {
@@ -261,7 +261,7 @@ struct Builder {
     if (root->shape.dims != operand->shape.dims) return false;   // reached through a reshaping alias
     for (auto* u : root->users) {
       if (is_alias_op(u)) return false;
-      bool as_b = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands[1] == root && u->operands[0] != root &&
+      bool as_b = u->is_gemm() && u->operands[1] == root && u->operands[0] != root &&
                   (u->operands.size() < 3 || u->operands[2] != root) && u->gemm.rhs_contracting == rhs_contracting;
       if (!as_b) return false;
     }
@@ -485,7 +485,7 @@ struct Builder {
       if (c->opcode != "constant" || c->is_scalar_constant() || c->shape.rank() != 2) continue;
       bool all = !c->users.empty();
       for (auto* u : c->users) {
-        bool good = u->opcode == "custom-call" && u->custom_call_target == "__cublas$gemm" && u->operands.size() >= 2 &&
+        bool good = u->is_gemm() && u->operands.size() >= 2 &&
                     u->operands[1] == c && u->operands[0] != c && u->gemm.rhs_contracting == 0 && c->shape.dims[0] % 32 == 0 &&
                     u->gemm.lhs_contracting == u->operands[0]->shape.rank() - 1 && (u->operands.size() < 3 || u->operands[2] != c);
         if (!good) all = false;

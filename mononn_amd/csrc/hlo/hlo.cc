@@ -34,7 +34,7 @@ const DTypeInfo kDTypes[] = {
 const std::set<std::string>& known_opcodes() {
   static const std::set<std::string> s = {
       "abs", "add", "bitcast", "broadcast", "clamp", "compare", "concatenate", "constant", "convert",
-      "convolution", "copy", "custom-call", "divide", "dynamic-slice", "dynamic-update-slice",
+      "convolution", "copy", "custom-call", "divide", "dot", "dynamic-slice", "dynamic-update-slice",
       "exponential", "gather", "get-tuple-element", "iota", "log", "maximum", "minimum", "multiply",
       "negate", "pad", "parameter", "reduce", "reduce-window", "reshape", "rsqrt", "select", "sign",
       "slice", "subtract", "tanh", "transpose", "tuple", "fusion", "sqrt", "power", "and", "or", "not"};
@@ -289,7 +289,9 @@ Shape parse_shape(Lexer& lx) {
 void decode_gemm_config(Instr* ins) {
   auto it = ins->attrs.find("backend_config");
   MONONN_CHECK(it != ins->attrs.end(), kParseError) << ins->hlo_name << ": __cublas$gemm without backend_config";
-  Json j = Json::parse(it->second);
+  Json top = Json::parse(it->second);
+  // newer XLA nests the fields: {"gemm_backend_config": {...}}
+  const Json& j = top.contains("gemm_backend_config") ? top.at("gemm_backend_config") : top;
   GemmConfig& g = ins->gemm;
   g.alpha_real = j.at("alpha_real").as_double();
   if (j.contains("alpha_imag")) g.alpha_imag = j.at("alpha_imag").as_double();
@@ -416,6 +418,34 @@ void decode_conv_config(Instr* ins) {
   ins->shape = arr;
 }
 
+// dot(lhs, rhs), lhs_batch_dims={0,1}, lhs_contracting_dims={3}, rhs_batch_dims={0,1}, rhs_contracting_dims={2}
+// -> the same GemmConfig a __cublas$gemm call carries (alpha 1, beta 0)
+void decode_dot_config(Instr* ins) {
+  auto dims = [&](const char* k) {
+    auto it = ins->attrs.find(k);
+    return it == ins->attrs.end() ? std::vector<int64_t>() : ints_of(it->second);
+  };
+  MONONN_CHECK(ins->operands.size() == 2, kParseError) << ins->hlo_name << ": dot takes two operands";
+  auto lc = dims("lhs_contracting_dims"), rc = dims("rhs_contracting_dims"), lb = dims("lhs_batch_dims"), rb = dims("rhs_batch_dims");
+  MONONN_CHECK(lc.size() == 1 && rc.size() == 1, kUnsupported) << ins->hlo_name << ": exactly one contracting dimension per operand is supported";
+  MONONN_CHECK(lb == rb, kUnsupported) << ins->hlo_name << ": batch dimensions of the two operands must be the same";
+  for (size_t i = 0; i < lb.size(); ++i)
+    MONONN_CHECK(lb[i] == static_cast<int64_t>(i), kUnsupported) << ins->hlo_name << ": batch dimensions must be the leading dimensions, in order";
+  MONONN_CHECK(static_cast<int>(lb.size()) == ins->operands[0]->shape.rank() - 2, kUnsupported)
+      << ins->hlo_name << ": every operand must have exactly two non-batch dimensions";
+  GemmConfig& g = ins->gemm;
+  g.alpha_real = 1;
+  g.beta = 0;
+  g.lhs_contracting = static_cast<int>(lc[0]);
+  g.rhs_contracting = static_cast<int>(rc[0]);
+  g.batch_size = 1;
+  for (size_t i = 0; i < lb.size(); ++i) {
+    g.lhs_batch.push_back(static_cast<int>(lb[i]));
+    g.rhs_batch.push_back(static_cast<int>(rb[i]));
+    g.batch_size *= ins->operands[0]->shape.dims[lb[i]];
+  }
+}
+
 void decode_attrs(Instr* ins, Module* mod) {
   auto has = [&](const char* k) { return ins->attrs.count(k) > 0; };
   auto get = [&](const char* k) -> const std::string& { return ins->attrs.at(k); };
@@ -511,6 +541,7 @@ void decode_attrs(Instr* ins, Module* mod) {
       MONONN_FAIL(kUnsupported) << ins->hlo_name << ": custom-call target '" << ins->custom_call_target << "' is not supported";
     }
   }
+  if (op == "dot") decode_dot_config(ins);
   if (op == "convolution") {
     // a bare convolution aborts in the reference as well (ir_parser_fused.cc:728-732)
     MONONN_FAIL(kUnsupported) << ins->hlo_name << ": bare convolution is not supported; expected custom-call __cudnn$convForward";

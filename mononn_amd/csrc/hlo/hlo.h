@@ -92,6 +92,9 @@ struct Instr {
   GemmConfig gemm;
   ConvConfig conv;
   bool is_conv() const { return opcode == "custom-call" && custom_call_target == "__cudnn$convForward"; }
+  // a dense contraction with a decoded GemmConfig: the cuBLAS custom call, or a plain `dot` (what a stock XLA
+  // prints before its GEMM rewriter has run)
+  bool is_gemm() const { return (opcode == "custom-call" && custom_call_target == "__cublas$gemm") || opcode == "dot"; }
 
   std::vector<Instr*> users;           // within the same computation
   bool is_scalar_constant() const { return opcode == "constant" && shape.num_elements() == 1 && !literal_elided; }

@@ -120,33 +120,36 @@ void MonoNNModule::set_constant(const std::string& name, const void* host_data, 
   }
 }
 
+// bytes of the module global for a payload given in the HLO's layout
+static std::vector<char> device_payload(const codegen::ConstantInfo& ci, const std::vector<char>& payload) {
+  if (ci.transform != graph::ConstantTransform::kPackMfmaB) return payload;
+  // [K,N] row-major -> [ceil(N/16)][K/32][64][8]: one MFMA B operand per contiguous KiB
+  const int es = hlo::dtype_bytes(ci.dtype);
+  const int64_t K = ci.dims[0], N = ci.dims[1];
+  const int64_t nt_count = (N + 15) / 16, ksteps = K / 32;
+  MONONN_CHECK(es == 2 && K % 32 == 0, kInternal) << "constant " << ci.hlo_name << " cannot be packed";
+  std::vector<char> t(static_cast<size_t>(ci.device_bytes), 0);
+  const uint16_t* src = reinterpret_cast<const uint16_t*>(payload.data());
+  uint16_t* dstp = reinterpret_cast<uint16_t*>(t.data());
+  for (int64_t nt = 0; nt < nt_count; ++nt)
+    for (int64_t ks = 0; ks < ksteps; ++ks)
+      for (int l = 0; l < 64; ++l) {
+        const int64_t n = nt * 16 + (l & 15);
+        if (n >= N) continue;
+        const int64_t k0 = ks * 32 + (l >> 4) * 8;
+        uint16_t* o = dstp + ((nt * ksteps + ks) * 64 + l) * 8;
+        for (int j = 0; j < 8; ++j) o[j] = src[(k0 + j) * N + n];
+      }
+  return t;
+}
+
 void MonoNNModule::upload_constant(const codegen::ConstantInfo& ci, const std::vector<char>& payload) {
   size_t n = 0;
   void* dst = dev_.global(ci.symbol, &n);
   MONONN_CHECK(static_cast<int64_t>(n) >= ci.bytes, kRuntimeError) << "global " << ci.symbol << " is smaller than its constant";
-  if (ci.transform == graph::ConstantTransform::kPackMfmaB) {
-    // [K,N] row-major -> [ceil(N/16)][K/32][64][8]: one MFMA B operand per contiguous KiB
-    const int es = hlo::dtype_bytes(ci.dtype);
-    const int64_t K = ci.dims[0], N = ci.dims[1];
-    const int64_t nt_count = (N + 15) / 16, ksteps = K / 32;
-    MONONN_CHECK(es == 2 && K % 32 == 0, kInternal) << "constant " << ci.hlo_name << " cannot be packed";
-    std::vector<char> t(static_cast<size_t>(ci.device_bytes), 0);
-    const uint16_t* src = reinterpret_cast<const uint16_t*>(payload.data());
-    uint16_t* dstp = reinterpret_cast<uint16_t*>(t.data());
-    for (int64_t nt = 0; nt < nt_count; ++nt)
-      for (int64_t ks = 0; ks < ksteps; ++ks)
-        for (int l = 0; l < 64; ++l) {
-          const int64_t n = nt * 16 + (l & 15);
-          if (n >= N) continue;
-          const int64_t k0 = ks * 32 + (l >> 4) * 8;
-          uint16_t* o = dstp + ((nt * ksteps + ks) * 64 + l) * 8;
-          for (int j = 0; j < 8; ++j) o[j] = src[(k0 + j) * N + n];
-        }
-    MONONN_CHECK(static_cast<int64_t>(n) >= ci.device_bytes, kRuntimeError) << "global " << ci.symbol << " is smaller than its packed constant";
-    dev_.upload(dst, t.data(), t.size());
-  } else {
-    dev_.upload(dst, payload.data(), payload.size());
-  }
+  std::vector<char> t = device_payload(ci, payload);
+  MONONN_CHECK(n >= t.size(), kRuntimeError) << "global " << ci.symbol << " is smaller than its constant in device layout";
+  dev_.upload(dst, t.data(), t.size());
   uploaded_[ci.name] = true;
 }
 
@@ -295,6 +298,22 @@ void MonoNNModule::dump_best(const std::string& dump_dir) const {
   make_dirs(dir);
   write_file(dir + "/best_tuning_spec.json", tuning_spec_json());
   if (has_code_object()) write_file(dir + "/best_tuning_spec.hsaco", code_object_);
+  // source of the kernel and of the standalone driver (host_main.cpp), and what that driver feeds the module
+  // globals with: literal constants always, elided ones when the host has supplied them and the module has not
+  // been loaded yet (payloads are handed to the device at load time)
+  make_dirs(dir + "/best_tuning_spec_src");
+  for (auto& kv : hip_.files) write_file(dir + "/best_tuning_spec_src/" + kv.first, kv.second);
+  bool any = false;
+  for (auto& c : hip_.constants) {
+    std::vector<char> bytes;
+    auto it = host_constants_.find(c.name);
+    if (!c.literal.empty()) bytes = device_payload(c, literal_payload(c));
+    else if (it != host_constants_.end()) bytes = device_payload(c, it->second);
+    else continue;
+    if (!any) make_dirs(dir + "/constants");
+    any = true;
+    write_file(dir + "/constants/" + c.symbol + ".bin", bytes);
+  }
 }
 
 }  // namespace module

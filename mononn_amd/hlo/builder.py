@@ -262,6 +262,24 @@ class Computation:
                           attrs=f'custom_call_target="__cublas$gemm", backend_config="{cfg_s}"',
                           name_hint="cublas-batch-gemm" if batch > 1 else "cublas-gemm")
 
+    def dot(self, a: Value, b: Value, lhs_contract: int, rhs_contract: int, batch_dims: Sequence[int] = ()) -> Value:
+        """Plain `dot` with the same operand conventions as `gemm` (what XLA prints before its GEMM rewriter)."""
+        r = len(a.dims)
+        nb = len(batch_dims)
+        assert len(b.dims) == r and list(batch_dims) == list(range(nb)) and nb == r - 2
+        m_dim = r - 1 if lhs_contract == r - 2 else r - 2
+        n_dim = r - 1 if rhs_contract == r - 2 else r - 2
+        out_dims = list(a.dims[:nb]) + [a.dims[m_dim], b.dims[n_dim]]
+        attrs = ""
+        if nb:
+            bd = ",".join(str(d) for d in batch_dims)
+            attrs = f"lhs_batch_dims={{{bd}}}, "
+        attrs += f"lhs_contracting_dims={{{lhs_contract}}}, "
+        if nb:
+            attrs += f"rhs_batch_dims={{{bd}}}, "
+        attrs += f"rhs_contracting_dims={{{rhs_contract}}}"
+        return self._emit("dot", a.dtype, out_dims, [a, b], attrs=attrs, name_hint="dot")
+
     def conv_forward(self, x: Value, filt: Value, stride: Sequence[int] = (1, 1), pad: Sequence[int] = (0, 0),
                      result_scale: float = 1.0) -> Value:
         """`__cudnn$convForward` custom call on an N,H,W,C input and a K,R,S,C filter (dim_labels

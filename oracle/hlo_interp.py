@@ -361,6 +361,18 @@ class Evaluator:
             sizes = _ints(ins.attrs["dynamic_slice_sizes"])
             starts = [int(np.clip(int(s), 0, x[0].shape[i] - sizes[i])) for i, s in enumerate(x[1:])]
             return x[0][tuple(slice(s, s + n) for s, n in zip(starts, sizes))]
+        if op == "dot":
+            lc, rc = _ints(ins.attrs["lhs_contracting_dims"])[0], _ints(ins.attrs["rhs_contracting_dims"])[0]
+            A, B = x[0].astype(np.float32), x[1].astype(np.float32)
+            r = A.ndim
+            if _ints(ins.attrs.get("lhs_batch_dims", "")) != list(range(r - 2)):
+                raise NotImplementedError("dot: batch dims must be the leading dims")
+            if lc == r - 2:
+                A = np.swapaxes(A, -1, -2)
+            if rc == r - 1:
+                B = np.swapaxes(B, -1, -2)
+            with np.errstate(over="ignore"):
+                return np.matmul(A, B).astype(dt)
         if op == "custom-call":
             target = ins.attrs["custom_call_target"].strip('"')
             if target == "__cublas$gemm":
@@ -395,6 +407,7 @@ class Evaluator:
 
     def _gemm(self, ins: Instr, x, dt):
         cfg = json.loads(ins.attrs["backend_config"][1:-1].replace('\\"', '"'))
+        cfg = cfg.get("gemm_backend_config", cfg)
         dn = cfg["dot_dimension_numbers"]
         lc = int(dn["lhs_contracting_dimensions"][0])
         rc = int(dn["rhs_contracting_dimensions"][0])

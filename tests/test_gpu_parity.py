@@ -30,7 +30,7 @@ def check_close(got, want32, atol=2e-2, cos_min=0.9999):
     return err, cos
 
 
-def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=False):
+def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=False, as_dot=False):
     mb = HloModuleBuilder("cluster_7__gemm_test.1")
     e = mb.entry
     r = len(batch) + 2
@@ -40,7 +40,10 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
     b_dims = list(batch) + ([K, N] if rhs_c == r - 2 else [N, K])
     a = e.parameter("f16", a_dims, "a")
     b = e.elided_constant("f16", b_dims, "w/kernel") if b_const else e.parameter("f16", b_dims, "b")
-    d = e.gemm(a, b, lhs_c, rhs_c, batch_dims=tuple(range(len(batch))), alpha=alpha)
+    if as_dot:
+        d = e.dot(a, b, lhs_c, rhs_c, batch_dims=tuple(range(len(batch))))
+    else:
+        d = e.gemm(a, b, lhs_c, rhs_c, batch_dims=tuple(range(len(batch))), alpha=alpha)
     e.set_tuple_root([d])
     return mb, a_dims, b_dims, list(batch) + [M, N]
 
@@ -53,6 +56,8 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
     dict(M=100, N=52, K=96, rhs_c=1),                             # ragged M / N on the MFMA path
     dict(M=64, N=48, K=40, rhs_c=1),                              # K not a multiple of 32
     dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                     # A stored [K,M]
+    dict(M=128, N=256, K=256, b_const=True, as_dot=True),         # plain `dot` with a constant right operand
+    dict(M=48, N=80, K=64, batch=(3,), rhs_c=2, as_dot=True),     # batched `dot`, both operands k-contiguous
 ])
 def test_gemm_cases(gpu_device, case):
     mb, a_dims, b_dims, d_dims = gemm_module(**case)

@@ -281,3 +281,46 @@ def test_unsupported_convolutions_are_rejected(edit, fragment):
         MonoNNModule.compile(text, build=False)
     assert e.value.status == "UNSUPPORTED", str(e.value)
     assert fragment in str(e.value)
+
+
+def test_plain_dot_and_nested_backend_config_are_gemms():
+    mb = HloModuleBuilder("cluster_5__dot.1")
+    e = mb.entry
+    a = e.parameter("f16", (128, 256), "a")
+    w = e.elided_constant("f16", (256, 512), "w/kernel")
+    e.set_tuple_root([e.dot(a, w, 1, 0)])
+    m = MonoNNModule.compile(mb.text(), build=False)
+    assert "gemm    dot_" in m.summary() and "f16_b1_m128_n512_k256_ak_bp" in m.summary()   # constant packed for the MFMA path
+    # newer XLA prints the cuBLAS fields one level down, under "gemm_backend_config"
+    mb2 = HloModuleBuilder("cluster_5__gemm.1")
+    e2 = mb2.entry
+    a2 = e2.parameter("f16", (128, 256), "a")
+    b2 = e2.parameter("f16", (256, 64), "b")
+    e2.set_tuple_root([e2.gemm(a2, b2, 1, 0, alpha=0.5)])
+    text = mb2.text()
+    nested = text.replace('backend_config="{', 'backend_config="{\\"gemm_backend_config\\":{').replace('}", ', '}}", ', 1) \
+        if '}", ' in text else text.replace('backend_config="{', 'backend_config="{\\"gemm_backend_config\\":{').replace('}"\n', '}}"\n', 1)
+    assert nested != text and "gemm_backend_config" in nested
+    m1 = MonoNNModule.compile(text, build=False)
+    m2 = MonoNNModule.compile(nested, build=False)
+    assert m1.summary() == m2.summary()
+    assert m1.get_source("main.hip") == m2.get_source("main.hip")
+
+
+def test_dump_contains_a_standalone_driver_and_the_constants(layer, tmp_path):
+    # host_codegen.cc:31-73 counterpart: the dump can be run without the library
+    m = MonoNNModule.compile(layer.hlo_text, build=True)
+    consts = layer.make_constants(3, "random")
+    m.set_constants(consts)
+    m.dump(str(tmp_path))
+    cluster = os.path.join(tmp_path, "cluster_0")
+    src = open(os.path.join(cluster, "best_tuning_spec_src", "host_main.cpp")).read()
+    assert "hipModuleLoadData" in src and 'kKernel = "mononn_cluster_0"' in src
+    info = m.buffer_info()
+    assert f"kTempBytes = {info['temp']}" in src
+    names = sorted(os.listdir(os.path.join(cluster, "constants")))
+    assert len(names) == len(consts)
+    # a packed GEMM weight is dumped in the layout of its module global (padded to 16 columns)
+    for c in m.constants():
+        path = os.path.join(cluster, "constants", "buffer_for_" + c["name"].lstrip("%").replace(".", "_").replace("-", "_") + ".bin")
+        assert os.path.getsize(path) >= c["bytes"]

@@ -299,3 +299,24 @@ def test_vit_encoder_against_torch():
     want = F.layer_norm(h, (H,), R["vit/layernorm/gamma"], R["vit/layernorm/beta"], 1e-6).numpy()
     assert got.shape == want.shape
     assert np.abs(got - want).max() < 5e-5
+
+
+def test_dot_matches_einsum_and_the_gemm_call():
+    # a plain `dot` means the same contraction as the cuBLAS call with alpha 1 / beta 0
+    rng = np.random.default_rng(33)
+    A = rng.normal(0, 1, (3, 40, 64)).astype(np.float16)
+    B = rng.normal(0, 1, (3, 24, 64)).astype(np.float16)
+    texts = []
+    for kind in ("dot", "gemm"):
+        mb = HloModuleBuilder("cluster_5__dot.1")
+        e = mb.entry
+        a = e.parameter("f16", A.shape, "a")
+        b = e.parameter("f16", B.shape, "b")
+        d = e.dot(a, b, 2, 2, batch_dims=(0,)) if kind == "dot" else e.gemm(a, b, 2, 2, batch_dims=(0,))
+        e.set_tuple_root([d])
+        texts.append(mb.text())
+    got_dot = hlo_interp.evaluate(texts[0], [A, B], {}, "fp32")[0]
+    got_gemm = hlo_interp.evaluate(texts[1], [A, B], {}, "fp32")[0]
+    want = np.einsum("bmk,bnk->bmn", A.astype(np.float64), B.astype(np.float64))
+    assert np.abs(got_dot - want).max() < 2e-5
+    assert np.array_equal(got_dot, got_gemm)
