@@ -275,7 +275,7 @@ class MonoNNModule:
         self.launch_raw(self.buffer_pointers(), stream)
         torch.cuda.synchronize()
         outs = []
-        npdt = {"f16": np.float16, "f32": np.float32, "s32": np.int32, "pred": np.bool_, "s64": np.int64}
+        npdt = {"f16": np.float16, "f32": np.float32, "s32": np.int32, "pred": np.bool_, "s64": np.int64, "u8": np.uint8, "s8": np.int8}
         for t, o in zip(b["liveouts"], out_dtypes_dims):
             outs.append(t.cpu().numpy().view(npdt[o["dtype"]]).reshape(o["dims"]).copy())
         return outs
