@@ -998,13 +998,19 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
 // tiles t with t % KW == kw and runs the epilogue on them.
 NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,
                            const Instr* g2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epi_members,
-                           const std::vector<const Instr*>& outputs, const LaunchShape& ls) {
+                           const std::vector<const Instr*>& outputs, const LaunchShape& ls, int key_waves) {
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
   MONONN_CHECK(K1 % 32 == 0 && N1 % 32 == 0 && N2 % 16 == 0, kUnsupported) << "attention fusion: extents must be MFMA multiples";
   int KW = 1;
   while (KW * 2 <= NW && N1 % (32 * KW * 2) == 0 && N1 / (KW * 2) >= 32) KW *= 2;
+  if (key_waves > 0) {
+    // tuning knob: fewer key slices per row block mean fewer exchanges through LDS but fewer, longer units
+    MONONN_CHECK(NW % key_waves == 0 && N1 % (32 * key_waves) == 0, kSpecError)
+        << "attention: " << key_waves << " key waves do not divide " << NW << " waves / " << N1 << " keys";
+    KW = key_waves;
+  }
   const int RW = NW / KW;
   const int64_t NKW = N1 / KW;   // keys per wave
   const int KS1 = static_cast<int>(K1 / 32), NT1 = static_cast<int>(NKW / 16), KS2 = static_cast<int>(NKW / 32), NT2 = static_cast<int>(N2 / 16);
@@ -1195,10 +1201,16 @@ NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchSh
   return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores);
 }
 
-NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls) {
+NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves) {
   std::vector<const Instr*> row(node.members.begin() + 1, node.members.begin() + node.gemm2_index);
   std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.end());
-  return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls);
+  return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls, key_waves);
+}
+
+int default_attention_key_waves(const graph::GemmDesc& d1, const LaunchShape& ls) {
+  int KW = 1;
+  while (KW * 2 <= ls.waves() && d1.N % (32 * KW * 2) == 0 && d1.N / (KW * 2) >= 32) KW *= 2;
+  return KW;
 }
 
 bool can_fuse_prologue(const Program& prog, const std::vector<const Instr*>& row_members, const std::vector<const Instr*>& gemm_members,
@@ -1229,7 +1241,7 @@ bool can_fuse_attention(const Program& prog, const Instr* gemm1, const graph::Ge
     if (outs.empty()) return false;
     graph::GemmDesc d2k = d2;
     d2k.b_k_contig = true;   // the layout pass stores the operand k-contiguous before real generation
-    gen_attention(prog, gemm1, d1, row_members, gemm2, d2k, epilogue_members, outs, LaunchShape{});
+    gen_attention(prog, gemm1, d1, row_members, gemm2, d2k, epilogue_members, outs, LaunchShape{}, 0);
     return true;
   } catch (const Error& e) {
     if (e.code() == kUnsupported) return false;

@@ -49,7 +49,10 @@ NodeFunction generate_cluster(const graph::Program& prog, const graph::Node& nod
 NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls,
                            const GemmTuning& t);
 
-NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls);
+// key_waves: waves of a workgroup that share one block of 16 query rows by splitting the keys between them
+// (0 = as many as the key count allows); the remaining factor of the workgroup's waves takes further row blocks
+NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls, int key_waves = 0);
+int default_attention_key_waves(const graph::GemmDesc& first_gemm, const LaunchShape& ls);
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus);
 // throws Error(kSpecError) when the tile / wave arrangement cannot be generated for this GEMM

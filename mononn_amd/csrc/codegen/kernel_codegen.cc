@@ -133,7 +133,23 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   for (auto& n : prog.nodes) {
     NodeFunction f;
     if (n.kind == NodeKind::kAttention) {
-      f = generate_attention(prog, n, ls);
+      // the fused node borrows a gemm_spec_list entry; of its fields only wave_arrangement.k (key waves) is used
+      auto it = spec.gemm_spec_list.find(n.name);
+      if (it == spec.gemm_spec_list.end()) {
+        spec::GemmSpec g;
+        g.wave_k = default_attention_key_waves(n.gemm, ls);
+        g.wave_m = ls.waves() / g.wave_k;
+        g.wave_n = 1;
+        g.tb_m = 16 * g.wave_m;
+        g.tb_n = static_cast<int>(n.gemm.N);
+        g.warp_m = 16;
+        g.warp_n = static_cast<int>(n.gemm.N / g.wave_k);
+        g.warp_k = static_cast<int>(n.gemm.K);
+        auto bc = n.members[0]->attrs.find("backend_config");
+        if (bc != n.members[0]->attrs.end()) g.backend_config = Json::parse(bc->second);
+        it = spec.gemm_spec_list.emplace(n.name, g).first;
+      }
+      f = generate_attention(prog, n, ls, it->second.wave_k);
     } else if (n.kind == NodeKind::kGemm) {
       auto it = spec.gemm_spec_list.find(n.name);
       GemmTuning t;

@@ -263,6 +263,20 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           std::snprintf(lbl, sizeof lbl, "tile%dx%d_waves%dx%dx%d", t.bm, t.bn, t.wm, t.wn, t.wk);
           add(lbl, s);
         }
+      } else if (c.kind == "attention") {
+        // key waves per row block: 1 (no exchange through LDS, a wave owns whole rows) .. all waves
+        for (int kw = 1; kw <= cx.block / 64; kw *= 2) {
+          if (c.sample->gemm.N % (32 * kw) != 0) continue;
+          GraphSpecification s = filled;
+          for (auto& n : c.nodes) {
+            spec::GemmSpec& g = s.gemm_spec_list[n];
+            g.wave_k = kw;
+            g.wave_m = cx.block / 64 / kw;
+            g.tb_m = 16 * g.wave_m;
+            g.warp_n = static_cast<int>(c.sample->gemm.N / kw);
+          }
+          add("key_waves" + std::to_string(kw), s);
+        }
       } else if (c.kind == "cluster_reduce") {
         for (int tier : {1, 2})
           for (int ilp : {1, 2, 4, 8}) {
@@ -377,7 +391,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       if (best_class < 0) continue;
       const GraphSpecification& w = trials[best_i].spec;
       for (auto& n : c.nodes) {
-        if (c.kind == "gemm") stitched.gemm_spec_list[n] = w.gemm_spec_list.at(n);
+        if (c.kind == "gemm" || c.kind == "attention") stitched.gemm_spec_list[n] = w.gemm_spec_list.at(n);
         else if (c.kind == "cluster_reduce") stitched.cluster_reduce_spec[n] = w.cluster_reduce_spec.at(n);
         else if (c.kind == "cluster_elewise") stitched.cluster_elewise_spec[n] = w.cluster_elewise_spec.at(n);
         report << ctx_str << "," << n << "," << best_class << "\n";

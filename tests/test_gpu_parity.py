@@ -172,3 +172,22 @@ def test_repeated_launches_are_bit_identical(gpu_device):
     changed = m.run(other, fx.outputs)[0]
     want = hlo_interp.evaluate(fx.hlo_text, other, consts, "fp32")[0]
     check_close(changed, want)
+
+
+@pytest.mark.parametrize("key_waves", [1, 2, 4])
+def test_attention_key_wave_arrangements(gpu_device, key_waves):
+    """The fused attention node with 1, 2 or 4 waves sharing a block of 16 query rows (the others take further
+    row blocks): same result up to the order in which the key slices are added."""
+    import json
+    fx = models.bert_encoder(L=1, B=2, S=128, H=256, NH=4, F=512, vocab=300, max_pos=128, mask_kind="length_mask")
+    consts = fx.make_constants(24, "random")
+    inputs = fx.make_inputs(24)
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    names = [n for n in spec["gemm_spec_list"] if n.startswith("cublas_batch_gemm_")]
+    assert names, "the attention block did not fuse"
+    for n in names:
+        spec["gemm_spec_list"][n]["cutlass_config"]["wave_arrangement"].update(k=key_waves, m=4 // key_waves)
+    (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, json.dumps(spec))
+    assert f"kw = mononn_dev::wave_id() % {key_waves}" in m.get_source("main.hip")
+    check_close(got, want)

@@ -100,7 +100,7 @@ def test_spec_round_trip_and_reload(layer, tmp_path):
     for key in ("cluster_elewise_spec", "cluster_reduce_spec", "gemm_spec_list", "conv_spec_list", "codegen_allow_list",
                 "codegen_reject_list", "feeds", "fetches", "input_data_files", "hlo_module_proto_file"):
         assert key in spec
-    g = next(iter(spec["gemm_spec_list"].values()))
+    g = next(v for k, v in spec["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))
     assert set(g["cutlass_config"]) >= {"threadblockshape", "warpshape", "instructionshape", "operatorclass", "archtag", "stages"}
     assert "alpha_real" in g["gemm_backend_config"]
     m2 = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
@@ -126,7 +126,7 @@ def test_spec_round_trip_and_reload(layer, tmp_path):
 def test_spec_changes_generated_code(layer):
     m = MonoNNModule.compile(layer.hlo_text, build=False)
     spec = json.loads(m.get_tuning_spec())
-    name = next(n for n in spec["gemm_spec_list"] if "fusion" in n)
+    name = next(n for n in spec["gemm_spec_list"] if n.startswith("cublas_gemm_") and "fusion" in n)
     cc = spec["gemm_spec_list"][name]["cutlass_config"]
     cc["threadblockshape"].update(m=16, n=64)
     cc["wave_arrangement"].update(m=1, n=2, k=2)
@@ -141,7 +141,8 @@ def test_spec_changes_generated_code(layer):
     (lambda s: s["cuda_context"]["cuda_runtime_context"]["grid_dim"].update(x=5000), "SPEC_ERROR"),
     (lambda s: s["codegen_allow_list"].append("ghost"), "SPEC_ERROR"),
     (lambda s: s["mononn_hip"].update(barrier="semaphore"), "SPEC_ERROR"),
-    (lambda s: next(iter(s["gemm_spec_list"].values()))["cutlass_config"]["wave_arrangement"].update(m=3), "SPEC_ERROR"),
+    (lambda s: next(v for k, v in s["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))["cutlass_config"]["wave_arrangement"].update(m=3), "SPEC_ERROR"),
+    (lambda s: next(v for k, v in s["gemm_spec_list"].items() if k.startswith("cublas_batch_gemm_"))["cutlass_config"]["wave_arrangement"].update(k=3), "SPEC_ERROR"),
 ])
 def test_bad_specs_are_rejected(layer, mutate, status):
     spec = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
