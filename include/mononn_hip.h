@@ -95,8 +95,12 @@ int mononn_module_set_constant(mononn_module* m, const char* name, const void* h
  * (mononn_engine/module/mononn_module_tuner.cc:99-131). */
 int mononn_module_load(mononn_module* m, int device);
 
-/* One forward pass = one cooperative launch.  device_ptrs: entry parameters in parameter order, then
+/* One forward pass = one launch of the persistent kernel.  device_ptrs: entry parameters in parameter order, then
  * live-out buffers, then the temp buffer (argument order of mononn_engine/module/mononn_module.cc:91-143).
+ * The launch is an ordinary one, as in the reference; the grid was checked against the co-resident capacity at
+ * load time.  Launches of such kernels must not overlap on one device (two partly resident grids would wait for
+ * each other at their first grid barrier): use one stream, or build with "mononn_hip": {"cooperative_launch": true}
+ * in the specification, which lets the runtime keep them apart.
  * Replaces: Launch(...) of profile_kernel (mononn_module_tuner.cc:135-139); the call is asynchronous
  *           on `stream` (a hipStream_t, NULL = default stream). */
 int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);

@@ -1,5 +1,5 @@
 // MonoNNModule: one HLO module + one tuning specification -> HIP source -> gfx950 code object,
-// and, once loaded on a GPU, a single cooperative launch per forward pass.
+// and, once loaded on a GPU, a single kernel launch per forward pass.
 //
 // Mirrors mononn_engine/module/mononn_module.h:31-87 (generate_code, build_assembly, get_ptx /
 // get_cubin / get_tuning_spec / get_cuda_program).  Differences forced by the platform: the HLO
