@@ -2,6 +2,9 @@
 
 #include <sys/stat.h>
 
+#include <unistd.h>
+
+#include <atomic>
 #include <cstring>
 #include <fstream>
 #include <sstream>
@@ -82,9 +85,27 @@ void MonoNNModule::generate_code() {
 
 void MonoNNModule::build_assembly() {
   MONONN_CHECK(program_ != nullptr, kInvalidArgument) << "build_assembly called before generate_code";
-  auto res = runtime::compile_hip(hip_.files, "main.hip", spec_.device.cuda_arch);
-  code_object_ = std::move(res.code_object);
-  compile_log_ = res.log;
+  try {
+    auto res = runtime::compile_hip(hip_.files, "main.hip", spec_.device.cuda_arch);
+    code_object_ = std::move(res.code_object);
+    compile_log_ = res.log;
+  } catch (const Error& e) {
+    // Keep what failed for inspection, as the reference's tuner does before it aborts
+    // (mononn_module_tuner.cc:261-285: sources and graph_spec.json under /tmp/mononn_codegen/<uuid>); here the
+    // caller gets the error code and the directory instead of an abort.
+    static std::atomic<unsigned> serial{0};
+    std::string dir = "/tmp/mononn_codegen/" + std::to_string(static_cast<long long>(getpid())) + "_" + std::to_string(serial.fetch_add(1));
+    std::string where;
+    try {
+      make_dirs(dir);
+      for (auto& kv : hip_.files) write_file(dir + "/" + kv.first, kv.second);
+      write_file(dir + "/graph_spec.json", tuning_spec_json());
+      where = " [sources and graph_spec.json kept in " + dir + "]";
+    } catch (const Error&) {
+      // the dump is a convenience; the compile error is what the caller needs to see
+    }
+    throw Error(e.code(), std::string(e.what()) + where);
+  }
 }
 
 std::string MonoNNModule::summary() const {

@@ -213,6 +213,10 @@ def test_compile_error_is_reported_not_fatal(layer):
     with pytest.raises(MonoNNError) as e:
         MonoNNModule.compile(layer.hlo_text, None, "not an identifier", build=True)
     assert e.value.status == "COMPILE_ERROR" and "error" in str(e.value)
+    # what failed is kept for inspection (mononn_module_tuner.cc:261-285 dumps to /tmp/mononn_codegen/<uuid>)
+    kept = re.search(r"kept in (/tmp/mononn_codegen/\S+)\]", str(e.value)).group(1)
+    assert sorted(os.listdir(kept)) == ["graph_spec.json", "headers.h", "host_main.cpp", "main.hip"]
+    assert "not an identifier" in open(os.path.join(kept, "main.hip")).read()
 
 
 def test_cli_compiles_and_dumps(layer, tmp_path):
