@@ -283,6 +283,13 @@ struct Builder {
       if (r.members.empty() || r.kind != NodeKind::kCluster) continue;
       auto outs = codegen::external_outputs(p, r.members);
       if (outs.size() != 1) continue;
+      // a row program that adds up the partial sums of a split-K GEMM stays a stage of its own
+      bool reads_split = false;
+      for (auto* in : external_inputs(r.members)) {
+        auto sk = opt.gemm_split_k.find(in->name);
+        reads_split = reads_split || (sk != opt.gemm_split_k.end() && sk->second > 1);
+      }
+      if (reads_split) continue;
       const Instr* h = outs[0];
       auto succ = successors();
       std::vector<int> takers;

@@ -329,3 +329,21 @@ def test_dump_contains_a_standalone_driver_and_the_constants(layer, tmp_path):
     for c in m.constants():
         path = os.path.join(cluster, "constants", "buffer_for_" + c["name"].lstrip("%").replace(".", "_").replace("-", "_") + ".bin")
         assert os.path.getsize(path) >= c["bytes"]
+
+
+def test_prologue_fusion_leaves_split_k_consumers_alone(layer):
+    # a LayerNorm that adds up split-K partial sums must stay a stage of its own even when LayerNorm-in-GEMM is on
+    spec = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
+    template = next(v for k, v in spec["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))
+    gemms = [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", layer.hlo_text)]
+    ffn2 = gemms[-1]
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}, {}
+    entry = json.loads(json.dumps(template))
+    entry["cutlass_config"]["split_k"] = 2
+    spec["gemm_spec_list"][ffn2] = entry
+    spec["mononn_hip"]["gemm_prologue_fusion"] = True
+    m = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
+    text = m.summary()
+    assert "+row-prologue" in text                      # the first LayerNorm went into FFN1
+    assert re.search(rf"gemm\s+{ffn2}\s", text)          # FFN2 is split: bare node, no fused epilogue
+    assert re.search(r"rowred\s+\S+\s+members=4", text)  # its consumer: bias + residual + LayerNorm over the partial sums
