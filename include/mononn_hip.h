@@ -77,9 +77,9 @@ int mononn_module_buffer_info(const mononn_module* m, int* n_params, const int64
                               int* n_liveouts, const int64_t** liveout_bytes, int64_t* temp_bytes);
 /* grid / block / dynamic LDS of the launch (best_tuning_spec.json keys grid_dim, block_dim, smem_size;
  * README.md:199-200) and the number of grid-wide barriers in the kernel. */
-/* 1 when the kernel hands data between stages through a module-owned coherent (uncached) temp arena:
- * the caller then passes NULL in the temp slot of mononn_launch.  0: the caller brings the temp buffer
- * (the reference's contract), at the price of cache maintenance in every grid barrier. */
+/* Whether the module brings its own temp arena (the caller would then pass NULL in the temp slot of
+ * mononn_launch).  Always 0 today: the caller brings the temp buffer, as in the reference's contract
+ * (temp_buffer argument, mononn_engine/module/mononn_module.cc:91-143). */
 int mononn_module_owns_temp(const mononn_module* m);
 int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int* smem, int* barriers);
 

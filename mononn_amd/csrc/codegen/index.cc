@@ -236,8 +236,6 @@ std::vector<LinExpr> delinearize(const LinExpr& lin, const std::vector<int64_t>&
 
   // general fallback: run-time division of the materialised linear index
   std::string e = lin.str(vars);
-  int64_t total = 1;
-  for (auto d : dims) total *= d;
   for (int i = 0; i < r; ++i) {
     if (dims[i] == 1) {
       out[i] = LinExpr::constant(0);

@@ -642,7 +642,7 @@ struct Builder {
 std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, const BuildOptions& opt) {
   auto prog = std::make_unique<Program>();
   prog->module = std::move(module);
-  Builder b{*prog, opt};
+  Builder b{*prog, opt, {}, {}};
   b.make_nodes();
   // epilogues first: a bias + residual fusion behind a GEMM belongs to that GEMM, not to the LayerNorm
   // row program that follows it

@@ -405,7 +405,9 @@ void decode_conv_config(Instr* ins) {
   if (bc != ins->attrs.end()) {
     Json j = Json::parse(bc->second);
     if (j.contains("conv_result_scale")) c.result_scale = j.at("conv_result_scale").as_double();
-    if (j.contains("side_input_scale")) MONONN_CHECK(j.at("side_input_scale").as_double() == 0, kUnsupported) << ins->hlo_name << ": side input is not supported";
+    if (j.contains("side_input_scale")) {
+      MONONN_CHECK(j.at("side_input_scale").as_double() == 0, kUnsupported) << ins->hlo_name << ": side input is not supported";
+    }
     if (j.contains("activation_mode")) {
       const Json& a = j.at("activation_mode");
       const std::string mode = a.is_string() ? a.as_string() : std::to_string(a.as_int());

@@ -58,9 +58,7 @@ MonoNNModule::MonoNNModule(const std::string& hlo_text, const std::string& spec_
   }
 }
 
-MonoNNModule::~MonoNNModule() {
-  if (own_temp_) runtime::coherent_release(dev_.device(), own_temp_);
-}
+MonoNNModule::~MonoNNModule() = default;
 
 void MonoNNModule::generate_code() {
   auto mod = hlo::parse_module(hlo_text_);
@@ -240,11 +238,6 @@ void MonoNNModule::load(int device) {
   size_t flag_bytes = 0;
   void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
   dev_.zero(flags, flag_bytes);
-  if (own_temp_) {
-    runtime::coherent_release(device, own_temp_);
-    own_temp_ = nullptr;
-  }
-  if (owns_temp()) own_temp_ = runtime::coherent_alloc(device, static_cast<size_t>(std::max<int64_t>(hip_.temp_bytes, 256)));
   uploaded_.clear();
   for (auto& ci : hip_.constants) {
     if (!ci.literal.empty()) {

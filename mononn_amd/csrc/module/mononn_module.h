@@ -83,7 +83,6 @@ class MonoNNModule {
   std::string compile_log_;
   runtime::DeviceModule dev_;
   int grid_ = 0;
-  void* own_temp_ = nullptr;     // coherent arena used when the kernel's barrier does no cache maintenance
   std::map<std::string, std::vector<char>> host_constants_;   // canonical name -> payload as given
   std::map<std::string, bool> uploaded_;
 };

@@ -45,42 +45,6 @@ DeviceProperties query_device(int device) {
   return d;
 }
 
-namespace {
-struct Arena {
-  int device;
-  void* ptr;
-  size_t bytes;
-  bool in_use;
-};
-std::mutex g_arena_mu;
-std::vector<Arena> g_arenas;
-}  // namespace
-
-void* coherent_alloc(int device, size_t bytes) {
-  std::lock_guard<std::mutex> lock(g_arena_mu);
-  bytes = std::max<size_t>((bytes + 4095) / 4096 * 4096, 4096);
-  Arena* best = nullptr;
-  for (auto& a : g_arenas)
-    if (a.device == device && !a.in_use && a.bytes >= bytes && (!best || a.bytes < best->bytes)) best = &a;
-  if (best) {
-    best->in_use = true;
-    return best->ptr;
-  }
-  HIP_OK(hipSetDevice(device));
-  void* p = nullptr;
-  HIP_OK(hipExtMallocWithFlags(&p, bytes, hipDeviceMallocUncached));
-  HIP_OK(hipMemset(p, 0, bytes));
-  HIP_OK(hipDeviceSynchronize());
-  g_arenas.push_back({device, p, bytes, true});
-  return p;
-}
-
-void coherent_release(int device, void* ptr) {
-  std::lock_guard<std::mutex> lock(g_arena_mu);
-  for (auto& a : g_arenas)
-    if (a.device == device && a.ptr == ptr) a.in_use = false;
-}
-
 DeviceModule::~DeviceModule() {
   if (module_) (void)hipModuleUnload(module_);
 }

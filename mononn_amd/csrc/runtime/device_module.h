@@ -26,12 +26,6 @@ struct DeviceProperties {
   std::string name;
 };
 
-// Device memory that no cache level keeps (every access goes to the memory side, so it is coherent
-// across the XCDs of one GPU without cache maintenance).  Arenas are pooled per device and handed
-// back with coherent_release; they are never returned to the driver before the process ends.
-void* coherent_alloc(int device, size_t bytes);
-void coherent_release(int device, void* ptr);
-
 int device_count();                           // 0 when no GPU is visible (never throws)
 DeviceProperties query_device(int device);    // throws Error(kRuntimeError) without a GPU
 

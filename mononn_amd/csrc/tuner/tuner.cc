@@ -73,10 +73,6 @@ void DeviceBuffers::ensure_temp(size_t bytes) {
   temp_capacity = std::max<size_t>(bytes, 256);
 }
 
-struct GemmCandidate {
-  codegen::GemmTuning t;
-};
-
 // Every wave arrangement x per-wave fragment tile that the code generator accepts for this problem
 // (reference: all CUTLASS tiles that fit, tuning_space_generator.cc:139-307).
 std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int waves, int budget) {
