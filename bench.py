@@ -138,16 +138,17 @@ def stage_profile(module, fx, consts, inputs, args):
             acc = p
         else:
             for a, b in zip(acc, p):
-                for k in ("busy_us", "barrier_us", "mean_wg_us"):
+                for k in ("busy_us", "barrier_us", "mean_wg_us", "step_us"):
                     a[k] += b[k]
     for a in acc:
-        for k in ("busy_us", "barrier_us", "mean_wg_us"):
+        for k in ("busy_us", "barrier_us", "mean_wg_us", "step_us"):
             a[k] /= n
     print(f"stage clocks, mean of {n} launches; busy = first workgroup in -> last workgroup done, "
-          f"barrier = last workgroup done -> first workgroup in the next stage")
-    print(f"{'stage':>5} {'busy_us':>8} {'mean_wg_us':>10} {'barrier_us':>10}  nodes")
+          f"barrier = last workgroup done -> first workgroup in the next stage, "
+          f"step = last workgroup done in the previous stage -> last workgroup done in this one")
+    print(f"{'stage':>5} {'busy_us':>8} {'mean_wg_us':>10} {'barrier_us':>10} {'step_us':>8}  nodes")
     for a in acc:
-        print(f"{a['stage']:5d} {a['busy_us']:8.2f} {a['mean_wg_us']:10.2f} {a['barrier_us']:10.2f}  {a['nodes'][:90]}")
+        print(f"{a['stage']:5d} {a['busy_us']:8.2f} {a['mean_wg_us']:10.2f} {a['barrier_us']:10.2f} {a['step_us']:8.2f}  {a['nodes'][:90]}")
     busy, bar = sum(a["busy_us"] for a in acc), sum(a["barrier_us"] for a in acc)
     print(f"total: busy {busy:.1f} us in {len(acc)} stages, barriers {bar:.1f} us ({len(acc) - 1} barriers)")
     prof_mod.close()

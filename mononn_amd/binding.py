@@ -228,20 +228,26 @@ class MonoNNModule:
     def stage_profile(self) -> List[dict]:
         """Per-stage timing of the last launch (kernel compiled with mononn_hip.profile_stages):
         `busy_us` = first workgroup in to last workgroup done, `barrier_us` = last workgroup done to the
-        first workgroup entering the next stage, `mean_wg_us` = average per-workgroup work time."""
+        first workgroup entering the next stage, `mean_wg_us` = average per-workgroup work time, `step_us` =
+        last workgroup done in the previous stage to last workgroup done in this one (what the stage adds to
+        the kernel's duration, whatever of its operand traffic overlaps the barrier).  Workgroups that had no
+        unit in a stage leave zero stamps and are left out."""
         ns, grid, tpu = ctypes.c_int(), ctypes.c_int(), ctypes.c_double()
         _check(_lib.mononn_module_stage_clock(self._h, None, 0, ctypes.byref(ns), ctypes.byref(grid), ctypes.byref(tpu)))
         n = ns.value * grid.value * 2
         buf = (ctypes.c_uint64 * n)()
         _check(_lib.mononn_module_stage_clock(self._h, buf, n, ctypes.byref(ns), ctypes.byref(grid), ctypes.byref(tpu)))
         t = np.frombuffer(buf, dtype=np.uint64).astype(np.float64).reshape(ns.value, grid.value, 2) / tpu.value
+        live = [(t[s, :, 0] > 0) & (t[s, :, 1] > 0) for s in range(ns.value)]
+        begin = [t[s, live[s], 0].min() if live[s].any() else np.nan for s in range(ns.value)]
+        done = [t[s, live[s], 1].max() if live[s].any() else np.nan for s in range(ns.value)]
         out = []
         for s in range(ns.value):
-            begin, done = t[s, :, 0].min(), t[s, :, 1].max()
-            nxt = t[s + 1, :, 0].min() if s + 1 < ns.value else done
+            nxt = begin[s + 1] if s + 1 < ns.value else done[s]
+            prev = done[s - 1] if s > 0 else begin[s]
             out.append({"stage": s, "nodes": _lib.mononn_module_stage_name(self._h, s).decode(),
-                        "busy_us": done - begin, "barrier_us": nxt - done,
-                        "mean_wg_us": float((t[s, :, 1] - t[s, :, 0]).mean())})
+                        "busy_us": done[s] - begin[s], "barrier_us": nxt - done[s], "step_us": done[s] - prev,
+                        "mean_wg_us": float((t[s, live[s], 1] - t[s, live[s], 0]).mean()) if live[s].any() else 0.0})
         return out
 
     # torch is used for device memory and streams only

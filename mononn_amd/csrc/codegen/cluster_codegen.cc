@@ -906,7 +906,9 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
   Epilogue epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, ptrs, first_epi);
   CodeBuffer fb;
-  std::string conv_struct;
+  std::string conv_struct, preload_body;
+  bool preload = false;
+  int preload_regs = 0;
   if (g.split_k <= 1) fb.line(epi.init_line);
   if (has_pro) fb.line(pro.init_line);
   int64_t units = 0;
@@ -948,10 +950,36 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
            << ", @NAME@_epi, mononn_dev::NoPrologue, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
            << ", bidx, tile_m, tile_n, epi, smem, mononn_dev::NoPrologue(), @NAME@_amap());";
     } else {
+      std::ostringstream b_expr;
+      b_expr << pb << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS);
+      preload = t.preload_b && g.b_packed && !has_pro;   // a row-program prologue fixes the chunking of the left operand
       call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
-           << (g.b_packed ? "true" : "false") << ", " << g.K << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << KS << ", " << pb
-           << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS) << ", " << g.M << ", " << g.N << ", " << g.K << ", "
-           << g.K << ", bidx, tile_m, tile_n, epi, smem" << (has_pro ? ", pro" : "") << ");";
+           << (g.b_packed ? "true" : "false") << ", " << g.K;
+      if (preload) call << ", @NAME@_epi, mononn_dev::NoPrologue, mononn_dev::RowMajorA, true, @NAME@_preb";
+      call << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << KS << ", " << b_expr.str() << ", " << g.M << ", " << g.N << ", "
+           << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
+      if (preload) call << ", mononn_dev::NoPrologue(), mononn_dev::RowMajorA(), &pre_b";
+      else if (has_pro) call << ", pro";
+      call << ");";
+      if (preload) {
+        // the companion repeats the unit decoding as far as the right operand needs it
+        const int TM = t.bm / t.wm / 16, TN = t.bn / t.wn / 16;
+        const int my_steps = static_cast<int>((KS / 32 + t.wk - 1) / t.wk);
+        const int ch_max = 32 / (TM + TN) > 0 ? 32 / (TM + TN) : 1;   // mirrors mononn_dev::gemm_chunk_steps
+        preload_regs = (my_steps * (TM + TN) <= 56 ? my_steps : std::min(my_steps, ch_max)) * TN;
+        CodeBuffer pf;
+        pf.line("const int bidx = unit / " + S(per_batch) + ";");
+        pf.line("const int rem0 = unit % " + S(per_batch) + ";");
+        pf.line("const int ksplit = rem0 % " + S(S_) + ";");
+        pf.line("const int rem = rem0 / " + S(S_) + ";");
+        if (tiles_n % 8 == 0 && S_ == 1) pf.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
+        else pf.line("const int tile_n = rem / " + S(tiles_m) + ";");
+        std::ostringstream pc;
+        pc << "mononn_dev::gemm_b_preload<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", " << g.K << ">("
+           << b_expr.str() << ", " << g.N << ", tile_n, pre_b);";
+        pf.line(pc.str());
+        preload_body = pf.text();
+      }
     }
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
@@ -979,7 +1007,18 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   }
   std::vector<std::string> globals = epi.globals;
   for (auto& gl : pro.globals) globals.push_back(gl);
-  return finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text + conv_struct);
+  NodeFunction f = finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text + conv_struct);
+  if (preload) {
+    const std::string tail = ", char* smem) {";
+    size_t at = f.text.find(tail);
+    MONONN_CHECK(at != std::string::npos, kInternal) << "node function signature not found";
+    f.text.replace(at, tail.size(), ", char* smem, const @NAME@_preb& pre_b) {");
+    f.text = "typedef mononn_dev::PreB<" + S(preload_regs) + "> @NAME@_preb;\n" + f.text;
+    std::string sig = signature(ptrs.entries);
+    sig = sig.substr(0, sig.rfind(", char* smem"));
+    f.preload_text = "__device__ __forceinline__ void @NAME@_pre(" + sig + ", @NAME@_preb& pre_b) {\n" + preload_body + "}\n";
+  }
+  return f;
 }
 
 // GEMM -> row program -> GEMM with everything between the two contractions on chip.

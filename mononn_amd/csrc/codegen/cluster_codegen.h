@@ -31,6 +31,9 @@ struct GemmTuning {
   int bm = 32, bn = 32;      // workgroup tile
   int wm = 1, wn = 1, wk = 4;   // wave arrangement; wm*wn*wk == waves per workgroup
   int split_k = 1;              // k range also split over workgroups (fp32 partial sums to memory)
+  // the function takes the first chunk of packed weights from registers filled by a companion function
+  // (NodeFunction::preload_text) that the kernel calls before it waits at the grid barrier
+  bool preload_b = false;
 };
 
 struct NodeFunction {
@@ -39,6 +42,10 @@ struct NodeFunction {
   int64_t num_units = 0;                       // independent work units (one workgroup each)
   int smem_bytes = 0;
   std::vector<std::string> globals;            // device-global definitions the function needs
+  // Optional companion `@NAME@_pre(unit, <pointers>, @NAME@_preb&)`: requests operands that do not depend on
+  // the previous stage.  When present, `text` defines the register block type `@NAME@_preb` and takes a trailing
+  // `const @NAME@_preb&` after `smem`.
+  std::string preload_text;
 };
 
 // fills has_reduce / row_program / rows / row_len

@@ -127,6 +127,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     int64_t units;
   };
   std::map<std::string, int> fn_ids;
+  std::set<int> preload_fns;   // functions with a companion that requests constant operands ahead of the barrier wait
   std::map<int, std::vector<std::string>> fn_arg_types;   // fn id -> pointer types of its arguments
   std::map<int, std::vector<Call>> by_stage;
   int smem = 0;
@@ -176,6 +177,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         t.wk = it->second.wave_k;
       }
       t.split_k = n.gemm.split_k;
+      t.preload_b = spec.hip.operand_preload;
       f = generate_gemm(prog, n, ls, t);
     } else {
       ClusterTuning t;
@@ -216,6 +218,12 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       size_t pos;
       while ((pos = def.find("@NAME@")) != std::string::npos) def.replace(pos, 6, fn);
       fn_defs.push_back(def);
+      if (!f.preload_text.empty()) {
+        std::string pdef = f.preload_text;
+        while ((pos = pdef.find("@NAME@")) != std::string::npos) pdef.replace(pos, 6, fn);
+        fn_defs.push_back(pdef);
+        preload_fns.insert(fn_ids[fn]);
+      }
       for (auto& g : f.globals) globals.insert(g);
     }
     NodeReport rep;
@@ -323,6 +331,12 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
   src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags);\n";
   src << "  int stage = -1;\n";
+  const bool lazy = !preload_fns.empty();
+  if (lazy) {
+    // The wait half of a barrier is put off until the workgroup's first unit of the new stage, behind the
+    // requests for that unit's constant operands; a workgroup without a unit in a stage does not wait for it.
+    src << "  bool pending = false;   // announced the end of the previous stage, not yet waited for the others\n";
+  }
   src << "  for (int c = 0; c < " << flat.size() << "; ++c) {\n";
   src << "    int fn = 0, units = 0, first = 0, total = 0;\n    bool new_stage = false;\n";
   src << "    char*";
@@ -337,27 +351,59 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     src << " break;   // " << f.call->node->name.substr(0, 50) << "\n";
   }
   src << "      default: break;\n    }\n";
+  // stage clocks: [stage][workgroup][0] = first unit of the stage may start, [1] = the workgroup's part is done;
+  // a workgroup that has no unit in a stage leaves both at zero
+  const std::string clk = "mononn_stage_clock[(stage * " + std::to_string(hp.grid) + " + blockIdx.x) * 2";
   src << "    if (new_stage) {\n";
-  if (hp.profiled) {
-    src << "      if (stage >= 0) {\n        __syncthreads();\n";
-    src << "        if (threadIdx.x == 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n      }\n";
+  if (!lazy) {
+    if (hp.profiled) {
+      src << "      if (stage >= 0) {\n        __syncthreads();\n";
+      src << "        if (threadIdx.x == 0) " << clk << " + 1] = wall_clock64();\n      }\n";
+    }
+    src << "      if (stage >= 0) barrier.sync();\n      ++stage;\n";
+    if (hp.profiled) src << "      if (threadIdx.x == 0) " << clk << "] = wall_clock64();\n";
+  } else {
+    src << "      if (stage >= 0) {\n";
+    if (hp.profiled) {
+      src << "        __syncthreads();\n";
+      src << "        if (threadIdx.x == 0) {\n";
+      src << "          if (pending) " << clk << "] = 0;\n";
+      src << "          " << clk << " + 1] = pending ? 0 : wall_clock64();\n        }\n";
+    }
+    src << "        barrier.arrive();\n        pending = true;\n      }\n      ++stage;\n";
+    if (hp.profiled) src << "      if (stage == 0 && threadIdx.x == 0) " << clk << "] = wall_clock64();\n";
   }
-  src << "      if (stage >= 0) barrier.sync();\n      ++stage;\n";
-  if (hp.profiled) src << "      if (threadIdx.x == 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2] = wall_clock64();\n";
   src << "    }\n";
   src << "    for (int u = blockIdx.x; u < total; u += gridDim.x) {\n";
   src << "      const int unit = u - first;\n";
   src << "      if (unit < 0 || unit >= units) continue;\n";
+  // One dispatch switch; in the lazy form every case first requests what it can, then waits if a barrier is pending
+  // (the wait is spelled out per case so that the requested registers flow straight into the function that uses
+  // them instead of meeting at a join of all cases).
+  std::string wait_text;
+  if (lazy) {
+    wait_text = "if (pending) { barrier.wait(); pending = false;";
+    if (hp.profiled) wait_text += " if (threadIdx.x == 0) " + clk + "] = wall_clock64();";
+    wait_text += " } ";
+  }
   src << "      switch (fn) {\n";
   for (auto& kv : fn_arg_types) {
-    src << "        case " << kv.first << ": node_fn_" << kv.first << "(unit";
-    for (size_t i = 0; i < kv.second.size(); ++i) src << ", (" << kv.second[i] << ")p" << i;
-    src << ", smem); break;\n";
+    std::ostringstream args;
+    for (size_t i = 0; i < kv.second.size(); ++i) args << ", (" << kv.second[i] << ")p" << i;
+    src << "        case " << kv.first << ": { ";
+    const bool pre = preload_fns.count(kv.first) > 0;
+    if (pre) src << "node_fn_" << kv.first << "_preb pre_b; node_fn_" << kv.first << "_pre(unit" << args.str() << ", pre_b); ";
+    src << wait_text << "node_fn_" << kv.first << "(unit" << args.str() << ", smem" << (pre ? ", pre_b" : "") << "); } break;\n";
   }
   src << "        default: break;\n      }\n    }\n  }\n";
   if (hp.profiled) {
     src << "  __syncthreads();\n";
-    src << "  if (threadIdx.x == 0 && stage >= 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
+    if (lazy) {
+      src << "  if (threadIdx.x == 0 && stage >= 0) {\n    if (pending) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2] = 0;\n";
+      src << "    mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2 + 1] = pending ? 0 : wall_clock64();\n  }\n";
+    } else {
+      src << "  if (threadIdx.x == 0 && stage >= 0) mononn_stage_clock[(stage * " << hp.grid << " + blockIdx.x) * 2 + 1] = wall_clock64();\n";
+    }
   }
   src << "}\n";
   hp.preamble = pre.str();

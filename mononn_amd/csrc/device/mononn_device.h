@@ -63,11 +63,12 @@ struct GridBarrier {
     epoch = __hip_atomic_load(&flags[blockIdx.x * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  // MONONN_BARRIER_FENCE: 0 = one thread per workgroup performs the release / acquire cache
-  // maintenance (an agent-scope acquire invalidates the XCD's whole L2, so issuing it from every
-  // wave multiplies that cost by the number of resident waves); 1 = every thread fences;
-  // 2 = no cache maintenance at all (valid with MONONN_COHERENT_STORES and a write-once temp arena).
-  __device__ __forceinline__ void sync() {
+  // A workgroup announces that its part of the stage is written (arrive) and, before it reads anything another
+  // workgroup wrote in that stage, makes sure that every workgroup has announced (wait).  Between the two it may
+  // do whatever does not depend on the stage: requesting constant operands of its next unit, for instance.  A
+  // workgroup without work in a stage need not wait for it at all: flags only grow, so it may announce the next
+  // stage right away and wait, when it has work again, for the latest one.
+  __device__ __forceinline__ void arrive() {
     __syncthreads();
     epoch += 1;
     if (threadIdx.x == 0) {
@@ -77,6 +78,9 @@ struct GridBarrier {
       __hip_atomic_store(&flags[blockIdx.x * kFlagStride], epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 #endif
     }
+  }
+
+  __device__ __forceinline__ void wait() {
 #if MONONN_BARRIER_FENCE == 0
     if (threadIdx.x < kWaveSize) {
       for (int b = threadIdx.x; b < (int)gridDim.x; b += kWaveSize) {
@@ -97,6 +101,15 @@ struct GridBarrier {
 #endif
 #endif
     __syncthreads();
+  }
+
+  // MONONN_BARRIER_FENCE: 0 = one thread per workgroup performs the release / acquire cache
+  // maintenance (an agent-scope acquire invalidates the XCD's whole L2, so issuing it from every
+  // wave multiplies that cost by the number of resident waves); 1 = every thread fences;
+  // 2 = no cache maintenance at all (valid with MONONN_COHERENT_STORES and a write-once temp arena).
+  __device__ __forceinline__ void sync() {
+    arrive();
+    wait();
   }
 };
 
@@ -272,20 +285,68 @@ struct RowMajorA {
   __device__ __forceinline__ const half_t* operator()(const half_t* A, int m, int k, int lda) const { return A + (long)m * lda + k; }
 };
 
-// K is the k extent this call contracts over; KTOTAL the k extent of the operands in memory (they differ
-// when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
-template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA>
-__device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
-                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
-                                          const AMap& amap = AMap()) {
+// k steps of one wave that are loaded together: (TM + TN) * 4 * CH * 2 (double buffer) stays within ~256 VGPRs.
+// With the right operand requested ahead of the tile (pre_b) a wave whose whole k range fits into 224 VGPRs takes
+// it as one chunk: there is nothing left to double-buffer.
+__device__ constexpr int gemm_chunk_steps(int TM, int TN, int my_steps, bool pre_b = false) {
+  if (pre_b && my_steps * (TM + TN) <= 56) return my_steps;
+  const int ch_max = 32 / (TM + TN) > 0 ? 32 / (TM + TN) : 1;
+  return my_steps < ch_max ? my_steps : ch_max;
+}
+
+// Right-operand fragments of a wave's first chunk, requested before the tile's left operand exists.  Packed weights
+// are constants of the module: a workgroup asks for them between announcing the end of its previous stage and
+// waiting for the other workgroups, so their way from memory overlaps the barrier instead of following it.
+template <int REGS>
+struct PreB {
+  half8_t v[REGS];
+};
+struct NoPreB {
+  half8_t v[1];
+};
+
+template <int BM, int BN, int WM, int WN, int WK, int K, int KTOTAL, class Pre>
+__device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_n, Pre& pb) {
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int KSTEPS = K / 32;
   constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
-  // chunk size: keep (TM + TN) * 4 * CH * 2 (double buffer) within ~256 VGPRs
-  constexpr int CH_MAX = 32 / (TM + TN) > 0 ? 32 / (TM + TN) : 1;
-  constexpr int CH = MY_STEPS < CH_MAX ? MY_STEPS : CH_MAX;
+  constexpr int CH = gemm_chunk_steps(TM, TN, MY_STEPS, true);
+  static_assert(CH * TN * sizeof(half8_t) <= sizeof(pb.v), "preload buffer too small for this tile");
+  const int lane = lane_id();
+  const int wave = wave_id();
+  const int wk = wave % WK;
+  const int wn = (wave / WK) % WN;
+  const int n_base = tile_n * BN + wn * (TN * 16);
+  const int nt_max = (N + 15) / 16 - 1;
+#pragma unroll
+  for (int s = 0; s < CH; ++s) {
+    int ks = s * WK + wk;
+    ks = ks < KSTEPS ? ks : KSTEPS - 1;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int nt = (n_base >> 4) + j;
+      nt = nt < nt_max ? nt : nt_max;
+      pb.v[s * TN + j] = *reinterpret_cast<const half8_t*>(B + (((long)nt * (KTOTAL / 32) + ks) * 64 + lane) * 8);
+    }
+  }
+}
+
+// K is the k extent this call contracts over; KTOTAL the k extent of the operands in memory (they differ
+// when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
+// PRE_B: the right operand's first chunk was requested by gemm_b_preload with the same parameters and comes in `pb`.
+template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA,
+          bool PRE_B = false, class Pre = NoPreB>
+__device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
+                                          int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
+                                          const AMap& amap = AMap(), const Pre* pb = nullptr) {
+  constexpr int TM = BM / WM / 16;
+  constexpr int TN = BN / WN / 16;
+  constexpr int KSTEPS = K / 32;
+  constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
+  constexpr int CH = gemm_chunk_steps(TM, TN, MY_STEPS, PRE_B);
   constexpr int NCHUNK = (MY_STEPS + CH - 1) / CH;
+  static_assert(!PRE_B || PACKED_B, "only packed weights can be requested ahead of the tile");
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
   static_assert(K % 32 == 0, "K must be a multiple of 32");
   const int lane = lane_id();
@@ -330,7 +391,10 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       int ks = (c * CH + s) * WK + wk;
       ks = ks < KSTEPS ? ks : KSTEPS - 1;   // surplus steps re-read a valid block and are not accumulated
 #pragma unroll
-      for (int j = 0; j < TN; ++j) b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
+      for (int j = 0; j < TN; ++j) {
+        if (PRE_B && c == 0) b[buf][s][j] = pb->v[s * TN + j];
+        else b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);

@@ -304,6 +304,13 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       }
     });
     GraphSpecification stitched = filled;
+    // runners-up of every class by the isolated stage clocks, for the whole-kernel refinement below
+    struct Alternative {
+      std::string label;
+      double us;
+      GraphSpecification spec;
+    };
+    std::map<std::string, std::vector<Alternative>> runners_up;   // class function -> candidates after the best
     const bool verbose = env::is_true("TF_MONONN_ENABLE_WORKER_THRAED_LOGGING") || env::is_true("MONONN_TUNER_VERBOSE");
     // Compiles the candidates `live` as one translation unit (shared preamble, one namespace per candidate),
     // loads it once and times the profiled stages of every candidate.
@@ -346,13 +353,23 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             dm.launch(hp.grid, hp.block, hp.smem, args.data(), nullptr);
             if (it < warm) continue;
             dm.download(ticks.data(), clk, cb);
+            // A stage is charged from the moment the last workgroup finished the stage before it (the first stage:
+            // from its first workgroup's entry) to the moment its own last workgroup finishes: the barrier in front
+            // of it is included, and so is whatever of its operand traffic a candidate hides behind that barrier.
+            // Workgroups without a unit in a stage leave zero stamps.
+            unsigned long long prev_hi = 0;
             for (int st = 0; st < hp.num_stages; ++st) {
               unsigned long long lo = ~0ull, hi = 0;
               for (int w = 0; w < hp.grid; ++w) {
-                lo = std::min(lo, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2]);
-                hi = std::max(hi, ticks[(static_cast<size_t>(st) * hp.grid + w) * 2 + 1]);
+                const unsigned long long in = ticks[(static_cast<size_t>(st) * hp.grid + w) * 2], out = ticks[(static_cast<size_t>(st) * hp.grid + w) * 2 + 1];
+                if (in == 0 || out == 0) continue;
+                lo = std::min(lo, in);
+                hi = std::max(hi, out);
               }
-              total += static_cast<double>(hi - lo) / tpu;
+              if (hi == 0) continue;
+              const unsigned long long from = st == 0 || prev_hi == 0 ? lo : prev_hi;
+              total += static_cast<double>(hi - from) / tpu;
+              prev_hi = hi;
               ++count;
             }
           }
@@ -381,10 +398,19 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           }
       } catch (const Error& e) {
         log << "  [" << ctx_str << "] class of " << c.nodes[0] << " failed: " << e.what() << "\n";
+        if (verbose) std::fprintf(stderr, "[mononn tuner] %s class of %s failed: %.300s\n", ctx_str.c_str(), c.nodes[0].c_str(), e.what());
       }
       for (size_t i : trials_of_class[c.function]) trials[i].mod.reset();
       if (verbose) std::fprintf(stderr, "[mononn tuner] %s %s x%zu: %zu candidates, best %.2f us\n", ctx_str.c_str(), c.kind.c_str(), c.nodes.size(), live.size(), best_class);
       if (best_class < 0) continue;
+      if (budget <= 1 && c.nodes.size() >= 2) {
+        std::vector<size_t> order;
+        for (size_t i : live)
+          if (i != best_i && trials[i].us > 0 && trials[i].us < 1.25 * best_class) order.push_back(i);
+        std::sort(order.begin(), order.end(), [&](size_t a, size_t b) { return trials[a].us < trials[b].us; });
+        const size_t keep = budget == 0 ? 6 : 2;
+        for (size_t k = 0; k < order.size() && k < keep; ++k) runners_up[c.function].push_back({trials[order[k]].label, trials[order[k]].us, trials[order[k]].spec});
+      }
       const GraphSpecification& w = trials[best_i].spec;
       for (auto& n : c.nodes) {
         if (c.kind == "gemm" || c.kind == "attention") stitched.gemm_spec_list[n] = w.gemm_spec_list.at(n);
@@ -417,7 +443,57 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         return -1;
       }
     };
-    if (!env::is_true("MONONN_TUNER_NO_SPLIT_K")) {
+    // ---- whole-kernel refinement ------------------------------------------------------------------------
+    // A class is timed above in a kernel that holds nothing but its own stages, where every workgroup reaches
+    // the barrier at the same moment and the caches hold only that class's operands.  In the real kernel the
+    // stage follows a different one, part of its operand traffic hides behind the barrier wait, and the
+    // ranking of close candidates can change: the runners-up of every class are tried in the whole kernel and
+    // the fastest whole kernel wins.
+    // A launch context that starts out well behind the best one so far is not worth the whole-kernel builds.
+    bool promising = true;
+    if (!env::is_true("MONONN_TUNER_NO_REFINEMENT")) {
+      stitched_us = whole_kernel_us(stitched);
+      promising = best_us < 0 || (stitched_us > 0 && stitched_us < 1.08 * best_us);
+      if (!promising) log << "  [" << ctx_str << "] " << stitched_us << " us before refinement, best context so far " << best_us << " us: not refined\n";
+    }
+    if (promising && !runners_up.empty() && !env::is_true("MONONN_TUNER_NO_REFINEMENT")) {
+      for (auto& kv : classes) {
+        ClassInfo& c = kv.second;
+        auto ru = runners_up.find(c.function);
+        if (ru == runners_up.end() || stitched_us < 0) continue;
+        std::string line;
+        double best_alt_us = -1;
+        const Alternative* best_alt = nullptr;
+        for (auto& alt : ru->second) {
+          GraphSpecification s = stitched;
+          for (auto& n : c.nodes) {
+            if (c.kind == "gemm" || c.kind == "attention") s.gemm_spec_list[n] = alt.spec.gemm_spec_list.at(n);
+            else if (c.kind == "cluster_reduce") s.cluster_reduce_spec[n] = alt.spec.cluster_reduce_spec.at(n);
+            else if (c.kind == "cluster_elewise") s.cluster_elewise_spec[n] = alt.spec.cluster_elewise_spec.at(n);
+          }
+          const double us = whole_kernel_us(s);
+          char buf[160];
+          std::snprintf(buf, sizeof buf, " %s=%.2f", alt.label.c_str(), us);
+          line += buf;
+          if (us > 0 && (best_alt_us < 0 || us < best_alt_us)) {
+            best_alt_us = us;
+            best_alt = &alt;
+          }
+        }
+        log << "  [" << ctx_str << "] whole kernel with runners-up of " << c.kind << " x" << c.nodes.size() << " (" << c.nodes[0] << "): now " << stitched_us
+            << " us;" << line << "\n";
+        if (verbose) std::fprintf(stderr, "[mononn tuner] %s refinement %s (%s): now %.2f us;%s\n", ctx_str.c_str(), c.kind.c_str(), c.nodes[0].c_str(), stitched_us, line.c_str());
+        if (best_alt && best_alt_us < 0.997 * stitched_us) {
+          for (auto& n : c.nodes) {
+            if (c.kind == "gemm" || c.kind == "attention") stitched.gemm_spec_list[n] = best_alt->spec.gemm_spec_list.at(n);
+            else if (c.kind == "cluster_reduce") stitched.cluster_reduce_spec[n] = best_alt->spec.cluster_reduce_spec.at(n);
+            else if (c.kind == "cluster_elewise") stitched.cluster_elewise_spec[n] = best_alt->spec.cluster_elewise_spec.at(n);
+          }
+          stitched_us = best_alt_us;
+        }
+      }
+    }
+    if (promising && !env::is_true("MONONN_TUNER_NO_SPLIT_K")) {
       for (auto& kv : classes) {
         ClassInfo& c = kv.second;
         if (c.kind != "gemm" || !c.sample || !c.sample->prologue.empty()) continue;
@@ -583,18 +659,76 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         if (verbose)
           std::fprintf(stderr, "[mononn tuner] %s split-K x%zu (%s): %zu candidates, unsplit %.2f us, best %s %.2f us\n", ctx_str.c_str(), instrs.size(),
                        instrs[0].c_str(), live.size(), trials[first].total_us / per, trials[best_i].label.c_str(), trials[best_i].total_us / per);
-        // The stage clocks leave out barrier skew and cache effects between stages, so the winner is adopted
-        // only when the whole kernel with it is faster than the whole kernel without.
-        if (best_i != first && trials[best_i].total_us < 0.97 * trials[first].total_us) {
-          GraphSpecification adopted = trials[best_i].spec;
-          drop_unknown(adopted, trials[best_i].mod->program());
+        // The stage clocks leave out barrier skew and cache effects between stages, so the best few candidates
+        // are built into the whole kernel and one is adopted only when that kernel is faster than without.
+        // Candidates: per split factor the best one or two by the stage clocks, as long as they are not far behind
+        // the unsplit pair of stages (what a split saves is partly hidden in the clocks of the isolated stages).
+        std::vector<size_t> order;
+        {
+          std::map<std::string, std::vector<size_t>> by_factor;   // "split4" -> trials
+          for (size_t i : live)
+            if (i != first && trials[i].total_us > 0 && trials[first].total_us > 0 && trials[i].total_us < 1.2 * trials[first].total_us)
+              by_factor[trials[i].label.substr(0, trials[i].label.find('_'))].push_back(i);
+          for (auto& bf : by_factor) {
+            std::sort(bf.second.begin(), bf.second.end(), [&](size_t a, size_t b) { return trials[a].total_us < trials[b].total_us; });
+            for (size_t k = 0; k < bf.second.size() && k < (budget == 0 ? 3u : 1u); ++k) order.push_back(bf.second[k]);
+          }
+        }
+        if (!order.empty()) {
           if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);
-          const double with_split = whole_kernel_us(adopted);
-          log << "    whole kernel: " << stitched_us << " us without, " << with_split << " us with " << trials[best_i].label << "\n";
-          if (with_split > 0 && stitched_us > 0 && with_split < 0.995 * stitched_us) {
-            for (auto& in : instrs) report << ctx_str << "," << in << "," << trials[best_i].total_us / per << "\n";
-            stitched = std::move(adopted);
-            stitched_us = with_split;
+          double best_with = -1;
+          GraphSpecification best_spec;
+          size_t best_split = first;
+          log << "    whole kernel: " << stitched_us << " us without;";
+          for (size_t i : order) {
+            GraphSpecification adopted = trials[i].spec;
+            drop_unknown(adopted, trials[i].mod->program());
+            const double with_split = whole_kernel_us(adopted);
+            log << " " << trials[i].label << "=" << with_split;
+            if (with_split > 0 && (best_with < 0 || with_split < best_with)) {
+              best_with = with_split;
+              best_spec = std::move(adopted);
+              best_split = i;
+            }
+          }
+          log << "\n";
+          if (verbose) std::fprintf(stderr, "[mononn tuner] %s   whole kernel %.2f us without, %.2f us with %s\n", ctx_str.c_str(), stitched_us, best_with, trials[best_split].label.c_str());
+          if (best_with > 0 && stitched_us > 0 && best_with < 0.995 * stitched_us) {
+            for (auto& in : instrs) report << ctx_str << "," << in << "," << trials[best_split].total_us / per << "\n";
+            stitched = std::move(best_spec);
+            stitched_us = best_with;
+            // the row programs that now add up the partial sums do more loading than before: their knobs again
+            std::vector<std::string> allow, consumers;
+            names_and_consumers(trials[best_split].mod->program(), instr_set, &allow, &consumers);
+            std::string line;
+            GraphSpecification best_knobs;
+            double best_knobs_us = -1;
+            for (int tier : {1, 2})
+              for (int ilp : {1, 2, 4}) {
+                GraphSpecification s = stitched;
+                bool changed = false;
+                for (auto& n : consumers) {
+                  auto it = s.cluster_reduce_spec.find(n);
+                  if (it == s.cluster_reduce_spec.end()) continue;
+                  changed = changed || it->second.locality_tier != tier || it->second.ilp_factor != ilp;
+                  it->second.locality_tier = tier;
+                  it->second.ilp_factor = ilp;
+                }
+                if (!changed) continue;
+                const double us = whole_kernel_us(s);
+                char buf[64];
+                std::snprintf(buf, sizeof buf, " tier%d_ilp%d=%.2f", tier, ilp, us);
+                line += buf;
+                if (us > 0 && (best_knobs_us < 0 || us < best_knobs_us)) {
+                  best_knobs_us = us;
+                  best_knobs = std::move(s);
+                }
+              }
+            log << "    consumers of the split GEMM, whole kernel: now " << stitched_us << " us;" << line << "\n";
+            if (best_knobs_us > 0 && best_knobs_us < 0.997 * stitched_us) {
+              stitched = std::move(best_knobs);
+              stitched_us = best_knobs_us;
+            }
           }
         }
         for (size_t i = first; i < trials.size(); ++i) trials[i].mod.reset();

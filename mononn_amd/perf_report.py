@@ -40,10 +40,10 @@ def stage_report(hlo_text: str, constants, inputs, outputs, spec_dir=None, launc
             acc = p
         else:
             for a, b in zip(acc, p):
-                for k in ("busy_us", "barrier_us", "mean_wg_us"):
+                for k in ("busy_us", "barrier_us", "mean_wg_us", "step_us"):
                     a[k] += b[k]
     for a in acc:
-        for k in ("busy_us", "barrier_us", "mean_wg_us"):
+        for k in ("busy_us", "barrier_us", "mean_wg_us", "step_us"):
             a[k] /= launches
     m.close()
     return acc
@@ -73,9 +73,9 @@ def main(argv=None):
     rows = stage_report(text, consts, inputs, outputs, args.spec_dir, args.launches)
     out = open(args.csv, "w", newline="") if args.csv else sys.stdout
     w = csv.writer(out)
-    w.writerow(["stage", "busy_us", "mean_workgroup_us", "barrier_us", "nodes"])
+    w.writerow(["stage", "busy_us", "mean_workgroup_us", "barrier_us", "step_us", "nodes"])
     for r in rows:
-        w.writerow([r["stage"], f"{r['busy_us']:.3f}", f"{r['mean_wg_us']:.3f}", f"{r['barrier_us']:.3f}", r["nodes"]])
+        w.writerow([r["stage"], f"{r['busy_us']:.3f}", f"{r['mean_wg_us']:.3f}", f"{r['barrier_us']:.3f}", f"{r['step_us']:.3f}", r["nodes"]])
     busy, bar = sum(r["busy_us"] for r in rows), sum(r["barrier_us"] for r in rows)
     print(f"# total: {busy:.1f} us busy in {len(rows)} stages, {bar:.1f} us in {len(rows) - 1} barriers", file=sys.stderr)
 

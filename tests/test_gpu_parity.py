@@ -99,7 +99,7 @@ def test_gather_bit_exact(gpu_device):
     assert np.array_equal(got.view(np.uint16), t[i].view(np.uint16))
 
 
-def _spec_with(hlo_text, gemm_overrides=None, hip=None):
+def _spec_with(hlo_text, gemm_overrides=None, hip=None, grid=None):
     """Default specification with some entries replaced; per-node maps are cleared so that nodes whose names
     change with the fusion decisions get fresh defaults."""
     import json
@@ -113,6 +113,8 @@ def _spec_with(hlo_text, gemm_overrides=None, hip=None):
         entry["cutlass_config"].update(cc)
         spec["gemm_spec_list"][name] = entry
     spec["mononn_hip"].update(hip or {})
+    if grid:
+        spec["cuda_context"]["cuda_runtime_context"]["grid_dim"]["x"] = grid
     return json.dumps(spec)
 
 
@@ -144,6 +146,11 @@ def test_fusion_variants_agree(gpu_device):
         "plain weight layout": _spec_with(fx.hlo_text, hip={"transpose_constant_b": False, "assign_operand_layouts": False}),
         "split-K": _spec_with(fx.hlo_text, gemm_overrides=split),
         "cooperative launch": _spec_with(fx.hlo_text, hip={"cooperative_launch": True}),
+        # by default a GEMM stage asks for its packed weights before it waits at the grid barrier
+        "weights requested inside the tile": _spec_with(fx.hlo_text, hip={"operand_preload": False}),
+        "the same with split-K": _spec_with(fx.hlo_text, hip={"operand_preload": False}, gemm_overrides=split),
+        # a grid of 8 workgroups: several units per workgroup and stage, only the first of them behind a barrier wait
+        "small grid": _spec_with(fx.hlo_text, grid=8),
     }
     for name, spec in variants.items():
         (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, spec)
@@ -155,6 +162,9 @@ def test_fusion_variants_agree(gpu_device):
     assert np.array_equal(fenced.view(np.uint16), base.view(np.uint16)), "barrier flavour must not change any bit"
     (coop,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants["cooperative launch"])
     assert np.array_equal(coop.view(np.uint16), base.view(np.uint16)), "the launch entry point must not change any bit"
+    for name in ("weights requested inside the tile", "small grid"):
+        (other,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants[name])
+        assert np.array_equal(other.view(np.uint16), base.view(np.uint16)), f"{name}: when an operand is requested must not change any bit"
 
 
 def test_repeated_launches_are_bit_identical(gpu_device):

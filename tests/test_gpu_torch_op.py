@@ -47,7 +47,7 @@ def test_perf_report_lists_every_stage(gpu_device, tmp_path):
     fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
     rows = perf_report.stage_report(fx.hlo_text, fx.make_constants(5, "baseline"), fx.make_inputs(5), fx.outputs, launches=5, device=gpu_device)
     assert len(rows) == 15 and [r["stage"] for r in rows] == list(range(15))
-    assert all(r["busy_us"] > 0 and r["mean_wg_us"] > 0 for r in rows)
+    assert all(r["busy_us"] > 0 and r["mean_wg_us"] > 0 and r["step_us"] > 0 for r in rows)
     assert all(r["barrier_us"] > 0 for r in rows[:-1])
     assert any("cublas_gemm" in r["nodes"] for r in rows)
     hlo = tmp_path / "m.hlo"
@@ -55,4 +55,4 @@ def test_perf_report_lists_every_stage(gpu_device, tmp_path):
     out = tmp_path / "report.csv"
     perf_report.main(["--hlo", str(hlo), "--csv", str(out), "--launches", "3"])
     table = list(csv.reader(open(out)))
-    assert table[0] == ["stage", "busy_us", "mean_workgroup_us", "barrier_us", "nodes"] and len(table) == 16
+    assert table[0] == ["stage", "busy_us", "mean_workgroup_us", "barrier_us", "step_us", "nodes"] and len(table) == 16

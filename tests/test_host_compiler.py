@@ -236,7 +236,8 @@ def test_write_once_temp_addresses(layer):
     spec = json.loads(coherent.get_tuning_spec())
     assert spec["mononn_hip"]["barrier"] == "flags_coherent"
     src = coherent.get_source()
-    sigs = {int(i): [p.strip() for p in sig.split(",")][:-1] for i, sig in re.findall(r"void node_fn_(\d+)\(int unit, ([^)]*)\)", src)}
+    sigs = {int(i): [p.strip() for p in sig.split(",") if not re.search(r"\b(smem|pre_b)$", p.strip())]
+            for i, sig in re.findall(r"void node_fn_(\d+)\(int unit, ([^)]*)\)", src)}
     written = []
     for fn, rest in re.findall(r"case \d+: fn = (\d+); units = \d+; first = \d+; total = \d+; new_stage = \w+;(.*?) break;", src):
         ptrs = dict(re.findall(r"p(\d+) = ([^;]*);", rest))
