@@ -78,7 +78,7 @@ Index leading_index(int var, int64_t extent, const std::vector<int64_t>& dims, c
 }
 
 void store(const Program& prog, CodeBuffer& cb, PointerTable& ptrs, const VarTable& vars, const Instr* out, const Index& idx, const std::string& v) {
-  cb.line("mononn_dev::st1(" + ptrs.output(out) + " + " + physical_offset(prog, out, idx).str(vars) + ", " + v + ");");
+  cb.line("mononn_dev::st1(" + ptrs.output(out) + " + " + physical_offset(prog, out, idx, &vars).str(vars) + ", " + v + ");");
 }
 
 std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs);
@@ -259,7 +259,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
             LinExpr lin = LinExpr::variable(row, ROWS).scaled(R).plus(col_of(k, v));
             Index oi = delinearize(lin, o->shape.dims, vars);
             vals.push_back(em.value(em.resolve_output(o), oi));
-            offs.push_back(physical_offset(prog, o, oi));
+            offs.push_back(physical_offset(prog, o, oi, &vars));
           }
           // one packed store when the V elements are adjacent in memory and the pack is 4/8/16 bytes
           const int bytes = V * hlo::dtype_bytes(o->shape.dtype);
@@ -634,8 +634,8 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
       }
       std::string v = em.value(em.resolve_output(out.o), out.idx);
       if (vec4) {
-        LinExpr full = physical_offset(prog, out.o, out.idx);
-        LinExpr base = physical_offset(prog, out.o, out.idx_base);
+        LinExpr full = physical_offset(prog, out.o, out.idx, &vars);
+        LinExpr base = physical_offset(prog, out.o, out.idx_base, &vars);
         out.vector_store = full.equals(base.plus(LinExpr::variable(vr, 4))) && out.o->shape.dtype == DType::kF16;
         if (out.vector_store) cb.line(out.stage + "[r] = " + v + ";");
         else store(prog, cb, ptrs, vars, out.o, out.idx, v);
@@ -649,7 +649,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   if (vec4) {
     for (auto& out : outs)
       if (out.vector_store) {
-        std::string lin = physical_offset(prog, out.o, out.idx_base).str(vars);
+        std::string lin = physical_offset(prog, out.o, out.idx_base, &vars).str(vars);
         cb.line("mononn_dev::stN<_Float16, 4>(" + ptrs.output(out.o) + " + " + lin + ", " + out.stage + ");");
       }
   }
@@ -845,7 +845,7 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
       cb.line("const _Float16 " + arr + "[8] = {" + init + "};");
       cb.line("a[" + S(s) + "][" + S(i) + "] = half8_t{" + arr + "[0], " + arr + "[1], " + arr + "[2], " + arr + "[3], " + arr + "[4], " + arr + "[5], " + arr + "[6], " + arr + "[7]};");
       if (stores) {
-        LinExpr off = physical_offset(prog, H, primary_index(i, s, 0));
+        LinExpr off = physical_offset(prog, H, primary_index(i, s, 0), &vars);
         cb.line("if (store && mv" + S(i) + ") mononn_dev::stN<_Float16, 8>(" + ptrs.output(H) + " + " + off.str(vars) + ", " + arr + ");");
       }
     }
@@ -953,13 +953,13 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
       std::ostringstream b_expr;
       b_expr << pb << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS);
       preload = t.preload_b && g.b_packed && !has_pro;   // a row-program prologue fixes the chunking of the left operand
+      MONONN_CHECK(!g.a_packed || !has_pro, kInternal) << gi->hlo_name << ": fragment-order left operand under a prologue";
       call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
-           << (g.b_packed ? "true" : "false") << ", " << g.K;
-      if (preload) call << ", @NAME@_epi, mononn_dev::NoPrologue, mononn_dev::RowMajorA, true, @NAME@_preb";
-      call << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << KS << ", " << b_expr.str() << ", " << g.M << ", " << g.N << ", "
-           << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
-      if (preload) call << ", mononn_dev::NoPrologue(), mononn_dev::RowMajorA(), &pre_b";
-      else if (has_pro) call << ", pro";
+           << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
+           << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ">("
+           << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
+           << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
+           << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");
       call << ");";
       if (preload) {
         // the companion repeats the unit decoding as far as the right operand needs it

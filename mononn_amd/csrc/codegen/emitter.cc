@@ -45,7 +45,14 @@ std::string PointerTable::output(const Instr* root, DType as) {
   return entries.back().name;
 }
 
-LinExpr physical_offset(const graph::Program& prog, const Instr* root, const Index& idx) {
+LinExpr physical_offset(const graph::Program& prog, const Instr* root, const Index& idx, const VarTable* vars) {
+  auto tile = prog.physical_tile.find(root);
+  if (tile != prog.physical_tile.end()) {
+    MONONN_CHECK(vars != nullptr, kInternal) << root->hlo_name << ": fragment-order buffer addressed without a variable table";
+    const int64_t K = tile->second, R = root->shape.num_elements() / K;
+    Index d = delinearize(linearize(idx, root->shape.dims), {R / 16, 16, K / 32, 4, 8}, *vars);
+    return linearize({d[0], d[2], d[3], d[1], d[4]}, {R / 16, K / 32, 4, 16, 8});
+  }
   auto it = prog.physical_perm.find(root);
   if (it == prog.physical_perm.end()) return linearize(idx, root->shape.dims);
   Index pi;
@@ -215,7 +222,7 @@ std::string Emitter::value(const Instr* ins, const Index& idx) {
 }
 
 std::string Emitter::load(const Instr* root, const Index& idx) {
-  LinExpr lin = physical_offset(prog_, root, idx);
+  LinExpr lin = physical_offset(prog_, root, idx, &vars_);
   auto sk = prog_.split_k.find(root);
   if (sk != prog_.split_k.end()) {
     // split-K GEMM result: S fp32 partial sums, added in a fixed order, then rounded to the f16 value

@@ -52,7 +52,9 @@ struct PointerTable {
 };
 
 // element offset of `idx` inside the buffer of storage root `root`, honouring a permuted physical layout
-LinExpr physical_offset(const graph::Program& prog, const hlo::Instr* root, const Index& idx);
+// element offset of logical index `idx` in the buffer of storage root `root`; `vars` is needed for roots kept in
+// fragment order (digits of the index are re-split)
+LinExpr physical_offset(const graph::Program& prog, const hlo::Instr* root, const Index& idx, const VarTable* vars = nullptr);
 
 class Emitter {
  public:

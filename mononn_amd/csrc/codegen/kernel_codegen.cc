@@ -26,6 +26,7 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.assign_operand_layouts = s.hip.assign_operand_layouts;
   o.fuse_attention = s.hip.fuse_attention;
   o.fuse_gemm_prologue = s.hip.gemm_prologue_fusion;
+  o.pack_left_operands = s.hip.pack_left_operands;
   o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
   for (auto& kv : s.gemm_spec_list)
     if (kv.second.split_k > 1) o.gemm_split_k[kv.first] = kv.second.split_k;

@@ -253,6 +253,9 @@ __device__ __forceinline__ T sign_of(T x) {
 // a chunk are issued back to back (and the next chunk's before the current chunk's MFMAs), which
 // leaves one exposed memory latency per tile instead of one per k step.
 //
+// A is row-major [M, lda] or, when the producing stage of this kernel stores it so (PACKED_A), in the same
+// fragment order as packed weights: a lane's 16 rows x 16 bytes of a row-major operand touch 16 cache lines per
+// quarter wave, a fragment-order operand is one contiguous KiB per MFMA step.
 // B comes in one of two layouts:
 //   PACKED_B = false : Bt[n][k], k contiguous (activation operands such as K in Q.K^T)
 //   PACKED_B = true  : fragment order [n/16][k/32][lane][8] written by the host at upload for
@@ -336,7 +339,7 @@ __device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_
 // when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
 // PRE_B: the right operand's first chunk was requested by gemm_b_preload with the same parameters and comes in `pb`.
 template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA,
-          bool PRE_B = false, class Pre = NoPreB>
+          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
                                           int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
                                           const AMap& amap = AMap(), const Pre* pb = nullptr) {
@@ -347,6 +350,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   constexpr int CH = gemm_chunk_steps(TM, TN, MY_STEPS, PRE_B);
   constexpr int NCHUNK = (MY_STEPS + CH - 1) / CH;
   static_assert(!PRE_B || PACKED_B, "only packed weights can be requested ahead of the tile");
+  static_assert(!PACKED_A || (AMap::kRowMajor && !Pro::enabled), "a fragment-order left operand takes neither a row map nor a prologue");
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
   static_assert(K % 32 == 0, "K must be a multiple of 32");
   const int lane = lane_id();
@@ -367,8 +371,17 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     int m = m_base + i * 16 + r16;
     m = m < M ? m : M - 1;
     a_row[i] = m;
-    a_ptr[i] = A + (long)m * lda + kq;
+    if constexpr (PACKED_A) {
+      // fragment order [m/16][k/32][lane][8], written that way by the producing stage (M is a multiple of 16)
+      int mt = (m_base >> 4) + i;
+      const int mt_max = M / 16 - 1;
+      mt = mt < mt_max ? mt : mt_max;
+      a_ptr[i] = A + ((long)mt * (KTOTAL / 32) * 64 + lane) * 8;
+    } else {
+      a_ptr[i] = A + (long)m * lda + kq;
+    }
   }
+  constexpr int A_STEP = PACKED_A ? 64 * 8 : 32;   // halves between consecutive k steps
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     if (PACKED_B) {
@@ -397,7 +410,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + ks * 32);
+        if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + (long)ks * A_STEP);
         else a[buf][s][i] = *reinterpret_cast<const half8_t*>(amap(A, a_row[i], ks * 32 + kq, lda));
       }
     }

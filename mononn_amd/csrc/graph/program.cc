@@ -533,6 +533,40 @@ struct Builder {
     each_gemm([&](const Instr* g, GemmDesc& d) {
       if (p.physical_perm.count(p.storage_root(g->operands[1]))) d.b_k_contig = true;
     });
+    if (opt.pack_left_operands && enabled("LeftOperandLayoutPass")) pack_left_operands();
+  }
+
+  // A left-hand GEMM operand [M, K] that this kernel produces itself is stored in MFMA fragment order when every
+  // node that addresses the buffer directly (GEMM and attention nodes: operand pointers, not the element
+  // emitter) is a plain MFMA GEMM reading it as its left operand with the same K.
+  void pack_left_operands() {
+    std::map<const Instr*, int64_t> want;    // root -> K
+    std::set<const Instr*> spoiled;
+    auto raw_use = [&](const Instr* operand) { spoiled.insert(p.storage_root(operand)); };
+    std::set<const Instr*> live(p.live_outs.begin(), p.live_outs.end());
+    for (auto& n : p.nodes) {
+      if (n.kind == NodeKind::kAttention) {
+        raw_use(n.members[0]->operands[0]);
+        raw_use(n.members[0]->operands[1]);
+        raw_use(n.members[n.gemm2_index]->operands[1]);
+        continue;
+      }
+      if (n.kind != NodeKind::kGemm) continue;
+      const Instr* g = n.members[0];
+      const GemmDesc& d = n.gemm;
+      const Instr* root = p.storage_root(g->operands[0]);
+      raw_use(g->operands[1]);
+      const bool mfma = d.a_k_contig && (d.b_k_contig || d.b_packed) && d.K % 32 == 0;
+      const bool fits = mfma && !d.is_conv && n.prologue.empty() && d.batch == 1 && d.M % 16 == 0 && p.producer.count(root) && !live.count(root) &&
+                        !p.physical_perm.count(root) && root->shape.dtype == hlo::DType::kF16 && root->shape.num_elements() == d.M * d.K &&
+                        (!want.count(root) || want[root] == d.K);
+      if (fits) want[root] = d.K;
+      else spoiled.insert(root);
+    }
+    for (auto& kv : want)
+      if (!spoiled.count(kv.first)) p.physical_tile[kv.first] = kv.second;
+    for (auto& n : p.nodes)
+      if (n.kind == NodeKind::kGemm && p.physical_tile.count(p.storage_root(n.members[0]->operands[0]))) n.gemm.a_packed = true;
   }
 
   void apply_split_k() {

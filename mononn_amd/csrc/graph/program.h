@@ -29,6 +29,7 @@ struct GemmDesc {
   bool a_k_contig = true;    // A stored [.., M, K]; false: [.., K, M]
   bool b_k_contig = false;   // B stored [.., N, K]; false: [.., K, N]
   bool b_packed = false;     // B is a constant that the host stores in MFMA fragment order at upload
+  bool a_packed = false;     // A is a value of this kernel that its producer stores in MFMA fragment order
   int split_k = 1;           // k range split over workgroups, fp32 partial sums as output
   int64_t a_batch_stride = 0, b_batch_stride = 0, d_batch_stride = 0;
   double alpha = 1.0, beta = 0.0;
@@ -96,6 +97,11 @@ struct Program {
   // storage roots kept in a permuted physical order: physical dim i = logical dim perm[i]
   // (right-hand GEMM operands produced inside the kernel are stored with k minor-most)
   std::map<const hlo::Instr*, std::vector<int>> physical_perm;
+  // storage roots kept in MFMA left-operand fragment order instead of row-major: the row-major linear index is
+  // read as (row, k) of a [rows, K] matrix (K = mapped value) and element (row, k) lives at
+  // ((row/16 * K/32 + k/32) * 4 + k%32/8) * 128 + row%16 * 8 + k%8, so that the 64 lanes' operands of one
+  // 16x32 MFMA step are one contiguous KiB.  Every reader and the writer go through codegen::physical_offset.
+  std::map<const hlo::Instr*, int64_t> physical_tile;
   // GEMM results kept as S fp32 partial sums [S][elements] (split-K); readers add them up
   std::map<const hlo::Instr*, int> split_k;
   std::vector<const hlo::Instr*> live_outs;                        // storage roots, root-tuple order
@@ -116,6 +122,7 @@ struct BuildOptions {
   bool fuse_gemm_prologue = false;      // row programs feeding a GEMM's left operand run inside that GEMM
   bool fuse_attention = true;           // GEMM -> soft-max style row program -> GEMM in one stage
   bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
+  bool pack_left_operands = true;       // store in-kernel left-hand GEMM operands in MFMA fragment order
   std::map<std::string, int> gemm_split_k;   // GEMM instruction (canonical name) -> k split over workgroups
   bool reuse_temp_slots = true;         // false: every temp value gets its own address (written once per launch)
   std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)

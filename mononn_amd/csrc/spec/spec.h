@@ -90,6 +90,8 @@ struct HipOptions {       // "mononn_hip" section
   // GEMM stages request their packed weights between announcing the end of the previous stage and waiting for the
   // other workgroups (the wait moves behind the requests; idle workgroups skip it)
   bool operand_preload = true;
+  // values of this kernel that only GEMMs read as their left operand are stored in MFMA fragment order
+  bool pack_left_operands = true;
 };
 
 struct GraphSpecification {
