@@ -1112,25 +1112,41 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.line("const int mt = (unit % " + S(blocks) + ") * " + S(RW) + " + rw;");
   cb.line("const bool m_valid = mt * 16 + r16 < " + S(M1) + ";");
   cb.line("const int m = m_valid ? mt * 16 + r16 : " + S(M1 - 1) + ";");
-  cb.line("const _Float16* qp = " + pq + " + (long)bidx * " + S(d1.a_batch_stride) + " + m * " + S(K1) + " + g * 8;");
-  cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + (kw * " + S(NKW) + " + r16) * " + S(K1) + " + g * 8;");
-  cb.line("const _Float16* vp = " + pv + " + (long)bidx * " + S(d2.b_batch_stride) + " + r16 * " + S(N1) + " + kw * " + S(NKW) + " + g * 4;");
+  // Operands in fragment order (stored so by the stage that produced them) are one contiguous KiB per MFMA step;
+  // row-major ones cost a lane's 16 rows x 16 bytes = 16 cache lines per quarter wave.
+  MONONN_CHECK(!d1.a_packed || M1 % 16 == 0, kInternal) << "fragment-order queries need whole row blocks";
+  if (d1.a_packed) {
+    cb.line("const int mt_c = mt < " + S(M1 / 16) + " ? mt : " + S(M1 / 16 - 1) + ";");
+    cb.line("const _Float16* qp = " + pq + " + (((long)bidx * " + S(M1 / 16) + " + mt_c) * " + S(KS1 * 64) + " + lane) * 8;");
+  } else {
+    cb.line("const _Float16* qp = " + pq + " + (long)bidx * " + S(d1.a_batch_stride) + " + m * " + S(K1) + " + g * 8;");
+  }
+  if (d1.b_tiled) cb.line("const _Float16* kp = " + pk + " + (((long)bidx * " + S(N1 / 16) + " + kw * " + S(NKW / 16) + ") * " + S(KS1 * 64) + " + lane) * 8;");
+  else cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + (kw * " + S(NKW) + " + r16) * " + S(K1) + " + g * 8;");
+  if (d2.b_tiled) cb.line("const _Float16* vp = " + pv + " + (((long)bidx * " + S(N2 / 16) + ") * " + S(N1 / 32) + " + kw * " + S(NKW / 32) + ") * 512 + lane * 8;");
+  else cb.line("const _Float16* vp = " + pv + " + (long)bidx * " + S(d2.b_batch_stride) + " + r16 * " + S(N1) + " + kw * " + S(NKW) + " + g * 4;");
   // all operand loads up front: one exposed memory latency for the whole unit
   cb.line("half8_t qf[" + S(KS1) + "], kf[" + S(NT1) + "][" + S(KS1) + "];");
-  cb.line("half4_t vf[" + S(NT2) + "][" + S(KS2) + "][2];");
+  cb.line("half8_t vf[" + S(NT2) + "][" + S(KS2) + "];");
   cb.line("#pragma unroll");
-  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qp + ks * 32);");
+  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qp + ks * " + S(d1.a_packed ? 512 : 32) + ");");
   cb.line("#pragma unroll");
   cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
   cb.line("#pragma unroll");
-  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + j * " + S(16 * K1) + " + ks * 32);");
+  if (d1.b_tiled) cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + (j * " + S(KS1) + " + ks) * 512);");
+  else cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + j * " + S(16 * K1) + " + ks * 32);");
   cb.close();
   cb.line("#pragma unroll");
   cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
   cb.line("#pragma unroll");
   cb.open("for (int ks = 0; ks < " + S(KS2) + "; ++ks)");
-  cb.line("vf[t][ks][0] = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32);");
-  cb.line("vf[t][ks][1] = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32 + 16);");
+  if (d2.b_tiled) {
+    cb.line("vf[t][ks] = *reinterpret_cast<const half8_t*>(vp + (t * " + S(N1 / 32) + " + ks) * 512);");
+  } else {
+    cb.line("const half4_t lo = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32);");
+    cb.line("const half4_t hi = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32 + 16);");
+    cb.line("vf[t][ks] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};");
+  }
   cb.close();
   cb.close();
   cb.line("float4_t sacc[" + S(NT1) + "];");
@@ -1190,8 +1206,7 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.line("const half8_t pf = {pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]};");
   cb.line("#pragma unroll");
   cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
-  cb.line("const half8_t vv = {vf[t][ks][0][0], vf[t][ks][0][1], vf[t][ks][0][2], vf[t][ks][0][3], vf[t][ks][1][0], vf[t][ks][1][1], vf[t][ks][1][2], vf[t][ks][1][3]};");
-  cb.line("oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv, pf, oacc[t], 0, 0, 0);");
+  cb.line("oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[t][ks], pf, oacc[t], 0, 0, 0);");
   cb.close();
   cb.close();
 

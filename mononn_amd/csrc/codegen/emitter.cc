@@ -49,9 +49,25 @@ LinExpr physical_offset(const graph::Program& prog, const Instr* root, const Ind
   auto tile = prog.physical_tile.find(root);
   if (tile != prog.physical_tile.end()) {
     MONONN_CHECK(vars != nullptr, kInternal) << root->hlo_name << ": fragment-order buffer addressed without a variable table";
-    const int64_t K = tile->second, R = root->shape.num_elements() / K;
-    Index d = delinearize(linearize(idx, root->shape.dims), {R / 16, 16, K / 32, 4, 8}, *vars);
-    return linearize({d[0], d[2], d[3], d[1], d[4]}, {R / 16, K / 32, 4, 16, 8});
+    Index pi = idx;
+    std::vector<int64_t> pd = root->shape.dims;
+    auto perm = prog.physical_perm.find(root);
+    if (perm != prog.physical_perm.end()) {
+      pi.clear();
+      pd.clear();
+      for (int d : perm->second) {
+        pi.push_back(idx[d]);
+        pd.push_back(root->shape.dims[d]);
+      }
+    }
+    const int64_t K = tile->second.k, R = root->shape.num_elements() / K;
+    if (tile->second.order == graph::Program::TileOrder::kRunsOf8) {
+      Index d = delinearize(linearize(pi, pd), {R / 16, 16, K / 32, 4, 8}, *vars);
+      return linearize({d[0], d[2], d[3], d[1], d[4]}, {R / 16, K / 32, 4, 16, 8});
+    }
+    // k % 32 = 16 * half + 4 * g + e  ->  lane group g, element 4 * half + e
+    Index d = delinearize(linearize(pi, pd), {R / 16, 16, K / 32, 2, 4, 4}, *vars);
+    return linearize({d[0], d[2], d[4], d[1], d[3], d[5]}, {R / 16, K / 32, 4, 16, 2, 4});
   }
   auto it = prog.physical_perm.find(root);
   if (it == prog.physical_perm.end()) return linearize(idx, root->shape.dims);

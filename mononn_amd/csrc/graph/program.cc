@@ -536,37 +536,61 @@ struct Builder {
     if (opt.pack_left_operands && enabled("LeftOperandLayoutPass")) pack_left_operands();
   }
 
-  // A left-hand GEMM operand [M, K] that this kernel produces itself is stored in MFMA fragment order when every
-  // node that addresses the buffer directly (GEMM and attention nodes: operand pointers, not the element
-  // emitter) is a plain MFMA GEMM reading it as its left operand with the same K.
+  // Operands that GEMM and attention nodes fetch with their own address arithmetic (not through the element
+  // emitter) are stored in MFMA fragment order when this kernel produces them itself and every such node reads
+  // them the same way: the left operand [M, K] of a plain MFMA GEMM, and the three operands of a fused attention
+  // (queries and keys contracted over their minor dimension, values over the key dimension).
   void pack_left_operands() {
-    std::map<const Instr*, int64_t> want;    // root -> K
+    using Order = Program::TileOrder;
+    struct Want {
+      int64_t k;
+      Order order;
+    };
+    std::map<const Instr*, Want> want;
     std::set<const Instr*> spoiled;
-    auto raw_use = [&](const Instr* operand) { spoiled.insert(p.storage_root(operand)); };
     std::set<const Instr*> live(p.live_outs.begin(), p.live_outs.end());
+    // a use of `operand` as [rows, k] in the given order; `perm_ok`: the root may carry the k-contiguous transposition
+    auto use = [&](const Instr* operand, bool fits, int64_t rows, int64_t k, Order order, bool perm_ok) {
+      const Instr* root = p.storage_root(operand);
+      fits = fits && rows % 16 == 0 && k % 32 == 0 && p.producer.count(root) && !live.count(root) && (perm_ok || !p.physical_perm.count(root)) &&
+             root->shape.dtype == hlo::DType::kF16 && root->shape.num_elements() == rows * k &&
+             (!want.count(root) || (want[root].k == k && want[root].order == order));
+      if (fits) want[root] = {k, order};
+      else spoiled.insert(root);
+    };
     for (auto& n : p.nodes) {
       if (n.kind == NodeKind::kAttention) {
-        raw_use(n.members[0]->operands[0]);
-        raw_use(n.members[0]->operands[1]);
-        raw_use(n.members[n.gemm2_index]->operands[1]);
+        const GemmDesc& d1 = n.gemm;
+        const GemmDesc& d2 = n.gemm2;
+        const Instr* g1 = n.members[0];
+        const Instr* g2 = n.members[n.gemm2_index];
+        const bool dense = d1.a_k_contig && d1.b_k_contig && d2.b_k_contig && d1.a_batch_stride == d1.M * d1.K && d1.b_batch_stride == d1.N * d1.K &&
+                           d2.b_batch_stride == d2.N * d2.K && d1.M % 16 == 0 && d1.N % 16 == 0 && d2.N % 16 == 0;
+        use(g1->operands[0], dense, d1.batch * d1.M, d1.K, Order::kRunsOf8, false);
+        use(g1->operands[1], dense, d1.batch * d1.N, d1.K, Order::kRunsOf8, false);
+        // values: stored [.., N2, keys] (transposed by the operand layout pass), contracted over the keys
+        use(g2->operands[1], dense && p.physical_perm.count(p.storage_root(g2->operands[1])), d2.batch * d2.N, d2.K, Order::kPairsOf4, true);
         continue;
       }
       if (n.kind != NodeKind::kGemm) continue;
       const Instr* g = n.members[0];
       const GemmDesc& d = n.gemm;
-      const Instr* root = p.storage_root(g->operands[0]);
-      raw_use(g->operands[1]);
+      spoiled.insert(p.storage_root(g->operands[1]));
       const bool mfma = d.a_k_contig && (d.b_k_contig || d.b_packed) && d.K % 32 == 0;
-      const bool fits = mfma && !d.is_conv && n.prologue.empty() && d.batch == 1 && d.M % 16 == 0 && p.producer.count(root) && !live.count(root) &&
-                        !p.physical_perm.count(root) && root->shape.dtype == hlo::DType::kF16 && root->shape.num_elements() == d.M * d.K &&
-                        (!want.count(root) || want[root] == d.K);
-      if (fits) want[root] = d.K;
-      else spoiled.insert(root);
+      use(g->operands[0], mfma && !d.is_conv && n.prologue.empty() && d.batch == 1, d.M, d.K, Order::kRunsOf8, false);
     }
     for (auto& kv : want)
-      if (!spoiled.count(kv.first)) p.physical_tile[kv.first] = kv.second;
-    for (auto& n : p.nodes)
-      if (n.kind == NodeKind::kGemm && p.physical_tile.count(p.storage_root(n.members[0]->operands[0]))) n.gemm.a_packed = true;
+      if (!spoiled.count(kv.first)) p.physical_tile[kv.first] = {kv.second.k, kv.second.order};
+    auto tiled = [&](const Instr* operand) { return p.physical_tile.count(p.storage_root(operand)) > 0; };
+    for (auto& n : p.nodes) {
+      if (n.kind == NodeKind::kGemm) {
+        n.gemm.a_packed = tiled(n.members[0]->operands[0]);
+      } else if (n.kind == NodeKind::kAttention) {
+        n.gemm.a_packed = tiled(n.members[0]->operands[0]);
+        n.gemm.b_tiled = tiled(n.members[0]->operands[1]);
+        n.gemm2.b_tiled = tiled(n.members[n.gemm2_index]->operands[1]);
+      }
+    }
   }
 
   void apply_split_k() {

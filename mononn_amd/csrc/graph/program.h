@@ -30,6 +30,7 @@ struct GemmDesc {
   bool b_k_contig = false;   // B stored [.., N, K]; false: [.., K, N]
   bool b_packed = false;     // B is a constant that the host stores in MFMA fragment order at upload
   bool a_packed = false;     // A is a value of this kernel that its producer stores in MFMA fragment order
+  bool b_tiled = false;      // likewise B (only operands of the fused attention; weights use b_packed)
   int split_k = 1;           // k range split over workgroups, fp32 partial sums as output
   int64_t a_batch_stride = 0, b_batch_stride = 0, d_batch_stride = 0;
   double alpha = 1.0, beta = 0.0;
@@ -97,11 +98,20 @@ struct Program {
   // storage roots kept in a permuted physical order: physical dim i = logical dim perm[i]
   // (right-hand GEMM operands produced inside the kernel are stored with k minor-most)
   std::map<const hlo::Instr*, std::vector<int>> physical_perm;
-  // storage roots kept in MFMA left-operand fragment order instead of row-major: the row-major linear index is
-  // read as (row, k) of a [rows, K] matrix (K = mapped value) and element (row, k) lives at
-  // ((row/16 * K/32 + k/32) * 4 + k%32/8) * 128 + row%16 * 8 + k%8, so that the 64 lanes' operands of one
-  // 16x32 MFMA step are one contiguous KiB.  Every reader and the writer go through codegen::physical_offset.
-  std::map<const hlo::Instr*, int64_t> physical_tile;
+  // Storage roots kept in MFMA operand fragment order.  The buffer is seen as a [rows, K] matrix (the row-major
+  // linear index, after `physical_perm` if the root has one, is row * K + k); the 16 rows x 32 k of one MFMA step
+  // form one contiguous KiB [lane = g * 16 + row % 16][8 halves] at block (row / 16) * (K / 32) + k / 32, so that
+  // a wave loads an operand with one fully coalesced instruction.  Two enumerations of k inside a step:
+  //   kRunsOf8:  lane group g holds k % 32 in [8g, 8g + 8)            (operands contracted over their minor dim)
+  //   kPairsOf4: lane group g holds k % 32 in {4g..4g+3, 16+4g..+3}   (the order in which a lane of the fused
+  //              attention holds its probabilities: the right operand of the second contraction)
+  // Every reader and the writer of such a root go through codegen::physical_offset.
+  enum class TileOrder { kRunsOf8, kPairsOf4 };
+  struct TileLayout {
+    int64_t k = 0;
+    TileOrder order = TileOrder::kRunsOf8;
+  };
+  std::map<const hlo::Instr*, TileLayout> physical_tile;
   // GEMM results kept as S fp32 partial sums [S][elements] (split-K); readers add them up
   std::map<const hlo::Instr*, int> split_k;
   std::vector<const hlo::Instr*> live_outs;                        // storage roots, root-tuple order

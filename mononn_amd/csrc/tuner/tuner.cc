@@ -456,7 +456,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       promising = best_us < 0 || (stitched_us > 0 && stitched_us < 1.08 * best_us);
       if (!promising) log << "  [" << ctx_str << "] " << stitched_us << " us before refinement, best context so far " << best_us << " us: not refined\n";
     }
-    if (promising && !runners_up.empty() && !env::is_true("MONONN_TUNER_NO_REFINEMENT")) {
+    // two sweeps: what the first one changes in one class can change the ranking in another
+    for (int sweep = 0, changed = 1; sweep < (budget == 0 ? 2 : 1) && changed && promising && !runners_up.empty() && !env::is_true("MONONN_TUNER_NO_REFINEMENT"); ++sweep) {
+      changed = 0;
       for (auto& kv : classes) {
         ClassInfo& c = kv.second;
         auto ru = runners_up.find(c.function);
@@ -484,12 +486,18 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             << " us;" << line << "\n";
         if (verbose) std::fprintf(stderr, "[mononn tuner] %s refinement %s (%s): now %.2f us;%s\n", ctx_str.c_str(), c.kind.c_str(), c.nodes[0].c_str(), stitched_us, line.c_str());
         if (best_alt && best_alt_us < 0.997 * stitched_us) {
+          const Alternative replaced{"previous", stitched_us, stitched};   // stays a candidate of the next sweep
+          const Alternative adopted = *best_alt;
+          best_alt = &adopted;
+          for (auto& alt : ru->second)
+            if (alt.label == adopted.label) alt = replaced;
           for (auto& n : c.nodes) {
             if (c.kind == "gemm" || c.kind == "attention") stitched.gemm_spec_list[n] = best_alt->spec.gemm_spec_list.at(n);
             else if (c.kind == "cluster_reduce") stitched.cluster_reduce_spec[n] = best_alt->spec.cluster_reduce_spec.at(n);
             else if (c.kind == "cluster_elewise") stitched.cluster_elewise_spec[n] = best_alt->spec.cluster_elewise_spec.at(n);
           }
           stitched_us = best_alt_us;
+          changed = 1;
         }
       }
     }
