@@ -474,13 +474,18 @@ namespace {
 // are all entries from `first_epi` on.
 struct Epilogue {
   std::string struct_text;   // struct @NAME@_epi { ... };
+  bool along_m = false;      // the four values of a call are four consecutive rows of one column (else columns of one row)
+  int vector_stores = 0;     // outputs written with one 8-byte store per call
   std::string init_line;     // @NAME@_epi epi{...};
   std::vector<std::string> globals;
 };
 
+// along_m: the MFMA is issued with the operands swapped, so that a lane holds four consecutive rows m of one
+// column n; outputs that are stored with m as the fast dimension (a transposed result) then take one packed
+// store instead of four scattered ones.
 Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<const Instr*>& cluster_members,
                         const std::vector<const Instr*>& outputs, const graph::GemmDesc& g, bool mfma, PointerTable& ptrs,
-                        size_t first_epi) {
+                        size_t first_epi, bool along_m = false) {
   if (g.split_k > 1) {
     // fp32 partial sums [split][batch][M][N]; the consumers add them up and apply the rounding
     MONONN_CHECK(mfma && g.N % 4 == 0 && cluster_members.empty() && outputs.size() == 1 && outputs[0] == gi && !g.has_addend, kSpecError)
@@ -502,26 +507,40 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     e.init_line = "@NAME@_epi epi{" + po + ", ksplit};";
     return e;
   }
-  const bool vec4 = mfma && g.N % 4 == 0;
+  MONONN_CHECK(!along_m || (mfma && g.M % 4 == 0 && !g.is_conv), kUnsupported) << gi->hlo_name << ": rows cannot be taken four at a time";
+  const bool vec4 = mfma && (along_m || g.N % 4 == 0);
   CodeBuffer cb;   // epilogue body
   VarTable vars;
   Emitter em(prog, cluster_members, cb, vars, ptrs);
   const hlo::Shape& D = gi->shape;
   std::vector<int64_t> batch_dims(D.dims.begin(), D.dims.end() - 2);
   int vb = vars.add("bidx", g.batch);
-  int vm = vars.add("m", g.M);
-  int vn4 = -1, vr = -1, vnn = -1;
-  if (vec4) {
-    vn4 = vars.add("n4", g.N / 4);
+  int vm = -1, vm4 = -1, vn4 = -1, vr = -1, vnn = -1;
+  if (along_m) {
+    vm4 = vars.add("m4", g.M / 4);
     vr = vars.add("r", 4);
-  } else {
     vnn = vars.add("nn", g.N);
+  } else {
+    vm = vars.add("m", g.M);
+    if (vec4) {
+      vn4 = vars.add("n4", g.N / 4);
+      vr = vars.add("r", 4);
+    } else {
+      vnn = vars.add("nn", g.N);
+    }
   }
   auto gemm_index = [&](bool with_r) {
     Index idx;
     if (g.is_conv) {
       // the GEMM row m enumerates the output pixels (n, p, q) in row-major order
       idx = delinearize(LinExpr::variable(vm, g.M), std::vector<int64_t>(D.dims.begin(), D.dims.end() - 1), vars);
+    } else if (along_m) {
+      idx = delinearize(LinExpr::variable(vb, g.batch), batch_dims, vars);
+      LinExpr m = LinExpr::variable(vm4, g.M / 4).scaled(4);
+      if (with_r) m = m.plus(LinExpr::variable(vr, 4));
+      idx.push_back(m);
+      idx.push_back(LinExpr::variable(vnn, g.N));
+      return idx;
     } else {
       idx = delinearize(LinExpr::variable(vb, g.batch), batch_dims, vars);
       idx.push_back(LinExpr::variable(vm, g.M));
@@ -562,7 +581,8 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   if (alpha_lit.find_first_of(".e") == std::string::npos) alpha_lit += ".0";
   alpha_lit += "f";
 
-  if (vec4) cb.line("const int n4 = n0 >> 2;");
+  if (along_m) cb.line("const int m4 = m0 >> 2;");
+  else if (vec4) cb.line("const int n4 = n0 >> 2;");
   // per-output staging arrays for the vector store
   struct Out {
     const Instr* o;
@@ -572,6 +592,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     std::string stage;
   };
   std::vector<Out> outs;
+  int n_vector_stores = 0;
   for (auto* o : outputs) {
     MONONN_CHECK(o->shape.num_elements() == D.num_elements(), kUnsupported)
         << o->hlo_name << ": epilogue output has a different element count than the GEMM result";
@@ -637,6 +658,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
         LinExpr full = physical_offset(prog, out.o, out.idx, &vars);
         LinExpr base = physical_offset(prog, out.o, out.idx_base, &vars);
         out.vector_store = full.equals(base.plus(LinExpr::variable(vr, 4))) && out.o->shape.dtype == DType::kF16;
+        if (out.vector_store) ++n_vector_stores;
         if (out.vector_store) cb.line(out.stage + "[r] = " + v + ";");
         else store(prog, cb, ptrs, vars, out.o, out.idx, v);
       } else {
@@ -675,9 +697,11 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
       for (size_t i = 0; i < preloads.size(); ++i) pre += "    " + preloads[i].second + " v" + S(i) + "[4];\n";
     }
     pre += "  };\n";
-    pre += "  __device__ __forceinline__ void preload(int bidx, int m, int n0, Pre& pre) const {\n";
+    pre += along_m ? "  __device__ __forceinline__ void preload(int bidx, int m0, int nn, Pre& pre) const {\n"
+                   : "  __device__ __forceinline__ void preload(int bidx, int m, int n0, Pre& pre) const {\n";
     if (!preloads.empty()) {
-      pre += "    const int n4 = n0 >> 2;\n    #pragma unroll\n    for (int r = 0; r < 4; ++r) {\n";
+      pre += along_m ? "    const int m4 = m0 >> 2;\n" : "    const int n4 = n0 >> 2;\n";
+      pre += "    #pragma unroll\n    for (int r = 0; r < 4; ++r) {\n";
       for (size_t i = 0; i < preloads.size(); ++i) pre += "      pre.v" + S(i) + "[r] = " + preloads[i].first + ";\n";
       pre += "    }\n";
     }
@@ -688,7 +712,8 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
       for (size_t pos = body_text.find(ref); pos != std::string::npos; pos = body_text.find(ref, pos + with.size())) body_text.replace(pos, ref.size(), with);
     }
   }
-  if (vec4) pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4], const Pre& pre) const {\n";
+  if (along_m) pre += "  __device__ __forceinline__ void operator()(int bidx, int m0, int nn, const float (&acc)[4], const Pre& pre) const {\n";
+  else if (vec4) pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4], const Pre& pre) const {\n";
   else if (mfma) {
     pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&accv)[4], const Pre&) const {\n";
     pre += "    for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") { const float acc = accv[r]; one(bidx, m, nn, acc); } }\n  }\n";
@@ -705,6 +730,8 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
 
   Epilogue out_e;
   out_e.struct_text = pre;
+  out_e.along_m = along_m;
+  out_e.vector_stores = n_vector_stores;
   std::string init = "@NAME@_epi epi{";
   for (size_t i = first_epi; i < ptrs.entries.size(); ++i) init += (i > first_epi ? ", " : "") + ptrs.entries[i].name;
   init += "};";
@@ -904,7 +931,27 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   }
   const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
   std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
-  Epilogue epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, ptrs, first_epi);
+  Epilogue epi;
+  {
+    // both orientations of the accumulator tile are generated; rows-per-lane wins when it packs more stores
+    PointerTable p_n = ptrs;
+    epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, p_n, first_epi);
+    bool use_m = false;
+    if (mfma && g.split_k <= 1 && !g.is_conv && g.M % 4 == 0) {
+      try {
+        PointerTable p_m = ptrs;
+        Epilogue e_m = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, p_m, first_epi, true);
+        if (e_m.vector_stores > epi.vector_stores) {
+          epi = std::move(e_m);
+          ptrs = std::move(p_m);
+          use_m = true;
+        }
+      } catch (const Error& e) {
+        if (e.code() != kUnsupported) throw;
+      }
+    }
+    if (!use_m) ptrs = std::move(p_n);
+  }
   CodeBuffer fb;
   std::string conv_struct, preload_body;
   bool preload = false;
@@ -956,7 +1003,8 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
       MONONN_CHECK(!g.a_packed || !has_pro, kInternal) << gi->hlo_name << ": fragment-order left operand under a prologue";
       call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
            << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
-           << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ">("
+           << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
+           << (epi.along_m ? "true" : "false") << ">("
            << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
            << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
            << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");

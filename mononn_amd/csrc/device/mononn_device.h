@@ -264,7 +264,8 @@ __device__ __forceinline__ T sign_of(T x) {
 //
 // The MFMA is issued with the B fragment as first operand so that a lane ends up with four
 // consecutive n of one row m (n = n0 + 4*(lane/16) + r, m = m0 + lane%16): the epilogue then
-// stores 8 contiguous bytes per lane.
+// stores 8 contiguous bytes per lane.  D_ALONG_M swaps the operands: four consecutive m of one
+// column n (m = m0 + 4*(lane/16) + r, n = n0 + lane%16), for results that are stored transposed.
 //
 // Epilogue functor:  struct Pre;  void preload(int batch, int m, int n, Pre&) const   (loads what operator() will read)
 //                    void operator()(int batch, int m, int n, const float (&v)[4])   (n % 4 == 0)
@@ -339,7 +340,7 @@ __device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_
 // when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
 // PRE_B: the right operand's first chunk was requested by gemm_b_preload with the same parameters and comes in `pb`.
 template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA,
-          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false>
+          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
                                           int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
                                           const AMap& amap = AMap(), const Pre* pb = nullptr) {
@@ -437,10 +438,15 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   for (int q = 0; q < NSLOT; ++q) {
     int f = q * WK + wk;
     f = f < TM * TN ? f : TM * TN - 1;
-    int m = m_base + (f / TN) * 16 + r16;
-    int n = n_base + (f % TN) * 16 + (lane >> 4) * 4;
-    m = m < M ? m : M - 1;
-    n = n < N ? n : (N >= 4 ? N - 4 : 0);
+    int m = m_base + (f / TN) * 16 + (D_ALONG_M ? (lane >> 4) * 4 : r16);
+    int n = n_base + (f % TN) * 16 + (D_ALONG_M ? r16 : (lane >> 4) * 4);
+    if (D_ALONG_M) {
+      m = m < M ? m : (M >= 4 ? M - 4 : 0);
+      n = n < N ? n : N - 1;
+    } else {
+      m = m < M ? m : M - 1;
+      n = n < N ? n : (N >= 4 ? N - 4 : 0);
+    }
     epi.preload(batch, m, n, pre[q]);
   }
 #pragma unroll
@@ -455,7 +461,8 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[c & 1][s][j], a[c & 1][s][i], acc[i][j], 0, 0, 0);
+            acc[i][j] = D_ALONG_M ? __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c & 1][s][i], b[c & 1][s][j], acc[i][j], 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_16x16x32_f16(b[c & 1][s][j], a[c & 1][s][i], acc[i][j], 0, 0, 0);
       }
     }
   }
@@ -486,8 +493,8 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         float4_t s = part[0];
 #pragma unroll
         for (int w = 1; w < WK; ++w) s += part[w];
-        const int m = m_base + i * 16 + r16;
-        const int n = n_base + j * 16 + (lane >> 4) * 4;
+        const int m = m_base + i * 16 + (D_ALONG_M ? (lane >> 4) * 4 : r16);
+        const int n = n_base + j * 16 + (D_ALONG_M ? r16 : (lane >> 4) * 4);
         if (m < M && n < N) {
           float v[4] = {s[0], s[1], s[2], s[3]};
           epi(batch, m, n, v, pre[f / WK]);
@@ -498,8 +505,8 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int m = m_base + i * 16 + r16;
-        const int n = n_base + j * 16 + (lane >> 4) * 4;
+        const int m = m_base + i * 16 + (D_ALONG_M ? (lane >> 4) * 4 : r16);
+        const int n = n_base + j * 16 + (D_ALONG_M ? r16 : (lane >> 4) * 4);
         if (m < M && n < N) {
           float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
           epi(batch, m, n, v, pre[i * TN + j]);
