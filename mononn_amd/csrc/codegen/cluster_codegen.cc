@@ -1069,6 +1069,39 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   return f;
 }
 
+// Output projection inside the attention node: the context of batch element bidx = (b, h), rows m, columns n must be
+// exactly element (b * M + m, h * N2 + n) of the projection's left operand, moved there by the epilogue clusters
+// without any arithmetic.  Proven on the code generator itself: the second GEMM's value is bound to a register at
+// (bidx, m, n) and the left operand is requested at the expected place; it must come back as that register.
+void check_out_proj_mapping(const Program& prog, const Instr* g2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epi_members,
+                            const Instr* g3, const graph::GemmDesc& d3, int heads) {
+  MONONN_CHECK(heads >= 1 && d2.batch % heads == 0 && d3.K == heads * d2.N && d3.M == d2.batch / heads * d2.M, kUnsupported)
+      << g3->hlo_name << ": not a projection of merged heads";
+  MONONN_CHECK(d2.N % 32 == 0 && d3.N % 16 == 0 && d3.a_k_contig && d3.batch == 1, kUnsupported) << g3->hlo_name << ": projection extents do not fit MFMA steps";
+  const Instr* c = nullptr;   // entry-level value whose storage the projection reads
+  for (auto* o : external_outputs(prog, [&] {
+         std::vector<const Instr*> tail{g2};
+         tail.insert(tail.end(), epi_members.begin(), epi_members.end());
+         return tail;
+       }()))
+    if (prog.storage_root(g3->operands[0]) == o) c = o;
+  MONONN_CHECK(c != nullptr && c != g2, kUnsupported) << g3->hlo_name << ": left operand is not the merged context";
+  CodeBuffer scratch;
+  VarTable vars;
+  PointerTable ptrs;
+  Emitter em(prog, epi_members, scratch, vars, ptrs);
+  int vb = vars.add("bidx", d2.batch), vm = vars.add("m", d2.M), vn = vars.add("n", d2.N);
+  const hlo::Shape& D2 = g2->shape;
+  Index gidx = delinearize(LinExpr::variable(vb, d2.batch), std::vector<int64_t>(D2.dims.begin(), D2.dims.end() - 2), vars);
+  gidx.push_back(LinExpr::variable(vm, d2.M));
+  gidx.push_back(LinExpr::variable(vn, d2.N));
+  em.bind(g2, gidx, "GV");
+  Index bh = delinearize(LinExpr::variable(vb, d2.batch), {d2.batch / heads, static_cast<int64_t>(heads)}, vars);
+  LinExpr lin = linearize({bh[0], LinExpr::variable(vm, d2.M), bh[1], LinExpr::variable(vn, d2.N)}, {d2.batch / heads, d2.M, static_cast<int64_t>(heads), d2.N});
+  std::string v = em.value(em.resolve_output(c), delinearize(lin, c->shape.dims, vars));
+  MONONN_CHECK(v == "GV", kUnsupported) << g3->hlo_name << ": the clusters between the attention and the projection do more than move data";
+}
+
 // GEMM -> row program -> GEMM with everything between the two contractions on chip.
 //
 // A workgroup owns RW blocks of 16 rows m of one batch element; the KW waves of a block split the
@@ -1085,7 +1118,8 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
 // tiles t with t % KW == kw and runs the epilogue on them.
 NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,
                            const Instr* g2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epi_members,
-                           const std::vector<const Instr*>& outputs, const LaunchShape& ls, int key_waves) {
+                           const std::vector<const Instr*>& outputs, const LaunchShape& ls, int key_waves,
+                           const Instr* g3 = nullptr, const graph::GemmDesc* d3p = nullptr, int heads = 0, bool preload_w = false) {
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
@@ -1151,6 +1185,9 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   }
   const int o_off = smem;
   if (KW > 1) smem += RW * KW * NT2 * 64 * 16;
+  // absorbed projection: the context rows of a row block as f16 left-operand fragments [N2 / 32][64 lanes][8]
+  const int cx_off = smem;
+  if (g3) smem += RW * static_cast<int>(N2) * 16 * 2;
 
   cb.line("const int lane = mononn_dev::lane_id();");
   cb.line("const int r16 = lane & 15, g = lane >> 4;");
@@ -1173,6 +1210,36 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   else cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + (kw * " + S(NKW) + " + r16) * " + S(K1) + " + g * 8;");
   if (d2.b_tiled) cb.line("const _Float16* vp = " + pv + " + (((long)bidx * " + S(N2 / 16) + ") * " + S(N1 / 32) + " + kw * " + S(NKW / 32) + ") * 512 + lane * 8;");
   else cb.line("const _Float16* vp = " + pv + " + (long)bidx * " + S(d2.b_batch_stride) + " + r16 * " + S(N1) + " + kw * " + S(NKW) + " + g * 4;");
+  // ---- absorbed output projection: this head's K3 slice of the packed weights, all N3 columns split over the KW waves
+  std::string pw, po, preload_body;
+  int NT3 = 0, NJ = 0, KS3 = 0;
+  if (g3) {
+    const graph::GemmDesc& d3 = *d3p;
+    MONONN_CHECK(!d2.has_addend && N2 % 32 == 0 && d3.N % 16 == 0 && d3.K == heads * N2 && d1.batch % heads == 0 && !d3.has_addend, kUnsupported)
+        << g3->hlo_name << ": projection cannot run inside the attention node";
+    pw = ptrs.input(prog.storage_root(g3->operands[1]));
+    po = ptrs.output(g3, DType::kF32);
+    NT3 = static_cast<int>(d3.N / 16);
+    NJ = (NT3 + KW - 1) / KW;
+    KS3 = static_cast<int>(N2 / 32);
+    CodeBuffer wl;
+    wl.line("#pragma unroll");
+    wl.open("for (int jj = 0; jj < " + S(NJ) + "; ++jj)");
+    wl.line("int nt = jj * " + S(KW) + " + kw;");
+    wl.line("nt = nt < " + S(NT3) + " ? nt : " + S(NT3 - 1) + ";");
+    wl.line("#pragma unroll");
+    wl.line("for (int s = 0; s < " + S(KS3) + "; ++s) pre_w.v[jj * " + S(KS3) + " + s] = *reinterpret_cast<const half8_t*>(" + pw + " + (((long)nt * " +
+            S(d3.K / 32) + " + head * " + S(KS3) + " + s) * 64 + lane) * 8);");
+    wl.close();
+    preload_body = wl.text();
+    cb.line("const int head = bidx % " + S(heads) + ";");
+    if (!preload_w) {
+      cb.line("@NAME@_preb pre_w;");
+      std::istringstream is(preload_body);
+      std::string l;
+      while (std::getline(is, l)) cb.line(l);
+    }
+  }
   // all operand loads up front: one exposed memory latency for the whole unit
   cb.line("half8_t qf[" + S(KS1) + "], kf[" + S(NT1) + "][" + S(KS1) + "];");
   cb.line("half8_t vf[" + S(NT2) + "][" + S(KS2) + "];");
@@ -1259,6 +1326,81 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.close();
 
   std::vector<std::string> globals = tables_of(em);
+  if (g3) {
+    const graph::GemmDesc& d3 = *d3p;
+    auto lit = [](double v) {
+      std::ostringstream o;
+      o.precision(9);
+      o << v;
+      std::string t = o.str();
+      if (t.find_first_of(".e") == std::string::npos) t += ".0";
+      return t + "f";
+    };
+    const std::string a2 = d2.alpha == 1.0 ? "" : " * " + lit(d2.alpha);
+    // The context (second GEMM's result, rounded to f16 as the HLO defines it) goes to LDS in left-operand fragment
+    // order: element d of row r16 belongs to step d / 32, lane (d % 32 / 8) * 16 + r16, slot d % 8; a lane holds
+    // d = 16 t + 4 g + r, r < 4.
+    cb.line("_Float16* cx = reinterpret_cast<_Float16*>(smem + " + S(cx_off) + ") + rw * " + S(N2 * 16) + ";");
+    auto write_ctx = [&](const std::string& o) {
+      cb.line("const half4_t ch = {(_Float16)(" + o + "[0]" + a2 + "), (_Float16)(" + o + "[1]" + a2 + "), (_Float16)(" + o + "[2]" + a2 + "), (_Float16)(" + o + "[3]" + a2 + ")};");
+      cb.line("*reinterpret_cast<half4_t*>(cx + (((t >> 1) * 64 + ((t & 1) * 2 + (g >> 1)) * 16 + r16) * 8 + (g & 1) * 4)) = ch;");
+    };
+    if (KW > 1) {
+      cb.line("float4_t* ob = reinterpret_cast<float4_t*>(smem + " + S(o_off) + ") + rw * " + S(KW * NT2 * 64) + ";");
+      cb.line("#pragma unroll");
+      cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+      cb.line("if (t % " + S(KW) + " != kw) ob[(kw * " + S(NT2) + " + t) * 64 + lane] = oacc[t];");
+      cb.close();
+      cb.line("__syncthreads();");
+      cb.line("#pragma unroll");
+      cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+      cb.line("if (t % " + S(KW) + " != kw) continue;");
+      cb.line("float4_t o = oacc[t];");
+      cb.line("#pragma unroll");
+      cb.line("for (int w = 0; w < " + S(KW) + "; ++w) if (w != kw) o += ob[(w * " + S(NT2) + " + t) * 64 + lane];");
+      write_ctx("o");
+      cb.close();
+    } else {
+      cb.line("#pragma unroll");
+      cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
+      write_ctx("oacc[t]");
+      cb.close();
+    }
+    cb.line("__syncthreads();");
+    cb.line("half8_t af[" + S(KS3) + "];");
+    cb.line("#pragma unroll");
+    cb.line("for (int s = 0; s < " + S(KS3) + "; ++s) af[s] = *reinterpret_cast<const half8_t*>(cx + (s * 64 + lane) * 8);");
+    // one fp32 partial sum per head: [heads][M3][N3]; the consuming row program adds them up
+    cb.line("float* prow = " + po + " + ((long)head * " + S(d3.M) + " + (bidx / " + S(heads) + ") * " + S(M1) + " + m) * " + S(d3.N) + " + g * 4;");
+    cb.line("#pragma unroll");
+    cb.open("for (int jj = 0; jj < " + S(NJ) + "; ++jj)");
+    cb.line("float4_t pacc = {0.f, 0.f, 0.f, 0.f};");
+    cb.line("#pragma unroll");
+    cb.line("for (int s = 0; s < " + S(KS3) + "; ++s) pacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pre_w.v[jj * " + S(KS3) + " + s], af[s], pacc, 0, 0, 0);");
+    cb.line("const int nt = jj * " + S(KW) + " + kw;");
+    cb.open("if (m_valid && nt < " + S(NT3) + ")");
+    const std::string a3 = d3.alpha == 1.0 ? "" : " * " + lit(d3.alpha);
+    cb.line("const float pv4[4] = {pacc[0]" + a3 + ", pacc[1]" + a3 + ", pacc[2]" + a3 + ", pacc[3]" + a3 + "};");
+    cb.line("mononn_dev::stN<float, 4>(prow + nt * 16, pv4);");
+    cb.close();
+    cb.close();
+    cb.line("__syncthreads();   // LDS is reused by the next unit");
+    NodeFunction f = finish(cb.text(), ptrs, globals, d1.batch * blocks, smem, "typedef mononn_dev::PreB<" + S(NJ * KS3) + "> @NAME@_preb;\n");
+    if (preload_w) {
+      const std::string tail = ", char* smem) {";
+      size_t at = f.text.find(tail);
+      MONONN_CHECK(at != std::string::npos, kInternal) << "node function signature not found";
+      f.text.replace(at, tail.size(), ", char* smem, const @NAME@_preb& pre_w) {");
+      std::string sig = signature(ptrs.entries);
+      sig = sig.substr(0, sig.rfind(", char* smem"));
+      CodeBuffer pf;
+      pf.line("const int lane = mononn_dev::lane_id();");
+      pf.line("const int kw = mononn_dev::wave_id() % " + S(KW) + ";");
+      pf.line("const int head = (unit / " + S(blocks) + ") % " + S(heads) + ";");
+      f.preload_text = "__device__ __forceinline__ void @NAME@_pre(" + sig + ", @NAME@_preb& pre_w) {\n" + pf.text() + preload_body + "}\n";
+    }
+    return f;
+  }
   Epilogue epi = build_epilogue(prog, g2, epi_members, outputs, d2, true, ptrs, first_epi);
   for (auto& gl : epi.globals) globals.push_back(gl);
   cb.line(epi.init_line);
@@ -1303,10 +1445,27 @@ NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchSh
   return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores);
 }
 
-NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves) {
+NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves, bool preload_weights) {
   std::vector<const Instr*> row(node.members.begin() + 1, node.members.begin() + node.gemm2_index);
+  if (node.gemm3_index != 0) {
+    std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.begin() + node.gemm3_index);
+    return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls, key_waves,
+                         node.members[node.gemm3_index], &node.gemm3, node.heads, preload_weights);
+  }
   std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.end());
   return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls, key_waves);
+}
+
+bool can_fuse_out_proj(const Program& prog, const Instr* gemm2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epilogue_members,
+                       const Instr* gemm3, const graph::GemmDesc& d3, int heads) {
+  try {
+    check_out_proj_mapping(prog, gemm2, d2, epilogue_members, gemm3, d3, heads);
+    return !d2.has_addend && !d3.has_addend;
+  } catch (const Error& e) {
+    if (getenv("MONONN_DEBUG_PASSES")) fprintf(stderr, "[attention out-projection fusion rejected] %s\n", e.what());
+    if (e.code() == kUnsupported) return false;
+    throw;
+  }
 }
 
 int default_attention_key_waves(const graph::GemmDesc& d1, const LaunchShape& ls) {

@@ -58,7 +58,13 @@ NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, 
 
 // key_waves: waves of a workgroup that share one block of 16 query rows by splitting the keys between them
 // (0 = as many as the key count allows); the remaining factor of the workgroup's waves takes further row blocks
-NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls, int key_waves = 0);
+// preload_weights: an absorbed output projection takes its weight fragments from a companion function
+// (NodeFunction::preload_text), as generate_gemm does under GemmTuning::preload_b
+NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls, int key_waves = 0,
+                                bool preload_weights = false);
+// the GEMM `gemm3` reads nothing but the heads that the attention's second GEMM produces, merged by pure data movement
+bool can_fuse_out_proj(const graph::Program& prog, const hlo::Instr* gemm2, const graph::GemmDesc& d2,
+                       const std::vector<const hlo::Instr*>& epilogue_members, const hlo::Instr* gemm3, const graph::GemmDesc& d3, int heads);
 int default_attention_key_waves(const graph::GemmDesc& first_gemm, const LaunchShape& ls);
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus);

@@ -27,6 +27,7 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.fuse_attention = s.hip.fuse_attention;
   o.fuse_gemm_prologue = s.hip.gemm_prologue_fusion;
   o.pack_left_operands = s.hip.pack_left_operands;
+  o.fuse_attention_out_proj = s.hip.attention_out_proj_fusion;
   o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
   for (auto& kv : s.gemm_spec_list)
     if (kv.second.split_k > 1) o.gemm_split_k[kv.first] = kv.second.split_k;
@@ -151,7 +152,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         if (bc != n.members[0]->attrs.end()) g.backend_config = Json::parse(bc->second);
         it = spec.gemm_spec_list.emplace(n.name, g).first;
       }
-      f = generate_attention(prog, n, ls, it->second.wave_k);
+      f = generate_attention(prog, n, ls, it->second.wave_k, spec.hip.operand_preload);
     } else if (n.kind == NodeKind::kGemm) {
       auto it = spec.gemm_spec_list.find(n.name);
       GemmTuning t;

@@ -53,6 +53,8 @@ struct Builder {
   const BuildOptions& opt;
   std::vector<Node> nodes;
   std::map<const Instr*, int> node_of_member;   // entry instr -> index in nodes (alive)
+  std::set<std::string> absorb;                 // GEMMs (canonical names) an attention node is going to take in
+  std::set<std::string> absorbed;               // ... and those it did take in
 
   bool enabled(const char* pass) const { return !opt.disabled_passes.count(pass); }
 
@@ -237,6 +239,7 @@ struct Builder {
         Node& g = nodes[gi];
         if (g.members.empty() || g.kind != NodeKind::kGemm) continue;
         if (opt.gemm_split_k.count(g.members[0]->name) && opt.gemm_split_k.at(g.members[0]->name) > 1) continue;   // epilogue moves to the consumer
+        if (absorb.count(g.members[0]->name)) continue;   // likewise
         for (int ci : succ[gi]) {
           Node& c = nodes[ci];
           if (c.members.empty() || c.kind != NodeKind::kCluster) continue;
@@ -287,7 +290,7 @@ struct Builder {
       bool reads_split = false;
       for (auto* in : external_inputs(r.members)) {
         auto sk = opt.gemm_split_k.find(in->name);
-        reads_split = reads_split || (sk != opt.gemm_split_k.end() && sk->second > 1);
+        reads_split = reads_split || (sk != opt.gemm_split_k.end() && sk->second > 1) || absorbed.count(in->name);
       }
       if (reads_split) continue;
       const Instr* h = outs[0];
@@ -386,6 +389,59 @@ struct Builder {
         nodes[g2i].members.clear();
         changed = true;
       }
+    }
+  }
+
+
+  // GEMMs that directly consume the single output of an attention node with a constant right operand
+  std::vector<std::pair<int, int>> out_proj_candidates() const {
+    std::vector<std::pair<int, int>> out;
+    auto succ = successors();
+    for (size_t ai = 0; ai < nodes.size(); ++ai) {
+      const Node& a = nodes[ai];
+      if (a.members.empty() || a.kind != NodeKind::kAttention || a.gemm3_index != 0) continue;
+      auto outs = codegen::external_outputs(p, a.members);
+      if (outs.size() != 1 || succ[ai].size() != 1) continue;
+      const Node& g = nodes[succ[ai][0]];
+      if (g.kind != NodeKind::kGemm || !g.prologue.empty() || g.gemm.is_conv) continue;
+      const Instr* gi = g.members[0];
+      if (!gi->is_gemm() || gi->operands.size() != 2 || p.storage_root(gi->operands[0]) != outs[0]) continue;
+      const Instr* w = gi->operands[1];
+      if (w->opcode != "constant" || w->shape.rank() != 2 || w->users.size() != 1) continue;
+      out.emplace_back(static_cast<int>(ai), succ[ai][0]);
+    }
+    return out;
+  }
+
+  void fuse_attention_out_proj() {
+    for (auto& pr : out_proj_candidates()) {
+      Node& a = nodes[pr.first];
+      Node& g = nodes[pr.second];
+      const Instr* gi = g.members[0];
+      if (!absorb.count(gi->name) || g.members.size() != 1) continue;
+      const GemmDesc& d3 = g.gemm;
+      const GemmDesc& d2 = a.gemm2;
+      if (d3.batch != 1 || !d3.a_k_contig || d3.b_k_contig || d3.has_addend || d3.K % d2.N != 0 || d2.N % 32 != 0 || d3.N % 16 != 0) continue;
+      const int64_t heads = d3.K / d2.N;
+      if (heads < 1 || d2.batch % heads != 0 || d3.M != d2.batch / heads * d2.M) continue;
+      if (gi->operands[1]->shape.dims[0] % 32 != 0 || !opt.transpose_constant_b || !enabled("ConstantLayoutPass")) continue;
+      // every reader of the projection must go through the element emitter (it adds up the per-head partial sums)
+      bool ok = true;
+      for (auto* u : gi->users)
+        if (u->is_gemm() || u->opcode == "tuple" || is_alias_op(u)) ok = false;
+      if (p.module->entry->root == gi) ok = false;
+      if (!ok) continue;
+      std::vector<const Instr*> epi(a.members.begin() + a.gemm2_index + 1, a.members.end());
+      if (!codegen::can_fuse_out_proj(p, a.members[a.gemm2_index], d2, epi, gi, d3, static_cast<int>(heads))) continue;
+      a.gemm3 = d3;
+      a.gemm3.split_k = static_cast<int>(heads);
+      a.gemm3_index = a.members.size();
+      a.heads = static_cast<int>(heads);
+      a.members.push_back(gi);
+      a.name += "_" + g.name;
+      node_of_member[gi] = pr.first;
+      g.members.clear();
+      absorbed.insert(gi->name);
     }
   }
 
@@ -500,6 +556,13 @@ struct Builder {
       if (all) ok[c] = true;
     }
     for (auto& n : p.nodes) {
+      if (n.kind == NodeKind::kAttention && n.gemm3_index != 0) {
+        const Instr* b = n.members[n.gemm3_index]->operands[1];
+        MONONN_CHECK(ok.count(b), kInternal) << "weights of the absorbed projection " << n.members[n.gemm3_index]->hlo_name << " cannot be packed";
+        n.gemm3.b_packed = true;
+        p.constant_transform[b] = ConstantTransform::kPackMfmaB;
+        continue;
+      }
       if (n.kind != NodeKind::kGemm) continue;
       const Instr* b = n.members[0]->operands[1];
       if (ok.count(b)) {
@@ -594,6 +657,9 @@ struct Builder {
   }
 
   void apply_split_k() {
+    // a projection absorbed by an attention node leaves it as one partial sum per head
+    for (auto& n : p.nodes)
+      if (n.kind == NodeKind::kAttention && n.gemm3_index != 0) p.split_k[n.members[n.gemm3_index]] = n.heads;
     for (auto& kv : opt.gemm_split_k) {
       if (kv.second <= 1) continue;
       Node* node = nullptr;
@@ -700,13 +766,34 @@ struct Builder {
 std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, const BuildOptions& opt) {
   auto prog = std::make_unique<Program>();
   prog->module = std::move(module);
-  Builder b{*prog, opt, {}, {}};
-  b.make_nodes();
-  // epilogues first: a bias + residual fusion behind a GEMM belongs to that GEMM, not to the LayerNorm
-  // row program that follows it
-  if (opt.fuse_gemm_epilogue && b.enabled("GemmEpilogueFusionPass")) b.fuse_gemm_epilogues();
-  if (opt.merge_dependent && b.enabled("MergeDependentPass")) b.merge_dependent();
-  if (opt.fuse_attention && b.enabled("AttentionFusionPass")) b.fuse_attention();
+  auto run_fusions = [&](Builder& b) {
+    b.make_nodes();
+    // epilogues first: a bias + residual fusion behind a GEMM belongs to that GEMM, not to the LayerNorm
+    // row program that follows it
+    if (opt.fuse_gemm_epilogue && b.enabled("GemmEpilogueFusionPass")) b.fuse_gemm_epilogues();
+    if (opt.merge_dependent && b.enabled("MergeDependentPass")) b.merge_dependent();
+    if (opt.fuse_attention && b.enabled("AttentionFusionPass")) b.fuse_attention();
+  };
+  // An output projection that an attention node can absorb must keep its epilogue out of the GEMM (it moves
+  // into the consuming row program), which has to be known before the epilogue pass runs: a first trial run
+  // of the fusion passes finds the candidates, a second one proves them, the third is the real one.
+  std::set<std::string> take;
+  const bool want_out_proj = opt.fuse_attention_out_proj && opt.fuse_attention && Builder{*prog, opt, {}, {}, {}, {}}.enabled("AttentionOutProjFusionPass");
+  if (want_out_proj) {
+    Builder probe{*prog, opt, {}, {}, {}, {}};
+    run_fusions(probe);
+    std::set<std::string> cand;
+    for (auto& pr : probe.out_proj_candidates()) cand.insert(probe.nodes[pr.second].members[0]->name);
+    if (!cand.empty()) {
+      Builder trial{*prog, opt, {}, {}, cand, {}};
+      run_fusions(trial);
+      trial.fuse_attention_out_proj();
+      take = trial.absorbed;
+    }
+  }
+  Builder b{*prog, opt, {}, {}, take, {}};
+  run_fusions(b);
+  if (!take.empty()) b.fuse_attention_out_proj();
   if (opt.fuse_gemm_prologue && b.enabled("GemmPrologueFusionPass")) b.fuse_gemm_prologues();
   b.finalize();
   b.decide_constant_layouts();

@@ -72,6 +72,11 @@ struct Node {
   // kAttention: second GEMM and where it sits in `members`
   GemmDesc gemm2;
   size_t gemm2_index = 0;
+  // kAttention with the output projection absorbed: a third GEMM (constant weights) applied per batch element
+  // (head) to that head's slice of the context; its result leaves the node as one fp32 partial sum per head
+  GemmDesc gemm3;
+  size_t gemm3_index = 0;   // 0 = none
+  int heads = 0;            // batch elements of the attention GEMMs per row of the projected matrix
   const hlo::Instr* gemm_instr() const { return kind == NodeKind::kGemm ? members[0] : nullptr; }
 };
 
@@ -133,6 +138,9 @@ struct BuildOptions {
   bool fuse_attention = true;           // GEMM -> soft-max style row program -> GEMM in one stage
   bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
   bool pack_left_operands = true;       // store in-kernel left-hand GEMM operands in MFMA fragment order
+  // the GEMM that consumes the merged heads of an attention node runs inside that node, head by head; its
+  // bias / residual epilogue moves into the consuming row program together with the sum over the heads
+  bool fuse_attention_out_proj = false;
   std::map<std::string, int> gemm_split_k;   // GEMM instruction (canonical name) -> k split over workgroups
   bool reuse_temp_slots = true;         // false: every temp value gets its own address (written once per launch)
   std::set<std::string> disabled_passes;   // MONONN_OPTIMIZATION_DISABLED_PASS (config.cc:82-86)

@@ -92,6 +92,9 @@ struct HipOptions {       // "mononn_hip" section
   bool operand_preload = true;
   // values of this kernel that only GEMMs read as their left operand are stored in MFMA fragment order
   bool pack_left_operands = true;
+  // the projection of the merged heads runs inside the attention stage, one fp32 partial sum per head; the stage
+  // of the projection disappears, its bias / residual epilogue moves into the row program that follows
+  bool attention_out_proj_fusion = false;
 };
 
 struct GraphSpecification {

@@ -151,6 +151,10 @@ def test_fusion_variants_agree(gpu_device):
         "the same with split-K": _spec_with(fx.hlo_text, hip={"operand_preload": False}, gemm_overrides=split),
         # a grid of 8 workgroups: several units per workgroup and stage, only the first of them behind a barrier wait
         "small grid": _spec_with(fx.hlo_text, grid=8),
+        # the projection of the merged heads inside the attention stage: one stage less per layer, the LayerNorm
+        # stage adds one fp32 partial sum per head
+        "output projection inside the attention stage": _spec_with(fx.hlo_text, hip={"attention_out_proj_fusion": True}),
+        "the same, weights requested inside the stage": _spec_with(fx.hlo_text, hip={"attention_out_proj_fusion": True, "operand_preload": False}),
     }
     for name, spec in variants.items():
         (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, spec)
@@ -158,6 +162,8 @@ def test_fusion_variants_agree(gpu_device):
         diff = np.abs(got.astype(np.float32) - base.astype(np.float32)).max()
         print(f"{name}: barriers={m.launch_dims()['barriers']} max_abs_err={err:.2e} vs default {diff:.2e}")
         assert diff <= 8e-3, name
+        if name.startswith("output projection inside"):
+            assert m.launch_dims()["barriers"] == m0.launch_dims()["barriers"] - 2, "one stage less per layer"
     (fenced,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants["fenced barrier, reused temp slots"])
     assert np.array_equal(fenced.view(np.uint16), base.view(np.uint16)), "barrier flavour must not change any bit"
     (coop,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants["cooperative launch"])
