@@ -124,17 +124,19 @@ std::vector<std::string> tables_of(const Emitter& em) {
 // needed after a workgroup reduction would be issued after that reduction's barrier, putting one more trip
 // to memory on the critical path.  Such loads are moved up to the head of the program: definitions of the
 // form `const T vN = <expression of inK[..], row, qK>;` go right behind the last `const int qK = ...;`.
-std::string hoist_row_loads(const std::string& text) {
+std::string hoist_row_loads(const std::string& text, bool prologue = false) {
   std::vector<std::string> lines;
   {
     std::istringstream is(text);
     std::string l;
     while (std::getline(is, l)) lines.push_back(l);
   }
-  static const std::regex q_def(R"(^\s*const int q\d+ = .*;$)");
+  static const std::regex q_def_row(R"(^\s*const int q\d+ = .*;$)");
+  static const std::regex q_def_pro(R"(^\s*const int m\d+ = .*;$)");   // a GEMM prologue: rows m0, m1, .. come last
+  const std::regex& q_def = prologue ? q_def_pro : q_def_row;
   static const std::regex v_def(R"(^\s*const [A-Za-z_][\w ]* v\d+ = (.*);$)");
   static const std::regex ident(R"((^|[^\w.])([A-Za-z_]\w*))");
-  static const std::regex allowed(R"(^(in\d+|q\d+|row|lane|tid|float|double|_Float16|int|long|unsigned|short|char|bool|int8_t|uint8_t|int16_t|uint16_t|int32_t|uint32_t|int64_t|uint64_t)$)");
+  static const std::regex allowed(R"(^(in\d+|q\d+|m\d+|wk|g|r16|row|lane|tid|float|double|_Float16|int|long|unsigned|short|char|bool|int8_t|uint8_t|int16_t|uint16_t|int32_t|uint32_t|int64_t|uint64_t)$)");
   int anchor = -1;
   for (size_t i = 0; i < lines.size(); ++i)
     if (std::regex_match(lines[i], q_def)) anchor = static_cast<int>(i);
@@ -146,6 +148,9 @@ std::string hoist_row_loads(const std::string& text) {
     if (std::regex_match(lines[i], m, v_def)) {
       const std::string rhs = m[1].str();
       hoist = rhs.find('[') != std::string::npos;
+      // in front of a GEMM registers are scarce (operand fragments are resident): only the partial sums of a split
+      // GEMM, which come from another XCD's stores, are requested ahead; constants of the row program hit nearby caches
+      if (prologue && lines[i].find("const float v") == std::string::npos) hoist = false;
       for (auto it = std::sregex_iterator(rhs.begin(), rhs.end(), ident); hoist && it != std::sregex_iterator(); ++it)
         hoist = std::regex_match((*it)[2].str(), allowed);
     }
@@ -156,7 +161,7 @@ std::string hoist_row_loads(const std::string& text) {
   for (auto& l : hoisted) out += l + "\n";
   // keeps the instruction scheduler from sinking a load to its first use (it would then wait for each
   // load in turn instead of having all of them in flight)
-  if (!hoisted.empty()) out += "    __builtin_amdgcn_sched_barrier(0);\n";
+  if (!hoisted.empty()) out += std::string(prologue ? "" : "  ") + "  __builtin_amdgcn_sched_barrier(0);\n";
   for (auto& l : rest) out += l + "\n";
   return out;
 }
@@ -454,7 +459,9 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
   if (has_prologue) {
     const int tm = t.bm / std::max(t.wm, 1) / 16, tn = t.bn / std::max(t.wn, 1) / 16;
     const int64_t ksteps = g.K / 32;
-    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && ksteps / t.wk <= 32 / (tm + tn), kSpecError)
+    // mirrors mononn_dev::gemm_chunk_steps: with the weights requested ahead of the tile a wave keeps up to 56 fragments
+    const bool wide = t.preload_b && g.b_packed && t.wk >= 1 && ksteps / t.wk * (tm + tn) <= 56;
+    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && (wide || ksteps / t.wk <= 32 / (tm + tn)), kSpecError)
         << "GEMM with a row-program prologue: a wave's whole k range (" << ksteps / std::max(t.wk, 1) << " steps) must fit one register chunk";
   }
   MONONN_CHECK(t.split_k >= 1 && g.K % (32 * t.split_k) == 0, kSpecError) << "split_k " << t.split_k << " does not divide the k steps of the GEMM";
@@ -497,12 +504,24 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     std::string a = al.str();
     if (a.find_first_of(".e") == std::string::npos) a += ".0";
     Epilogue e;
+    // where element (bidx, m, n0) of one partial sum lives: row-major, or in fragment order when the consumer
+    // takes the rows as MFMA fragments (a row program fused in front of the next GEMM)
+    std::string where = "(long)bidx * " + S(g.M * g.N) + " + m * " + S(g.N) + " + n0";
+    if (prog.physical_tile.count(gi)) {
+      VarTable tv;
+      int vbi = tv.add("bidx", g.batch), vmi = tv.add("m", g.M), vni = tv.add("n4", g.N / 4);
+      Index gidx = delinearize(LinExpr::variable(vbi, g.batch), std::vector<int64_t>(gi->shape.dims.begin(), gi->shape.dims.end() - 2), tv);
+      gidx.push_back(LinExpr::variable(vmi, g.M));
+      gidx.push_back(LinExpr::variable(vni, g.N / 4).scaled(4));
+      where = physical_offset(prog, gi, gidx, &tv).str(tv);
+    }
     e.struct_text = "struct @NAME@_epi {\n  float* out;\n  int ksplit;\n"
                     "  struct Pre {};\n"
                     "  __device__ __forceinline__ void preload(int, int, int, Pre&) const {}\n"
                     "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4], const Pre&) const {\n"
+                    "    const int n4 = n0 >> 2;\n    (void)n4;\n"
                     "    const float v[4] = {acc[0] * " + a + "f, acc[1] * " + a + "f, acc[2] * " + a + "f, acc[3] * " + a + "f};\n"
-                    "    mononn_dev::stN<float, 4>(out + (long)ksplit * " + S(g.batch * g.M * g.N) + " + (long)bidx * " + S(g.M * g.N) + " + m * " + S(g.N) + " + n0, v);\n"
+                    "    mononn_dev::stN<float, 4>(out + (long)ksplit * " + S(g.batch * g.M * g.N) + " + " + where + ", v);\n"
                     "  }\n};\n";
     e.init_line = "@NAME@_epi epi{" + po + ", ksplit};";
     return e;
@@ -753,6 +772,24 @@ struct Prologue {
   const Instr* primary = nullptr;   // the [M,K] input whose rows arrive as MFMA fragments
 };
 
+}  // namespace
+
+// primary input of a row program fused in front of a GEMM: an [M,K] f16 value that the cluster reads from outside
+// and that is stored as such (not as the partial sums of a split GEMM); its rows arrive as MFMA fragments
+const Instr* prologue_primary(const Program& prog, const std::vector<const Instr*>& row_members, int64_t M, int64_t K) {
+  std::set<const Instr*> mem(row_members.begin(), row_members.end());
+  for (auto* m : row_members)
+    for (auto* o : m->operands) {
+      const Instr* r = prog.storage_root(o);
+      if (mem.count(r) || (r->opcode == "get-tuple-element" && mem.count(r->operands[0]))) continue;
+      if (prog.split_k.count(r)) continue;
+      if (r->shape.dtype == DType::kF16 && r->shape.dims == std::vector<int64_t>({M, K})) return r;
+    }
+  return nullptr;
+}
+
+namespace {
+
 Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& row_members, const Instr* gi, const graph::GemmDesc& g,
                         const GemmTuning& t, const LaunchShape& ls, bool stores, PointerTable& ptrs) {
   (void)ls;
@@ -765,18 +802,8 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
                kUnsupported)
       << "GEMM prologue: the row program must produce exactly the f16 [M,K] left operand";
   const Instr* H = outs[0];
-  const int TM = t.bm / t.wm / 16, WK = t.wk, CH = static_cast<int>(g.K / 32 / WK);
-  // primary input: a [M,K] f16 value read by the cluster from outside
-  const Instr* primary = nullptr;
-  {
-    std::set<const Instr*> mem(row_members.begin(), row_members.end());
-    for (auto* m : row_members)
-      for (auto* o : m->operands) {
-        const Instr* r = prog.storage_root(o);
-        if (mem.count(r) || (r->opcode == "get-tuple-element" && mem.count(r->operands[0]))) continue;
-        if (!primary && r->shape.dtype == DType::kF16 && r->shape.dims == std::vector<int64_t>({g.M, g.K})) primary = r;
-      }
-  }
+  const int TM = t.bm / t.wm / 16, WK = t.wk, CH = static_cast<int>(g.K / 32 / WK);   // the wave's whole k range (one chunk)
+  const Instr* primary = prologue_primary(prog, row_members, g.M, g.K);
   MONONN_CHECK(primary != nullptr, kUnsupported) << "GEMM prologue: no [M,K] f16 input to take the place of the left operand";
   Prologue out;
   out.primary = primary;
@@ -887,7 +914,8 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
   }
   st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, char* smem) const {\n";
   {
-    std::istringstream is(cb.text());
+    // every operand of the row program is requested before the first of them is used: one trip to memory
+    std::istringstream is(hoist_row_loads(cb.text(), true));
     std::string l;
     while (std::getline(is, l)) st += "  " + l + "\n";
   }
@@ -999,8 +1027,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     } else {
       std::ostringstream b_expr;
       b_expr << pb << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS);
-      preload = t.preload_b && g.b_packed && !has_pro;   // a row-program prologue fixes the chunking of the left operand
-      MONONN_CHECK(!g.a_packed || !has_pro, kInternal) << gi->hlo_name << ": fragment-order left operand under a prologue";
+      preload = t.preload_b && g.b_packed;
       call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
            << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
            << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "

@@ -62,6 +62,8 @@ NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, 
 // (NodeFunction::preload_text), as generate_gemm does under GemmTuning::preload_b
 NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls, int key_waves = 0,
                                 bool preload_weights = false);
+// the input of a row program fused in front of a GEMM whose rows the GEMM loads as its left-operand fragments
+const hlo::Instr* prologue_primary(const graph::Program& prog, const std::vector<const hlo::Instr*>& row_members, int64_t M, int64_t K);
 // the GEMM `gemm3` reads nothing but the heads that the attention's second GEMM produces, merged by pure data movement
 bool can_fuse_out_proj(const graph::Program& prog, const hlo::Instr* gemm2, const graph::GemmDesc& d2,
                        const std::vector<const hlo::Instr*>& epilogue_members, const hlo::Instr* gemm3, const graph::GemmDesc& d3, int heads);

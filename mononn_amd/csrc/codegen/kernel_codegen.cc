@@ -299,21 +299,33 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     const Call* call;
     int first_unit, stage_total;
     bool new_stage;
+    int rot;   // unit u of the stage runs on workgroup (u + rot) % grid
   };
   std::vector<Flat> flat;
+  // A workgroup that had a unit in the previous stage reaches the barrier later than an idle one and has asked for
+  // its constant operands later: when the units of two consecutive stages fit side by side, the second stage is
+  // placed on the workgroups the first one left idle.  Offsets are multiples of 8 so that a unit keeps its XCD.
+  int64_t prev_total = 0, prev_rot = 0;
+  bool any_rot = false;
   for (auto& st : by_stage) {
     int64_t total = 0;
     for (auto& c : st.second) total += c.units;
     MONONN_CHECK(total < (int64_t(1) << 31), kResourceExhausted) << "stage has too many work units";
+    int64_t rot = 0;
+    if (spec.hip.stage_rotation && hp.grid % 8 == 0 && prev_total > 0 && total + (prev_total + 7) / 8 * 8 <= hp.grid)
+      rot = (prev_rot + (prev_total + 7) / 8 * 8) % hp.grid;
+    any_rot = any_rot || rot != 0;
     hp.stage_nodes.emplace_back();
     int64_t first = 0;
     bool ns = true;
     for (auto& c : st.second) {
       hp.stage_nodes.back().push_back(c.node->name);
-      flat.push_back({&c, static_cast<int>(first), static_cast<int>(total), ns});
+      flat.push_back({&c, static_cast<int>(first), static_cast<int>(total), ns, static_cast<int>(rot)});
       ns = false;
       first += c.units;
     }
+    prev_total = total;
+    prev_rot = rot;
   }
   hp.num_barriers = by_stage.empty() ? 0 : static_cast<int>(by_stage.size()) - 1;
   auto base_expr = [&](const Operand& o) -> std::string {
@@ -340,7 +352,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     src << "  bool pending = false;   // announced the end of the previous stage, not yet waited for the others\n";
   }
   src << "  for (int c = 0; c < " << flat.size() << "; ++c) {\n";
-  src << "    int fn = 0, units = 0, first = 0, total = 0;\n    bool new_stage = false;\n";
+  src << "    int fn = 0, units = 0, first = 0, total = 0" << (any_rot ? ", rot = 0" : "") << ";\n    bool new_stage = false;\n";
   src << "    char*";
   for (size_t i = 0; i < max_ptrs; ++i) src << (i ? ", *" : " ") << "p" << i << " = nullptr";
   src << ";\n";
@@ -349,6 +361,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     const Flat& f = flat[i];
     src << "      case " << i << ": fn = " << f.call->fn_id << "; units = " << f.call->units << "; first = " << f.first_unit << "; total = "
         << f.stage_total << "; new_stage = " << (f.new_stage ? "true" : "false") << ";";
+    if (f.rot) src << " rot = " << f.rot << ";";
     for (size_t a = 0; a < f.call->args.size(); ++a) src << " p" << a << " = " << base_expr(f.call->args[a]) << ";";
     src << " break;   // " << f.call->node->name.substr(0, 50) << "\n";
   }
@@ -376,7 +389,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     if (hp.profiled) src << "      if (stage == 0 && threadIdx.x == 0) " << clk << "] = wall_clock64();\n";
   }
   src << "    }\n";
-  src << "    for (int u = blockIdx.x; u < total; u += gridDim.x) {\n";
+  if (any_rot) src << "    for (int u = blockIdx.x >= rot ? blockIdx.x - rot : blockIdx.x + gridDim.x - rot; u < total; u += gridDim.x) {\n";
+  else src << "    for (int u = blockIdx.x; u < total; u += gridDim.x) {\n";
   src << "      const int unit = u - first;\n";
   src << "      if (unit < 0 || unit >= units) continue;\n";
   // One dispatch switch; in the lazy form every case first requests what it can, then waits if a barrier is pending

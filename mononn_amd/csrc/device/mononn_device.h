@@ -351,7 +351,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   constexpr int CH = gemm_chunk_steps(TM, TN, MY_STEPS, PRE_B);
   constexpr int NCHUNK = (MY_STEPS + CH - 1) / CH;
   static_assert(!PRE_B || PACKED_B, "only packed weights can be requested ahead of the tile");
-  static_assert(!PACKED_A || (AMap::kRowMajor && !Pro::enabled), "a fragment-order left operand takes neither a row map nor a prologue");
+  static_assert(!PACKED_A || AMap::kRowMajor, "a fragment-order left operand takes no row map");
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
   static_assert(K % 32 == 0, "K must be a multiple of 32");
   const int lane = lane_id();

@@ -290,7 +290,8 @@ struct Builder {
       bool reads_split = false;
       for (auto* in : external_inputs(r.members)) {
         auto sk = opt.gemm_split_k.find(in->name);
-        reads_split = reads_split || (sk != opt.gemm_split_k.end() && sk->second > 1) || absorbed.count(in->name);
+        (void)sk;   // partial sums of a split GEMM reach the row program through the element emitter, fused or not
+        reads_split = reads_split || absorbed.count(in->name);
       }
       if (reads_split) continue;
       const Instr* h = outs[0];
@@ -640,14 +641,32 @@ struct Builder {
       const GemmDesc& d = n.gemm;
       spoiled.insert(p.storage_root(g->operands[1]));
       const bool mfma = d.a_k_contig && (d.b_k_contig || d.b_packed) && d.K % 32 == 0;
-      use(g->operands[0], mfma && !d.is_conv && n.prologue.empty() && d.batch == 1, d.M, d.K, Order::kRunsOf8, false);
+      if (!n.prologue.empty()) {
+        // the tile loads the rows of the row program's primary input in place of the left operand
+        const Instr* primary = codegen::prologue_primary(p, n.prologue, d.M, d.K);
+        if (primary) use(primary, mfma && d.batch == 1, d.M, d.K, Order::kRunsOf8, false);
+        continue;
+      }
+      use(g->operands[0], mfma && !d.is_conv && d.batch == 1, d.M, d.K, Order::kRunsOf8, false);
+    }
+    // Partial sums of a split GEMM that a fused row program takes row fragment by row fragment: same order, fp32.
+    for (auto& n : p.nodes) {
+      if (n.kind != NodeKind::kGemm || n.prologue.empty()) continue;
+      for (auto* r : n.inputs) {
+        auto sk = p.split_k.find(r);
+        if (sk == p.split_k.end() || p.physical_tile.count(r) || r->shape.rank() != 2) continue;
+        const int64_t M = r->shape.dims[0], N = r->shape.dims[1];
+        if (M == n.gemm.M && N == n.gemm.K && M % 16 == 0 && N % 32 == 0) p.physical_tile[r] = {N, Order::kRunsOf8};
+      }
     }
     for (auto& kv : want)
       if (!spoiled.count(kv.first)) p.physical_tile[kv.first] = {kv.second.k, kv.second.order};
     auto tiled = [&](const Instr* operand) { return p.physical_tile.count(p.storage_root(operand)) > 0; };
     for (auto& n : p.nodes) {
       if (n.kind == NodeKind::kGemm) {
-        n.gemm.a_packed = tiled(n.members[0]->operands[0]);
+        // with a row program in front, the tile loads that program's primary input in place of the left operand
+        const Instr* a = n.prologue.empty() ? n.members[0]->operands[0] : codegen::prologue_primary(p, n.prologue, n.gemm.M, n.gemm.K);
+        n.gemm.a_packed = a != nullptr && tiled(a);
       } else if (n.kind == NodeKind::kAttention) {
         n.gemm.a_packed = tiled(n.members[0]->operands[0]);
         n.gemm.b_tiled = tiled(n.members[0]->operands[1]);
@@ -676,7 +695,7 @@ struct Builder {
           if (r == g) {
             bool via_emitter = n.kind == NodeKind::kCluster;
             if (n.kind == NodeKind::kGemm) {   // allowed inside an epilogue, not as a matrix operand
-              via_emitter = p.storage_root(n.members[0]->operands[0]) != g && p.storage_root(n.members[0]->operands[1]) != g && n.prologue.empty();
+              via_emitter = p.storage_root(n.members[0]->operands[0]) != g && p.storage_root(n.members[0]->operands[1]) != g;
             }
             MONONN_CHECK(via_emitter, kSpecError) << "split_k: " << kv.first << " is read by " << n.name << " as a matrix operand";
           }
@@ -797,8 +816,8 @@ std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, cons
   if (opt.fuse_gemm_prologue && b.enabled("GemmPrologueFusionPass")) b.fuse_gemm_prologues();
   b.finalize();
   b.decide_constant_layouts();
-  b.assign_operand_layouts();
   b.apply_split_k();
+  b.assign_operand_layouts();
   for (auto& n : prog->nodes)
     if (n.kind == NodeKind::kCluster) codegen::classify_cluster(*prog, n);
   b.assign_buffers();

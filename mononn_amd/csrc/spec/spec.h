@@ -95,6 +95,8 @@ struct HipOptions {       // "mononn_hip" section
   // the projection of the merged heads runs inside the attention stage, one fp32 partial sum per head; the stage
   // of the projection disappears, its bias / residual epilogue moves into the row program that follows
   bool attention_out_proj_fusion = false;
+  // a stage whose units fit beside those of the stage before it runs on the workgroups that stage left idle
+  bool stage_rotation = true;
 };
 
 struct GraphSpecification {

@@ -143,6 +143,7 @@ def test_fusion_variants_agree(gpu_device):
         "no attention fusion": _spec_with(fx.hlo_text, hip={"fuse_attention": False}),
         "no epilogue fusion": _spec_with(fx.hlo_text, hip={"gemm_epilogue_fusion": False}),
         "LayerNorm as GEMM prologue": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}),
+        "LayerNorm as GEMM prologue over split-K partial sums": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}, gemm_overrides=split),
         "plain weight layout": _spec_with(fx.hlo_text, hip={"transpose_constant_b": False, "assign_operand_layouts": False}),
         "split-K": _spec_with(fx.hlo_text, gemm_overrides=split),
         "cooperative launch": _spec_with(fx.hlo_text, hip={"cooperative_launch": True}),
