@@ -114,7 +114,9 @@ int mononn_time_kernel(mononn_module* m, void* const* device_ptrs, size_t n_ptrs
 
 /* Per-stage wall-clock stamps of the last launch, for kernels compiled from a specification with
  * mononn_hip.profile_stages = true: ticks[(stage * grid + workgroup) * 2 + {0: stage begin, 1: work done}].
- * Copies at most `capacity` values; n_stages / grid / ticks_per_us describe the layout.  Stage names
+ * "stage begin" is stamped when the workgroup's first unit of the stage may start (after its barrier wait, behind
+ * which requests for constant operands may already be in flight); a workgroup without a unit in a stage leaves both
+ * values at zero.  Copies at most `capacity` values; n_stages / grid / ticks_per_us describe the layout.  Stage names
  * (node names joined by '+') come from mononn_module_stage_name.
  * Replaces: the per-node report of dump_performance_report (mononn_engine/module/mononn_module_tuner.cc:422-448). */
 int mononn_module_stage_clock(mononn_module* m, uint64_t* ticks, size_t capacity, int* n_stages, int* grid,

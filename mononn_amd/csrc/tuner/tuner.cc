@@ -186,6 +186,23 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     MonoNNModule def(params.hlo_text, base.to_json().dump(0), params.kernel_name);
     def.generate_code();
     GraphSpecification filled = def.tuning_spec();
+    // MONONN_TUNER_SEED_SPEC_DIR: a dump directory of an earlier tuning run of the same module.  Its entries join
+    // the candidates that are tried in the whole kernel, so a new run ends no worse than the one it starts from
+    // (the stage clocks are noisy, and the order in which classes are decided matters).
+    std::unique_ptr<GraphSpecification> seed;
+    {
+      const char* sd = std::getenv("MONONN_TUNER_SEED_SPEC_DIR");
+      if (sd && *sd) {
+        try {
+          std::string text;
+          MONONN_CHECK(module::read_file(def.cluster_dir(sd) + "/best_tuning_spec.json", &text), kInvalidArgument) << "no best_tuning_spec.json";
+          auto sp = std::make_unique<GraphSpecification>(GraphSpecification::from_json(Json::parse(text)));
+          if (sp->context_string() == ctx_str) seed = std::move(sp);
+        } catch (const Error& e) {
+          log << "  seed specification in " << sd << " not usable: " << e.what() << "\n";
+        }
+      }
+    }
     if (bufs.ptrs.empty()) {
       hipError_t e = hipSetDevice(params.device);
       if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipSetDevice: " << hipGetErrorString(e);
@@ -403,6 +420,15 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       for (size_t i : trials_of_class[c.function]) trials[i].mod.reset();
       if (verbose) std::fprintf(stderr, "[mononn tuner] %s %s x%zu: %zu candidates, best %.2f us\n", ctx_str.c_str(), c.kind.c_str(), c.nodes.size(), live.size(), best_class);
       if (best_class < 0) continue;
+      if (seed) {
+        bool all = true;
+        for (auto& n : c.nodes) {
+          if (c.kind == "gemm" || c.kind == "attention") all = all && seed->gemm_spec_list.count(n) && seed->gemm_spec_list.at(n).split_k <= 1;
+          else if (c.kind == "cluster_reduce") all = all && seed->cluster_reduce_spec.count(n);
+          else if (c.kind == "cluster_elewise") all = all && seed->cluster_elewise_spec.count(n);
+        }
+        if (all) runners_up[c.function].push_back({"seed", -1.0, *seed});
+      }
       if (budget <= 1 && c.nodes.size() >= 2) {
         std::vector<size_t> order;
         for (size_t i : live)
@@ -449,10 +475,26 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     // stage follows a different one, part of its operand traffic hides behind the barrier wait, and the
     // ranking of close candidates can change: the runners-up of every class are tried in the whole kernel and
     // the fastest whole kernel wins.
+    // The seed as a whole: its classes were tuned against each other, which a class-by-class comparison cannot see.
+    if (seed) {
+      GraphSpecification whole = filled;
+      whole.gemm_spec_list = seed->gemm_spec_list;
+      whole.cluster_reduce_spec = seed->cluster_reduce_spec;
+      whole.cluster_elewise_spec = seed->cluster_elewise_spec;
+      if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);
+      const double seed_us = whole_kernel_us(whole);
+      log << "  [" << ctx_str << "] whole kernel: " << stitched_us << " us with the best of every class by the stage clocks, " << seed_us
+          << " us with the seed specification; the search goes on from the faster one\n";
+      if (verbose) std::fprintf(stderr, "[mononn tuner] %s whole kernel %.2f us tuned, %.2f us seed\n", ctx_str.c_str(), stitched_us, seed_us);
+      if (seed_us > 0 && (stitched_us < 0 || seed_us < 0.999 * stitched_us)) {
+        stitched = std::move(whole);
+        stitched_us = seed_us;
+      }
+    }
     // A launch context that starts out well behind the best one so far is not worth the whole-kernel builds.
     bool promising = true;
     if (!env::is_true("MONONN_TUNER_NO_REFINEMENT")) {
-      stitched_us = whole_kernel_us(stitched);
+      if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);
       promising = best_us < 0 || (stitched_us > 0 && stitched_us < 1.08 * best_us);
       if (!promising) log << "  [" << ctx_str << "] " << stitched_us << " us before refinement, best context so far " << best_us << " us: not refined\n";
     }
@@ -609,7 +651,22 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           }
           std::vector<std::string> both = allow;
           both.insert(both.end(), consumers.begin(), consumers.end());
-          for (auto& t : gemm_candidates(part, cx.block / 64, std::max(budget, 1))) {
+          std::vector<codegen::GemmTuning> tiles = gemm_candidates(part, cx.block / 64, std::max(budget, 1));
+          size_t seed_tile = tiles.size();
+          if (seed) {
+            auto it = seed->gemm_spec_list.find(instrs[0]);
+            if (it != seed->gemm_spec_list.end() && it->second.split_k == S) {
+              codegen::GemmTuning st;
+              st.bm = it->second.tb_m;
+              st.bn = it->second.tb_n;
+              st.wm = it->second.wave_m;
+              st.wn = it->second.wave_n;
+              st.wk = it->second.wave_k;
+              tiles.push_back(st);
+            }
+          }
+          for (size_t ti = 0; ti < tiles.size(); ++ti) {
+            const codegen::GemmTuning& t = tiles[ti];
             GraphSpecification s = s0;
             for (auto& in : instrs) {
               apply_gemm(s, in, t, part.K);
@@ -624,7 +681,12 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             s.codegen_allow_list = both;
             Trial tr;
             char lbl[112];
-            std::snprintf(lbl, sizeof lbl, "split%d_tile%dx%d_waves%dx%dx%d", S, t.bm, t.bn, t.wm, t.wn, t.wk);
+            std::snprintf(lbl, sizeof lbl, "split%d_%stile%dx%d_waves%dx%dx%d", S, ti == seed_tile ? "seed_" : "", t.bm, t.bn, t.wm, t.wn, t.wk);
+            if (ti == seed_tile)
+              for (auto& n : consumers) {
+                auto it = seed->cluster_reduce_spec.find(n);
+                if (it != seed->cluster_reduce_spec.end()) s.cluster_reduce_spec[n] = it->second;
+              }
             tr.label = lbl;
             tr.spec = std::move(s);
             cand.push_back(std::move(tr));
@@ -681,6 +743,10 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             std::sort(bf.second.begin(), bf.second.end(), [&](size_t a, size_t b) { return trials[a].total_us < trials[b].total_us; });
             for (size_t k = 0; k < bf.second.size() && k < (budget == 0 ? 3u : 1u); ++k) order.push_back(bf.second[k]);
           }
+          for (size_t i : live)
+            if (i != first && trials[i].total_us > 0 && trials[i].label.find("_seed_") != std::string::npos &&
+                std::find(order.begin(), order.end(), i) == order.end())
+              order.push_back(i);
         }
         if (!order.empty()) {
           if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);

@@ -332,8 +332,8 @@ def test_dump_contains_a_standalone_driver_and_the_constants(layer, tmp_path):
         assert os.path.getsize(path) >= c["bytes"]
 
 
-def test_prologue_fusion_leaves_split_k_consumers_alone(layer):
-    # a LayerNorm that adds up split-K partial sums must stay a stage of its own even when LayerNorm-in-GEMM is on
+def test_split_k_consumer_without_a_following_gemm_stays_a_row_program(layer):
+    # the last LayerNorm adds up split-K partial sums and feeds no GEMM: a stage of its own, LayerNorm-in-GEMM or not
     spec = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
     template = next(v for k, v in spec["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))
     gemms = [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", layer.hlo_text)]
@@ -348,3 +348,98 @@ def test_prologue_fusion_leaves_split_k_consumers_alone(layer):
     assert "+row-prologue" in text                      # the first LayerNorm went into FFN1
     assert re.search(rf"gemm\s+{ffn2}\s", text)          # FFN2 is split: bare node, no fused epilogue
     assert re.search(r"rowred\s+\S+\s+members=4", text)  # its consumer: bias + residual + LayerNorm over the partial sums
+
+
+def _hip_spec(hlo_text, **hip):
+    spec = json.loads(MonoNNModule.compile(hlo_text, build=False).get_tuning_spec())
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}, {}
+    spec["mononn_hip"].update(hip)
+    return spec
+
+
+def test_hip_options_have_defaults_and_are_checked(layer):
+    hip = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())["mononn_hip"]
+    assert hip["operand_preload"] is True and hip["pack_left_operands"] is True and hip["stage_rotation"] is True
+    assert hip["attention_out_proj_fusion"] is False and hip["gemm_prologue_fusion"] is False and hip["cooperative_launch"] is False
+    with pytest.raises(MonoNNError) as e:
+        MonoNNModule.compile(layer.hlo_text, json.dumps(_hip_spec(layer.hlo_text, operand_prefetch=True)), build=False)
+    assert e.value.status == "SPEC_ERROR"
+
+
+def test_weights_are_requested_between_arrive_and_wait(layer):
+    src = MonoNNModule.compile(layer.hlo_text, build=False).get_source()
+    # every packed-weight GEMM has a companion that loads the first chunk of its right operand ...
+    pre = set(re.findall(r"void (node_fn_\d+)_pre\(", src))
+    assert pre and all(f"typedef mononn_dev::PreB<" in src for _ in pre)
+    # ... called in the dispatch switch before the pending barrier wait, the function proper after it
+    for fn in pre:
+        case = re.search(rf"case \d+: {{ {fn}_preb pre_b; {fn}_pre\(unit.*?pre_b\); if \(pending\) {{ barrier\.wait\(\); pending = false; }} {fn}\(unit.*?smem, pre_b\); }} break;", src)
+        assert case, fn
+    assert "barrier.arrive();" in src and "barrier.sync()" not in src
+    off = MonoNNModule.compile(layer.hlo_text, json.dumps(_hip_spec(layer.hlo_text, operand_preload=False)), build=False).get_source()
+    assert "_pre(" not in off and "barrier.sync();" in off and "barrier.arrive()" not in off
+
+
+def test_fragment_order_writer_and_reader_agree(layer):
+    """A left GEMM operand produced in the kernel is written by its producer through the index machinery of the
+    code generator and read by the GEMM tile as block (row / 16) * (K / 32) + k / 32, lane (k % 32 / 8) * 16 + row % 16,
+    element k % 8: both must name the same address for every (row, k)."""
+    src = MonoNNModule.compile(layer.hlo_text, build=False).get_source()
+    # the LayerNorm between attention and FFN1 writes [32, 128] f16 rows, 4 or 8 consecutive columns per store
+    stores = re.findall(r"stN<_Float16, (\d)>\(out0 \+ ([^,]*\(row / 16\)[^,]*), pk\d+\)", src)
+    assert stores, "no fragment-order store of a row program found"
+    width, expr = int(stores[0][0]), stores[0][1]
+    K, rows = 128, 32
+    seen = set()
+    for row in range(rows):
+        for q0 in range(K // width):
+            base = eval(expr.replace("/", "//"), {"row": row, "q0": q0})
+            for e in range(width):
+                k = q0 * width + e
+                want = (((row // 16) * (K // 32) + k // 32) * 64 + ((k % 32) // 8) * 16 + row % 16) * 8 + k % 8
+                assert base + e == want, (row, k)
+                seen.add(base + e)
+    assert seen == set(range(rows * K))
+    plain = MonoNNModule.compile(layer.hlo_text, json.dumps(_hip_spec(layer.hlo_text, pack_left_operands=False)), build=False).get_source()
+    assert "(row / 16)" not in plain
+
+
+def test_stage_is_placed_on_idle_workgroups_when_it_fits(layer):
+    # LayerNorm: 32 units; FFN1 with 32x64 tiles: 1 x 4 = 4 units: both fit into the grid side by side
+    spec = _hip_spec(layer.hlo_text)
+    m = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False)
+    src = m.get_source()
+    assert re.search(r"rot = \d+;", src) and "blockIdx.x >= rot ? blockIdx.x - rot : blockIdx.x + gridDim.x - rot" in src
+    rots = [int(r) for r in re.findall(r" rot = (\d+);", src)]
+    assert all(r % 8 == 0 for r in rots), "a unit must keep its XCD"
+    spec["mononn_hip"]["stage_rotation"] = False
+    assert " rot = " not in MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False).get_source()
+
+
+def test_output_projection_inside_the_attention_stage(layer):
+    base = MonoNNModule.compile(layer.hlo_text, build=False)
+    fused = MonoNNModule.compile(layer.hlo_text, json.dumps(_hip_spec(layer.hlo_text, attention_out_proj_fusion=True)))   # hipRTC build
+    assert fused.launch_dims()["barriers"] == base.launch_dims()["barriers"] - 1
+    src = fused.get_source()
+    assert "float* prow" in src and "pre_w.v[" in src
+    # one fp32 partial sum per head, added up by the row program that follows: 4 heads in this fixture
+    assert fused.buffer_info()["temp"] > base.buffer_info()["temp"]
+
+
+def test_layernorm_in_gemm_over_split_k_partial_sums():
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
+    gemms = [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", fx.hlo_text)]
+    spec = _hip_spec(fx.hlo_text)
+    template = next(v for k, v in json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())["gemm_spec_list"].items()
+                    if k.startswith("cublas_gemm_"))
+    for g, s in ((gemms[3], 2), (gemms[5], 4)):
+        entry = json.loads(json.dumps(template))
+        entry["cutlass_config"]["split_k"] = s
+        spec["gemm_spec_list"][g] = entry
+    plain = MonoNNModule.compile(fx.hlo_text, json.dumps(spec), build=False)
+    spec["mononn_hip"]["gemm_prologue_fusion"] = True
+    fused = MonoNNModule.compile(fx.hlo_text, json.dumps(spec))   # hipRTC build
+    assert fused.launch_dims()["barriers"] < plain.launch_dims()["barriers"]
+    src = fused.get_source()
+    # the partial sums of the split GEMMs are stored in fragment order for the row program in front of the next GEMM
+    assert re.search(r"stN<float, 4>\(out \+ \(long\)ksplit \* \d+ \+ \(m % 16\) \* 8", src)
