@@ -429,12 +429,12 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         }
         if (all) runners_up[c.function].push_back({"seed", -1.0, *seed});
       }
-      if (budget <= 1 && c.nodes.size() >= 2) {
+      if (c.nodes.size() >= 2) {
         std::vector<size_t> order;
         for (size_t i : live)
           if (i != best_i && trials[i].us > 0 && trials[i].us < 1.25 * best_class) order.push_back(i);
         std::sort(order.begin(), order.end(), [&](size_t a, size_t b) { return trials[a].us < trials[b].us; });
-        const size_t keep = budget == 0 ? 6 : 2;
+        const size_t keep = budget == 0 ? 6 : budget == 1 ? 2 : 1;
         for (size_t k = 0; k < order.size() && k < keep; ++k) runners_up[c.function].push_back({trials[order[k]].label, trials[order[k]].us, trials[order[k]].spec});
       }
       const GraphSpecification& w = trials[best_i].spec;

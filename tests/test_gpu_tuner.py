@@ -1,0 +1,81 @@
+"""GPU tests of the tuner (MonoNNModuleTuner::tune, mononn_module_tuner.cc:620-991): it must hand back a module that
+computes the same function as the default one, leave the reference's dump tree behind, and that tree must be enough
+to rebuild the same kernel (TF_MONONN_EXISTING_TUNING_SPEC_DIR contract, README.md:145-149)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from mononn_amd import MonoNNModule, MonoNNModuleTuner
+from mononn_amd.hlo import models
+from oracle import hlo_interp
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(got, want32):
+    g, w = got.astype(np.float64).ravel(), want32.astype(np.float64).ravel()
+    assert np.abs(g - w).max() <= 2e-2                                         # the north star's tolerance
+    assert float(g @ w / (np.linalg.norm(g) * np.linalg.norm(w))) >= 0.9999
+
+
+@pytest.fixture(scope="module")
+def encoder():
+    # FFN2 contracts over 1024: long enough for the split-K phase to consider it
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=1024, vocab=300, max_pos=64)
+    consts, inputs = fx.make_constants(31, "random"), fx.make_inputs(31)
+    return fx, consts, inputs, hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+
+
+def test_tuned_module_dump_tree_and_reload(gpu_device, encoder, tmp_path, monkeypatch):
+    fx, consts, inputs, want = encoder
+    monkeypatch.setenv("MONONN_TUNER_VERBOSE", "0")
+    dump = str(tmp_path / "dump")
+    tuned = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, dump, budget=2)   # fastest: one launch shape, few tiles
+    tuned.set_constants(consts)
+    tuned.load(gpu_device)
+    got = tuned.run(inputs, fx.outputs)[0]
+    _check(got, want)
+    # dump tree (mononn_module_tuner.cc:374-383, 457-603)
+    cluster = os.path.join(dump, "cluster_0")
+    names = set(os.listdir(cluster))
+    assert {"best_tuning_spec.json", "best_tuning_spec.hsaco", "best_tuning_spec_src", "tuning_log.log", "performance_report.csv"} <= names
+    contexts = [n[:-5] for n in names if n.endswith(".json") and n != "best_tuning_spec.json"]
+    assert contexts and all(f"{c}.hsaco" in names and f"{c}_src" in names for c in contexts)
+    log = open(os.path.join(cluster, "tuning_log.log")).read()
+    assert "Tuning result for each thread grid setting" in log and "gemm x" in log and " ms\n" in log
+    assert "whole kernel" in log                         # the class winners were confirmed in the whole kernel
+    report = open(os.path.join(cluster, "performance_report.csv")).read().splitlines()
+    assert len(report) > 10 and all(len(r.split(",")) == 3 for r in report[1:])
+    # the tree is enough to get the same kernel back, bit for bit
+    again = MonoNNModule.from_spec_dir(fx.hlo_text, dump)
+    assert json.loads(again.get_tuning_spec()) == json.loads(tuned.get_tuning_spec())
+    again.set_constants(consts)
+    again.load(gpu_device)
+    assert np.array_equal(again.run(inputs, fx.outputs)[0].view(np.uint16), got.view(np.uint16))
+    # and the tuned kernel is not slower than the default one (same launch shape family, 5% slack for noise)
+    import torch
+    default = MonoNNModule.compile(fx.hlo_text)
+    default.set_constants(consts)
+    default.load(gpu_device)
+    default.run(inputs, fx.outputs)
+    stream = torch.cuda.current_stream().cuda_stream
+    t_def, _ = default.time_raw(default.buffer_pointers(), stream, 10, 100)
+    t_tuned, _ = tuned.time_raw(tuned.buffer_pointers(), stream, 10, 100)
+    print(f"default {t_def * 1e3:.1f} us, tuned {t_tuned * 1e3:.1f} us")
+    assert t_tuned <= 1.05 * t_def
+
+
+def test_tuning_from_a_seed_specification(gpu_device, encoder, tmp_path, monkeypatch):
+    fx, consts, inputs, want = encoder
+    first = str(tmp_path / "first")
+    MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, first, budget=2).close()
+    monkeypatch.setenv("MONONN_TUNER_SEED_SPEC_DIR", first)
+    second = str(tmp_path / "second")
+    tuned = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, second, budget=2)
+    log = open(os.path.join(second, "cluster_0", "tuning_log.log")).read()
+    assert "with the seed specification" in log
+    tuned.set_constants(consts)
+    tuned.load(gpu_device)
+    _check(tuned.run(inputs, fx.outputs)[0], want)
