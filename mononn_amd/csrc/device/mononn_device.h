@@ -227,12 +227,6 @@ __device__ __forceinline__ float fast_tanh(float x) {
   float e = __expf(2.0f * x);
   return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
 }
-// keep a value (and the load that produced it) alive without using it
-template <class T>
-__device__ __forceinline__ void touch(T v) {
-  float f = (float)v;
-  asm volatile("" ::"v"(f));
-}
 template <class T>
 __device__ __forceinline__ T sign_of(T x) {
   return (T)((x > (T)0) - (x < (T)0));
