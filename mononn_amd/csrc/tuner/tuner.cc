@@ -498,8 +498,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       promising = best_us < 0 || (stitched_us > 0 && stitched_us < 1.08 * best_us);
       if (!promising) log << "  [" << ctx_str << "] " << stitched_us << " us before refinement, best context so far " << best_us << " us: not refined\n";
     }
-    // two sweeps: what the first one changes in one class can change the ranking in another
-    for (int sweep = 0, changed = 1; sweep < (budget == 0 ? 2 : 1) && changed && promising && !runners_up.empty() && !env::is_true("MONONN_TUNER_NO_REFINEMENT"); ++sweep) {
+    // several sweeps: what one sweep changes in one class can change the ranking in another
+    auto refine = [&](int max_sweeps) {
+    for (int sweep = 0, changed = 1; sweep < max_sweeps && changed && promising && !runners_up.empty() && !env::is_true("MONONN_TUNER_NO_REFINEMENT"); ++sweep) {
       changed = 0;
       for (auto& kv : classes) {
         ClassInfo& c = kv.second;
@@ -543,6 +544,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         }
       }
     }
+    };
+    refine(budget == 0 ? 3 : 1);
+    bool split_adopted = false;
     if (promising && !env::is_true("MONONN_TUNER_NO_SPLIT_K")) {
       for (auto& kv : classes) {
         ClassInfo& c = kv.second;
@@ -771,6 +775,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             for (auto& in : instrs) report << ctx_str << "," << in << "," << trials[best_split].total_us / per << "\n";
             stitched = std::move(best_spec);
             stitched_us = best_with;
+            split_adopted = true;
             // the row programs that now add up the partial sums do more loading than before: their knobs again
             std::vector<std::string> allow, consumers;
             names_and_consumers(trials[best_split].mod->program(), instr_set, &allow, &consumers);
@@ -808,6 +813,8 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         for (size_t i = first; i < trials.size(); ++i) trials[i].mod.reset();
       }
     }
+    // the classes that kept their node names once more, now against the split GEMMs and their consumers
+    if (split_adopted) refine(budget == 0 ? 2 : 1);
     // ---- whole kernel of this context --------------------------------------------------------------
     stitched.codegen_allow_list.clear();
     stitched.hip.profile_stages = false;
