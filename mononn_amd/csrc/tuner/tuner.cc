@@ -815,6 +815,111 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     }
     // the classes that kept their node names once more, now against the split GEMMs and their consumers
     if (split_adopted) refine(budget == 0 ? 2 : 1);
+    // ---- stages made of several GEMM calls: a tile per call ---------------------------------------------
+    // The GEMMs of one stage (the Q, K and V projections) have been tuned as one class, with one tile.  Their calls
+    // occupy consecutive ranges of workgroups, and the workgroups differ: those that had a unit in the stage before
+    // ask for their weights later than those that were idle, and some may have no unit at all.  Giving every call
+    // position its own tile, under the condition that the stage still fits the grid in one round, lets the late
+    // workgroups take the small tiles.  Judged on the whole kernel.
+    if (promising && budget <= 1 && !env::is_true("MONONN_TUNER_NO_REFINEMENT")) {
+      MonoNNModule probe(params.hlo_text, [&] {
+        GraphSpecification s = stitched;
+        s.codegen_allow_list.clear();
+        s.hip.profile_stages = false;
+        return s.to_json().dump(0);
+      }(), "mononn_probe");
+      bool ok = true;
+      try {
+        probe.generate_code();
+      } catch (const Error&) {
+        ok = false;
+      }
+      if (ok) {
+        const codegen::HipProgram& php = probe.hip_program();
+        std::map<std::string, const codegen::NodeReport*> report_of;
+        for (auto& r : php.nodes) report_of[r.name] = &r;
+        std::map<std::string, const graph::Node*> node_of;
+        for (auto& n : probe.program().nodes) node_of[n.name] = &n;
+        // (function of the class under this specification, position in the stage) -> nodes; stage totals
+        std::map<std::pair<std::string, int>, std::vector<std::string>> groups;
+        std::map<std::string, int64_t> stage_total_of;   // node -> units of its whole stage
+        for (auto& st : php.stage_nodes) {
+          int gemms = 0;
+          int64_t total = 0;
+          for (auto& n : st) {
+            auto it = report_of.find(n);
+            if (it == report_of.end()) continue;
+            total += it->second->units;
+            gemms += it->second->kind == "gemm";
+          }
+          if (gemms < 2) continue;
+          for (size_t pos = 0; pos < st.size(); ++pos) {
+            auto it = report_of.find(st[pos]);
+            if (it == report_of.end() || it->second->kind != "gemm") continue;
+            auto nd = node_of.find(st[pos]);
+            if (nd == node_of.end() || !nd->second->prologue.empty() || nd->second->gemm.split_k > 1 || !codegen::gemm_uses_mfma(nd->second->gemm)) continue;
+            groups[{nd->second->gemm.problem_hash(), static_cast<int>(pos)}].push_back(st[pos]);
+            stage_total_of[st[pos]] = total;
+          }
+        }
+        if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);
+        // the calls of one problem shape, in stage order; a candidate tile is given to the first p of them (the
+        // workgroups with the lowest numbers are the ones that were busy in the stage before), p = 1 .. all
+        std::map<std::string, std::vector<int>> positions_of;
+        for (auto& gr : groups) positions_of[gr.first.first].push_back(gr.first.second);
+        for (auto& fam : positions_of) {
+          std::vector<int>& pos = fam.second;
+          std::sort(pos.begin(), pos.end());
+          const std::vector<std::string>& first_names = groups.at({fam.first, pos[0]});
+          const graph::GemmDesc& g = node_of.at(first_names[0])->gemm;
+          const int64_t total = stage_total_of.at(first_names[0]);
+          const int64_t grid = php.grid;
+          std::string line;
+          double best_us2 = -1;
+          GraphSpecification best_spec2;
+          for (size_t p = 1; p <= pos.size(); ++p) {
+            int64_t cur = 0;
+            for (size_t i = 0; i < p; ++i) cur += report_of.at(groups.at({fam.first, pos[i]})[0])->units;
+            struct Cand {
+              codegen::GemmTuning t;
+              int64_t units;
+            };
+            std::vector<Cand> cands;
+            for (auto& t : gemm_candidates(g, cx.block / 64, 1)) {
+              const int64_t u = ((g.M + t.bm - 1) / t.bm) * ((g.N + t.bn - 1) / t.bn) * g.batch;
+              const int64_t new_total = total - cur + static_cast<int64_t>(p) * u;
+              if (static_cast<int64_t>(p) * u == cur || new_total > grid || 8 * new_total < 7 * grid || t.wk != cx.block / 64) continue;
+              cands.push_back({t, u});
+            }
+            // fullest grid first; a handful is enough
+            std::sort(cands.begin(), cands.end(), [&](const Cand& a, const Cand& b) { return a.units > b.units; });
+            if (cands.size() > 4) cands.resize(4);
+            for (auto& cd : cands) {
+              GraphSpecification s2 = stitched;
+              for (size_t i = 0; i < p; ++i)
+                for (auto& n : groups.at({fam.first, pos[i]})) apply_gemm(s2, n, cd.t, g.K);
+              const double us2 = whole_kernel_us(s2);
+              char buf[112];
+              std::snprintf(buf, sizeof buf, " first%zu:tile%dx%d_waves%dx%dx%d(%lld units each)=%.2f", p, cd.t.bm, cd.t.bn, cd.t.wm, cd.t.wn, cd.t.wk,
+                            static_cast<long long>(cd.units), us2);
+              line += buf;
+              if (us2 > 0 && (best_us2 < 0 || us2 < best_us2)) {
+                best_us2 = us2;
+                best_spec2 = std::move(s2);
+              }
+            }
+          }
+          if (line.empty()) continue;
+          log << "  [" << ctx_str << "] tiles per call in the stages of " << first_names[0] << " (x" << first_names.size() << ", " << pos.size() << " calls, " << total
+              << " units): now " << stitched_us << " us;" << line << "\n";
+          if (verbose) std::fprintf(stderr, "[mononn tuner] %s tiles per call (%s): now %.2f us;%s\n", ctx_str.c_str(), first_names[0].c_str(), stitched_us, line.c_str());
+          if (best_us2 > 0 && best_us2 < 0.997 * stitched_us) {
+            stitched = std::move(best_spec2);
+            stitched_us = best_us2;
+          }
+        }
+      }
+    }
     // ---- whole kernel of this context --------------------------------------------------------------
     stitched.codegen_allow_list.clear();
     stitched.hip.profile_stages = false;
