@@ -359,7 +359,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           bufs.ensure_temp(static_cast<size_t>(hp.temp_bytes));
           std::vector<void*> vals = bufs.ptrs, args(vals.size());
           for (size_t a = 0; a < vals.size(); ++a) args[a] = &vals[a];
-          const int warm = 2, iters = budget >= 1 ? 4 : 8;
+          const int warm = 3, iters = budget >= 1 ? 8 : 20;   // launches are short: the compilation of the candidates dominates
           size_t cb = 0;
           void* clk = dm.global("mononn_stage_clock", &cb);
           std::vector<unsigned long long> ticks(cb / sizeof(unsigned long long));
