@@ -433,7 +433,9 @@ bool can_merge_clusters(const Program& prog, const std::vector<const Instr*>& pr
 // ------------------------------------------------------------------------------------------
 bool gemm_uses_mfma(const graph::GemmDesc& g) {
   if (g.is_conv && !g.conv_fragment_loads()) return false;
-  return g.a_k_contig && (g.b_k_contig || g.b_packed) && g.K % 32 == 0;
+  if (!g.a_k_contig || !(g.b_k_contig || g.b_packed)) return false;
+  // a k extent that is not a multiple of 32 is zero-filled in the last step, from plain row-major operands only
+  return g.K % 32 == 0 || (!g.is_conv && !g.b_packed && !g.a_packed && g.split_k <= 1);
 }
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus) {
@@ -483,7 +485,8 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
     MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && (wide || ksteps / t.wk <= 32 / (tm + tn)), kSpecError)
         << "GEMM with a row-program prologue: a wave's whole k range (" << ksteps / std::max(t.wk, 1) << " steps) must fit one register chunk";
   }
-  MONONN_CHECK(t.split_k >= 1 && g.K % (32 * t.split_k) == 0, kSpecError) << "split_k " << t.split_k << " does not divide the k steps of the GEMM";
+  MONONN_CHECK(t.split_k >= 1 && (t.split_k == 1 || g.K % (32 * t.split_k) == 0), kSpecError)
+      << "split_k " << t.split_k << " does not divide the k steps of the GEMM";
   MONONN_CHECK(t.wm >= 1 && t.wn >= 1 && t.wk >= 1 && t.wm * t.wn * t.wk == ls.waves(), kSpecError)
       << "GEMM wave arrangement " << t.wm << "x" << t.wn << "x" << t.wk << " does not use " << ls.waves() << " waves";
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)

@@ -307,7 +307,8 @@ template <int BM, int BN, int WM, int WN, int WK, int K, int KTOTAL, class Pre>
 __device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_n, Pre& pb) {
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
-  constexpr int KSTEPS = K / 32;
+  constexpr bool RAGGED_K = K % 32 != 0;   // the last k step is partly past the end: its missing elements are zeros
+  constexpr int KSTEPS = (K + 31) / 32;
   constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
   constexpr int CH = gemm_chunk_steps(TM, TN, MY_STEPS, true);
   static_assert(CH * TN * sizeof(half8_t) <= sizeof(pb.v), "preload buffer too small for this tile");
@@ -340,14 +341,16 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
                                           const AMap& amap = AMap(), const Pre* pb = nullptr) {
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
-  constexpr int KSTEPS = K / 32;
+  constexpr bool RAGGED_K = K % 32 != 0;   // the last k step is partly past the end: its missing elements are zeros
+  constexpr int KSTEPS = (K + 31) / 32;
   constexpr int MY_STEPS = (KSTEPS + WK - 1) / WK;
   constexpr int CH = gemm_chunk_steps(TM, TN, MY_STEPS, PRE_B);
   constexpr int NCHUNK = (MY_STEPS + CH - 1) / CH;
   static_assert(!PRE_B || PACKED_B, "only packed weights can be requested ahead of the tile");
   static_assert(!PACKED_A || AMap::kRowMajor, "a fragment-order left operand takes no row map");
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
-  static_assert(K % 32 == 0, "K must be a multiple of 32");
+  static_assert(!RAGGED_K || (!PACKED_A && !PACKED_B && !PRE_B && AMap::kRowMajor && K == KTOTAL && !Pro::enabled),
+                "a k extent that is not a multiple of 32 is taken from plain k-contiguous operands only");
   const int lane = lane_id();
   const int wave = wave_id();
   const int wk = wave % WK;
@@ -393,6 +396,18 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   constexpr int B_STEP = PACKED_B ? 64 * 8 : 32;   // halves between consecutive k steps
 
   half8_t a[2][CH][TM], b[2][CH][TN];
+  // Rows whose k extent is not a multiple of 32 start at odd element offsets, so their fragments are read
+  // without an alignment promise, and the lanes whose 8 elements cross the end read them one by one.
+  auto load_ragged = [&](const half_t* p, int k0) {
+    half8_t v;
+    if (k0 + 8 <= K) {
+      __builtin_memcpy(&v, p, sizeof(v));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = k0 + e < K ? p[e] : half_t(0);
+    }
+    return v;
+  };
   auto load_chunk = [&](int c, int buf) {
 #pragma unroll
     for (int s = 0; s < CH; ++s) {
@@ -401,11 +416,13 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         if (PRE_B && c == 0) b[buf][s][j] = pb->v[s * TN + j];
+        else if constexpr (RAGGED_K) b[buf][s][j] = load_ragged(b_ptr[j] + (long)ks * B_STEP, ks * 32 + kq);
         else b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + (long)ks * A_STEP);
+        if constexpr (RAGGED_K) a[buf][s][i] = load_ragged(a_ptr[i] + (long)ks * A_STEP, ks * 32 + kq);
+        else if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + (long)ks * A_STEP);
         else a[buf][s][i] = *reinterpret_cast<const half8_t*>(amap(A, a_row[i], ks * 32 + kq, lda));
       }
     }

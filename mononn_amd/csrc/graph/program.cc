@@ -584,7 +584,7 @@ struct Builder {
       }
     };
     each_gemm([&](const Instr* g, GemmDesc& d) {
-      if (d.b_k_contig || d.b_packed || !d.a_k_contig || d.K % 32 != 0) return;
+      if (d.b_k_contig || d.b_packed || !d.a_k_contig) return;
       const Instr* root = p.storage_root(g->operands[1]);
       if (!p.producer.count(root)) return;   // parameter / constant
       if (!can_store_k_contig(root, g->operands[1], g->gemm.rhs_contracting)) return;

@@ -78,7 +78,7 @@ void DeviceBuffers::ensure_temp(size_t bytes) {
 std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int waves, int budget) {
   std::vector<codegen::GemmTuning> out;
   if (!codegen::gemm_uses_mfma(g)) return out;
-  const int ksteps = static_cast<int>(g.K / 32);
+  const int ksteps = static_cast<int>((g.K + 31) / 32);
   for (int wk = 1; wk <= waves; wk *= 2) {
     if (wk > ksteps) break;
     for (int wm = 1; wm * wk <= waves; wm *= 2) {

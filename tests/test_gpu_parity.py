@@ -54,7 +54,10 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
     dict(M=128, N=128, K=64, batch=(1, 12), rhs_c=3, alpha=0.125),  # scores: both operands k-contiguous
     dict(M=128, N=64, K=128, batch=(2, 3)),                       # context: B stored [K,N]
     dict(M=100, N=52, K=96, rhs_c=1),                             # ragged M / N on the MFMA path
-    dict(M=64, N=48, K=40, rhs_c=1),                              # K not a multiple of 32
+    dict(M=64, N=48, K=40, rhs_c=1),                              # K not a multiple of 32: zero-filled last MFMA step
+    dict(M=197, N=64, K=197, batch=(2, 3), rhs_c=3),              # odd row length: fragments start at unaligned addresses
+    dict(M=33, N=20, K=17, rhs_c=1),                              # K below one MFMA step
+    dict(M=64, N=48, K=40),                                       # K not a multiple of 32 and B stored [K,N] -> fallback path
     dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                     # A stored [K,M]
     dict(M=128, N=256, K=256, b_const=True, as_dot=True),         # plain `dot` with a constant right operand
     dict(M=48, N=80, K=64, batch=(3,), rhs_c=2, as_dot=True),     # batched `dot`, both operands k-contiguous

@@ -272,6 +272,15 @@ def test_convolution_call_is_lowered_as_implicit_gemm():
     assert m2.buffer_info()["liveouts"] == [2 * 5 * 10 * 6 * 2]
 
 
+def test_contraction_length_off_the_mfma_step_still_takes_mfma_tiles():
+    # ViT's P.V product contracts over 197 keys: the tile zero-fills the last step instead of falling back to one
+    # thread per element; V is stored transposed by the stage that writes it, so both operands are k-contiguous
+    fx = models.vit(L=1, B=1)
+    src = MonoNNModule.compile(fx.hlo_text, build=False).get_source("main.hip")
+    assert "gemm_naive_element" not in src
+    assert re.search(r"gemm_tile<\d+, \d+, \d+, \d+, \d+, 197, false, 197,", src)
+
+
 @pytest.mark.parametrize("edit,fragment", [
     (lambda t: t.replace("window={size=16x16 stride=16x16}", "window={size=16x16 stride=16x16 rhs_dilate=2x2}"), "dilated"),
     (lambda t: t.replace("window={size=16x16 stride=16x16}", "window={size=16x16 stride=16x16 pad=0_1x0_0}"), "symmetric"),
