@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <functional>
+#include <sstream>
 
 #include "common/status.h"
 
@@ -285,6 +286,77 @@ std::string Emitter::serial_reduce(const Instr* ins, const Index& idx) {
   return acc;
 }
 
+std::vector<std::string> Emitter::inline_scalar_computation(const hlo::Computation* c, const std::vector<std::string>& args) {
+  MONONN_CHECK(c->params.size() == args.size(), kUnsupported) << "computation " << c->hlo_name << " takes " << c->params.size() << " parameters, " << args.size() << " given";
+  for (auto* p : c->params) MONONN_CHECK(p->shape.rank() == 0, kUnsupported) << c->hlo_name << ": reducer parameters must be scalars";
+  push_scope();
+  for (size_t i = 0; i < args.size(); ++i) bind(c->params[i], {}, args[i]);
+  std::vector<std::string> out;
+  if (c->root->opcode == "tuple") {
+    for (auto* o : c->root->operands) out.push_back(value(o, {}));
+  } else {
+    out.push_back(value(c->root, {}));
+  }
+  for (auto* p : c->params) unbind(p);
+  pop_scope();
+  return out;
+}
+
+// (value, index) reductions and their like (ir_parser_fused.cc:1169-1213, tuple functors of
+// reduction_functor_generator.cc:246-283): the elements are combined in ascending order by the thread that owns
+// the output element.
+std::vector<std::string> Emitter::serial_reduce_variadic(const Instr* ins, const Index& idx) {
+  const size_t n = ins->operands.size() / 2;
+  MONONN_CHECK(n >= 1 && ins->operands.size() == 2 * n && ins->dimensions.size() == 1 && ins->shape.is_tuple() && ins->shape.tuple.size() == n, kUnsupported)
+      << ins->hlo_name << ": a variadic reduce takes N operands, N init values and yields an N-tuple over one reduced dimension";
+  const std::string k = "variadic:" + key(ins, idx);
+  for (auto it = scopes_.rbegin(); it != scopes_.rend(); ++it) {
+    auto f = it->find(k);
+    if (f == it->end()) continue;
+    std::vector<std::string> cached;
+    std::istringstream is(f->second);
+    std::string name;
+    while (is >> name) cached.push_back(name);
+    return cached;
+  }
+  const Instr* x0 = ins->operands[0];
+  const int d = static_cast<int>(ins->dimensions[0]);
+  const int64_t R = x0->shape.dims[d];
+  std::vector<std::string> acc, types;
+  for (size_t i = 0; i < n; ++i) {
+    MONONN_CHECK(ins->operands[i]->shape.dims == x0->shape.dims, kUnsupported) << ins->hlo_name << ": operands of different shapes";
+    types.push_back(hlo::dtype_ctype(ins->shape.tuple[i].dtype));
+    acc.push_back(fresh("acc"));
+    out_.line(types[i] + " " + acc[i] + " = " + value(ins->operands[n + i], {}) + ";");
+  }
+  std::string rk = fresh("rk");
+  int var = vars_.add(rk, R);
+  out_.open("for (int " + rk + " = 0; " + rk + " < " + std::to_string(R) + "; ++" + rk + ")");
+  push_scope();
+  Index xi;
+  for (int i = 0, j = 0; i < x0->shape.rank(); ++i) {
+    if (i == d) xi.push_back(LinExpr::variable(var, R));
+    else xi.push_back(idx[j++]);
+  }
+  std::vector<std::string> args = acc;
+  for (size_t i = 0; i < n; ++i) args.push_back(value(ins->operands[i], xi));
+  std::vector<std::string> res = inline_scalar_computation(ins->called, args);
+  MONONN_CHECK(res.size() == n, kUnsupported) << ins->hlo_name << ": the reducer yields " << res.size() << " values for " << n << " operands";
+  // all results are taken before any accumulator changes (a reducer may pass an accumulator through to another slot)
+  std::vector<std::string> tmp;
+  for (size_t i = 0; i < n; ++i) {
+    tmp.push_back(fresh("nx"));
+    out_.line("const " + types[i] + " " + tmp[i] + " = (" + types[i] + ")" + res[i] + ";");
+  }
+  for (size_t i = 0; i < n; ++i) out_.line(acc[i] + " = " + tmp[i] + ";");
+  pop_scope();
+  out_.close();
+  std::string joined;
+  for (auto& a : acc) joined += a + " ";
+  scopes_.back()[k] = joined;
+  return acc;
+}
+
 std::string Emitter::emit(const Instr* ins, const Index& idx) {
   const std::string& op = ins->opcode;
   const DType dt = ins->shape.dtype;
@@ -321,6 +393,11 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
     std::string name = "lit_" + std::to_string(std::hash<std::string>{}(T + flat));
     literal_tables_[name] = "__device__ const " + T + " " + name + "[] = {" + flat + "};";
     return def(dt, name + "[" + linearize(idx, ins->shape.dims).str(vars_) + "]");
+  }
+  if (op == "get-tuple-element" && ins->operands[0]->opcode == "reduce" && (!entry || is_member(ins->operands[0]))) {
+    auto all = serial_reduce_variadic(ins->operands[0], idx);
+    MONONN_CHECK(ins->tuple_index >= 0 && static_cast<size_t>(ins->tuple_index) < all.size(), kParseError) << ins->hlo_name << ": tuple index out of range";
+    return all[ins->tuple_index];
   }
   if (entry && !is_member(ins)) {
     // value produced outside this cluster: follow pure renames, load at the storage root
@@ -440,7 +517,90 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
     }
     return value(x, xi);
   }
-  if (op == "reduce") return serial_reduce(ins, idx);
+  if (op == "dynamic-update-slice") {
+    // the update where the index falls inside it (start indices clamped so that it fits), the operand elsewhere
+    const Instr* x = ins->operands[0];
+    const Instr* u = ins->operands[1];
+    std::string cond;
+    Index ui;
+    for (int i = 0; i < x->shape.rank(); ++i) {
+      const int64_t un = u->shape.dims[i], hi = x->shape.dims[i] - un;
+      if (hi == 0) {
+        ui.push_back(idx[i]);
+        continue;
+      }
+      std::string s = value(ins->operands[2 + i], {});
+      std::string c = fresh("us");
+      out_.line("const int " + c + " = (" + idx[i].str(vars_) + ") - min(max((int)" + s + ", 0), " + std::to_string(hi) + ");");
+      cond += (cond.empty() ? "" : " && ") + c + " >= 0 && " + c + " < " + std::to_string(un);
+      ui.push_back(LinExpr::opaque(c, un));
+    }
+    if (cond.empty()) return value(u, ui);
+    std::string v = fresh();
+    out_.line(T + " " + v + ";");
+    out_.open("if (" + cond + ")");
+    push_scope();
+    out_.line(v + " = " + value(u, ui) + ";");
+    pop_scope();
+    out_.close();
+    out_.open("else");
+    push_scope();
+    out_.line(v + " = " + value(x, idx) + ";");
+    pop_scope();
+    out_.close();
+    return v;
+  }
+  if (op == "reduce-window") {
+    // acc = init; for every window position: acc = reducer(acc, inside the operand ? operand : init)
+    // (index map of index_tracer.cc's reduce-window: input = output * stride + window offset - low padding)
+    const Instr* x = ins->operands[0];
+    const int r = x->shape.rank();
+    std::string init = value(ins->operands[1], {});
+    std::string acc = fresh("acc");
+    out_.line(T + " " + acc + " = " + init + ";");
+    std::vector<std::string> w(r);
+    int opened = 0;
+    for (int i = 0; i < r; ++i) {
+      if (ins->window_size[i] == 1) continue;
+      w[i] = fresh("w");
+      out_.open("for (int " + w[i] + " = 0; " + w[i] + " < " + std::to_string(ins->window_size[i]) + "; ++" + w[i] + ")");
+      ++opened;
+    }
+    push_scope();
+    std::string cond;
+    Index xi;
+    for (int i = 0; i < r; ++i) {
+      const int64_t lo = ins->window_pad_low[i], hi = ins->window_pad_high[i], st = ins->window_stride[i], n = x->shape.dims[i];
+      if (ins->window_size[i] == 1 && st == 1 && lo == 0 && hi == 0) {
+        xi.push_back(idx[i]);
+        continue;
+      }
+      std::string p = fresh("p");
+      out_.line("const int " + p + " = (" + idx[i].str(vars_) + ") * " + std::to_string(st) + (w[i].empty() ? "" : " + " + w[i]) + " - " + std::to_string(lo) + ";");
+      if (lo > 0 || hi > 0) cond += (cond.empty() ? "" : " && ") + p + " >= 0 && " + p + " < " + std::to_string(n);
+      xi.push_back(LinExpr::opaque(p, n));
+    }
+    std::string v;
+    if (cond.empty()) {
+      v = value(x, xi);
+    } else {
+      v = fresh();
+      out_.line(T + " " + v + " = " + init + ";");
+      out_.open("if (" + cond + ")");
+      push_scope();
+      out_.line(v + " = " + value(x, xi) + ";");
+      pop_scope();
+      out_.close();
+    }
+    out_.line(acc + " = (" + T + ")" + reducer_expr(ins, acc, v) + ";");
+    pop_scope();
+    for (int i = 0; i < opened; ++i) out_.close();
+    return acc;
+  }
+  if (op == "reduce") {
+    MONONN_CHECK(!ins->shape.is_tuple(), kUnsupported) << ins->hlo_name << ": tuple-valued reduce read without get-tuple-element";
+    return serial_reduce(ins, idx);
+  }
 
   // ---- element-wise -----------------------------------------------------------------------
   std::vector<std::string> a;

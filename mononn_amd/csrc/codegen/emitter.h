@@ -91,6 +91,10 @@ class Emitter {
   std::string emit(const hlo::Instr* ins, const Index& idx);
   std::string load(const hlo::Instr* root, const Index& idx);
   std::string serial_reduce(const hlo::Instr* ins, const Index& idx);
+  // N-operand reduce with a tuple-valued reducer: one loop for all N results, which are returned in tuple order
+  std::vector<std::string> serial_reduce_variadic(const hlo::Instr* ins, const Index& idx);
+  // the scalar computation `c` with its parameters replaced by the C expressions `args`: C expressions of its results
+  std::vector<std::string> inline_scalar_computation(const hlo::Computation* c, const std::vector<std::string>& args);
   std::string key(const hlo::Instr* ins, const Index& idx) const;
   std::string def(hlo::DType t, const std::string& rhs);
   bool is_member(const hlo::Instr* v) const { return members_.count(v) > 0; }

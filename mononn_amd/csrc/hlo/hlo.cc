@@ -525,6 +525,41 @@ void decode_attrs(Instr* ins, Module* mod) {
     }
   }
   if (op == "dynamic-slice") ins->dynamic_slice_sizes = ints_of(need("dynamic_slice_sizes"));
+  if (op == "dynamic-update-slice") {
+    MONONN_CHECK(ins->operands.size() >= 2 && static_cast<int>(ins->operands.size()) == 2 + ins->shape.rank() &&
+                     ins->operands[0]->shape.dims == ins->shape.dims && ins->operands[1]->shape.rank() == ins->shape.rank(),
+                 kUnsupported)
+        << ins->hlo_name << ": dynamic-update-slice takes the operand, the update and one scalar start index per dimension";
+    for (int i = 0; i < ins->shape.rank(); ++i)
+      MONONN_CHECK(ins->operands[1]->shape.dims[i] <= ins->shape.dims[i], kInvalidArgument) << ins->hlo_name << ": the update is larger than the operand";
+  }
+  if (op == "reduce-window") {
+    // one operand and its init value, no dilation (ir_parser_fused.cc:1218-1222, :1246-1250)
+    MONONN_CHECK(ins->operands.size() == 2 && !ins->shape.is_tuple(), kUnsupported) << ins->hlo_name << ": reduce-window takes one operand and one init value";
+    auto w = window_fields(need("window"));
+    MONONN_CHECK(!w.count("lhs_dilate") && !w.count("rhs_dilate"), kUnsupported) << ins->hlo_name << ": window dilation is not supported";
+    const hlo::Shape& x = ins->operands[0]->shape;
+    const size_t r = static_cast<size_t>(x.rank());
+    MONONN_CHECK(w.count("size") && w["size"].size() == r && ins->shape.rank() == x.rank(), kParseError) << ins->hlo_name << ": window size does not match the operand's rank";
+    for (size_t i = 0; i < r; ++i) {
+      ins->window_size.push_back(std::strtoll(w["size"][i].c_str(), nullptr, 10));
+      ins->window_stride.push_back(w.count("stride") && w["stride"].size() == r ? std::strtoll(w["stride"][i].c_str(), nullptr, 10) : 1);
+      int64_t lo = 0, hi = 0;
+      if (w.count("pad") && w["pad"].size() == r) {
+        const std::string& pd = w["pad"][i];
+        size_t us = pd.find('_');
+        MONONN_CHECK(us != std::string::npos, kParseError) << ins->hlo_name << ": bad window padding '" << pd << "'";
+        lo = std::strtoll(pd.substr(0, us).c_str(), nullptr, 10);
+        hi = std::strtoll(pd.substr(us + 1).c_str(), nullptr, 10);
+      }
+      ins->window_pad_low.push_back(lo);
+      ins->window_pad_high.push_back(hi);
+      MONONN_CHECK(ins->window_size[i] >= 1 && ins->window_stride[i] >= 1 && lo >= 0 && hi >= 0, kUnsupported) << ins->hlo_name << ": negative window padding is not supported";
+      const int64_t span = x.dims[i] + lo + hi - ins->window_size[i];
+      MONONN_CHECK(span >= 0 && ins->shape.dims[i] == span / ins->window_stride[i] + 1, kInvalidArgument)
+          << ins->hlo_name << ": output extent " << ins->shape.dims[i] << " of dimension " << i << " does not follow from the window";
+    }
+  }
   if (op == "gather") {
     ins->offset_dims = ints_of(need("offset_dims"));
     ins->collapsed_slice_dims = ints_of(need("collapsed_slice_dims"));

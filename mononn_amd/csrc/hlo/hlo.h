@@ -84,6 +84,7 @@ struct Instr {
   std::vector<int64_t> slice_starts, slice_limits, slice_strides;
   std::vector<int64_t> pad_low, pad_high, pad_interior;
   std::vector<int64_t> dynamic_slice_sizes;
+  std::vector<int64_t> window_size, window_stride, window_pad_low, window_pad_high;   // reduce-window
   // gather
   std::vector<int64_t> offset_dims, collapsed_slice_dims, start_index_map, slice_sizes;
   int64_t index_vector_dim = -1;

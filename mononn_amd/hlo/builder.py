@@ -192,6 +192,35 @@ class Computation:
         return self._emit("reduce", x.dtype, dims, [x, init],
                           attrs=f"dimensions={{{dim}}}, to_apply=%{reducer}")
 
+    def reduce_window(self, x: Value, init: Value, size: Sequence[int], stride: Sequence[int],
+                      pad: Sequence[Sequence[int]], reducer: str) -> Value:
+        """Window reduction without dilation (ir_parser_fused.cc:1215-1262): out = (in + lo + hi - size) / stride + 1."""
+        dims = [(n + lo + hi - w) // st + 1 for n, w, st, (lo, hi) in zip(x.dims, size, stride, pad)]
+        window = ("size=" + "x".join(map(str, size)) + " stride=" + "x".join(map(str, stride)) +
+                  " pad=" + "x".join(f"{lo}_{hi}" for lo, hi in pad))
+        return self._emit("reduce-window", x.dtype, dims, [x, init], attrs=f"window={{{window}}}, to_apply=%{reducer}")
+
+    def dynamic_update_slice(self, x: Value, update: Value, starts: Sequence[Value]) -> Value:
+        return self._emit("dynamic-update-slice", x.dtype, x.dims, [x, update] + list(starts))
+
+    def reduce_variadic(self, xs: Sequence[Value], inits: Sequence[Value], dim: int, reducer: str) -> List[Value]:
+        """N-operand reduce with a tuple-valued reducer, e.g. (value, index) for arg-max
+        (ir_parser_fused.cc:1169-1213).  Returns the get-tuple-element values."""
+        dims = tuple(d for i, d in enumerate(xs[0].dims) if i != dim)
+        outs = [Value("", x.dtype, dims) for x in xs]
+        tshape = "(" + ", ".join(o.shape_str for o in outs) + ")"
+        name = self.module.fresh("reduce")
+        ops = ", ".join(o.operand_str for o in list(xs) + list(inits))
+        self.lines.append(f"%{name} = {tshape} reduce({ops}), dimensions={{{dim}}}, to_apply=%{reducer}")
+        res = []
+        for i, o in enumerate(outs):
+            g = self.module.fresh("get-tuple-element")
+            self.lines.append(f"%{g} = {o.shape_str} get-tuple-element({tshape} %{name}), index={i}")
+            res.append(Value(g, o.dtype, o.dims))
+        self.root = res[-1]
+        self.root_is_tuple = False
+        return res
+
     def gather_rows(self, table: Value, indices: Value) -> Value:
         """Row gather out[i..., :] = table[indices[i...], :] in XLA's gather form
         (dimension numbers as recorded by ir_parser_fused.cc:1034-1066)."""
@@ -352,6 +381,25 @@ class HloModuleBuilder:
             a = c.parameter(dtype, (), "x")
             b = c.parameter(dtype, (), "y")
             c.binary(opcode, a, b)
+            self.computations.append(c)
+            self._reducers[key] = c.name
+        return self._reducers[key]
+
+    def arg_reducer(self, direction: str, dtype: str, index_dtype: str = "s32") -> str:
+        """(value, index) reducer: keeps the larger (direction GE/GT) or smaller (LE/LT) value, and on
+        equal values the smaller index -- the form XLA gives tf.argmax / tf.argmin."""
+        key = ("arg", direction, dtype, index_dtype)
+        if key not in self._reducers:
+            c = Computation(self, self.fresh(f"arg_{direction.lower()}_{dtype}_reducer"))
+            av = c.parameter(dtype, (), "acc_value")
+            ai = c.parameter(index_dtype, (), "acc_index")
+            xv = c.parameter(dtype, (), "value")
+            xi = c.parameter(index_dtype, (), "index")
+            better = c.compare(av, xv, direction)
+            same = c.compare(av, xv, "EQ")
+            first = c.compare(ai, xi, "LT")
+            keep = c.binary("or", better, c.binary("and", same, first))
+            c.set_tuple_root([c.select(keep, av, xv), c.select(keep, ai, xi)])
             self.computations.append(c)
             self._reducers[key] = c.name
         return self._reducers[key]

@@ -15,8 +15,12 @@ reference attaches to each instruction when it lowers it:
     init, reducer = called computation)  ir_parser_fused.cc:1169-1213,
                                           mononn_engine/codegen/reduction_functor_generator.cc:224-294
   * broadcast/transpose/slice/pad/
-    concatenate/gather/dynamic-slice
-    index maps ......................... mononn_engine/core/context/index_tracer.cc:67-456
+    concatenate/gather/dynamic-slice/
+    reduce-window index maps ........... mononn_engine/core/context/index_tracer.cc:67-456
+  * reduce-window (operand + init, no
+    dilation), dynamic-update-slice,
+    variadic (value, index) reduce ..... ir_parser_fused.cc:1215-1262, :973-978, :1169-1213,
+                                          reduction_functor_generator.cc:246-283
   * row gather ......................... index_tracer.cc:235-280
   * element-wise op -> functor ......... mononn_engine/core/gpu/functor.cc:42-88, :145-168
   * __cublas$gemm backend_config ....... mononn_engine/core/op_impl/gemm_impl.cc:182-231, :233-499
@@ -28,8 +32,9 @@ not shared between the thing under test and its checker.
 Pinning (what fixes these functions besides the formulae above): tests/test_oracle_pinning.py
 checks the evaluator against closed forms and library routines -- fp64 triple-loop GEMM on tiny
 shapes, the two worked backend_config examples of gemm_impl.cc:290-316 against numpy einsum,
-torch.nn.functional soft-max / layer_norm / gelu(tanh), brute-force gather, and a whole BERT
-layer against an independent torch restatement.  Bit-level results of the CUDA build (CUTLASS
+torch.nn.functional soft-max / layer_norm / gelu(tanh), brute-force gather, torch max/avg
+pooling for reduce-window, NumPy slice assignment for dynamic-update-slice, np.argmax/argmin for
+the variadic reduce, and a whole BERT layer against an independent torch restatement.  Bit-level results of the CUDA build (CUTLASS
 accumulation order, -use_fast_math intrinsics) are not reproducible offline: parity unpinned at
 that level; the north-star tolerance is defined against fp32 evaluation, which this is.
 
@@ -254,6 +259,7 @@ class Evaluator:
         self.constants = constants or {}
         self.fp32 = precision == "fp32"
         self.trace: Dict[str, np.ndarray] = {}
+        self._vector_depth = 0
 
     def np_dtype(self, hlo_dtype: str):
         if self.fp32 and hlo_dtype == "f16":
@@ -285,6 +291,8 @@ class Evaluator:
         sh = ins.shape
         dt = self.np_dtype(sh.dtype) if sh.tuple_shapes is None else None
         if op == "parameter":
+            if self._vector_depth:   # a reducer body applied to whole arrays at once: its scalar shapes are not checked
+                return np.asarray(args[int(ins.literal)]).astype(self.np_dtype(sh.dtype), copy=False)
             return self._cast_in(args[int(ins.literal)], sh)
         if op == "constant":
             if ins.literal.replace(" ", "") == "{...}":
@@ -361,6 +369,15 @@ class Evaluator:
             sizes = _ints(ins.attrs["dynamic_slice_sizes"])
             starts = [int(np.clip(int(s), 0, x[0].shape[i] - sizes[i])) for i, s in enumerate(x[1:])]
             return x[0][tuple(slice(s, s + n) for s, n in zip(starts, sizes))]
+        if op == "dynamic-update-slice":
+            # start indices are clamped so that the update fits (XLA semantics, as for dynamic-slice)
+            upd = x[1]
+            starts = [int(np.clip(int(s), 0, x[0].shape[i] - upd.shape[i])) for i, s in enumerate(x[2:])]
+            out = np.array(x[0], dtype=dt, copy=True)
+            out[tuple(slice(s, s + n) for s, n in zip(starts, upd.shape))] = upd
+            return out
+        if op == "reduce-window":
+            return self._reduce_window(ins, x, dt)
         if op == "dot":
             lc, rc = _ints(ins.attrs["lhs_contracting_dims"])[0], _ints(ins.attrs["rhs_contracting_dims"])[0]
             A, B = x[0].astype(np.float32), x[1].astype(np.float32)
@@ -382,10 +399,61 @@ class Evaluator:
             raise NotImplementedError(f"custom-call target {target}")
         raise NotImplementedError(f"opcode {op}")
 
+    def _apply_reducer(self, red: Comp, args):
+        self._vector_depth += 1
+        try:
+            return self._run_comp(red, list(args))
+        finally:
+            self._vector_depth -= 1
+
+    def _reduce_window(self, ins: Instr, x, dt):
+        # out[o] = reducer over w of padded(x)[o * stride + w], padding = the init value, the accumulator
+        # starts at the init value (ir_parser_fused.cc:1215-1262: two operands, no dilation)
+        if len(x) != 2:
+            raise NotImplementedError("reduce-window takes one operand and one init value")
+        win = dict(kv.split("=") for kv in ins.attrs["window"].strip("{}").split())
+        if "lhs_dilate" in win or "rhs_dilate" in win:
+            raise NotImplementedError("reduce-window with dilation")
+        size = [int(v) for v in win["size"].split("x")]
+        stride = [int(v) for v in win["stride"].split("x")] if "stride" in win else [1] * len(size)
+        pad = [tuple(int(v) for v in p.split("_")) for p in win["pad"].split("x")] if "pad" in win else [(0, 0)] * len(size)
+        red = self.mod["comps"][ins.attrs["to_apply"].lstrip("%")]
+        init = np.asarray(x[1])
+        padded = np.empty([lo + n + hi for (lo, hi), n in zip(pad, x[0].shape)], x[0].dtype)
+        padded[...] = init
+        padded[tuple(slice(lo, lo + n) for (lo, _), n in zip(pad, x[0].shape))] = x[0]
+        acc = np.empty(ins.shape.dims, x[0].dtype)
+        acc[...] = init
+        with np.errstate(all="ignore"):
+            for w in np.ndindex(*size):
+                part = padded[tuple(slice(wi, wi + (o - 1) * st + 1, st) for wi, o, st in zip(w, ins.shape.dims, stride))]
+                acc = self._apply_reducer(red, [acc, part])
+        return np.asarray(acc).astype(dt, copy=False)
+
+    def _reduce_variadic(self, ins: Instr, x, d):
+        # N operands, N init values, a reducer of 2N parameters (accumulators first) returning an N-tuple
+        # (ir_parser_fused.cc:1169-1213: tuple functors, e.g. (value, index) for arg-max); elements are
+        # combined in ascending order of the reduced dimension
+        n = len(x) // 2
+        red = self.mod["comps"][ins.attrs["to_apply"].lstrip("%")]
+        out_dims = [e for i, e in enumerate(x[0].shape) if i != d]
+        acc = []
+        for i in range(n):
+            a = np.empty(out_dims, x[i].dtype)
+            a[...] = x[n + i]
+            acc.append(a)
+        with np.errstate(all="ignore"):
+            for k in range(x[0].shape[d]):
+                res = self._apply_reducer(red, acc + [np.take(x[i], k, axis=d) for i in range(n)])
+                acc = [np.asarray(r) for r in res]
+        return tuple(a.astype(self.np_dtype(t.dtype), copy=False) for a, t in zip(acc, ins.shape.tuple_shapes))
+
     def _reduce(self, ins: Instr, x, dt):
         dims = _ints(ins.attrs["dimensions"])
+        if len(dims) == 1 and len(x) > 2 and len(x) % 2 == 0:
+            return self._reduce_variadic(ins, x, dims[0])
         if len(dims) != 1 or len(x) != 2:
-            raise NotImplementedError("only single-dimension, single-operand reduce")
+            raise NotImplementedError("only single-dimension reduce")
         red = self.mod["comps"][ins.attrs["to_apply"].lstrip("%")]
         fn = _REDUCERS[red.root.opcode]
         init = x[1]

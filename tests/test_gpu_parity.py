@@ -211,3 +211,51 @@ def test_attention_key_wave_arrangements(gpu_device, key_waves):
     (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, json.dumps(spec))
     assert f"kw = mononn_dev::wave_id() % {key_waves}" in m.get_source("main.hip")
     check_close(got, want)
+
+
+@pytest.mark.parametrize("xd,size,stride,pad", [
+    ((2, 9, 10, 8), (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (1, 1), (1, 1), (0, 0))),
+    ((4, 56, 56, 64), (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (0, 1), (0, 1), (0, 0))),     # ResNet stem pooling
+    ((3, 7, 5, 2), (1, 3, 2, 1), (1, 1, 2, 1), ((0, 0), (1, 1), (0, 1), (0, 0))),
+])
+def test_reduce_window_bit_exact(gpu_device, xd, size, stride, pad):
+    # maximum never rounds; the f16 sum adds the window elements in the order the HLO's evaluation defines (ascending
+    # window offsets, rounding after every add), so both are bit-exact against the oracle run "as written"
+    from op_cases import pool_module
+    x = np.random.default_rng(51).normal(0, 1, xd).astype(np.float16)
+    for kind in ("max", "sum"):
+        text, od = pool_module(xd, size, stride, pad, kind)
+        (got,), _ = run_module(text, [x], {}, [{"dtype": "f16", "dims": od}])
+        want = hlo_interp.evaluate(text, [x], {})[0]
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), kind
+        want32 = hlo_interp.evaluate(text, [x], {}, "fp32")[0]
+        assert np.abs(got.astype(np.float32) - want32).max() <= 2e-2
+
+
+def test_dynamic_update_slice_bit_exact(gpu_device):
+    from op_cases import update_slice_module
+    rng = np.random.default_rng(53)
+    x = rng.normal(0, 1, (6, 10, 8)).astype(np.float16)
+    u = rng.normal(0, 1, (2, 4, 8)).astype(np.float16)
+    for scale in (None, 2.0):
+        text = update_slice_module(x.shape, u.shape, scale=scale)
+        m = MonoNNModule.compile(text)
+        m.load(0)
+        for starts in [(1, 3, 0), (0, 0, 0), (4, 6, 0), (9, -5, 3)]:      # the last one is clamped to (4, 0, 0)
+            ins = [x, u] + [np.array(s, np.int32) for s in starts]
+            (got,) = m.run(ins, [{"dtype": "f16", "dims": list(x.shape)}])
+            want = hlo_interp.evaluate(text, ins, {})[0]
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (scale, starts)
+        m.close()
+
+
+@pytest.mark.parametrize("rows,n,direction", [(7, 50, "GE"), (64, 1000, "GE"), (5, 333, "LE")])
+def test_variadic_reduce_bit_exact(gpu_device, rows, n, direction):
+    # (value, index) reduction: arg-max / arg-min with the first index on ties
+    from op_cases import arg_reduce_module
+    x = np.random.default_rng(57).integers(-6, 7, (rows, n)).astype(np.float16)      # many ties
+    text = arg_reduce_module(rows, n, direction)
+    (v, i), _ = run_module(text, [x], {}, [{"dtype": "f16", "dims": [rows]}, {"dtype": "s32", "dims": [rows]}])
+    wv, wi = hlo_interp.evaluate(text, [x], {})
+    assert np.array_equal(i, wi) and np.array_equal(v.view(np.uint16), wv.view(np.uint16))
+    assert np.array_equal(i, (np.argmax if direction == "GE" else np.argmin)(x, axis=1).astype(np.int32))

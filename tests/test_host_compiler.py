@@ -281,6 +281,29 @@ def test_contraction_length_off_the_mfma_step_still_takes_mfma_tiles():
     assert re.search(r"gemm_tile<\d+, \d+, \d+, \d+, \d+, 197, false, 197,", src)
 
 
+def test_reduce_window_update_slice_and_variadic_reduce_are_lowered():
+    # index maps of index_tracer.cc for reduce-window / dynamic-update-slice, tuple reducers of
+    # reduction_functor_generator.cc:246-283: each is one stage of plain per-element code
+    from op_cases import pool_module, update_slice_module, arg_reduce_module
+    text, od = pool_module((2, 9, 10, 8), (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (1, 1), (1, 1), (0, 0)), "max")
+    m = MonoNNModule.compile(text, build=False)
+    src = m.get_source("main.hip")
+    assert od == [2, 5, 5, 8] and m.buffer_info()["liveouts"] == [2 * 5 * 5 * 8 * 2]
+    assert re.search(r"for \(int w\d+ = 0; w\d+ < 3; \+\+w\d+\)", src) and "* 2 + w" in src and ">= 0 &&" in src
+    # without padding there is no bounds test
+    text, _ = pool_module((1, 8, 8, 4), (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0),) * 4, "sum")
+    assert ">= 0 &&" not in MonoNNModule.compile(text, build=False).get_source("main.hip")
+    src = MonoNNModule.compile(update_slice_module((6, 10, 8), (2, 4, 8)), build=False).get_source("main.hip")
+    assert "min(max((int)" in src and ", 0), 4)" in src and ", 0), 6)" in src and "else" in src     # starts clamped to extent - update
+    src = MonoNNModule.compile(arg_reduce_module(7, 50), build=False).get_source("main.hip")
+    assert "int32_t* out1" in src and re.search(r"for \(int rk\d+ = 0; rk\d+ < 50;", src)
+    # what the reference rejects is rejected here too: window dilation (ir_parser_fused.cc:1246-1250)
+    bad = pool_module((1, 8, 8, 4), (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0),) * 4)[0].replace("stride=1x2x2x1", "stride=1x2x2x1 rhs_dilate=1x2x2x1")
+    with pytest.raises(MonoNNError) as ei:
+        MonoNNModule.compile(bad, build=False)
+    assert "dilation" in str(ei.value)
+
+
 @pytest.mark.parametrize("edit,fragment", [
     (lambda t: t.replace("window={size=16x16 stride=16x16}", "window={size=16x16 stride=16x16 rhs_dilate=2x2}"), "dilated"),
     (lambda t: t.replace("window={size=16x16 stride=16x16}", "window={size=16x16 stride=16x16 pad=0_1x0_0}"), "symmetric"),

@@ -320,3 +320,54 @@ def test_dot_matches_einsum_and_the_gemm_call():
     want = np.einsum("bmk,bnk->bmn", A.astype(np.float64), B.astype(np.float64))
     assert np.abs(got_dot - want).max() < 2e-5
     assert np.array_equal(got_dot, got_gemm)
+
+
+@pytest.mark.parametrize("xd,size,stride,pad", [
+    ((2, 9, 10, 8), (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (1, 1), (1, 1), (0, 0))),
+    ((1, 8, 8, 4), (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0), (0, 0), (0, 0), (0, 0))),
+    ((3, 7, 5, 2), (1, 3, 2, 1), (1, 1, 2, 1), ((0, 0), (1, 1), (0, 1), (0, 0))),
+])
+def test_reduce_window_matches_torch_pooling(xd, size, stride, pad):
+    # max pooling against the library routine (padding = -inf); sum pooling against avg_pool2d * window size with
+    # zero padding counted in (padding = the init value 0)
+    from op_cases import pool_module
+    rng = np.random.default_rng(41)
+    x = rng.normal(0, 1, xd).astype(np.float16)
+    t = torch.tensor(x.astype(np.float32)).permute(0, 3, 1, 2)
+    sym = all(lo == hi for lo, hi in pad)
+    text, od = pool_module(xd, size, stride, pad, "max")
+    got = hlo_interp.evaluate(text, [x], {}, "fp32")[0]
+    tp = F.pad(t, (pad[2][0], pad[2][1], pad[1][0], pad[1][1]), value=float("-inf"))
+    want = F.max_pool2d(tp, size[1:3], stride[1:3]).permute(0, 2, 3, 1).numpy()
+    assert list(got.shape) == od == list(want.shape)
+    assert np.array_equal(got, want)
+    text, _ = pool_module(xd, size, stride, pad, "sum", dtype="f32")
+    got = hlo_interp.evaluate(text, [x.astype(np.float32)], {}, "fp32")[0]
+    tz = F.pad(t, (pad[2][0], pad[2][1], pad[1][0], pad[1][1]), value=0.0)
+    want = (F.avg_pool2d(tz, size[1:3], stride[1:3]) * (size[1] * size[2])).permute(0, 2, 3, 1).numpy()
+    assert np.abs(got - want).max() < 1e-5
+    assert sym or got.shape == want.shape
+
+
+def test_dynamic_update_slice_matches_numpy_assignment_with_clamped_starts():
+    from op_cases import update_slice_module
+    rng = np.random.default_rng(43)
+    x = rng.normal(0, 1, (6, 10, 8)).astype(np.float16)
+    u = rng.normal(0, 1, (2, 4, 8)).astype(np.float16)
+    text = update_slice_module(x.shape, u.shape)
+    for starts in [(1, 3, 0), (0, 0, 0), (4, 6, 0), (9, -5, 3)]:      # the last one is clamped to (4, 0, 0)
+        got = hlo_interp.evaluate(text, [x, u] + [np.array(s, np.int32) for s in starts], {})[0]
+        s = [min(max(v, 0), n - m) for v, n, m in zip(starts, x.shape, u.shape)]
+        want = x.copy()
+        want[s[0]:s[0] + 2, s[1]:s[1] + 4, s[2]:s[2] + 8] = u
+        assert np.array_equal(got, want)
+
+
+def test_variadic_reduce_is_argmax_with_first_index_on_ties():
+    from op_cases import arg_reduce_module
+    rng = np.random.default_rng(47)
+    x = rng.integers(-4, 5, (7, 50)).astype(np.float16)      # many ties
+    v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "GE"), [x], {})
+    assert np.array_equal(i, np.argmax(x, axis=1).astype(np.int32)) and np.array_equal(v, x.max(axis=1))
+    v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "LE"), [x], {})
+    assert np.array_equal(i, np.argmin(x, axis=1).astype(np.int32)) and np.array_equal(v, x.min(axis=1))
