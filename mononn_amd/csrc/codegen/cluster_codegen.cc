@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <functional>
 #include <set>
 #include <regex>
 #include <sstream>
@@ -49,7 +50,10 @@ RowInfo analyze_rows(const std::vector<const Instr*>& members) {
   info.row_program = true;
   for (auto* r : reds) {
     const hlo::Shape& x = r->operands[0]->shape;
-    bool ok = r->operands.size() == 2 && r->dimensions.size() == 1 && x.rank() >= 1 && r->dimensions[0] == x.rank() - 1;
+    // one operand and its init value, or N of each with a tuple-valued reducer ((value, index) reductions)
+    bool arity = r->operands.size() == 2 || (r->operands.size() > 2 && r->operands.size() % 2 == 0 && r->shape.is_tuple() &&
+                                              r->shape.tuple.size() == r->operands.size() / 2);
+    bool ok = arity && r->dimensions.size() == 1 && x.rank() >= 1 && r->dimensions[0] == x.rank() - 1;
     if (!ok) {
       info.row_program = false;
       break;
@@ -202,6 +206,88 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       if (block_tier) cb.line(acc + " = mononn_dev::block_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ", reinterpret_cast<" + T + "*>(smem));");
       else cb.line(acc + " = mononn_dev::wave_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
     };
+    // Tuple-valued reductions: N accumulators, the reducer computation inlined for every element and, as a local
+    // lambda, for the exchange between lanes and waves.  The lanes combine disjoint column sets in a butterfly, so
+    // the reducer has to be associative and commutative (XLA's contract for reduce), as arg-max with the
+    // first-index tie rule is.
+    struct TupleAcc {
+      std::vector<std::string> acc, types;
+    };
+    auto tuple_begin = [&](const Instr* r) {
+      TupleAcc ta;
+      const size_t n = r->operands.size() / 2;
+      for (size_t i = 0; i < n; ++i) {
+        ta.types.push_back(hlo::dtype_ctype(r->shape.tuple[i].dtype));
+        ta.acc.push_back(em.fresh("red"));
+        cb.line(ta.types[i] + " " + ta.acc[i] + " = " + em.value(r->operands[n + i], {}) + ";");
+      }
+      return ta;
+    };
+    // acc = reducer(acc, element) ; `guard` (may be empty) keeps the accumulators where it is false
+    auto tuple_update = [&](const Instr* r, const TupleAcc& ta, const std::vector<std::string>& vals, const std::string& guard) {
+      const size_t n = ta.acc.size();
+      std::vector<std::string> args = ta.acc;
+      args.insert(args.end(), vals.begin(), vals.end());
+      std::vector<std::string> res = em.inline_scalar_computation(r->called, args);
+      MONONN_CHECK(res.size() == n, kUnsupported) << r->hlo_name << ": the reducer yields " << res.size() << " values for " << n << " operands";
+      std::vector<std::string> tmp;
+      for (size_t i = 0; i < n; ++i) {
+        tmp.push_back(em.fresh("nx"));
+        cb.line("const " + ta.types[i] + " " + tmp[i] + " = (" + ta.types[i] + ")" + res[i] + ";");
+      }
+      for (size_t i = 0; i < n; ++i) cb.line(ta.acc[i] + " = " + (guard.empty() ? tmp[i] : guard + " ? " + tmp[i] + " : " + ta.acc[i]) + ";");
+    };
+    auto tuple_all_reduce = [&](const Instr* r, const TupleAcc& ta) {
+      const size_t n = ta.acc.size();
+      std::string comb = em.fresh("comb");
+      std::string params;
+      std::vector<std::string> a, b;
+      for (size_t i = 0; i < n; ++i) {
+        a.push_back("a" + S(i));
+        b.push_back("b" + S(i));
+        params += (i ? ", " : "") + ta.types[i] + "& a" + S(i);
+      }
+      for (size_t i = 0; i < n; ++i) params += ", const " + ta.types[i] + " b" + S(i);
+      cb.open("auto " + comb + " = [](" + params + ")");
+      {
+        TupleAcc inner{a, ta.types};
+        tuple_update(r, inner, b, "");
+      }
+      cb.close(";");
+      auto call = [&](const std::function<std::string(size_t)>& other) {
+        std::string args;
+        for (size_t i = 0; i < n; ++i) args += (i ? ", " : "") + ta.acc[i];
+        for (size_t i = 0; i < n; ++i) args += ", " + other(i);
+        return comb + "(" + args + ");";
+      };
+      cb.line("#pragma unroll");
+      cb.open("for (int off = 32; off >= 1; off >>= 1)");
+      cb.line(call([&](size_t i) { return "mononn_dev::lane_xor(" + ta.acc[i] + ", off)"; }));
+      cb.close();
+      if (!block_tier) return;
+      // across the waves: every wave leaves its tuple in LDS (member i at byte offset i * NW * 8), then every thread
+      // folds them in wave order
+      auto slot = [&](size_t i, const std::string& w) { return "reinterpret_cast<" + ta.types[i] + "*>(smem + " + S(static_cast<int64_t>(i) * NW * 8) + ")[" + w + "]"; };
+      cb.line("__syncthreads();");
+      cb.open("if (lane == 0)");
+      for (size_t i = 0; i < n; ++i) cb.line(slot(i, "mononn_dev::wave_id()") + " = " + ta.acc[i] + ";");
+      cb.close();
+      cb.line("__syncthreads();");
+      for (size_t i = 0; i < n; ++i) cb.line(ta.acc[i] + " = " + slot(i, "0") + ";");
+      cb.open("for (int w = 1; w < " + S(NW) + "; ++w)");
+      cb.line(call([&](size_t i) { return slot(i, "w"); }));
+      cb.close();
+    };
+    auto tuple_bind = [&](const Instr* r, const TupleAcc& ta) {
+      for (auto* u : r->users) {
+        MONONN_CHECK(u->opcode == "get-tuple-element" && u->tuple_index >= 0 && static_cast<size_t>(u->tuple_index) < ta.acc.size(), kUnsupported)
+            << r->hlo_name << ": a tuple-valued reduce is read through get-tuple-element only";
+        em.bind(u, leading_index(row, ROWS, u->shape.dims, vars), ta.acc[u->tuple_index]);
+      }
+    };
+    size_t max_tuple = 1;
+    for (auto* r : em.collect_reduces())
+      if (r->shape.is_tuple()) max_tuple = std::max(max_tuple, r->shape.tuple.size());
     auto operand_index = [&](const Instr* x, const LinExpr& col) {
       std::vector<int64_t> lead(x->shape.dims.begin(), x->shape.dims.end() - 1);
       Index xi = leading_index(row, ROWS, lead, vars);
@@ -241,6 +327,19 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       }
       auto col_of = [&](int64_t k, int v) { return LinExpr::variable(qvar[k], NQ).scaled(V).plus_const(v); };
       for (auto* r : em.collect_reduces()) {
+        if (r->shape.is_tuple()) {
+          TupleAcc ta = tuple_begin(r);
+          const size_t n = ta.acc.size();
+          for (int64_t k = 0; k < T; ++k)
+            for (int v = 0; v < V; ++v) {
+              std::vector<std::string> vals;
+              for (size_t i = 0; i < n; ++i) vals.push_back(em.value(r->operands[i], operand_index(r->operands[i], col_of(k, v))));
+              tuple_update(r, ta, vals, partial[k] ? "act" + S(k) : "");
+            }
+          tuple_all_reduce(r, ta);
+          tuple_bind(r, ta);
+          continue;
+        }
         std::string Tn = hlo::dtype_ctype(r->shape.dtype);
         std::string acc = em.fresh("red");
         cb.line(Tn + " " + acc + " = " + em.value(r->operands[1], {}) + ";");
@@ -291,6 +390,19 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       int col = vars.add("col", R);
       const std::string col_loop = "for (int col = tid; col < " + S(R) + "; col += " + S(stride) + ")";
       for (auto* r : em.collect_reduces()) {
+        if (r->shape.is_tuple()) {
+          TupleAcc ta = tuple_begin(r);
+          cb.open(col_loop);
+          em.push_scope();
+          std::vector<std::string> vals;
+          for (size_t i = 0; i < ta.acc.size(); ++i) vals.push_back(em.value(r->operands[i], operand_index(r->operands[i], LinExpr::variable(col, R))));
+          tuple_update(r, ta, vals, "");
+          em.pop_scope();
+          cb.close();
+          tuple_all_reduce(r, ta);
+          tuple_bind(r, ta);
+          continue;
+        }
         std::string Tn = hlo::dtype_ctype(r->shape.dtype);
         std::string acc = em.fresh("red");
         cb.line(Tn + " " + acc + " = " + em.value(r->operands[1], {}) + ";");
@@ -318,7 +430,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     }
     cb.close();
     int64_t units = block_tier ? ROWS : (ROWS + NW - 1) / NW;
-    return finish(T * V <= 32 ? hoist_row_loads(cb.text()) : cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 : 0);
+    return finish(T * V <= 32 ? hoist_row_loads(cb.text()) : cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 * static_cast<int>(max_tuple) : 0);
   }
 
   // element-wise loop(s); outputs of equal element count share one loop.  A thread owns V consecutive

@@ -77,6 +77,10 @@ class Emitter {
   // the instruction computing output `i` of an entry-level member (fusion root / tuple element)
   const hlo::Instr* resolve_output(const hlo::Instr* entry_value) const;
 
+  // the scalar computation `c` with its parameters replaced by the C expressions `args`: C expressions of its results
+  // (the statements they need are written to the code buffer)
+  std::vector<std::string> inline_scalar_computation(const hlo::Computation* c, const std::vector<std::string>& args);
+
   static std::string literal(const hlo::Instr* c);                    // scalar constant as C literal
   static std::string literal_of(hlo::DType t, const std::string& text);
   static std::string reducer_expr(const hlo::Instr* reduce, const std::string& a, const std::string& b);
@@ -93,8 +97,6 @@ class Emitter {
   std::string serial_reduce(const hlo::Instr* ins, const Index& idx);
   // N-operand reduce with a tuple-valued reducer: one loop for all N results, which are returned in tuple order
   std::vector<std::string> serial_reduce_variadic(const hlo::Instr* ins, const Index& idx);
-  // the scalar computation `c` with its parameters replaced by the C expressions `args`: C expressions of its results
-  std::vector<std::string> inline_scalar_computation(const hlo::Computation* c, const std::vector<std::string>& args);
   std::string key(const hlo::Instr* ins, const Index& idx) const;
   std::string def(hlo::DType t, const std::string& rhs);
   bool is_member(const hlo::Instr* v) const { return members_.count(v) > 0; }

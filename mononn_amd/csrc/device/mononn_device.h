@@ -202,6 +202,27 @@ __device__ __forceinline__ T wave_all_reduce(T v, Op op) {
   }
 }
 
+// value of `v` in lane (own lane ^ mask), for any type of up to 8 bytes (tuple reductions exchange every member)
+template <class T>
+__device__ __forceinline__ T lane_xor(T v, int mask) {
+  static_assert(sizeof(T) <= 8, "lane exchange of at most 8 bytes");
+  if constexpr (sizeof(T) <= 4) {
+    int b = 0;
+    __builtin_memcpy(&b, &v, sizeof(T));
+    b = __shfl_xor(b, mask, kWaveSize);
+    T r;
+    __builtin_memcpy(&r, &b, sizeof(T));
+    return r;
+  } else {
+    long long b;
+    __builtin_memcpy(&b, &v, 8);
+    b = __shfl_xor(b, mask, kWaveSize);
+    T r;
+    __builtin_memcpy(&r, &b, 8);
+    return r;
+  }
+}
+
 // `scratch` holds at least blockDim.x / 64 elements of T in LDS
 template <class T, class Op>
 __device__ __forceinline__ T block_all_reduce(T v, Op op, T* scratch) {

@@ -335,9 +335,19 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       std::map<std::string, std::string> files;
       std::string tu = trials[live[0]].mod->hip_program().preamble;
       std::set<std::string> decls;
+      // candidates that differ in their number of profiled stages (a split adds one) declare stamp arrays of different
+      // lengths: the translation unit gets the longest
+      const std::string clock_decl = "__device__ unsigned long long mononn_stage_clock[";
+      size_t clock_len = 0;
       for (size_t i : live)
-        for (auto& d : trials[i].mod->hip_program().global_decls)
+        for (auto& d : trials[i].mod->hip_program().global_decls) {
+          if (d.compare(0, clock_decl.size(), clock_decl) == 0) {
+            clock_len = std::max<size_t>(clock_len, std::strtoull(d.c_str() + clock_decl.size(), nullptr, 10));
+            continue;
+          }
           if (decls.insert(d).second) tu += d + "\n";
+        }
+      if (clock_len > 0) tu += clock_decl + std::to_string(clock_len) + "];\n";
       for (size_t i : live) tu += "namespace cand_" + std::to_string(i) + " {\n" + trials[i].mod->hip_program().body + "}\n";
       files["headers.h"] = trials[live[0]].mod->hip_program().files.at("headers.h");
       files["main.hip"] = tu;

@@ -386,8 +386,10 @@ class HloModuleBuilder:
         return self._reducers[key]
 
     def arg_reducer(self, direction: str, dtype: str, index_dtype: str = "s32") -> str:
-        """(value, index) reducer: keeps the larger (direction GE/GT) or smaller (LE/LT) value, and on
-        equal values the smaller index -- the form XLA gives tf.argmax / tf.argmin."""
+        """(value, index) reducer: keeps the larger (direction GT) or smaller (LT) value, and on equal values the
+        smaller index -- the form XLA gives tf.argmax / tf.argmin.  With GT / LT the reducer is commutative, which a
+        reduction spread over lanes needs; GE / LE keep the accumulator on ties whatever its index and only mean
+        "first index" when the elements arrive in ascending order."""
         key = ("arg", direction, dtype, index_dtype)
         if key not in self._reducers:
             c = Computation(self, self.fresh(f"arg_{direction.lower()}_{dtype}_reducer"))

@@ -35,18 +35,20 @@ def update_slice_module(xd, ud, dtype="f16", scale=None):
     return mb.text()
 
 
-def arg_reduce_module(rows, n, direction="GE", dtype="f16"):
-    """(value, index) of the largest (GE) / smallest (LE) element of every row, first one on ties."""
+def arg_reduce_module(rows, n, direction="GT", dtype="f16", axis=1):
+    """(value, index) of the largest (GT) / smallest (LT) element along `axis` of a [rows, n] (axis 1) or [n, rows]
+    (axis 0) matrix, first one on ties."""
     mb = HloModuleBuilder("cluster_10__argmax.1")
     e = mb.entry
-    x = e.parameter(dtype, (rows, n), "x")
+    xd = (rows, n) if axis == 1 else (n, rows)
+    x = e.parameter(dtype, xd, "x")
     red = mb.arg_reducer(direction, dtype)
 
     def body(f, p):
-        idx = f.iota("s32", (rows, n), 1)
+        idx = f.iota("s32", xd, axis)
         init_v = f.scalar(dtype, float("-inf") if direction in ("GE", "GT") else float("inf"))
         init_i = f.scalar("s32", 0)
-        return f.reduce_variadic([p, idx], [init_v, init_i], 1, red)
+        return f.reduce_variadic([p, idx], [init_v, init_i], axis, red)
     vals = e.fusion("kInput", [x], body)
     e.set_tuple_root(list(vals))
     return mb.text()

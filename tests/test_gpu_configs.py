@@ -170,3 +170,14 @@ def test_vit_full_size_properties(gpu_device):
     assert np.array_equal(out_rev[::-1], out)
     assert np.array_equal(m.run(inputs, fx.outputs)[0], out)
     m.close()
+    # the tuned specification shipped for this configuration computes the same function (other tiles, other
+    # summation orders: tolerance of two fp16 evaluations of one model)
+    import os
+    from mononn_amd import MonoNNModule, binding
+    spec_dir = os.path.join(os.path.dirname(binding.__file__), "specs", "vit_b16_b8")
+    if os.path.isdir(spec_dir):
+        t = MonoNNModule.from_spec_dir(fx.hlo_text, spec_dir)
+        t.set_constants(consts)
+        t.load(gpu_device)
+        _check(t.run(inputs, fx.outputs)[0], out.astype(np.float32), "vit tuned vs default")
+        t.close()

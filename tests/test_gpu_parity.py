@@ -249,13 +249,21 @@ def test_dynamic_update_slice_bit_exact(gpu_device):
         m.close()
 
 
-@pytest.mark.parametrize("rows,n,direction", [(7, 50, "GE"), (64, 1000, "GE"), (5, 333, "LE")])
-def test_variadic_reduce_bit_exact(gpu_device, rows, n, direction):
+@pytest.mark.parametrize("rows,n,direction,axis", [
+    (7, 50, "GT", 1),          # one wave per row, partly filled
+    (64, 1000, "GT", 1),       # one workgroup per row, register-resident
+    (5, 333, "LT", 1),
+    (16, 50257, "GT", 1),      # vocabulary-sized rows: column loop, exchange through LDS
+    (40, 50, "GT", 0),         # not the last dimension: serial loop per output element
+])
+def test_variadic_reduce_bit_exact(gpu_device, rows, n, direction, axis):
     # (value, index) reduction: arg-max / arg-min with the first index on ties
     from op_cases import arg_reduce_module
-    x = np.random.default_rng(57).integers(-6, 7, (rows, n)).astype(np.float16)      # many ties
-    text = arg_reduce_module(rows, n, direction)
+    x = np.random.default_rng(57).integers(-6, 7, (rows, n) if axis == 1 else (n, rows)).astype(np.float16)      # many ties
+    text = arg_reduce_module(rows, n, direction, axis=axis)
     (v, i), _ = run_module(text, [x], {}, [{"dtype": "f16", "dims": [rows]}, {"dtype": "s32", "dims": [rows]}])
-    wv, wi = hlo_interp.evaluate(text, [x], {})
-    assert np.array_equal(i, wi) and np.array_equal(v.view(np.uint16), wv.view(np.uint16))
-    assert np.array_equal(i, (np.argmax if direction == "GE" else np.argmin)(x, axis=1).astype(np.int32))
+    assert np.array_equal(i, (np.argmax if direction == "GT" else np.argmin)(x, axis=axis).astype(np.int32))
+    assert np.array_equal(v, x.max(axis=axis) if direction == "GT" else x.min(axis=axis))
+    if n <= 1000:
+        wv, wi = hlo_interp.evaluate(text, [x], {})
+        assert np.array_equal(i, wi) and np.array_equal(v.view(np.uint16), wv.view(np.uint16))

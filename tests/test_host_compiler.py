@@ -281,6 +281,25 @@ def test_contraction_length_off_the_mfma_step_still_takes_mfma_tiles():
     assert re.search(r"gemm_tile<\d+, \d+, \d+, \d+, \d+, 197, false, 197,", src)
 
 
+SHIPPED_SPECS = {"bert_base_b1_s128": models.bert_base, "vit_b16_b8": models.vit, "gpt2_b4_s512": models.gpt2}
+
+
+def test_shipped_specifications_load_against_their_models():
+    # every tuned specification in the package names the nodes of the model fixture it was tuned for: loading it
+    # through the spec-dir path must compile (a renamed node or a tile the generator rejects fails here)
+    root = os.path.join(os.path.dirname(binding.__file__), "specs")
+    found = sorted(os.listdir(root))
+    assert "bert_base_b1_s128" in found and set(found) <= set(SHIPPED_SPECS)
+    for name in found:
+        fx = SHIPPED_SPECS[name]()
+        m = MonoNNModule.from_spec_dir(fx.hlo_text, os.path.join(root, name))
+        spec = json.loads(m.get_tuning_spec())
+        shipped = json.load(open(os.path.join(root, name, "cluster_0", "best_tuning_spec.json")))
+        assert spec["gemm_spec_list"] == shipped["gemm_spec_list"] and spec["mononn_hip"] == shipped["mononn_hip"]
+        assert len(m.get_code_object()) > 0
+        m.close()
+
+
 def test_reduce_window_update_slice_and_variadic_reduce_are_lowered():
     # index maps of index_tracer.cc for reduce-window / dynamic-update-slice, tuple reducers of
     # reduction_functor_generator.cc:246-283: each is one stage of plain per-element code
@@ -295,8 +314,14 @@ def test_reduce_window_update_slice_and_variadic_reduce_are_lowered():
     assert ">= 0 &&" not in MonoNNModule.compile(text, build=False).get_source("main.hip")
     src = MonoNNModule.compile(update_slice_module((6, 10, 8), (2, 4, 8)), build=False).get_source("main.hip")
     assert "min(max((int)" in src and ", 0), 4)" in src and ", 0), 6)" in src and "else" in src     # starts clamped to extent - update
+    # a tuple-valued reduce over the last dimension is a row program (the lanes exchange whole tuples, the reducer is
+    # inlined as a local lambda); over another dimension it is a serial loop of the thread that owns the element
     src = MonoNNModule.compile(arg_reduce_module(7, 50), build=False).get_source("main.hip")
-    assert "int32_t* out1" in src and re.search(r"for \(int rk\d+ = 0; rk\d+ < 50;", src)
+    assert "int32_t* out1" in src and "mononn_dev::lane_xor(" in src and re.search(r"auto comb\d+ = \[\]\(_Float16& a0, int32_t& a1, const _Float16 b0, const int32_t b1\)", src)
+    src = MonoNNModule.compile(arg_reduce_module(64, 2000), build=False).get_source("main.hip")
+    assert "reinterpret_cast<int32_t*>(smem + 32)[w]" in src                         # long rows: one workgroup per row
+    src = MonoNNModule.compile(arg_reduce_module(7, 50, axis=0), build=False).get_source("main.hip")
+    assert "lane_xor" not in src and re.search(r"for \(int rk\d+ = 0; rk\d+ < 50;", src)
     # what the reference rejects is rejected here too: window dilation (ir_parser_fused.cc:1246-1250)
     bad = pool_module((1, 8, 8, 4), (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0),) * 4)[0].replace("stride=1x2x2x1", "stride=1x2x2x1 rhs_dilate=1x2x2x1")
     with pytest.raises(MonoNNError) as ei:

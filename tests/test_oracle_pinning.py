@@ -367,7 +367,7 @@ def test_variadic_reduce_is_argmax_with_first_index_on_ties():
     from op_cases import arg_reduce_module
     rng = np.random.default_rng(47)
     x = rng.integers(-4, 5, (7, 50)).astype(np.float16)      # many ties
-    v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "GE"), [x], {})
+    v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "GT"), [x], {})
     assert np.array_equal(i, np.argmax(x, axis=1).astype(np.int32)) and np.array_equal(v, x.max(axis=1))
-    v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "LE"), [x], {})
+    v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "LT"), [x], {})
     assert np.array_equal(i, np.argmin(x, axis=1).astype(np.int32)) and np.array_equal(v, x.min(axis=1))
