@@ -604,8 +604,8 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
     const int tm = t.bm / std::max(t.wm, 1) / 16, tn = t.bn / std::max(t.wn, 1) / 16;
     const int64_t ksteps = g.K / 32;
     // mirrors mononn_dev::gemm_chunk_steps: with the weights requested ahead of the tile a wave keeps up to 56 fragments
-    const bool wide = t.preload_b && g.b_packed && t.wk >= 1 && ksteps / t.wk * (tm + tn) <= 56;
-    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && (wide || ksteps / t.wk <= 32 / (tm + tn)), kSpecError)
+    const bool wide = t.preload_b && g.b_packed && t.wk >= 1 && ksteps / t.wk * (tm + tn) <= ls.whole_range_fragments();
+    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && (wide || ksteps / t.wk <= ls.chunk_fragments() / (tm + tn)), kSpecError)
         << "GEMM with a row-program prologue: a wave's whole k range (" << ksteps / std::max(t.wk, 1) << " steps) must fit one register chunk";
   }
   MONONN_CHECK(t.split_k >= 1 && (t.split_k == 1 || g.K % (32 * t.split_k) == 0), kSpecError)
@@ -1185,8 +1185,8 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         // the companion repeats the unit decoding as far as the right operand needs it
         const int TM = t.bm / t.wm / 16, TN = t.bn / t.wn / 16;
         const int my_steps = static_cast<int>((KS / 32 + t.wk - 1) / t.wk);
-        const int ch_max = 32 / (TM + TN) > 0 ? 32 / (TM + TN) : 1;   // mirrors mononn_dev::gemm_chunk_steps
-        preload_regs = (my_steps * (TM + TN) <= 56 ? my_steps : std::min(my_steps, ch_max)) * TN;
+        const int ch_max = ls.chunk_fragments() / (TM + TN) > 0 ? ls.chunk_fragments() / (TM + TN) : 1;   // mirrors mononn_dev::gemm_chunk_steps
+        preload_regs = (my_steps * (TM + TN) <= ls.whole_range_fragments() ? my_steps : std::min(my_steps, ch_max)) * TN;
         CodeBuffer pf;
         pf.line("const int bidx = unit / " + S(per_batch) + ";");
         pf.line("const int rem0 = unit % " + S(per_batch) + ";");

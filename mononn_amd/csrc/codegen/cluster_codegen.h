@@ -17,7 +17,12 @@ namespace codegen {
 
 struct LaunchShape {
   int block_size = 256;   // threads per workgroup (multiple of 64)
+  // waves that share a SIMD when the whole grid is resident (grid beyond one workgroup per CU): the register
+  // budget of a wave is 512 / waves_per_simd, and the operand chunks of the GEMM tile shrink with it
+  int waves_per_simd = 1;
   int waves() const { return block_size / 64; }
+  int chunk_fragments() const { return waves_per_simd >= 2 ? 16 : 32; }        // mirrors mononn_dev::gemm_chunk_steps
+  int whole_range_fragments() const { return waves_per_simd >= 2 ? 24 : 56; }
 };
 
 // per-cluster knobs; names follow the reference's cluster_*_spec fields

@@ -71,6 +71,12 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   ls.block_size = spec.runtime.block_dim.x;
   hp.block = ls.block_size;
   hp.grid = spec.runtime.grid_dim.x;
+  {
+    // more workgroups than compute units: they share the CUs' four SIMDs, and the register budget with them
+    const int cus = std::max(spec.device.sm_count, 1);
+    const int per_cu = (hp.grid + cus - 1) / cus;
+    ls.waves_per_simd = std::max(1, (per_cu * ls.waves() + 3) / 4);
+  }
   MONONN_CHECK(hp.grid <= hp.max_grid, kSpecError) << "grid of " << hp.grid << " workgroups exceeds the barrier capacity of " << hp.max_grid;
 
   // every node named by the spec must exist (mononn_module.cc:83-85)
@@ -258,6 +264,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   std::ostringstream pre, glob, src;
   pre << "// generated by mononn-hip for " << spec.device.cuda_arch << "\n";
   pre << "#define MONONN_BLOCK_SIZE " << hp.block << "\n";
+  if (ls.waves_per_simd > 1) pre << "#define MONONN_WAVES_PER_SIMD " << ls.waves_per_simd << "\n";
   if (spec.hip.barrier == "flags_allfence") pre << "#define MONONN_BARRIER_FENCE 1\n";
   else if (spec.hip.barrier == "flags_coherent") pre << "#define MONONN_BARRIER_FENCE 2\n#define MONONN_COHERENT_STORES 1\n";
   else MONONN_CHECK(spec.hip.barrier == "flags", kSpecError) << "unknown barrier flavour '" << spec.hip.barrier << "'";
@@ -338,7 +345,10 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     return o.off ? b + " + " + std::to_string(o.off) : b;
   };
 
-  src << "extern \"C\" __launch_bounds__(" << ls.block_size << ") __global__ void " << kernel_name << "(";
+  // the second bound (waves per SIMD) caps the registers of a wave so that the whole grid stays resident
+  src << "extern \"C\" __launch_bounds__(" << ls.block_size;
+  if (ls.waves_per_simd > 1) src << ", " << ls.waves_per_simd;
+  src << ") __global__ void " << kernel_name << "(";
   for (size_t i = 0; i < hp.param_bytes.size(); ++i) src << "void* arg" << i << ", ";
   for (size_t i = 0; i < hp.liveout_bytes.size(); ++i) src << "void* liveout_buffer_" << i << ", ";
   src << "void* temp_buffer) {\n";

@@ -41,6 +41,10 @@ typedef int int4_t __attribute__((ext_vector_type(4)));
 #ifndef MONONN_COHERENT_STORES
 #define MONONN_COHERENT_STORES 0
 #endif
+// waves that share a SIMD when the whole grid is resident: the kernel is compiled for 512 / this many VGPRs per wave
+#ifndef MONONN_WAVES_PER_SIMD
+#define MONONN_WAVES_PER_SIMD 1
+#endif
 
 namespace mononn_dev {
 
@@ -332,8 +336,9 @@ struct RowMajorA {
 // With the right operand requested ahead of the tile (pre_b) a wave whose whole k range fits into 224 VGPRs takes
 // it as one chunk: there is nothing left to double-buffer.
 __device__ constexpr int gemm_chunk_steps(int TM, int TN, int my_steps, bool pre_b = false) {
-  if (pre_b && my_steps * (TM + TN) <= 56) return my_steps;
-  const int ch_max = 32 / (TM + TN) > 0 ? 32 / (TM + TN) : 1;
+  constexpr int whole = MONONN_WAVES_PER_SIMD >= 2 ? 24 : 56, chunk = MONONN_WAVES_PER_SIMD >= 2 ? 16 : 32;   // half the registers: half the fragments
+  if (pre_b && my_steps * (TM + TN) <= whole) return my_steps;
+  const int ch_max = chunk / (TM + TN) > 0 ? chunk / (TM + TN) : 1;
   return my_steps < ch_max ? my_steps : ch_max;
 }
 

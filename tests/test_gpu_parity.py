@@ -155,6 +155,9 @@ def test_fusion_variants_agree(gpu_device):
         "the same with split-K": _spec_with(fx.hlo_text, hip={"operand_preload": False}, gemm_overrides=split),
         # a grid of 8 workgroups: several units per workgroup and stage, only the first of them behind a barrier wait
         "small grid": _spec_with(fx.hlo_text, grid=8),
+        # two workgroups per compute unit: the kernel is compiled for half the registers per wave, the whole grid
+        # must still be resident for the barrier
+        "two workgroups per compute unit": _spec_with(fx.hlo_text, grid=512),
         # the projection of the merged heads inside the attention stage: one stage less per layer, the LayerNorm
         # stage adds one fp32 partial sum per head
         "output projection inside the attention stage": _spec_with(fx.hlo_text, hip={"attention_out_proj_fusion": True}),

@@ -284,6 +284,23 @@ def test_contraction_length_off_the_mfma_step_still_takes_mfma_tiles():
 SHIPPED_SPECS = {"bert_base_b1_s128": models.bert_base, "vit_b16_b8": models.vit, "gpt2_b4_s512": models.gpt2}
 
 
+def test_register_budget_follows_the_workgroups_per_compute_unit():
+    # a persistent grid must be resident as a whole: with more than one workgroup per CU (or 512-thread workgroups)
+    # two waves share a SIMD, the kernel is compiled for 256 registers per wave and the GEMM tile loads smaller chunks
+    layer = models.bert_layer()
+    base = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
+    assert "__launch_bounds__(256)" in MonoNNModule.compile(layer.hlo_text, build=False).get_source("main.hip")
+    for grid, block, bounds in [(512, 256, "__launch_bounds__(256, 2)"), (256, 512, "__launch_bounds__(512, 2)"), (768, 256, "__launch_bounds__(256, 3)")]:
+        spec = json.loads(json.dumps(base))
+        spec["cuda_context"]["cuda_runtime_context"]["grid_dim"]["x"] = grid
+        spec["cuda_context"]["cuda_runtime_context"]["block_dim"]["x"] = block
+        spec["gemm_spec_list"] = {}
+        spec["cluster_reduce_spec"] = {}
+        spec["cluster_elewise_spec"] = {}
+        src = MonoNNModule.compile(layer.hlo_text, json.dumps(spec), build=False).get_source("main.hip")
+        assert bounds in src and "#define MONONN_WAVES_PER_SIMD " + bounds[-2] in src, (grid, block)
+
+
 def test_shipped_specifications_load_against_their_models():
     # every tuned specification in the package names the nodes of the model fixture it was tuned for: loading it
     # through the spec-dir path must compile (a renamed node or a tile the generator rejects fails here)
