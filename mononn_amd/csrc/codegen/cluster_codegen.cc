@@ -566,7 +566,12 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
   int waves = ls.waves();
   // Large problems: every wave owns a 64x64 (else 32x32) block of the result over the whole k range, no exchange
   // through LDS, as long as that still leaves a tile per compute unit (BERT-large at batch 16: 128x128 tiles run
-  // 2.1x faster than the small-problem default below).
+  // 2.1x faster than the small-problem default below).  Larger blocks per wave (64x128, 128x128) fetch fewer operand
+  // fragments per MFMA and are up to 1.5x faster on such a GEMM alone (its tiles are bound by what the L1
+  // delivers), but inside whole models they made the kernels slower more often than faster (BERT-large 9.9 ->
+  // 11.6 ms: stages whose code did not change, attention and LayerNorm, slow down with them), so they are
+  // neither the default nor tuner candidates (they win the isolated stage clocks and lose in the whole kernel);
+  // a specification may still name them (up to 64 accumulator fragments per wave).
   for (int per_wave : {64, 32}) {
     int wm = 1, wn = waves;
     while (wn > wm) {
@@ -605,7 +610,7 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
     const int64_t ksteps = g.K / 32;
     // mirrors mononn_dev::gemm_chunk_steps: with the weights requested ahead of the tile a wave keeps up to 56 fragments
     const bool wide = t.preload_b && g.b_packed && t.wk >= 1 && ksteps / t.wk * (tm + tn) <= ls.whole_range_fragments();
-    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && (wide || ksteps / t.wk <= ls.chunk_fragments() / (tm + tn)), kSpecError)
+    MONONN_CHECK(t.wk >= 1 && ksteps % t.wk == 0 && tm + tn > 0 && (wide || ksteps / t.wk <= (tm * tn > 32 ? ls.chunk_fragments() / 2 : ls.chunk_fragments()) / (tm + tn)), kSpecError)
         << "GEMM with a row-program prologue: a wave's whole k range (" << ksteps / std::max(t.wk, 1) << " steps) must fit one register chunk";
   }
   MONONN_CHECK(t.split_k >= 1 && (t.split_k == 1 || g.K % (32 * t.split_k) == 0), kSpecError)
@@ -615,7 +620,8 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)
       << "GEMM tile " << t.bm << "x" << t.bn << " is not a multiple of 16 per wave";
   int frags = (t.bm / t.wm / 16) * (t.bn / t.wn / 16);
-  MONONN_CHECK(frags <= 32, kSpecError) << "GEMM tile " << t.bm << "x" << t.bn << " needs " << frags << " accumulator fragments per wave (max 32)";
+  const int max_frags = ls.waves_per_simd >= 2 ? 32 : 64;   // 4 accumulator registers each, out of 512 / waves per SIMD
+  MONONN_CHECK(frags <= max_frags, kSpecError) << "GEMM tile " << t.bm << "x" << t.bn << " needs " << frags << " accumulator fragments per wave (max " << max_frags << ")";
 }
 
 namespace {
@@ -1185,7 +1191,8 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         // the companion repeats the unit decoding as far as the right operand needs it
         const int TM = t.bm / t.wm / 16, TN = t.bn / t.wn / 16;
         const int my_steps = static_cast<int>((KS / 32 + t.wk - 1) / t.wk);
-        const int ch_max = ls.chunk_fragments() / (TM + TN) > 0 ? ls.chunk_fragments() / (TM + TN) : 1;   // mirrors mononn_dev::gemm_chunk_steps
+        const int chunk = TM * TN > 32 ? ls.chunk_fragments() / 2 : ls.chunk_fragments();
+        const int ch_max = chunk / (TM + TN) > 0 ? chunk / (TM + TN) : 1;   // mirrors mononn_dev::gemm_chunk_steps
         preload_regs = (my_steps * (TM + TN) <= ls.whole_range_fragments() ? my_steps : std::min(my_steps, ch_max)) * TN;
         CodeBuffer pf;
         pf.line("const int bidx = unit / " + S(per_batch) + ";");

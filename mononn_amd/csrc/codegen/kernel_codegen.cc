@@ -3,6 +3,7 @@
 #include "codegen/host_codegen.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <set>
 #include <sstream>
 

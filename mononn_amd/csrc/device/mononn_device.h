@@ -336,8 +336,9 @@ struct RowMajorA {
 // With the right operand requested ahead of the tile (pre_b) a wave whose whole k range fits into 224 VGPRs takes
 // it as one chunk: there is nothing left to double-buffer.
 __device__ constexpr int gemm_chunk_steps(int TM, int TN, int my_steps, bool pre_b = false) {
-  constexpr int whole = MONONN_WAVES_PER_SIMD >= 2 ? 24 : 56, chunk = MONONN_WAVES_PER_SIMD >= 2 ? 16 : 32;   // half the registers: half the fragments
+  constexpr int whole = MONONN_WAVES_PER_SIMD >= 2 ? 24 : 56, chunk0 = MONONN_WAVES_PER_SIMD >= 2 ? 16 : 32;   // half the registers: half the fragments
   if (pre_b && my_steps * (TM + TN) <= whole) return my_steps;
+  const int chunk = TM * TN > 32 ? chunk0 / 2 : chunk0;   // more than 128 accumulator registers: smaller operand chunks
   const int ch_max = chunk / (TM + TN) > 0 ? chunk / (TM + TN) : 1;
   return my_steps < ch_max ? my_steps : ch_max;
 }
