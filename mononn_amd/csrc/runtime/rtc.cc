@@ -1,5 +1,8 @@
 #include "runtime/rtc.h"
 
+#include <cstdlib>
+#include <sstream>
+
 #include <hip/hiprtc.h>
 
 #include "common/status.h"
@@ -25,6 +28,12 @@ CompileResult compile_hip(const std::map<std::string, std::string>& files, const
                                    // keep the compiler from forming packed fp32 instructions
                                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
   for (auto& o : extra_options) opts.push_back(o);
+  // extra compiler options, blank separated (e.g. "-mllvm -amdgpu-sched-strategy=max-ilp")
+  if (const char* x = std::getenv("MONONN_HIPRTC_FLAGS")) {
+    std::istringstream is(x);
+    std::string tok;
+    while (is >> tok) opts.push_back(tok);
+  }
   std::vector<const char*> copts;
   for (auto& o : opts) copts.push_back(o.c_str());
   r = hiprtcCompileProgram(prog, static_cast<int>(copts.size()), copts.data());
