@@ -156,11 +156,15 @@ std::string hoist_row_loads(const std::string& text, bool prologue = false) {
   for (size_t i = 0; i < lines.size(); ++i)
     if (std::regex_match(lines[i], q_def)) anchor = static_cast<int>(i);
   if (anchor < 0) return text;
+  // Only loads of the straight-line part move: one that sits under a condition (the branches of a concatenate, a pad,
+  // a window's bounds test) is guarded by it, and its address is out of range exactly where the condition is false.
+  auto indent_of = [](const std::string& l) { return l.find_first_not_of(' '); };
+  const size_t base_indent = indent_of(lines[anchor]);
   std::vector<std::string> hoisted, rest;
   for (size_t i = static_cast<size_t>(anchor) + 1; i < lines.size(); ++i) {
     std::smatch m;
     bool hoist = false;
-    if (std::regex_match(lines[i], m, v_def)) {
+    if (indent_of(lines[i]) == base_indent && std::regex_match(lines[i], m, v_def)) {
       const std::string rhs = m[1].str();
       hoist = rhs.find('[') != std::string::npos;
       // in front of a GEMM registers are scarce (operand fragments are resident): only the partial sums of a split

@@ -250,13 +250,13 @@ std::string Emitter::load(const Instr* root, const Index& idx) {
     std::string sum;
     for (int i = 0; i < sk->second; ++i) {
       std::string ref = p + "[" + lin.plus_const(i * E).str(vars_) + "]";
-      if (lin.opaques().empty()) simple_loads_.emplace_back(ref, "float");
+      if (lin.opaques().empty() && guarded_ == 0) simple_loads_.emplace_back(ref, "float");
       sum += (i ? " + " : "") + def(DType::kF32, ref);
     }
     return def(root->shape.dtype, "(" + std::string(hlo::dtype_ctype(root->shape.dtype)) + ")(" + sum + ")");
   }
   std::string ref = ptrs_.input(root) + "[" + lin.str(vars_) + "]";
-  if (lin.opaques().empty()) simple_loads_.emplace_back(ref, hlo::dtype_ctype(root->shape.dtype));
+  if (lin.opaques().empty() && guarded_ == 0) simple_loads_.emplace_back(ref, hlo::dtype_ctype(root->shape.dtype));
   return def(root->shape.dtype, ref);
 }
 
@@ -273,6 +273,7 @@ std::string Emitter::serial_reduce(const Instr* ins, const Index& idx) {
   out_.line(t + " " + acc + " = " + init + ";");
   int var = vars_.add(rk, R);
   out_.open("for (int " + rk + " = 0; " + rk + " < " + std::to_string(R) + "; ++" + rk + ")");
+  ++guarded_;
   push_scope();
   Index xi;
   for (int i = 0, j = 0; i < x->shape.rank(); ++i) {
@@ -282,6 +283,7 @@ std::string Emitter::serial_reduce(const Instr* ins, const Index& idx) {
   std::string v = value(x, xi);
   out_.line(acc + " = (" + t + ")" + reducer_expr(ins, acc, v) + ";");
   pop_scope();
+  --guarded_;
   out_.close();
   return acc;
 }
@@ -332,6 +334,7 @@ std::vector<std::string> Emitter::serial_reduce_variadic(const Instr* ins, const
   std::string rk = fresh("rk");
   int var = vars_.add(rk, R);
   out_.open("for (int " + rk + " = 0; " + rk + " < " + std::to_string(R) + "; ++" + rk + ")");
+  ++guarded_;
   push_scope();
   Index xi;
   for (int i = 0, j = 0; i < x0->shape.rank(); ++i) {
@@ -350,6 +353,7 @@ std::vector<std::string> Emitter::serial_reduce_variadic(const Instr* ins, const
   }
   for (size_t i = 0; i < n; ++i) out_.line(acc[i] + " = " + tmp[i] + ";");
   pop_scope();
+  --guarded_;
   out_.close();
   std::string joined;
   for (auto& a : acc) joined += a + " ";
@@ -453,11 +457,13 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
       std::string head = (k == 0 ? "if (" : "else if (") + e + " < " + std::to_string(off + n) + ")";
       if (last) head = k == 0 ? "" : "else";
       out_.open(head);
+      ++guarded_;
       push_scope();
       Index xi = idx;
       xi[d] = idx[d].plus_const(-off);
       out_.line(v + " = " + value(x, xi) + ";");
       pop_scope();
+      --guarded_;
       out_.close();
       off += n;
     }
@@ -479,9 +485,11 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
     std::string v = fresh();
     out_.line(T + " " + v + " = " + padv + ";");
     out_.open("if (" + cond + ")");
+    ++guarded_;
     push_scope();
     out_.line(v + " = " + value(x, xi) + ";");
     pop_scope();
+    --guarded_;
     out_.close();
     return v;
   }
@@ -539,14 +547,18 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
     std::string v = fresh();
     out_.line(T + " " + v + ";");
     out_.open("if (" + cond + ")");
+    ++guarded_;
     push_scope();
     out_.line(v + " = " + value(u, ui) + ";");
     pop_scope();
+    --guarded_;
     out_.close();
     out_.open("else");
+    ++guarded_;
     push_scope();
     out_.line(v + " = " + value(x, idx) + ";");
     pop_scope();
+    --guarded_;
     out_.close();
     return v;
   }
@@ -564,6 +576,7 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
       if (ins->window_size[i] == 1) continue;
       w[i] = fresh("w");
       out_.open("for (int " + w[i] + " = 0; " + w[i] + " < " + std::to_string(ins->window_size[i]) + "; ++" + w[i] + ")");
+      ++guarded_;
       ++opened;
     }
     push_scope();
@@ -587,13 +600,16 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
       v = fresh();
       out_.line(T + " " + v + " = " + init + ";");
       out_.open("if (" + cond + ")");
+      ++guarded_;
       push_scope();
       out_.line(v + " = " + value(x, xi) + ";");
       pop_scope();
+      --guarded_;
       out_.close();
     }
     out_.line(acc + " = (" + T + ")" + reducer_expr(ins, acc, v) + ";");
     pop_scope();
+    guarded_ -= opened;
     for (int i = 0; i < opened; ++i) out_.close();
     return acc;
   }

@@ -88,7 +88,8 @@ class Emitter {
   // device-global arrays for non-scalar literal constants met inside fused computations
   const std::map<std::string, std::string>& literal_tables() const { return literal_tables_; }
   // "ptr[index]" of every plain load emitted so far whose index only involves loop variables
-  // loads whose address depends on the loop variables only, as (reference text, C type), in emission order
+  // loads whose address depends on the loop variables only, as (reference text, C type), in emission order; loads
+  // emitted under a condition or inside a loop of the emitter's own are left out: they may only run where they stand
   const std::vector<std::pair<std::string, std::string>>& simple_loads() const { return simple_loads_; }
 
  private:
@@ -117,6 +118,7 @@ class Emitter {
   std::map<std::string, std::string> literal_tables_;
   std::vector<std::pair<std::string, std::string>> simple_loads_;
   int counter_ = 0;
+  int guarded_ = 0;   // scopes (conditions, loops) this emitter has opened and not yet closed
 };
 
 }  // namespace codegen

@@ -1,0 +1,105 @@
+"""Bounds check of generated kernels on the CPU: the generated translation unit of a module made of element-wise and
+row-program stages is compiled for the host against tests/cpu_shim/headers.h and run thread by thread with every
+buffer placed against inaccessible guard pages, once flush with the page before it (catches reads in front of a
+buffer) and once flush with the page behind it (catches reads past its end).  An out-of-range access ends the run
+with the buffer, the offset and the thread that made it."""
+import json
+import os
+import subprocess
+import tempfile
+
+from mononn_amd import MonoNNModule
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CLANG = "/opt/rocm/lib/llvm/bin/clang++"
+
+DRIVER = r"""
+#include <csignal>
+#include <cstdio>
+#include <cstdlib>
+#include <sys/mman.h>
+#include <unistd.h>
+#include "headers.h"
+Dim3 threadIdx, blockIdx, gridDim, blockDim;
+extern "C" { alignas(16) char smem[1 << 17]; }
+#include "main.hip"
+
+struct Buf { const char* name; size_t bytes; char* base; char* lo; char* hi; };
+static Buf bufs[%(nbuf)d];
+static const size_t kGuard = size_t(64) << 20;
+static void on_fault(int, siginfo_t* si, void*) {
+  char* a = static_cast<char*>(si->si_addr);
+  for (auto& b : bufs)
+    if (a >= b.lo && a < b.hi) {
+      std::fprintf(stderr, "OUT OF BOUNDS: %%s (%%zu bytes) at byte offset %%ld, block %%u thread %%u\n", b.name, b.bytes, long(a - b.base), blockIdx.x, threadIdx.x);
+      _exit(3);
+    }
+  std::fprintf(stderr, "FAULT at %%p outside every buffer's guard range, block %%u thread %%u\n", (void*)a, blockIdx.x, threadIdx.x);
+  _exit(4);
+}
+int main(int argc, char** argv) {
+  const bool at_end = argc > 1 && argv[1][0] == 'e';
+  const char* names[] = {%(names)s};
+  const size_t sizes[] = {%(sizes)s};
+  const long page = sysconf(_SC_PAGESIZE);
+  for (int i = 0; i < %(nbuf)d; ++i) {
+    const size_t body = (std::max<size_t>(sizes[i], 1) + page - 1) / page * page;
+    char* r = static_cast<char*>(mmap(nullptr, body + 2 * kGuard, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0));
+    if (r == MAP_FAILED) { std::perror("mmap"); return 2; }
+    mprotect(r + kGuard, body, PROT_READ | PROT_WRITE);
+    char* base = at_end ? r + kGuard + ((body - sizes[i]) & ~size_t(15)) : r + kGuard;
+    for (size_t k = 0; k < sizes[i]; ++k) base[k] = char(k * 7 + i);     // finite halves, small integers as indices
+    bufs[i] = {names[i], sizes[i], base, r, r + body + 2 * kGuard};
+  }
+  struct sigaction sa = {};
+  sa.sa_sigaction = on_fault;
+  sa.sa_flags = SA_SIGINFO;
+  sigaction(SIGSEGV, &sa, nullptr);
+  sigaction(SIGBUS, &sa, nullptr);
+  gridDim.x = %(grid)d;
+  blockDim.x = %(block)d;
+  for (unsigned b = 0; b < %(grid)du; ++b)
+    for (unsigned t = 0; t < %(block)du; ++t) {
+      blockIdx.x = b;
+      threadIdx.x = t;
+      %(kernel)s(%(args)s);
+    }
+  std::printf("ok\n");
+  return 0;
+}
+"""
+
+
+def check_module(hlo_text, spec_json=None, workdir=None):
+    """Returns (ok, message)."""
+    m = MonoNNModule.compile(hlo_text, spec_json, build=False)
+    src = m.get_source("main.hip")
+    if "gemm_tile<" in src or "gemm_naive_element" in src or "mfma" in src:
+        raise ValueError("the host shim covers element-wise and row-program stages only")
+    info, dims = m.buffer_info(), m.launch_dims()
+    names, sizes = [], []
+    for i, b in enumerate(info["parameters"]):
+        names.append(f"parameter {i}")
+        sizes.append(b)
+    for i, b in enumerate(info["liveouts"]):
+        names.append(f"live-out {i}")
+        sizes.append(b)
+    names.append("temp arena")
+    sizes.append(max(info["temp"], 16))
+    tmp = workdir or tempfile.mkdtemp(prefix="mononn_cpu_bounds_")
+    open(os.path.join(tmp, "main.hip"), "w").write(src)
+    drv = DRIVER % {"nbuf": len(names), "names": ", ".join(json.dumps(n) for n in names), "sizes": ", ".join(f"{s}ul" for s in sizes),
+                    "grid": dims["grid"], "block": dims["block"], "kernel": m.kernel_name,
+                    "args": ", ".join(f"bufs[{i}].base" for i in range(len(names)))}
+    open(os.path.join(tmp, "driver.cpp"), "w").write(drv)
+    exe = os.path.join(tmp, "driver")
+    cp = subprocess.run([CLANG, "-x", "c++", "-std=c++17", "-O0", "-w", "-I", os.path.join(HERE, "cpu_shim"), "-I", tmp,
+                         os.path.join(tmp, "driver.cpp"), "-o", exe], capture_output=True, text=True)
+    m.close()
+    if cp.returncode != 0:
+        return False, "host build failed:\n" + cp.stderr[-3000:]
+    for mode in ("start", "end"):
+        r = subprocess.run([exe, mode], capture_output=True, text=True, timeout=300)
+        if r.returncode != 0:
+            return False, f"buffers flush with their {mode}: " + (r.stderr.strip() or f"exit code {r.returncode}")
+    return True, "ok"

@@ -1,0 +1,74 @@
+"""Differential tests on seeded random fused-HLO modules (tests/random_graphs.py): the oracle must evaluate them, the
+host compiler must lower them, and on the GPU the generated kernel must agree with the oracle."""
+import numpy as np
+import pytest
+
+from mononn_amd import MonoNNModule
+from oracle import hlo_interp
+from random_graphs import random_module
+
+SEEDS = list(range(36))
+
+
+def test_random_graphs_are_lowered_and_evaluated():
+    kinds = set()
+    for seed in SEEDS:
+        text, inputs, descs = random_module(seed)
+        want = hlo_interp.evaluate(text, inputs, {})
+        assert [list(w.shape) for w in want] == [d["dims"] for d in descs]
+        assert all(np.isfinite(w.astype(np.float64)).all() for w in want), seed
+        m = MonoNNModule.compile(text, build=False)
+        summary = m.summary()
+        kinds.update(k for k in ("rowred", "elewise") if k in summary)
+        m.close()
+    assert kinds == {"rowred", "elewise"}          # the seeds cover row programs and plain element-wise stages
+
+
+def test_random_graphs_stay_inside_their_buffers():
+    # the generated kernels run thread by thread on the CPU with every buffer against guard pages (tests/cpu_bounds.py)
+    from cpu_bounds import check_module
+    from op_cases import arg_reduce_module, pool_module, update_slice_module
+    cases = [(f"seed {s}", random_module(s)[0]) for s in SEEDS]
+    cases += [("max pooling with padding", pool_module((2, 9, 10, 8), (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (1, 1), (1, 1), (0, 0)))[0]),
+              ("sum pooling, ragged", pool_module((3, 7, 5, 2), (1, 3, 2, 1), (1, 1, 2, 1), ((0, 0), (1, 1), (0, 1), (0, 0)), "sum")[0]),
+              ("dynamic-update-slice", update_slice_module((6, 10, 8), (2, 4, 8), scale=2.0)),
+              ("arg-max, wave per row", arg_reduce_module(7, 50)),
+              ("arg-max, workgroup per row", arg_reduce_module(64, 2000)),
+              ("arg-max over the major dimension", arg_reduce_module(40, 50, axis=0))]
+    for name, text in cases:
+        ok, msg = check_module(text)
+        assert ok, f"{name}: {msg}"
+
+
+def test_loads_under_a_condition_are_not_requested_ahead_of_it():
+    # a row program asks for its operands at the top of the row; a load that sits in a branch of a concatenate is
+    # only in range where the branch is taken and has to stay there
+    text, _, _ = random_module(0)
+    src = MonoNNModule.compile(text, build=False).get_source("main.hip")
+    body = src[src.index("node_fn_0("):]
+    barrier = body.index("__builtin_amdgcn_sched_barrier(0)")
+    first_branch = body.index("if (q0 < ")
+    assert barrier < first_branch
+    assert "+ 247]" not in body[:barrier] and "+ -10]" not in body[:barrier]        # the two halves of the rotated row
+    assert "+ 247]" in body[first_branch:] and "+ -10]" in body[first_branch:]
+
+
+@pytest.mark.gpu
+def test_random_graphs_match_the_oracle(gpu_device):
+    worst = 0.0
+    for seed in SEEDS:
+        text, inputs, descs = random_module(seed)
+        want = hlo_interp.evaluate(text, inputs, {})
+        m = MonoNNModule.compile(text)
+        m.load(gpu_device)
+        got = m.run(inputs, descs)
+        m.close()
+        for g, w in zip(got, want):
+            g64, w64 = g.astype(np.float64), w.astype(np.float64)
+            assert np.isfinite(g64).all(), seed
+            # f16 results: the same rounding points as the oracle run as written, up to fast-math transcendental
+            # functions and the summation order of the f32 row sums
+            err = np.abs(g64 - w64) / (1.0 + np.abs(w64))
+            worst = max(worst, float(err.max()))
+            assert err.max() <= 2e-2, f"seed {seed}: relative error {err.max()} at {np.unravel_index(err.argmax(), err.shape)}"
+    print(f"random graphs: worst relative error {worst:.3e} over {len(SEEDS)} modules")
