@@ -182,6 +182,11 @@ class Computation:
         spec = ", ".join(f"[{s}:{l}]" for s, l in zip(starts, limits))
         return self._emit("slice", x.dtype, dims, [x], attrs="slice={" + spec + "}")
 
+    def pad(self, x: Value, value: Value, low: Sequence[int], high: Sequence[int]) -> Value:
+        """Edge padding without interior padding (ir_parser_fused.cc:1143-1147)."""
+        dims = [lo + n + hi for lo, n, hi in zip(low, x.dims, high)]
+        return self._emit("pad", x.dtype, dims, [x, value], attrs="padding=" + "x".join(f"{lo}_{hi}" for lo, hi in zip(low, high)))
+
     def concatenate(self, xs: Sequence[Value], dim: int) -> Value:
         dims = list(xs[0].dims)
         dims[dim] = sum(x.dims[dim] for x in xs)

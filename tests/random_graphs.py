@@ -39,7 +39,7 @@ def random_module(seed: int):
             n_ops = int(rng.integers(3, 9))
             for _ in range(n_ops):
                 kind = rng.choice(["binary", "unary", "rowvec", "colvec", "const", "select", "transpose", "rotate", "mask",
-                                   "reduce", "rowin"])
+                                   "reduce", "rowin", "shift", "window"])
                 a = pick()
                 if kind == "binary":
                     r = f.binary(str(rng.choice(["add", "subtract", "multiply", "maximum", "minimum"])), a, pick())
@@ -64,6 +64,16 @@ def random_module(seed: int):
                 elif kind == "rotate" and C >= 2:
                     c1 = int(rng.integers(1, C))
                     r = f.concatenate([f.slice(a, [0, c1], [R, C]), f.slice(a, [0, 0], [R, c1])], 1)
+                elif kind == "shift" and C >= 2:
+                    # shift the columns by k with zero fill: pad on one side, cut the other
+                    k = int(rng.integers(1, min(C, 9)))
+                    if rng.random() < 0.5:
+                        r = f.slice(f.pad(a, f.scalar("f32", 0.0), [0, k], [0, 0]), [0, 0], [R, C])
+                    else:
+                        r = f.slice(f.pad(a, f.scalar("f32", 0.0), [0, 0], [0, k]), [0, k], [R, C + k])
+                elif kind == "window" and C >= 3:
+                    # moving maximum over three columns, same size (padding = -inf)
+                    r = f.reduce_window(a, f.scalar("f32", float("-inf")), (1, 3), (1, 1), ((0, 0), (1, 1)), mb.reducer("maximum", "f32"))
                 elif kind == "mask":
                     col = f.iota("s32", (R, C), 1)
                     lim = f.splat("s32", int(rng.integers(0, C + 1)), (R, C))

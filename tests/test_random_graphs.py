@@ -7,7 +7,7 @@ from mononn_amd import MonoNNModule
 from oracle import hlo_interp
 from random_graphs import random_module
 
-SEEDS = list(range(36))
+SEEDS = list(range(48))
 
 
 def test_random_graphs_are_lowered_and_evaluated():
@@ -40,17 +40,35 @@ def test_random_graphs_stay_inside_their_buffers():
         assert ok, f"{name}: {msg}"
 
 
+def _rotated_row_sum_module(R=70, C=257, k=10):
+    """Row program over a row whose columns are rotated by k (slice + concatenate): the two slices are read under the
+    branches of the concatenate, at addresses that are in range only where the branch is taken."""
+    from mononn_amd.hlo.builder import HloModuleBuilder
+    mb = HloModuleBuilder("cluster_77__rotated_rows.1")
+    e = mb.entry
+    x = e.parameter("f16", (R, C), "x")
+
+    def body(f, p):
+        a = f.convert(p, "f32")
+        rot = f.concatenate([f.slice(a, [0, C - k], [R, C]), f.slice(a, [0, 0], [R, C - k])], 1)
+        red = f.reduce(rot, f.scalar("f32", 0.0), 1, mb.reducer("add", "f32"))
+        return f.convert(f.sub(rot, f.broadcast(red, (R, C), [0])), "f16")
+    e.set_tuple_root([e.fusion("kInput", [x], body)])
+    return mb.text()
+
+
 def test_loads_under_a_condition_are_not_requested_ahead_of_it():
     # a row program asks for its operands at the top of the row; a load that sits in a branch of a concatenate is
     # only in range where the branch is taken and has to stay there
-    text, _, _ = random_module(0)
+    from cpu_bounds import check_module
+    text = _rotated_row_sum_module()
     src = MonoNNModule.compile(text, build=False).get_source("main.hip")
     body = src[src.index("node_fn_0("):]
-    barrier = body.index("__builtin_amdgcn_sched_barrier(0)")
-    first_branch = body.index("if (q0 < ")
-    assert barrier < first_branch
-    assert "+ 247]" not in body[:barrier] and "+ -10]" not in body[:barrier]        # the two halves of the rotated row
+    first_branch = body.index("if (q0 < 10)")
+    assert "+ 247]" not in body[:first_branch] and "+ -10]" not in body[:first_branch]        # the two halves of the rotated row
     assert "+ 247]" in body[first_branch:] and "+ -10]" in body[first_branch:]
+    ok, msg = check_module(text)
+    assert ok, msg
 
 
 @pytest.mark.gpu
