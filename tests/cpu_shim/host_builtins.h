@@ -1,0 +1,42 @@
+// Pre-included in front of the real device prelude when a generated translation unit is built for the host (bounds
+// checks on the CPU, tests/cpu_bounds.py): HIP keywords, thread coordinates and the handful of GPU builtins the
+// prelude uses.  One thread runs at a time, so values that cross lanes or waves are not reproduced (a shuffle returns
+// the caller's own value, the MFMA stub only consumes its operands) and a spin on another workgroup's barrier flag
+// ends at once: only the addresses a thread touches are meaningful.
+#pragma once
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+
+#define __device__
+#define __global__
+#define __shared__
+#define __forceinline__ inline
+#define __launch_bounds__(...)
+#define __HIP_MEMORY_SCOPE_AGENT 0
+#define __hip_atomic_store(p, v, order, scope) (*(p) = (v))
+#define __hip_atomic_load(p, order, scope) (*(p))
+#define __builtin_amdgcn_s_sleep(x) break /* the only use is the body of a spin on a flag */
+#define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) (src)
+#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
+#define __shfl_xor(v, ...) (v)
+#define __syncthreads() ((void)0)
+#define __expf expf
+#define __logf logf
+
+struct Dim3 {
+  unsigned x = 0, y = 0, z = 0;
+};
+extern Dim3 threadIdx, blockIdx, gridDim, blockDim;
+using std::max;
+using std::min;
+inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
+inline unsigned long long wall_clock64() { return 1; }
+typedef _Float16 host_half8 __attribute__((ext_vector_type(8)));
+typedef float host_float4 __attribute__((ext_vector_type(4)));
+inline host_float4 __builtin_amdgcn_mfma_f32_16x16x32_f16(host_half8 a, host_half8 b, host_float4 c, int, int, int) {
+  c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
+  return c;
+}

@@ -1,0 +1,88 @@
+"""Every generated kernel keeps its accesses inside its buffers: the generated translation units (with the device
+prelude they ship with) run on the CPU, one thread at a time, every buffer against guard pages (tests/cpu_bounds.py).
+Covers what a GPU test could only report as a memory fault: MFMA tiles on ragged shapes, fragment-order operands,
+weights requested ahead of the barrier, fused attention, split-K, the launch variants and the tuned BERT-base kernel."""
+import json
+
+import numpy as np
+import pytest
+
+from cpu_bounds import check_module
+from mononn_amd import MonoNNModule
+from mononn_amd.hlo import models
+import test_gpu_parity as parity
+
+GEMM_CASES = [m for m in parity.test_gemm_cases.pytestmark if m.name == "parametrize"][0].args[1]
+
+
+def test_the_check_itself_reports_an_access_past_a_buffer():
+    mb, *_ = parity.gemm_module(M=100, N=52, K=96, rhs_c=1)
+    ok, _ = check_module(mb.text())
+    assert ok
+    for which in ("live-out 0", "parameter 0", "parameter 1"):      # the same kernel, one buffer declared 32 bytes short
+        ok, msg = check_module(mb.text(), shrink=(which, 32))
+        assert not ok and "OUT OF BOUNDS: " + which in msg, msg
+    ok, msg = check_module(models.bert_layer().hlo_text, shrink=("temp arena", 64))
+    assert not ok and "temp arena" in msg
+
+
+@pytest.mark.parametrize("case", GEMM_CASES)
+def test_gemm_layout_cases(case):
+    ok, msg = check_module(parity.gemm_module(**case)[0].text())
+    assert ok, msg
+
+
+def test_random_gemm_shapes_layouts_and_tiles():
+    rng = np.random.default_rng(5)
+    for _ in range(25):
+        batch = [(), (2,), (2, 3)][int(rng.integers(0, 3))]
+        r = len(batch) + 2
+        case = dict(M=int(rng.integers(1, 300)), N=int(rng.integers(1, 300)), K=int(rng.choice([8, 17, 32, 40, 64, 96, 100, 128, 197, 256])),
+                    batch=batch, lhs_c=int(rng.choice([r - 1, r - 2])), rhs_c=int(rng.choice([r - 1, r - 2])))
+        if not batch and rng.random() < 0.4:
+            case.update(b_const=True, lhs_c=r - 1, rhs_c=r - 2)
+        text = parity.gemm_module(**case)[0].text()
+        spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+        if rng.random() < 0.7:
+            c = next(iter(spec["gemm_spec_list"].values()))["cutlass_config"]
+            wk = int(rng.choice([1, 2, 4]))
+            wm = int(rng.choice([w for w in (1, 2, 4) if (4 // wk) % w == 0]))
+            wn = 4 // wk // wm
+            tm, tn = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+            c["threadblockshape"] = {"m": 16 * tm * wm, "n": 16 * tn * wn, "k": 32}
+            c["warpshape"] = {"m": 16 * tm, "n": 16 * tn, "k": c["warpshape"]["k"]}
+            c["wave_arrangement"] = {"m": wm, "n": wn, "k": wk}
+        ok, msg = check_module(text, json.dumps(spec))
+        assert ok, f"{case}: {msg}"
+
+
+def test_encoder_variants():
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
+    variants = {
+        "default": None,
+        "8 workgroups": parity._spec_with(fx.hlo_text, grid=8),
+        "2 workgroups per compute unit": parity._spec_with(fx.hlo_text, grid=512),
+        "LayerNorm inside the GEMM": parity._spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}),
+        "output projection inside the attention": parity._spec_with(fx.hlo_text, hip={"attention_out_proj_fusion": True}),
+        "no attention fusion": parity._spec_with(fx.hlo_text, hip={"fuse_attention": False}),
+        "no epilogue fusion": parity._spec_with(fx.hlo_text, hip={"gemm_epilogue_fusion": False}),
+        "plain layouts": parity._spec_with(fx.hlo_text, hip={"transpose_constant_b": False, "assign_operand_layouts": False}),
+        "weights requested inside the tile": parity._spec_with(fx.hlo_text, hip={"operand_preload": False}),
+        "row-major left operands": parity._spec_with(fx.hlo_text, hip={"pack_left_operands": False}),
+    }
+    for name, spec in variants.items():
+        ok, msg = check_module(fx.hlo_text, spec)
+        assert ok, f"{name}: {msg}"
+
+
+def test_other_model_families_and_the_tuned_bert_base_kernel():
+    import os
+    from mononn_amd import binding
+    for name, fx in [("GPT-2 style decoder", models.gpt2(L=2, B=2, S=64, H=256, NH=4, F=512, vocab=1000, max_pos=128)),
+                     ("ViT, 17 tokens", models.vit(L=2, B=2, image=64, patch=16, H=256, NH=4, F=512)),
+                     ("ViT-B/16 layer, 197 tokens", models.vit(L=1, B=1))]:
+        ok, msg = check_module(fx.hlo_text)
+        assert ok, f"{name}: {msg}"
+    spec = open(os.path.join(os.path.dirname(binding.__file__), "specs", "bert_base_b1_s128", "cluster_0", "best_tuning_spec.json")).read()
+    ok, msg = check_module(models.bert_base().hlo_text, spec)
+    assert ok, msg

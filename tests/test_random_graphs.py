@@ -40,6 +40,26 @@ def test_random_graphs_stay_inside_their_buffers():
         assert ok, f"{name}: {msg}"
 
 
+def test_tuning_knobs_keep_random_graphs_inside_their_buffers():
+    # the same bounds check under other specifications: vector widths, workgroup-per-row programs, small grids
+    # (several units per workgroup), other workgroup sizes
+    import json
+    from cpu_bounds import check_module
+    for seed in SEEDS[:10]:
+        text = random_module(seed)[0]
+        base = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+        for ilp, tier, grid, block in [(4, 2, 256, 256), (8, 1, 8, 256), (2, 2, 3, 512)]:
+            spec = json.loads(json.dumps(base))
+            for v in spec["cluster_reduce_spec"].values():
+                v["ilp_factor"], v["locality_tier"] = ilp, tier
+            for v in spec["cluster_elewise_spec"].values():
+                v["ilp_factor"] = ilp
+            spec["cuda_context"]["cuda_runtime_context"]["grid_dim"]["x"] = grid
+            spec["cuda_context"]["cuda_runtime_context"]["block_dim"]["x"] = block
+            ok, msg = check_module(text, json.dumps(spec))
+            assert ok, f"seed {seed}, ilp {ilp}, tier {tier}, grid {grid}, block {block}: {msg}"
+
+
 def _rotated_row_sum_module(R=70, C=257, k=10):
     """Row program over a row whose columns are rotated by k (slice + concatenate): the two slices are read under the
     branches of the concatenate, at addresses that are in range only where the branch is taken."""
