@@ -113,3 +113,31 @@ def random_module(seed: int):
     e.set_tuple_root(outs)
     descs = [{"dtype": o.dtype, "dims": list(o.dims)} for o in outs]
     return mb.text(), inputs, descs
+
+
+def random_gemm_cases(seed: int, count: int):
+    """Seeded GEMM modules over shapes, batch ranks, operand layouts and (mostly) explicit tiles: yields
+    (case dict for test_gpu_parity.gemm_module, hlo_text, specification json)."""
+    import json
+    from mononn_amd import MonoNNModule
+    import test_gpu_parity as parity
+    rng = np.random.default_rng(seed)
+    for _ in range(count):
+        batch = [(), (2,), (2, 3)][int(rng.integers(0, 3))]
+        r = len(batch) + 2
+        case = dict(M=int(rng.integers(1, 300)), N=int(rng.integers(1, 300)), K=int(rng.choice([8, 17, 32, 40, 64, 96, 100, 128, 197, 256])),
+                    batch=batch, lhs_c=int(rng.choice([r - 1, r - 2])), rhs_c=int(rng.choice([r - 1, r - 2])))
+        if not batch and rng.random() < 0.4:
+            case.update(b_const=True, lhs_c=r - 1, rhs_c=r - 2)
+        text = parity.gemm_module(**case)[0].text()
+        spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+        if rng.random() < 0.7:
+            c = next(iter(spec["gemm_spec_list"].values()))["cutlass_config"]
+            wk = int(rng.choice([1, 2, 4]))
+            wm = int(rng.choice([w for w in (1, 2, 4) if (4 // wk) % w == 0]))
+            wn = 4 // wk // wm
+            tm, tn = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+            c["threadblockshape"] = {"m": 16 * tm * wm, "n": 16 * tn * wn, "k": 32}
+            c["warpshape"] = {"m": 16 * tm, "n": 16 * tn, "k": c["warpshape"]["k"]}
+            c["wave_arrangement"] = {"m": wm, "n": wn, "k": wk}
+        yield case, text, json.dumps(spec)

@@ -33,26 +33,9 @@ def test_gemm_layout_cases(case):
 
 
 def test_random_gemm_shapes_layouts_and_tiles():
-    rng = np.random.default_rng(5)
-    for _ in range(25):
-        batch = [(), (2,), (2, 3)][int(rng.integers(0, 3))]
-        r = len(batch) + 2
-        case = dict(M=int(rng.integers(1, 300)), N=int(rng.integers(1, 300)), K=int(rng.choice([8, 17, 32, 40, 64, 96, 100, 128, 197, 256])),
-                    batch=batch, lhs_c=int(rng.choice([r - 1, r - 2])), rhs_c=int(rng.choice([r - 1, r - 2])))
-        if not batch and rng.random() < 0.4:
-            case.update(b_const=True, lhs_c=r - 1, rhs_c=r - 2)
-        text = parity.gemm_module(**case)[0].text()
-        spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
-        if rng.random() < 0.7:
-            c = next(iter(spec["gemm_spec_list"].values()))["cutlass_config"]
-            wk = int(rng.choice([1, 2, 4]))
-            wm = int(rng.choice([w for w in (1, 2, 4) if (4 // wk) % w == 0]))
-            wn = 4 // wk // wm
-            tm, tn = int(rng.integers(1, 5)), int(rng.integers(1, 5))
-            c["threadblockshape"] = {"m": 16 * tm * wm, "n": 16 * tn * wn, "k": 32}
-            c["warpshape"] = {"m": 16 * tm, "n": 16 * tn, "k": c["warpshape"]["k"]}
-            c["wave_arrangement"] = {"m": wm, "n": wn, "k": wk}
-        ok, msg = check_module(text, json.dumps(spec))
+    from random_graphs import random_gemm_cases
+    for case, text, spec in random_gemm_cases(5, 25):
+        ok, msg = check_module(text, spec)
         assert ok, f"{case}: {msg}"
 
 
