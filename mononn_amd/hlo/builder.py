@@ -205,6 +205,10 @@ class Computation:
                   " pad=" + "x".join(f"{lo}_{hi}" for lo, hi in pad))
         return self._emit("reduce-window", x.dtype, dims, [x, init], attrs=f"window={{{window}}}, to_apply=%{reducer}")
 
+    def dynamic_slice(self, x: Value, starts: Sequence[Value], sizes: Sequence[int]) -> Value:
+        return self._emit("dynamic-slice", x.dtype, sizes, [x] + list(starts),
+                          attrs="dynamic_slice_sizes={" + ",".join(str(n) for n in sizes) + "}")
+
     def dynamic_update_slice(self, x: Value, update: Value, starts: Sequence[Value]) -> Value:
         return self._emit("dynamic-update-slice", x.dtype, x.dims, [x, update] + list(starts))
 

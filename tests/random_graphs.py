@@ -18,20 +18,28 @@ def random_module(seed: int):
     x1 = e.parameter("f16", (R, C), "x1")
     v = e.parameter("f16", (C,), "v")
     w = e.parameter("f16", (R,), "w")
+    T = int(rng.choice([1, 7, 50]))
+    table = e.parameter("f16", (T, C), "table")
+    ids = e.parameter("s32", (R,), "ids")                 # partly out of range: row gathers clamp
+    wide = e.parameter("f16", (R, C + 6), "wide")
+    start = e.parameter("s32", (), "start")               # may be out of range: dynamic-slice clamps
     inputs = [rng.normal(0, 1, (R, C)).astype(np.float16), rng.normal(0, 1, (R, C)).astype(np.float16),
-              rng.normal(0, 1, (C,)).astype(np.float16), rng.normal(0, 1, (R,)).astype(np.float16)]
+              rng.normal(0, 1, (C,)).astype(np.float16), rng.normal(0, 1, (R,)).astype(np.float16),
+              rng.normal(0, 1, (T, C)).astype(np.float16), rng.integers(-3, T + 3, (R,)).astype(np.int32),
+              rng.normal(0, 1, (R, C + 6)).astype(np.float16), np.array(int(rng.integers(-4, 12)), np.int32)]
     full = [x0, x1]          # entry-level [R, C] f16 values available to later fusions
     rows = []                # entry-level [R] f32 values
     n_fusions = int(rng.integers(1, 4))
     for fi in range(n_fusions):
-        operands = list(full) + [v, w] + rows
+        operands = list(full) + [v, w] + rows + [table, ids, wide, start]
         state = {"has_reduce": False}
 
         def body(f, *ps):
             pf = [f.convert(p, "f32") for p in ps[:len(full)]]
             pv = f.convert(ps[len(full)], "f32")
             pw = f.convert(ps[len(full) + 1], "f32")
-            prow = list(ps[len(full) + 2:])
+            prow = list(ps[len(full) + 2:len(ps) - 4])
+            ptable, pids, pwide, pstart = ps[len(ps) - 4:]
             vals = list(pf)
 
             def pick():
@@ -39,7 +47,7 @@ def random_module(seed: int):
             n_ops = int(rng.integers(3, 9))
             for _ in range(n_ops):
                 kind = rng.choice(["binary", "unary", "rowvec", "colvec", "const", "select", "transpose", "rotate", "mask",
-                                   "reduce", "rowin", "shift", "window"])
+                                   "reduce", "rowin", "shift", "window", "gather", "dslice"])
                 a = pick()
                 if kind == "binary":
                     r = f.binary(str(rng.choice(["add", "subtract", "multiply", "maximum", "minimum"])), a, pick())
@@ -74,6 +82,11 @@ def random_module(seed: int):
                 elif kind == "window" and C >= 3:
                     # moving maximum over three columns, same size (padding = -inf)
                     r = f.reduce_window(a, f.scalar("f32", float("-inf")), (1, 3), (1, 1), ((0, 0), (1, 1)), mb.reducer("maximum", "f32"))
+                elif kind == "gather":
+                    r = f.binary("add", a, f.convert(f.gather_rows(ptable, pids), "f32"))
+                elif kind == "dslice":
+                    zero = f.scalar("s32", 0)
+                    r = f.binary("multiply", a, f.convert(f.dynamic_slice(pwide, [zero, pstart], (R, C)), "f32"))
                 elif kind == "mask":
                     col = f.iota("s32", (R, C), 1)
                     lim = f.splat("s32", int(rng.integers(0, C + 1)), (R, C))
