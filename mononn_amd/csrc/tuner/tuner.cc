@@ -170,6 +170,26 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
   std::vector<Ctx> contexts = {{1, 256}, {1, 512}};
   if (budget == 0) contexts.push_back({2, 256});
   if (budget >= 2) contexts = {{1, 256}};
+  // MONONN_TUNER_LAUNCH_CONTEXTS="1x256,2x256": workgroups per CU x threads, instead of the list above (large models:
+  // one context of a full search takes minutes)
+  {
+    const std::string only = env::get("MONONN_TUNER_LAUNCH_CONTEXTS", "");
+    std::vector<Ctx> chosen;
+    size_t st = 0;
+    while (!only.empty() && st <= only.size()) {
+      size_t e = only.find(',', st);
+      const std::string item = only.substr(st, e == std::string::npos ? std::string::npos : e - st);
+      const size_t x = item.find('x');
+      const int per_cu = x == std::string::npos ? 0 : std::atoi(item.substr(0, x).c_str());
+      const int block = x == std::string::npos ? 0 : std::atoi(item.substr(x + 1).c_str());
+      MONONN_CHECK(per_cu >= 1 && per_cu <= 4 && block >= 64 && block <= 1024 && block % 64 == 0, kInvalidArgument)
+          << "MONONN_TUNER_LAUNCH_CONTEXTS: '" << item << "' is not <workgroups per CU>x<threads per workgroup>";
+      chosen.push_back({per_cu, block});
+      if (e == std::string::npos) break;
+      st = e + 1;
+    }
+    if (!chosen.empty()) contexts = chosen;
+  }
 
   std::unique_ptr<MonoNNModule> best;
   double best_us = -1;

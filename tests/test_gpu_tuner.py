@@ -79,3 +79,22 @@ def test_tuning_from_a_seed_specification(gpu_device, encoder, tmp_path, monkeyp
     tuned.set_constants(consts)
     tuned.load(gpu_device)
     _check(tuned.run(inputs, fx.outputs)[0], want)
+
+
+def test_launch_contexts_can_be_named(gpu_device, encoder, tmp_path, monkeypatch):
+    # MONONN_TUNER_LAUNCH_CONTEXTS replaces the built-in list of (workgroups per CU) x (threads per workgroup)
+    from mononn_amd import MonoNNError
+    fx, consts, inputs, want = encoder
+    monkeypatch.setenv("MONONN_TUNER_LAUNCH_CONTEXTS", "1x512")
+    out = str(tmp_path / "ctx")
+    tuned = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, out, budget=2)
+    assert tuned.launch_dims()["block"] == 512
+    files = os.listdir(os.path.join(out, "cluster_0"))
+    assert any(f.endswith("__512_1_1.json") for f in files) and not any(f.endswith("__256_1_1.json") for f in files)
+    tuned.set_constants(consts)
+    tuned.load(gpu_device)
+    _check(tuned.run(inputs, fx.outputs)[0], want)
+    monkeypatch.setenv("MONONN_TUNER_LAUNCH_CONTEXTS", "two by four")
+    with pytest.raises(MonoNNError) as ei:
+        MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, None, budget=2)
+    assert "MONONN_TUNER_LAUNCH_CONTEXTS" in str(ei.value)
