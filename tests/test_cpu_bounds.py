@@ -58,6 +58,18 @@ def test_encoder_variants():
         assert ok, f"{name}: {msg}"
 
 
+ODD_ENCODERS = [dict(B=1, S=17, H=64, NH=1, F=100), dict(B=3, S=50, H=96, NH=2, F=100), dict(B=1, S=100, H=120, NH=3, F=256),
+                dict(B=3, S=64, H=128, NH=4, F=100), dict(B=1, S=50, H=120, NH=3, F=100), dict(B=3, S=17, H=96, NH=2, F=256)]
+
+
+@pytest.mark.parametrize("shape", ODD_ENCODERS)
+def test_encoders_with_sizes_off_the_mfma_steps(shape):
+    # sequence lengths, hidden sizes and head sizes that are not multiples of 16 / 32: ragged tiles, unfused attention
+    fx = models.bert_encoder(L=1, vocab=97, max_pos=128, **shape)
+    ok, msg = check_module(fx.hlo_text)
+    assert ok, msg
+
+
 def test_other_model_families_and_the_tuned_bert_base_kernel():
     import os
     from mononn_amd import binding

@@ -181,3 +181,16 @@ def test_vit_full_size_properties(gpu_device):
         t.load(gpu_device)
         _check(t.run(inputs, fx.outputs)[0], out.astype(np.float32), "vit tuned vs default")
         t.close()
+
+
+@pytest.mark.parametrize("shape", [dict(B=1, S=17, H=64, NH=1, F=100), dict(B=3, S=50, H=96, NH=2, F=100), dict(B=1, S=100, H=120, NH=3, F=256),
+                                   dict(B=3, S=64, H=128, NH=4, F=100), dict(B=1, S=50, H=120, NH=3, F=100), dict(B=3, S=17, H=96, NH=2, F=256)])
+def test_encoders_with_sizes_off_the_mfma_steps(gpu_device, shape):
+    # the shapes whose addresses tests/test_cpu_bounds.py checks on the CPU, here for their values
+    fx = models.bert_encoder(L=1, vocab=97, max_pos=128, **shape)
+    consts = fx.make_constants(1240, "random")
+    inputs = fx.make_inputs(1240)
+    m, got = _run(fx, consts, inputs, gpu_device)
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _check(got, want, f"encoder {shape}")
+    m.close()
