@@ -1,4 +1,6 @@
-"""Bounds check of generated kernels on the CPU: the generated translation unit of a module (its main.hip and the
+"""TEST INFRASTRUCTURE ONLY (an address checker, not an execution path: values that cross threads are not reproduced).
+
+Bounds check of generated kernels on the CPU: the generated translation unit of a module (its main.hip and the
 device prelude it includes, unchanged) is compiled for the host with tests/cpu_shim/host_builtins.h pre-included and
 run thread by thread with every buffer placed against inaccessible guard pages, once flush with the page before it (catches reads in front of a
 buffer) and once flush with the page behind it (catches reads past its end).  An out-of-range access ends the run

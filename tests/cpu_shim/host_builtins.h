@@ -1,3 +1,4 @@
+// TEST INFRASTRUCTURE ONLY: nothing in the product includes this file or runs kernels on the CPU.
 // Pre-included in front of the real device prelude when a generated translation unit is built for the host (bounds
 // checks on the CPU, tests/cpu_bounds.py): HIP keywords, thread coordinates and the handful of GPU builtins the
 // prelude uses.  One thread runs at a time, so values that cross lanes or waves are not reproduced (a shuffle returns
