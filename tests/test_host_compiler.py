@@ -284,6 +284,29 @@ def test_contraction_length_off_the_mfma_step_still_takes_mfma_tiles():
 SHIPPED_SPECS = {"bert_base_b1_s128": models.bert_base, "vit_b16_b8": models.vit, "gpt2_b4_s512": models.gpt2}
 
 
+def test_results_only_the_host_reads_are_stored_through_the_cache():
+    # a value that a later stage reads crosses XCDs through write-through stores; the last LayerNorm's result is read
+    # by the host alone and is written with plain stores (the L2 merges them; all of it is written out at kernel end)
+    fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
+    src = MonoNNModule.compile(fx.hlo_text, build=False).get_source("main.hip")
+    fns = re.split(r"(?=__device__ __forceinline__ void node_fn_\d+\()", src)
+    plain = [f for f in fns if "stN_plain<" in f or "st1_plain(" in f]
+    assert len(plain) == 1 and "mononn_dev::stN<" not in plain[0] and "mononn_dev::st1(" not in plain[0].split("extern \"C\"")[0]
+    assert sum("mononn_dev::stN<" in f or "mononn_dev::st1(" in f for f in fns) >= 5
+    # a module output that a later stage also reads keeps the write-through stores
+    mb = HloModuleBuilder("cluster_6__two_readers.1")
+    e = mb.entry
+    x = e.parameter("f16", (64, 128), "x")
+    w = e.elided_constant("f16", (128, 128), "w/kernel")
+    h = e.fusion("kLoop", [x], lambda f, p: f.tanh(p))
+    y = e.gemm(h, w, 1, 0)
+    e.set_tuple_root([h, y])
+    src = MonoNNModule.compile(mb.text(), build=False).get_source("main.hip")
+    first = [f for f in re.split(r"(?=__device__ __forceinline__ void node_fn_\d+\()", src) if "fast_tanh" in f][0]
+    first = re.split(r"\n(?:typedef|struct) ", first)[0]          # the next function's epilogue struct follows in the text
+    assert "_plain" not in first and ("mononn_dev::stN<" in first or "mononn_dev::st1(" in first)
+
+
 def test_register_budget_follows_the_workgroups_per_compute_unit():
     # a persistent grid must be resident as a whole: with more than one workgroup per CU (or 512-thread workgroups)
     # two waves share a SIMD, the kernel is compiled for 256 registers per wave and the GEMM tile loads smaller chunks
