@@ -448,6 +448,120 @@ void decode_dot_config(Instr* ins) {
   }
 }
 
+// Operand counts, attribute lengths and extents that every later stage relies on (index maps subscript these
+// vectors without further checks): a module that gets past here is consistent, whatever text it came from.
+void validate_shapes(const Instr* ins) {
+  const std::string& op = ins->opcode;
+  const Shape& sh = ins->shape;
+  auto arity = [&](size_t lo, size_t hi) {
+    MONONN_CHECK(ins->operands.size() >= lo && ins->operands.size() <= hi, kParseError)
+        << ins->hlo_name << " (" << op << "): " << ins->operands.size() << " operands, expected " << lo << (hi == lo ? "" : " to " + std::to_string(hi));
+  };
+  auto array_operand = [&](size_t i) -> const Shape& {
+    MONONN_CHECK(!ins->operands[i]->shape.is_tuple(), kParseError) << ins->hlo_name << ": operand " << i << " is a tuple";
+    return ins->operands[i]->shape;
+  };
+  auto in_range = [&](int64_t v, int64_t n, const char* what) {
+    MONONN_CHECK(v >= 0 && v < n, kParseError) << ins->hlo_name << ": " << what << " " << v << " out of range [0, " << n << ")";
+  };
+  static const std::set<std::string> unary = {"abs", "convert", "copy", "exponential", "log", "negate", "not", "rsqrt", "sign", "sqrt", "tanh"};
+  static const std::set<std::string> binary = {"add", "and", "divide", "maximum", "minimum", "multiply", "or", "power", "subtract", "compare"};
+  if (unary.count(op)) {
+    arity(1, 1);
+    MONONN_CHECK(array_operand(0).dims == sh.dims, kParseError) << ins->hlo_name << ": operand and result shapes differ";
+  } else if (binary.count(op)) {
+    arity(2, 2);
+    MONONN_CHECK(array_operand(0).dims == sh.dims && array_operand(1).dims == sh.dims, kParseError) << ins->hlo_name << ": operand and result shapes differ";
+  } else if (op == "select" || op == "clamp") {
+    arity(3, 3);
+    for (size_t i = 0; i < 3; ++i)
+      MONONN_CHECK(array_operand(i).dims == sh.dims || array_operand(i).rank() == 0, kParseError) << ins->hlo_name << ": operand " << i << " does not match the result shape";
+  } else if (op == "bitcast" || op == "reshape") {
+    arity(1, 1);
+    if (!ins->operands[0]->shape.is_tuple())
+      MONONN_CHECK(array_operand(0).num_elements() == sh.num_elements(), kParseError) << ins->hlo_name << ": element count changes";
+  } else if (op == "broadcast") {
+    arity(1, 1);
+    const Shape& x = array_operand(0);
+    MONONN_CHECK(static_cast<int>(ins->dimensions.size()) == x.rank(), kParseError) << ins->hlo_name << ": dimensions={} must name one result dimension per operand dimension";
+    for (int i = 0; i < x.rank(); ++i) {
+      in_range(ins->dimensions[i], sh.rank(), "broadcast dimension");
+      MONONN_CHECK(sh.dims[ins->dimensions[i]] == x.dims[i], kParseError) << ins->hlo_name << ": broadcast extent mismatch in operand dimension " << i;
+    }
+  } else if (op == "transpose") {
+    arity(1, 1);
+    const Shape& x = array_operand(0);
+    MONONN_CHECK(static_cast<int>(ins->dimensions.size()) == x.rank() && sh.rank() == x.rank(), kParseError) << ins->hlo_name << ": dimensions={} must be a permutation of the operand's dimensions";
+    std::vector<bool> seen(x.rank(), false);
+    for (int i = 0; i < x.rank(); ++i) {
+      in_range(ins->dimensions[i], x.rank(), "transpose dimension");
+      MONONN_CHECK(!seen[ins->dimensions[i]] && sh.dims[i] == x.dims[ins->dimensions[i]], kParseError) << ins->hlo_name << ": not a permutation of the operand's shape";
+      seen[ins->dimensions[i]] = true;
+    }
+  } else if (op == "slice") {
+    arity(1, 1);
+    const Shape& x = array_operand(0);
+    MONONN_CHECK(static_cast<int>(ins->slice_starts.size()) == x.rank() && sh.rank() == x.rank(), kParseError) << ins->hlo_name << ": slice={} must have one range per dimension";
+    for (int i = 0; i < x.rank(); ++i)
+      MONONN_CHECK(ins->slice_starts[i] >= 0 && ins->slice_limits[i] <= x.dims[i] && ins->slice_limits[i] - ins->slice_starts[i] == sh.dims[i], kParseError)
+          << ins->hlo_name << ": slice range of dimension " << i << " does not fit the operand / result";
+  } else if (op == "concatenate") {
+    arity(1, 1u << 20);
+    MONONN_CHECK(ins->dimensions.size() == 1, kParseError) << ins->hlo_name << ": concatenate needs dimensions={d}";
+    in_range(ins->dimensions[0], sh.rank(), "concatenate dimension");
+    int64_t total = 0;
+    for (size_t k = 0; k < ins->operands.size(); ++k) {
+      const Shape& x = array_operand(k);
+      MONONN_CHECK(x.rank() == sh.rank(), kParseError) << ins->hlo_name << ": operand " << k << " has another rank";
+      for (int i = 0; i < sh.rank(); ++i)
+        if (i != ins->dimensions[0]) MONONN_CHECK(x.dims[i] == sh.dims[i], kParseError) << ins->hlo_name << ": operand " << k << " differs outside the concatenated dimension";
+      total += x.dims[ins->dimensions[0]];
+    }
+    MONONN_CHECK(total == sh.dims[ins->dimensions[0]], kParseError) << ins->hlo_name << ": operand extents do not add up to the result";
+  } else if (op == "pad") {
+    arity(2, 2);
+    const Shape& x = array_operand(0);
+    MONONN_CHECK(static_cast<int>(ins->pad_low.size()) == x.rank() && sh.rank() == x.rank() && array_operand(1).rank() == 0, kParseError)
+        << ins->hlo_name << ": padding= must have one entry per dimension and a scalar padding value";
+    for (int i = 0; i < x.rank(); ++i)
+      MONONN_CHECK(ins->pad_low[i] + x.dims[i] + ins->pad_high[i] == sh.dims[i], kParseError) << ins->hlo_name << ": padded extent of dimension " << i << " does not match the result";
+  } else if (op == "iota") {
+    arity(0, 0);
+    in_range(ins->iota_dimension, std::max(sh.rank(), 1), "iota_dimension");
+  } else if (op == "reduce") {
+    MONONN_CHECK(ins->operands.size() >= 2 && ins->operands.size() % 2 == 0, kParseError) << ins->hlo_name << ": reduce takes N operands and N init values";
+    const Shape& x = array_operand(0);
+    MONONN_CHECK(!ins->dimensions.empty(), kParseError) << ins->hlo_name << ": reduce needs dimensions={..}";
+    for (auto d : ins->dimensions) in_range(d, x.rank(), "reduced dimension");
+    const size_t n = ins->operands.size() / 2;
+    MONONN_CHECK(ins->called && ins->called->params.size() == 2 * n, kParseError) << ins->hlo_name << ": the reducer must take " << 2 * n << " parameters";
+    MONONN_CHECK(sh.is_tuple() ? sh.tuple.size() == n : n == 1, kParseError) << ins->hlo_name << ": result arity does not match the operands";
+    const Shape& out = sh.is_tuple() ? sh.tuple[0] : sh;
+    MONONN_CHECK(out.rank() == x.rank() - static_cast<int>(ins->dimensions.size()), kParseError) << ins->hlo_name << ": result rank does not follow from the reduced dimensions";
+    for (size_t k = 0; k < n; ++k) MONONN_CHECK(array_operand(k).dims == x.dims && array_operand(n + k).rank() == 0, kParseError) << ins->hlo_name << ": operands must share a shape, init values must be scalars";
+  } else if (op == "dynamic-slice") {
+    MONONN_CHECK(!ins->operands.empty(), kParseError) << ins->hlo_name << ": no operand";
+    const Shape& x = array_operand(0);
+    MONONN_CHECK(static_cast<int>(ins->operands.size()) == 1 + x.rank() && static_cast<int>(ins->dynamic_slice_sizes.size()) == x.rank() && sh.rank() == x.rank(), kParseError)
+        << ins->hlo_name << ": dynamic-slice takes one scalar start index and one size per dimension";
+    for (int i = 0; i < x.rank(); ++i)
+      MONONN_CHECK(ins->dynamic_slice_sizes[i] == sh.dims[i] && sh.dims[i] <= x.dims[i] && array_operand(1 + i).rank() == 0, kParseError) << ins->hlo_name << ": slice size of dimension " << i << " does not fit";
+  } else if (op == "gather") {
+    arity(2, 2);
+    array_operand(0);
+    array_operand(1);
+  } else if (op == "get-tuple-element") {
+    arity(1, 1);
+    if (ins->operands[0]->shape.is_tuple()) in_range(ins->tuple_index, static_cast<int64_t>(ins->operands[0]->shape.tuple.size()), "tuple index");
+  } else if (op == "fusion") {
+    MONONN_CHECK(ins->called && ins->called->params.size() == ins->operands.size(), kParseError)
+        << ins->hlo_name << ": " << ins->operands.size() << " operands for a computation of " << (ins->called ? ins->called->params.size() : 0) << " parameters";
+    for (size_t i = 0; i < ins->operands.size(); ++i)
+      MONONN_CHECK(ins->called->params[i]->shape.dims == ins->operands[i]->shape.dims && ins->called->params[i]->shape.dtype == ins->operands[i]->shape.dtype, kParseError)
+          << ins->hlo_name << ": operand " << i << " does not match parameter " << i << " of " << ins->called->hlo_name;
+  }
+}
+
 void decode_attrs(Instr* ins, Module* mod) {
   auto has = [&](const char* k) { return ins->attrs.count(k) > 0; };
   auto get = [&](const char* k) -> const std::string& { return ins->attrs.at(k); };
@@ -583,6 +697,7 @@ void decode_attrs(Instr* ins, Module* mod) {
     // a bare convolution aborts in the reference as well (ir_parser_fused.cc:728-732)
     MONONN_FAIL(kUnsupported) << ins->hlo_name << ": bare convolution is not supported; expected custom-call __cudnn$convForward";
   }
+  validate_shapes(ins);
 }
 
 }  // namespace
