@@ -81,3 +81,28 @@ def test_other_model_families_and_the_tuned_bert_base_kernel():
     spec = open(os.path.join(os.path.dirname(binding.__file__), "specs", "bert_base_b1_s128", "cluster_0", "best_tuning_spec.json")).read()
     ok, msg = check_module(models.bert_base().hlo_text, spec)
     assert ok, msg
+
+
+def test_whatever_specification_is_accepted_stays_inside_the_buffers():
+    # numbers of a valid specification replaced at random (tiles, wave arrangements, knobs, launch shape): the host
+    # compiler either rejects the result or generates a kernel that passes the bounds check
+    import random
+    import re
+    from mononn_amd import MonoNNError
+    fx = models.bert_encoder(L=1, B=1, S=32, H=64, NH=2, F=128, vocab=50, max_pos=64)
+    spec = json.dumps(json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec()), indent=1)
+    numbers = list(re.finditer(r"(?<=: )-?\d+(?=,|\n)", spec))
+    rnd = random.Random(3)
+    accepted = 0
+    for _ in range(60):
+        t = spec
+        for m in sorted(rnd.sample(numbers, rnd.randint(1, 3)), key=lambda m: -m.start()):
+            t = t[:m.start()] + rnd.choice(["0", "1", "2", "3", "4", "5", "7", "8", "16", "17", "32", "48", "64", "96", "100", "128", "256", "512", "1024"]) + t[m.end():]
+        try:
+            MonoNNModule.compile(fx.hlo_text, t, build=False).close()
+        except MonoNNError:
+            continue
+        accepted += 1
+        ok, msg = check_module(fx.hlo_text, t)
+        assert ok, msg + "\n" + t
+    assert accepted >= 20
