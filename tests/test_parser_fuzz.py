@@ -69,3 +69,31 @@ def test_attributes_that_do_not_fit_the_shapes_are_parse_errors():
     perm = re.search(r"dimensions=\{([\d,]+)\}", t).group(1)
     with pytest.raises(MonoNNError):
         MonoNNModule.compile(text.replace(t, t.replace("{" + perm + "}", "{" + ",".join(["0"] * len(perm.split(","))) + "}")), build=False)
+
+
+def test_misuse_of_the_c_abi_returns_error_codes():
+    # NULL pointers, unknown names, calls in the wrong order: an error code and a message, never a crash
+    import ctypes
+    from mononn_amd import binding
+    lib = binding._lib
+    text = models.bert_layer().hlo_text.encode()
+    h = ctypes.c_void_p()
+    assert lib.mononn_compile(None, 0, None, None, 0, ctypes.byref(h)) != 0
+    assert lib.mononn_compile(text, len(text), None, None, 0, None) != 0
+    assert lib.mononn_compile(b"", 0, None, None, 0, ctypes.byref(h)) != 0 and b"HloModule" in lib.mononn_last_error()
+    assert lib.mononn_compile(text, len(text), b"{not json", None, 0, ctypes.byref(h)) != 0 and b"JSON" in lib.mononn_last_error()
+    assert lib.mononn_compile_from_spec_dir(text, len(text), b"/nonexistent/dir", ctypes.byref(h)) != 0
+    assert lib.mononn_compile(text, len(text), None, None, 0, ctypes.byref(h)) == 0
+    p, vp, n = ctypes.c_char_p(), ctypes.c_void_p(), ctypes.c_size_t()
+    assert lib.mononn_module_source(h, None, ctypes.byref(p), ctypes.byref(n)) != 0
+    assert lib.mononn_module_source(h, b"nope.txt", ctypes.byref(p), ctypes.byref(n)) != 0
+    assert lib.mononn_module_code_object(h, ctypes.byref(vp), ctypes.byref(n)) != 0 and b"not been built" in lib.mononn_last_error()
+    assert lib.mononn_module_set_constant(h, b"nope", b"abcd", 4) != 0 and b"no constant named" in lib.mononn_last_error()
+    assert lib.mononn_module_set_constant(h, None, b"abcd", 4) != 0
+    assert lib.mononn_module_load(h, 0) != 0                      # nothing built yet
+    assert lib.mononn_launch(h, None, 0, None) != 0
+    assert lib.mononn_module_dump(h, None) != 0
+    assert lib.mononn_module_load(None, 0) != 0 and lib.mononn_launch(None, None, 0, None) != 0
+    assert lib.mononn_module_summary(None, ctypes.byref(p), ctypes.byref(n)) != 0
+    lib.mononn_module_destroy(None)
+    lib.mononn_module_destroy(h)
