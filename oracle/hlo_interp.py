@@ -34,9 +34,22 @@ checks the evaluator against closed forms and library routines -- fp64 triple-lo
 shapes, the two worked backend_config examples of gemm_impl.cc:290-316 against numpy einsum,
 torch.nn.functional soft-max / layer_norm / gelu(tanh), brute-force gather, torch max/avg
 pooling for reduce-window, NumPy slice assignment for dynamic-update-slice, np.argmax/argmin for
-the variadic reduce, and a whole BERT layer against an independent torch restatement.  Bit-level results of the CUDA build (CUTLASS
+the variadic reduce, and a whole BERT layer against an independent torch restatement;
+tests/test_oracle_pinning_ops.py checks the remaining branches on hand-written HLO text against
+plain Python arithmetic and brute-force loops: integer divide (truncation toward zero), convert
+(float -> int truncation, int -> half rounding and overflow), power / log / negate / abs / sign /
+sqrt / exponential, the six compare directions, select, clamp, and / or / not, maximum / minimum,
+dynamic-slice with clamped starts, pad (low / high / value), slice + concatenate + broadcast + iota +
+transpose, and reduce with add / maximum / minimum / multiply / and / or reducers over the last and
+over another dimension.  Bit-level results of the CUDA build (CUTLASS
 accumulation order, -use_fast_math intrinsics) are not reproducible offline: parity unpinned at
 that level; the north-star tolerance is defined against fp32 evaluation, which this is.
+
+Reduce init values are used as the HLO writes them (XLA semantics).  The reference replaces an
+infinite init by the type's finite extreme (ir_parser_fused.cc:182-204: -inf -> -65504 for f16,
+-FLT_MAX for f32); the two readings differ only for a row that holds nothing but values beyond that
+extreme (e.g. a maximum over a row of -inf gives -inf here, -65504 there).  The HIP kernels follow
+the HLO as written, like this file; tests/test_oracle_pinning_ops.py pins that case.
 
 precision="as_written": every f16-typed instruction result is rounded to IEEE half (what the
 HLO says).  precision="fp32": f16 is carried as float32 without rounding (the "fp32 reference"
@@ -479,8 +492,8 @@ class Evaluator:
         dn = cfg["dot_dimension_numbers"]
         lc = int(dn["lhs_contracting_dimensions"][0])
         rc = int(dn["rhs_contracting_dimensions"][0])
-        A = x[0].astype(np.float32)
-        B = x[1].astype(np.float32)
+        A = x[0].astype(np.float32, copy=False)
+        B = x[1].astype(np.float32, copy=False)
         r = A.ndim
         if lc == r - 2:
             A = np.swapaxes(A, -1, -2)
@@ -488,9 +501,9 @@ class Evaluator:
             B = np.swapaxes(B, -1, -2)
         D = np.matmul(A, B) * np.float32(cfg["alpha_real"])
         if len(x) > 2 and float(cfg["beta"]) != 0.0:
-            D = D + np.float32(cfg["beta"]) * x[2].astype(np.float32)
+            D = D + np.float32(cfg["beta"]) * x[2].astype(np.float32, copy=False)
         with np.errstate(over="ignore"):
-            return D.astype(dt)
+            return D.astype(dt, copy=False)
 
 
     def _conv_forward(self, ins: Instr, x):

@@ -32,3 +32,8 @@ def test_standalone_driver_reproduces_the_library_result(gpu_device, tmp_path):
     assert re.search(r"mononn_cluster_0: grid \d+ x block \d+, 50 iterations, [\d.]+ us per launch", out.stdout), out.stdout
     got = np.fromfile(os.path.join(tmp_path, "liveout_0.bin"), dtype=np.float16).reshape(want.shape)
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    # and both against the fp32 oracle of the same HLO and weights
+    from oracle import hlo_interp
+    ref = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0].astype(np.float64).ravel()
+    g = got.astype(np.float64).ravel()
+    assert np.abs(g - ref).max() <= 2e-2 and g @ ref / (np.linalg.norm(g) * np.linalg.norm(ref)) >= 0.9999

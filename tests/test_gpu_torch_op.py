@@ -24,6 +24,11 @@ def test_custom_op_matches_the_ctypes_path_bit_for_bit(gpu_device):
     (got,) = torch_op.forward(fn, *tin)
     assert got.dtype == torch.float16 and tuple(got.shape) == tuple(fx.outputs[0]["dims"])
     assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # the operator's result against the fp32 oracle of the same HLO and weights
+    from oracle import hlo_interp
+    ref = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0].astype(np.float64).ravel()
+    g = got.cpu().numpy().astype(np.float64).ravel()
+    assert np.abs(g - ref).max() <= 2e-2 and g @ ref / (np.linalg.norm(g) * np.linalg.norm(ref)) >= 0.9999
     # on a side stream, ordered after work that torch queued there
     side = torch.cuda.Stream(device=dev)
     with torch.cuda.stream(side):
