@@ -105,6 +105,19 @@ int mononn_module_load(mononn_module* m, int device);
  *           on `stream` (a hipStream_t, NULL = default stream). */
 int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);
 
+/* Wait for `stream` and report what the kernel could not: MONONN_RUNTIME_ERROR when a grid-barrier wait of a launch
+ * gave up (the grid was not resident as a whole within mononn_hip.barrier_timeout_ms of the specification, e.g. an
+ * ordinary launch beside another kernel).  Every workgroup of such a launch still runs to its end, so the kernel
+ * terminates; its outputs are invalid.  The barrier state is reset and the module stays usable.
+ * Replaces: BlockHostUntilDone of profile_kernel (mononn_engine/module/mononn_module_tuner.cc:140-149), where a
+ *           failed wait is LOG(FATAL). */
+int mononn_module_synchronize(mononn_module* m, void* stream);
+
+/* Device address and size of a module global of the loaded code object: "buffer_for_<node>" (constants,
+ * mononn_engine/codegen/graph_codegen.cc:71-86), "mononn_barrier_flags", "mononn_barrier_error".
+ * Replaces: the cuModuleGetGlobal lookup a host would do on the reference's PTX (README.md:179-200). */
+int mononn_module_global(const mononn_module* m, const char* symbol, void** device_ptr, size_t* bytes);
+
 /* Time `iters` launches after `warmup` with HIP events on `stream`; avg_ms receives the mean,
  * each_ms (may be NULL, else iters floats) the individual launches.
  * Replaces: the CUPTI gpu__time_duration range of profile_in_batch

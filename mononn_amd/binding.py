@@ -61,6 +61,8 @@ def _load_library() -> ctypes.CDLL:
     lib.mononn_module_set_constant.argtypes = [c.c_void_p, c.c_char_p, c.c_void_p, c.c_size_t]
     lib.mononn_module_load.argtypes = [c.c_void_p, c.c_int]
     lib.mononn_launch.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p]
+    lib.mononn_module_synchronize.argtypes = [c.c_void_p, c.c_void_p]
+    lib.mononn_module_global.argtypes = [c.c_void_p, c.c_char_p, P(c.c_void_p), P(c.c_size_t)]
     lib.mononn_time_kernel.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p, c.c_int, c.c_int,
                                        P(c.c_float), P(c.c_float)]
     lib.mononn_module_stage_clock.argtypes = [c.c_void_p, P(c.c_uint64), c.c_size_t, P(c.c_int), P(c.c_int), P(c.c_double)]
@@ -79,7 +81,7 @@ EXPORTED_SYMBOLS = [
     "mononn_module_destroy", "mononn_module_kernel_name", "mononn_module_spec_json", "mononn_module_source",
     "mononn_module_code_object", "mononn_module_summary", "mononn_module_buffer_info", "mononn_module_launch_dims", "mononn_module_owns_temp",
     "mononn_module_num_constants", "mononn_module_constant_info", "mononn_module_set_constant", "mononn_module_load",
-    "mononn_launch", "mononn_time_kernel", "mononn_module_stage_clock", "mononn_module_stage_name", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
+    "mononn_launch", "mononn_module_synchronize", "mononn_module_global", "mononn_time_kernel", "mononn_module_stage_clock", "mononn_module_stage_name", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
 
 
 def _check(rc: int):
@@ -217,6 +219,16 @@ class MonoNNModule:
         arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
         _check(_lib.mononn_launch(self._h, arr, len(device_ptrs), ctypes.c_void_p(stream)))
 
+    def synchronize(self, stream: int = 0):
+        """Wait for `stream`; raises MonoNNError(RUNTIME_ERROR) when a grid-barrier wait of a launch gave up."""
+        _check(_lib.mononn_module_synchronize(self._h, ctypes.c_void_p(stream)))
+
+    def global_address(self, symbol: str):
+        """(device pointer, bytes) of a module global of the loaded code object."""
+        p, n = ctypes.c_void_p(), ctypes.c_size_t()
+        _check(_lib.mononn_module_global(self._h, symbol.encode(), ctypes.byref(p), ctypes.byref(n)))
+        return p.value, n.value
+
     def time_raw(self, device_ptrs: Sequence[int], stream: int = 0, warmup: int = 20, iters: int = 200):
         arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
         avg = ctypes.c_float()
@@ -279,7 +291,7 @@ class MonoNNModule:
             t.copy_(torch.from_numpy(a.view(np.uint8).reshape(-1)))
         stream = torch.cuda.current_stream().cuda_stream
         self.launch_raw(self.buffer_pointers(), stream)
-        torch.cuda.synchronize()
+        self.synchronize(stream)
         outs = []
         npdt = {"f16": np.float16, "f32": np.float32, "s32": np.int32, "pred": np.bool_, "s64": np.int64, "u8": np.uint8, "s8": np.int8}
         for t, o in zip(b["liveouts"], out_dtypes_dims):

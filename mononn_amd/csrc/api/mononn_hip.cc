@@ -208,6 +208,20 @@ int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, voi
   });
 }
 
+int mononn_module_synchronize(mononn_module* m, void* stream) {
+  return guarded([&] {
+    require(m != nullptr, "NULL module");
+    m->impl->synchronize(stream);
+  });
+}
+
+int mononn_module_global(const mononn_module* m, const char* symbol, void** device_ptr, size_t* bytes) {
+  return guarded([&] {
+    require(m && symbol && device_ptr, "NULL argument");
+    *device_ptr = m->impl->global_address(symbol, bytes);
+  });
+}
+
 int mononn_time_kernel(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream, int warmup, int iters,
                        float* avg_ms, float* each_ms) {
   return guarded([&] {

@@ -507,7 +507,7 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
     std::string iv = value(indices, ii);
     int64_t rows = table->shape.dims[0];
     std::string clamped = fresh("g");
-    out_.line("const int " + clamped + " = min(max((int)" + iv + ", 0), " + std::to_string(rows - 1) + ");");
+    out_.line("const int " + clamped + " = mononn_dev::clamp_index(" + iv + ", " + std::to_string(rows - 1) + ");");
     Index ti;
     ti.push_back(LinExpr::opaque(clamped, rows));
     for (size_t i = r; i < idx.size(); ++i) ti.push_back(idx[i]);
@@ -520,7 +520,7 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
       std::string s = value(ins->operands[1 + i], {});
       int64_t hi = x->shape.dims[i] - ins->dynamic_slice_sizes[i];
       std::string c = fresh("ds");
-      out_.line("const int " + c + " = min(max((int)" + s + ", 0), " + std::to_string(hi) + ");");
+      out_.line("const int " + c + " = mononn_dev::clamp_index(" + s + ", " + std::to_string(hi) + ");");
       xi.push_back(idx[i].plus(LinExpr::opaque(c, hi + 1)));
     }
     return value(x, xi);
@@ -539,7 +539,7 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
       }
       std::string s = value(ins->operands[2 + i], {});
       std::string c = fresh("us");
-      out_.line("const int " + c + " = (" + idx[i].str(vars_) + ") - min(max((int)" + s + ", 0), " + std::to_string(hi) + ");");
+      out_.line("const int " + c + " = (" + idx[i].str(vars_) + ") - mononn_dev::clamp_index(" + s + ", " + std::to_string(hi) + ");");
       cond += (cond.empty() ? "" : " && ") + c + " >= 0 && " + c + " < " + std::to_string(un);
       ui.push_back(LinExpr::opaque(c, un));
     }

@@ -117,6 +117,18 @@ int main(int argc, char** argv) {
   float ms = 0;
   CHECK(hipEventElapsedTime(&ms, t0, t1));
   std::printf("%s: grid %d x block %d, %d iterations, %.2f us per launch\n", kKernel, kGrid, kBlock, iters, ms * 1000.f / iters);
+  {
+    // a grid-barrier wait that ran out of time leaves the ordinal of its barrier here (the kernel still ends)
+    hipDeviceptr_t err;
+    size_t n = 0;
+    unsigned word = 0;
+    CHECK(hipModuleGetGlobal(&err, &n, mod, "mononn_barrier_error"));
+    CHECK(hipMemcpyDtoH(&word, err, sizeof(word)));
+    if (word != 0) {
+      std::fprintf(stderr, "a workgroup gave up waiting at grid barrier %u: the grid was not resident as a whole; results are invalid\n", word);
+      return 3;
+    }
+  }
 
   for (int i = 0; i < kNumLiveouts; ++i) {
     std::vector<char> out(kLiveoutBytes[i]);

@@ -269,6 +269,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   if (spec.hip.barrier == "flags_allfence") pre << "#define MONONN_BARRIER_FENCE 1\n";
   else if (spec.hip.barrier == "flags_coherent") pre << "#define MONONN_BARRIER_FENCE 2\n#define MONONN_COHERENT_STORES 1\n";
   else MONONN_CHECK(spec.hip.barrier == "flags", kSpecError) << "unknown barrier flavour '" << spec.hip.barrier << "'";
+  pre << "#define MONONN_BARRIER_BUDGET_TICKS " << static_cast<long long>(spec.hip.barrier_timeout_ms) * 100000 << "ull   // wall clock: 100 MHz\n";
   pre << "#include \"headers.h\"\n\n";
   for (auto& c : hp.constants) {
     std::ostringstream d;
@@ -279,6 +280,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     std::ostringstream d;
     d << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];";
     hp.global_decls.push_back(d.str());
+    hp.global_decls.push_back("__device__ unsigned mononn_barrier_error[4];   // [0]: 0, or the ordinal (from 1) of the first barrier a wait gave up on");
   }
   hp.profiled = spec.hip.profile_stages;
   hp.cooperative = spec.hip.cooperative_launch;
@@ -354,7 +356,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   for (size_t i = 0; i < hp.liveout_bytes.size(); ++i) src << "void* liveout_buffer_" << i << ", ";
   src << "void* temp_buffer) {\n";
   src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
-  src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags);\n";
+  src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags, mononn_barrier_error);\n";
   src << "  int stage = -1;\n";
   const bool lazy = !preload_fns.empty();
   if (lazy) {

@@ -57,14 +57,31 @@ __device__ __forceinline__ int wave_id() { return threadIdx.x / kWaveSize; }
 // ---------------------------------------------------------------------------------------------
 // grid-wide barrier
 // ---------------------------------------------------------------------------------------------
+// Waits are bounded: the kernel notes the wall clock (100 MHz) when it starts, and a wait that is still polling
+// MONONN_BARRIER_BUDGET_TICKS later gives up, records the barrier's ordinal in the error word and returns.  From
+// then on every wait of every workgroup that finds a flag missing returns after one look at the clock, so the
+// workgroups run through their remaining stages (on incomplete data, but every address they form is in range
+// whatever the data: run-time indices are clamped) and the kernel ends normally.  The host reads the error word
+// after synchronising.  What this guards against: a grid that is not resident as a whole (an ordinary launch next
+// to another kernel), where the resident workgroups would otherwise poll for ever.
+#ifndef MONONN_BARRIER_BUDGET_TICKS
+#define MONONN_BARRIER_BUDGET_TICKS 1000000000ull   // 10 s
+#endif
+
 struct GridBarrier {
   unsigned* flags;   // [gridDim.x * kFlagStride]
+  unsigned* error;   // [0]: 0, or 1 + ordinal of the first barrier a wait gave up on
   unsigned epoch;    // last epoch this workgroup has published
+  unsigned first;    // epoch at kernel start (for the ordinal in the error word)
+  unsigned long long deadline;
 
-  __device__ __forceinline__ void init(unsigned* f) {
+  __device__ __forceinline__ void init(unsigned* f, unsigned* err) {
     flags = f;
+    error = err;
     // all workgroups left the previous launch at the same epoch; pick it up from our own flag
     epoch = __hip_atomic_load(&flags[blockIdx.x * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    first = epoch;
+    deadline = wall_clock64() + MONONN_BARRIER_BUDGET_TICKS;
   }
 
   // A workgroup announces that its part of the stage is written (arrive) and, before it reads anything another
@@ -73,6 +90,12 @@ struct GridBarrier {
   // workgroup without work in a stage need not wait for it at all: flags only grow, so it may announce the next
   // stage right away and wait, when it has work again, for the latest one.
   __device__ __forceinline__ void arrive() {
+#if MONONN_BARRIER_FENCE == 2
+    // The flag is a relaxed store, and the workgroup barrier below waits for LDS traffic only: every wave first
+    // waits until its own write-through stores are acknowledged (vmcnt(0); expcnt / lgkmcnt fields left at their
+    // maxima), so that no byte of the stage is still on its way when thread 0 publishes the flag.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
     __syncthreads();
     epoch += 1;
     if (threadIdx.x == 0) {
@@ -84,22 +107,27 @@ struct GridBarrier {
     }
   }
 
+  // polls flag b until it reaches this workgroup's epoch or the kernel's time budget is spent
+  __device__ __forceinline__ void poll(int b) {
+    unsigned spins = 0;
+    while ((int)(__hip_atomic_load(&flags[b * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
+      __builtin_amdgcn_s_sleep(1);
+      if ((++spins & 63u) == 0u && wall_clock64() > deadline) {
+        unsigned expected = 0;
+        __hip_atomic_compare_exchange_strong(error, &expected, epoch - first, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+  }
+
   __device__ __forceinline__ void wait() {
 #if MONONN_BARRIER_FENCE == 0
     if (threadIdx.x < kWaveSize) {
-      for (int b = threadIdx.x; b < (int)gridDim.x; b += kWaveSize) {
-        while ((int)(__hip_atomic_load(&flags[b * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
-          __builtin_amdgcn_s_sleep(1);
-        }
-      }
+      for (int b = threadIdx.x; b < (int)gridDim.x; b += kWaveSize) poll(b);
       __atomic_thread_fence(__ATOMIC_ACQUIRE);   // agent scope: drop stale lines before the next stage reads
     }
 #else
-    for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
-      while ((int)(__hip_atomic_load(&flags[b * kFlagStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
-        __builtin_amdgcn_s_sleep(1);
-      }
-    }
+    for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) poll(b);
 #if MONONN_BARRIER_FENCE == 1
     __atomic_thread_fence(__ATOMIC_ACQUIRE);
 #endif
@@ -275,6 +303,12 @@ __device__ __forceinline__ float fast_tanh(float x) {
   // tanh(x) = 1 - 2 / (exp(2x) + 1); exact enough in fp32 and safe for large |x|
   float e = __expf(2.0f * x);
   return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+// A run-time index (gather row, dynamic-slice start) clamped to [0, hi] in the index's own type, then narrowed:
+// a 64-bit index far out of range must land on the nearest end, not on whatever its low 32 bits say.
+template <class T>
+__device__ __forceinline__ int clamp_index(T v, int hi) {
+  return v < (T)0 ? 0 : (v > (T)hi ? hi : (int)v);
 }
 template <class T>
 __device__ __forceinline__ T sign_of(T x) {

@@ -231,6 +231,7 @@ void MonoNNModule::load(int device) {
   // The grid barrier needs every workgroup resident at once.  The reference's barrier would
   // deadlock on an over-sized grid; here it is rejected from the occupancy query before launch.
   int capacity = dev_.max_coresident_blocks(hip_.block, hip_.smem);
+  if (capacity < hip_.grid) dev_.unload();   // a refused module must not be launchable
   MONONN_CHECK(capacity >= hip_.grid, kResourceExhausted)
       << "grid of " << hip_.grid << " workgroups x " << hip_.block << " threads exceeds the co-resident capacity of device " << device << " ("
       << capacity << ")";
@@ -238,6 +239,9 @@ void MonoNNModule::load(int device) {
   size_t flag_bytes = 0;
   void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
   dev_.zero(flags, flag_bytes);
+  size_t err_bytes = 0;
+  void* err = dev_.global("mononn_barrier_error", &err_bytes);
+  dev_.zero(err, err_bytes);
   uploaded_.clear();
   for (auto& ci : hip_.constants) {
     if (!ci.literal.empty()) {
@@ -260,6 +264,29 @@ void MonoNNModule::launch(void* const* device_ptrs, size_t n, void* stream) {
   prepare_args(vals);
   for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
   dev_.launch(grid_, hip_.block, hip_.smem, args.data(), stream, hip_.cooperative);
+}
+
+void MonoNNModule::synchronize(void* stream) {
+  MONONN_CHECK(dev_.loaded(), kInvalidArgument) << "synchronize called before load";
+  dev_.synchronize(stream);
+  size_t err_bytes = 0;
+  void* err = dev_.global("mononn_barrier_error", &err_bytes);
+  unsigned word[4] = {0, 0, 0, 0};
+  dev_.download(word, err, sizeof(word));
+  if (word[0] == 0) return;
+  // the workgroups left the kernel at different epochs: start over from a clean slate so that the module stays usable
+  size_t flag_bytes = 0;
+  void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
+  dev_.zero(flags, flag_bytes);
+  dev_.zero(err, err_bytes);
+  MONONN_FAIL(kRuntimeError) << "kernel " << kernel_name_ << ": a workgroup gave up waiting at grid barrier " << word[0] << " of " << hip_.num_barriers
+                             << " after " << spec_.hip.barrier_timeout_ms << " ms (mononn_hip.barrier_timeout_ms): the grid of " << grid_
+                             << " workgroups was not resident as a whole (another kernel running on the device?); the outputs of this launch are invalid";
+}
+
+void* MonoNNModule::global_address(const std::string& symbol, size_t* bytes) const {
+  MONONN_CHECK(dev_.loaded(), kInvalidArgument) << "module globals have addresses once the module is loaded";
+  return dev_.global(symbol, bytes);
 }
 
 double MonoNNModule::read_stage_clock(std::vector<unsigned long long>* ticks, int* n_stages, int* grid) {
@@ -289,7 +316,9 @@ float MonoNNModule::time_kernel(void* const* device_ptrs, size_t n, void* stream
   std::vector<void*> args(n);
   prepare_args(vals);
   for (size_t i = 0; i < n; ++i) args[i] = &vals[i];
-  return dev_.time_launches(grid_, hip_.block, hip_.smem, args.data(), stream, warmup, iters, each, hip_.cooperative);
+  float ms = dev_.time_launches(grid_, hip_.block, hip_.smem, args.data(), stream, warmup, iters, each, hip_.cooperative);
+  synchronize(stream);
+  return ms;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -52,6 +52,9 @@ class MonoNNModule {
   bool loaded() const { return dev_.loaded(); }
   // args: entry parameters in order, live-out buffers in order, temp buffer (device pointers)
   void launch(void* const* device_ptrs, size_t n, void* stream);
+  // waits for `stream` and reports a grid-barrier wait that gave up (kRuntimeError; flags are reset, the module stays usable)
+  void synchronize(void* stream);
+  void* global_address(const std::string& symbol, size_t* bytes) const;
   float time_kernel(void* const* device_ptrs, size_t n, void* stream, int warmup, int iters, std::vector<float>* each = nullptr);
   int grid() const { return grid_; }
   int block() const { return hip_.block; }

@@ -112,6 +112,11 @@ void DeviceModule::download(void* host_dst, const void* src, size_t bytes) const
   HIP_OK(hipMemcpy(host_dst, src, bytes, hipMemcpyDeviceToHost));
 }
 
+void DeviceModule::synchronize(void* stream) const {
+  HIP_OK(hipSetDevice(device_));
+  HIP_OK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+}
+
 double DeviceModule::wall_clock_ticks_per_us() const {
   int khz = 0;
   HIP_OK(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device_));

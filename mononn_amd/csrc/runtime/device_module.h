@@ -46,6 +46,7 @@ class DeviceModule {
   void upload(void* dst, const void* host_src, size_t bytes) const;
   void zero(void* dst, size_t bytes) const;
   void download(void* host_dst, const void* src, size_t bytes) const;   // synchronises the device first
+  void synchronize(void* stream) const;
   double wall_clock_ticks_per_us() const;
 
   // workgroups of `block` threads and `smem` bytes of LDS that can be resident on the whole device

@@ -87,6 +87,9 @@ struct HipOptions {       // "mononn_hip" section
   // (two half-resident grids would wait for each other at their first barrier).  true: cooperative launch, the
   // runtime keeps such kernels apart at the price of ~20 us more per launch.
   bool cooperative_launch = false;
+  // A grid-barrier wait that is still polling this long after the kernel started gives up (the kernel then runs to
+  // its end and the host finds an error word): what stands between a grid that is not wholly resident and a hang.
+  int barrier_timeout_ms = 10000;
   // GEMM stages request their packed weights between announcing the end of the previous stage and waiting for the
   // other workgroups (the wait moves behind the requests; idle workgroups skip it)
   bool operand_preload = true;

@@ -20,6 +20,8 @@
 #define __hip_atomic_load(p, order, scope) (*(p))
 #define __builtin_amdgcn_s_sleep(x) break /* the only use is the body of a spin on a flag */
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_s_waitcnt(x) ((void)0)
+#define __hip_atomic_compare_exchange_strong(p, expected, v, ok, fail, scope) (*(p) == *(expected) ? (*(p) = (v), true) : false)
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) (src)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __shfl_xor(v, ...) (v)

@@ -353,7 +353,7 @@ def test_reduce_window_update_slice_and_variadic_reduce_are_lowered():
     text, _ = pool_module((1, 8, 8, 4), (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0),) * 4, "sum")
     assert ">= 0 &&" not in MonoNNModule.compile(text, build=False).get_source("main.hip")
     src = MonoNNModule.compile(update_slice_module((6, 10, 8), (2, 4, 8)), build=False).get_source("main.hip")
-    assert "min(max((int)" in src and ", 0), 4)" in src and ", 0), 6)" in src and "else" in src     # starts clamped to extent - update
+    assert "mononn_dev::clamp_index(" in src and ", 4);" in src and ", 6);" in src and "else" in src     # starts clamped to extent - update
     # a tuple-valued reduce over the last dimension is a row program (the lanes exchange whole tuples, the reducer is
     # inlined as a local lambda); over another dimension it is a serial loop of the thread that owns the element
     src = MonoNNModule.compile(arg_reduce_module(7, 50), build=False).get_source("main.hip")
