@@ -105,6 +105,17 @@ int mononn_module_load(mononn_module* m, int device);
  *           on `stream` (a hipStream_t, NULL = default stream). */
 int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);
 
+/* mononn_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the temp arena is a fixed array of mononn_static_temp_bytes() bytes (64 MiB) in
+ * the library's own device image instead of a buffer of the caller, and the call allocates nothing.  device_ptrs:
+ * entry parameters in parameter order, then live-out buffers -- no temp slot.  A module whose temp arena is larger
+ * is refused with MONONN_RESOURCE_EXHAUSTED.  Each GPU holds one such array from the first mononn_module_load on it
+ * until the process ends; every call on a GPU, from any module, shares it, so calls that overlap on one GPU race.
+ * Nothing in the arena has to start at zero: every temp address is written before it is read in the same launch.
+ * No counterpart in the reference. */
+int mononn_launch_static_temp(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);
+size_t mononn_static_temp_bytes(void);
+
 /* Wait for `stream` and report what the kernel could not: MONONN_RUNTIME_ERROR when a grid-barrier wait of a launch
  * gave up (the grid was not resident as a whole within mononn_hip.barrier_timeout_ms of the specification, e.g. an
  * ordinary launch beside another kernel).  Every workgroup of such a launch still runs to its end, so the kernel

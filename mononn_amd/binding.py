@@ -61,6 +61,8 @@ def _load_library() -> ctypes.CDLL:
     lib.mononn_module_set_constant.argtypes = [c.c_void_p, c.c_char_p, c.c_void_p, c.c_size_t]
     lib.mononn_module_load.argtypes = [c.c_void_p, c.c_int]
     lib.mononn_launch.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p]
+    lib.mononn_launch_static_temp.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p]
+    lib.mononn_static_temp_bytes.restype = c.c_size_t
     lib.mononn_module_synchronize.argtypes = [c.c_void_p, c.c_void_p]
     lib.mononn_module_global.argtypes = [c.c_void_p, c.c_char_p, P(c.c_void_p), P(c.c_size_t)]
     lib.mononn_time_kernel.argtypes = [c.c_void_p, P(c.c_void_p), c.c_size_t, c.c_void_p, c.c_int, c.c_int,
@@ -81,7 +83,7 @@ EXPORTED_SYMBOLS = [
     "mononn_module_destroy", "mononn_module_kernel_name", "mononn_module_spec_json", "mononn_module_source",
     "mononn_module_code_object", "mononn_module_summary", "mononn_module_buffer_info", "mononn_module_launch_dims", "mononn_module_owns_temp",
     "mononn_module_num_constants", "mononn_module_constant_info", "mononn_module_set_constant", "mononn_module_load",
-    "mononn_launch", "mononn_module_synchronize", "mononn_module_global", "mononn_time_kernel", "mononn_module_stage_clock", "mononn_module_stage_name", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
+    "mononn_launch", "mononn_launch_static_temp", "mononn_static_temp_bytes", "mononn_module_synchronize", "mononn_module_global", "mononn_time_kernel", "mononn_module_stage_clock", "mononn_module_stage_name", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
 
 
 def _check(rc: int):
@@ -218,6 +220,11 @@ class MonoNNModule:
     def launch_raw(self, device_ptrs: Sequence[int], stream: int = 0):
         arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
         _check(_lib.mononn_launch(self._h, arr, len(device_ptrs), ctypes.c_void_p(stream)))
+
+    def launch_static_temp(self, device_ptrs: Sequence[int], stream: int = 0):
+        """mononn_launch_static_temp: parameters and live-outs only; the temp arena is the library's static device array."""
+        arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
+        _check(_lib.mononn_launch_static_temp(self._h, arr, len(device_ptrs), ctypes.c_void_p(stream)))
 
     def synchronize(self, stream: int = 0):
         """Wait for `stream`; raises MonoNNError(RUNTIME_ERROR) when a grid-barrier wait of a launch gave up."""

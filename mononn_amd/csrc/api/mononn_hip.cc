@@ -10,6 +10,7 @@
 #include "hlo/hlo.h"
 #include "module/mononn_module.h"
 #include "runtime/device_module.h"
+#include "runtime/static_scratch.h"
 #include "tuner/tuner.h"
 
 using mononn::Error;
@@ -207,6 +208,15 @@ int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, voi
     m->impl->launch(device_ptrs, n_ptrs, stream);
   });
 }
+
+int mononn_launch_static_temp(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream) {
+  return guarded([&] {
+    require(m && device_ptrs, "NULL argument");
+    m->impl->launch_static_temp(device_ptrs, n_ptrs, stream);
+  });
+}
+
+size_t mononn_static_temp_bytes(void) { return mononn::runtime::static_scratch_bytes(); }
 
 int mononn_module_synchronize(mononn_module* m, void* stream) {
   return guarded([&] {

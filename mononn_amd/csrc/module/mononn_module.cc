@@ -13,6 +13,7 @@
 #include "common/status.h"
 #include "hlo/hlo.h"
 #include "runtime/rtc.h"
+#include "runtime/static_scratch.h"
 
 namespace mononn {
 namespace module {
@@ -236,6 +237,9 @@ void MonoNNModule::load(int device) {
       << "grid of " << hip_.grid << " workgroups x " << hip_.block << " threads exceeds the co-resident capacity of device " << device << " ("
       << capacity << ")";
   grid_ = hip_.grid;
+  // once per device, with that device current: the address of the library's static temp arena on this GPU
+  static_scratch_error_.clear();
+  runtime::static_scratch_setup(device, &static_scratch_error_);
   size_t flag_bytes = 0;
   void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
   dev_.zero(flags, flag_bytes);
@@ -252,6 +256,34 @@ void MonoNNModule::load(int device) {
     if (it != host_constants_.end()) upload_constant(ci, it->second);
   }
   host_constants_.clear();
+}
+
+void MonoNNModule::launch_static_temp(void* const* device_ptrs, size_t n, void* stream) {
+  // Same kernel, same launch; the temp arena is the library's own fixed device array instead of a caller's buffer.
+  // Nothing here allocates device memory, and the argument tables live on the stack.
+  MONONN_CHECK(dev_.loaded(), kInvalidArgument) << "launch called before load";
+  MONONN_CHECK(n + 1 == num_args(), kInvalidArgument) << "kernel takes " << num_args() - 1 << " buffers (parameters, live-outs) besides the temp arena, got " << n;
+  constexpr size_t kMaxArgs = 1024;   // the reference's own limit on kernel arguments (mononn_module_tuner.cc:113-127)
+  MONONN_CHECK(n + 1 <= kMaxArgs, kInvalidArgument) << "more than " << kMaxArgs << " kernel arguments";
+  MONONN_CHECK(hip_.temp_bytes <= static_cast<int64_t>(runtime::static_scratch_bytes()), kResourceExhausted)
+      << "kernel " << kernel_name_ << " needs a temp arena of " << hip_.temp_bytes << " bytes, the library's static arena holds "
+      << runtime::static_scratch_bytes() << ": use mononn_launch with a buffer of the caller";
+  void* arena = runtime::static_scratch_address(dev_.device());
+  MONONN_CHECK(arena != nullptr, kRuntimeError) << "the static arena has no address on device " << dev_.device() << ": " << static_scratch_error_;
+  for (auto& c : hip_.constants)
+    MONONN_CHECK(!c.literal.empty() || uploaded_.count(c.name) || host_constants_.count(c.name), kInvalidArgument)
+        << "constant " << c.hlo_name << " has no payload yet";
+  void* vals[kMaxArgs];
+  void* args[kMaxArgs];
+  for (size_t i = 0; i < n; ++i) {
+    MONONN_CHECK(device_ptrs[i] != nullptr, kInvalidArgument) << "buffer " << i << " is null";
+    MONONN_CHECK(reinterpret_cast<uintptr_t>(device_ptrs[i]) % 16 == 0, kInvalidArgument) << "buffer " << i << " is not 16-byte aligned";
+    vals[i] = device_ptrs[i];
+    args[i] = &vals[i];
+  }
+  vals[n] = arena;
+  args[n] = &vals[n];
+  dev_.launch(grid_, hip_.block, hip_.smem, args, stream, hip_.cooperative);
 }
 
 void MonoNNModule::launch(void* const* device_ptrs, size_t n, void* stream) {

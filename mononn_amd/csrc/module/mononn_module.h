@@ -52,6 +52,8 @@ class MonoNNModule {
   bool loaded() const { return dev_.loaded(); }
   // args: entry parameters in order, live-out buffers in order, temp buffer (device pointers)
   void launch(void* const* device_ptrs, size_t n, void* stream);
+  // the same launch with the library's static device arena as temp buffer: device_ptrs = parameters, live-outs
+  void launch_static_temp(void* const* device_ptrs, size_t n, void* stream);
   // waits for `stream` and reports a grid-barrier wait that gave up (kRuntimeError; flags are reset, the module stays usable)
   void synchronize(void* stream);
   void* global_address(const std::string& symbol, size_t* bytes) const;
@@ -88,6 +90,7 @@ class MonoNNModule {
   int grid_ = 0;
   std::map<std::string, std::vector<char>> host_constants_;   // canonical name -> payload as given
   std::map<std::string, bool> uploaded_;
+  std::string static_scratch_error_;   // why the static temp arena has no address on this device ("" when it has)
 };
 
 // helpers shared with the tuner / CLI
