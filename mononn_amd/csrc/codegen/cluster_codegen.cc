@@ -576,6 +576,39 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
   // 11.6 ms: stages whose code did not change, attention and LayerNorm, slow down with them), so they are
   // neither the default nor tuner candidates (they win the isolated stage clocks and lose in the whole kernel);
   // a specification may still name them (up to 64 accumulator fragments per wave).
+  // Large problems (any MFMA-capable GEMM with k a multiple of 32): operand tiles go through LDS once per workgroup.
+  // Among the tile shapes the one that needs the least time by a simple model: rounds of tiles over the compute
+  // units x tile area / throughput of a compute unit that is busy with such a tile, relative to 256 x 256 (measured
+  // on [6144, 1024] x [1024, 4096] with both operands in fragment order: 1.0 PFLOP/s-equivalent for 256 x 256,
+  // which fills the chip only 1.5 times there; 0.87 for 192 x 256, which fills it twice).
+  if (gemm_uses_mfma(g) && g.K % 32 == 0 && g.K >= 128 && waves == 4 && ls.waves_per_simd == 1 && g.split_k <= 1) {
+    struct Cand { int bm, bn, bk; double eff; };
+    double best = 0;
+    const int cus = std::max(num_cus, 1);
+    for (const Cand& c : {Cand{256, 256, 32, 1.0}, Cand{192, 256, 32, 0.86}, Cand{256, 192, 32, 0.82}, Cand{256, 128, 64, 0.78}, Cand{128, 256, 64, 0.77},
+                          Cand{192, 128, 64, 0.74}, Cand{128, 128, 64, 0.65}}) {
+      if (g.M < c.bm || g.N < c.bn) continue;
+      const int64_t units = ((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn) * g.batch;
+      if (units < cus) continue;   // every compute unit gets a tile, or the small-problem paths below take over
+      const int64_t rounds = (units + cus - 1) / cus;
+      // per tile: its multiply-adds at the tile's efficiency plus a fixed cost (first operands on their way, epilogue,
+      // waves of a workgroup out of step) worth about ten million multiply-adds
+      const double cost = static_cast<double>(rounds) * (static_cast<double>(c.bm) * c.bn * g.K / c.eff + 1.0e7);
+      if (best == 0 || cost < best) {
+        best = cost;
+        t.bm = c.bm;
+        t.bn = c.bn;
+        t.bk = c.bk;
+      }
+    }
+    if (best > 0) {
+      t.wm = 2;
+      t.wn = 2;
+      t.wk = 1;
+      t.stages = 2;
+      return t;
+    }
+  }
   for (int per_wave : {64, 32}) {
     int wm = 1, wn = waves;
     while (wn > wm) {
@@ -623,6 +656,16 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
       << "GEMM wave arrangement " << t.wm << "x" << t.wn << "x" << t.wk << " does not use " << ls.waves() << " waves";
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)
       << "GEMM tile " << t.bm << "x" << t.bn << " is not a multiple of 16 per wave";
+  if (t.stages >= 2) {
+    MONONN_CHECK(!has_prologue && t.wk == 1 && g.K % 32 == 0, kSpecError) << "an LDS-staged GEMM tile takes no row-program prologue, no k split over waves and a k extent that is a multiple of 32";
+    MONONN_CHECK(t.stages == 2 && t.bk >= 32 && t.bk % 32 == 0 && t.bk <= 128, kSpecError)
+        << "LDS-staged GEMM tile: " << t.stages << " stages of " << t.bk << " k: two LDS buffers of 32, 64, 96 or 128 k";
+    const int kstp = t.bk / 16, ablk = t.bm / 32 * kstp, bblk = t.bn / 32 * kstp;   // 1 KiB blocks of 32 rows x 16 k
+    MONONN_CHECK(t.bm % (32 * t.wm) == 0 && t.bn % (32 * t.wn) == 0, kSpecError) << "LDS-staged GEMM tile " << t.bm << "x" << t.bn << " is not a multiple of 32 per wave";
+    MONONN_CHECK(ablk % ls.waves() == 0 && bblk % ls.waves() == 0, kSpecError)
+        << "LDS-staged GEMM tile " << t.bm << "x" << t.bn << "x" << t.bk << ": the " << ls.waves() << " waves cannot share the copy of a k tile evenly";
+    MONONN_CHECK((ablk + bblk) / ls.waves() <= 16, kSpecError) << "LDS-staged GEMM tile " << t.bm << "x" << t.bn << "x" << t.bk << ": more than 16 staged pieces per lane and k tile";
+  }
   int frags = (t.bm / t.wm / 16) * (t.bn / t.wn / 16);
   const int max_frags = ls.waves_per_simd >= 2 ? 32 : 64;   // 4 accumulator registers each, out of 512 / waves per SIMD
   MONONN_CHECK(frags <= max_frags, kSpecError) << "GEMM tile " << t.bm << "x" << t.bn << " needs " << frags << " accumulator fragments per wave (max " << max_frags << ")";
@@ -1157,7 +1200,27 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fb.line("const int ksplit = rem0 % " + S(S_) + ";");
     fb.line("const int rem = rem0 / " + S(S_) + ";");
     if (g.split_k > 1) fb.line(epi.init_line);
-    if (tiles_n % 8 == 0 && S_ == 1) {
+    // LDS-staged tiles (large problems): the 8 XCDs each take a rectangle of the tile grid, rm x rn tiles, walked
+    // row by row, so that the tiles an XCD works on at one time share few operand panels: every panel an XCD
+    // touches comes over the fabric once per XCD, and with a strip of single columns (below) the left operand
+    // would cross it once per XCD for every tile column.  The split of the grid into gm x gn rectangles is the
+    // one with the fewest panel bytes per XCD.
+    int gm = 0, gn = 0;
+    if (t.stages >= 2 && S_ == 1) {
+      int64_t best = -1;
+      for (int a : {1, 2, 4, 8}) {
+        const int b = 8 / a;
+        if (tiles_m % a || tiles_n % b) continue;
+        const int64_t cost = tiles_m / a * t.bm + tiles_n / b * t.bn;
+        if (best < 0 || cost < best) best = cost, gm = a, gn = b;
+      }
+    }
+    if (gm > 0) {
+      const int64_t rn = tiles_n / gn, rm = tiles_m / gm;
+      fb.line("const int xcd = rem & 7, q = rem >> 3;   // " + S(rm) + " x " + S(rn) + " tiles per XCD");
+      fb.line("const int tile_n = (xcd / " + S(gm) + ") * " + S(rn) + " + q % " + S(rn) + ";");
+      fb.line("const int tile_m = (xcd % " + S(gm) + ") * " + S(rm) + " + q / " + S(rn) + ";");
+    } else if (tiles_n % 8 == 0 && S_ == 1) {
       fb.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
       fb.line("const int tile_m = (rem >> 3) % " + S(tiles_m) + ";");
     } else {
@@ -1176,20 +1239,31 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
          << "    return in + (((long)n * " << c.H << " + p * " << c.stride_h << " + r) * " << c.W << " + q * " << c.stride_w << ") * " << c.C << " + sc;\n"
          << "  }\n};\n";
       conv_struct = am.str();
-      call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", false, " << g.K
-           << ", @NAME@_epi, mononn_dev::NoPrologue, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
-           << ", bidx, tile_m, tile_n, epi, smem, mononn_dev::NoPrologue(), @NAME@_amap());";
+      if (t.stages >= 2)
+        call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", false, false, false, "
+             << t.bk << ", @NAME@_epi, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
+             << ", bidx, tile_m, tile_n, epi, smem, @NAME@_amap());";
+      else
+        call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", false, " << g.K
+             << ", @NAME@_epi, mononn_dev::NoPrologue, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
+             << ", bidx, tile_m, tile_n, epi, smem, mononn_dev::NoPrologue(), @NAME@_amap());";
     } else {
       std::ostringstream b_expr;
       b_expr << pb << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS);
-      preload = t.preload_b && g.b_packed;
-      call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
-           << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
-           << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
-           << (epi.along_m ? "true" : "false") << ">("
-           << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
-           << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
-           << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");
+      preload = t.preload_b && g.b_packed && t.stages < 2;
+      if (t.stages >= 2)
+        call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", "
+             << (g.a_packed ? "true" : "false") << ", " << (g.b_packed ? "true" : "false") << ", " << (epi.along_m ? "true" : "false") << ", " << t.bk
+             << ", @NAME@_epi>(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
+             << b_expr.str() << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
+      else
+        call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
+             << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
+             << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
+             << (epi.along_m ? "true" : "false") << ">("
+             << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
+             << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
+             << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");
       call << ");";
       if (preload) {
         // the companion repeats the unit decoding as far as the right operand needs it
@@ -1214,6 +1288,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     }
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
+    if (t.stages >= 2) smem = 2 * (t.bm + t.bn) * t.bk * 2;
     smem = std::max(smem, pro.smem);
   } else {
     const int64_t total = g.batch * g.M * g.N;

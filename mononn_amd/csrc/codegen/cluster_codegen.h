@@ -39,6 +39,10 @@ struct GemmTuning {
   // the function takes the first chunk of packed weights from registers filled by a companion function
   // (NodeFunction::preload_text) that the kernel calls before it waits at the grid barrier
   bool preload_b = false;
+  // 2: operand tiles of bk k each are staged through two LDS buffers, once per workgroup
+  // (mononn_dev::gemm_tile_lds; wk must be 1); 1: every wave fetches its own fragments from global memory
+  int stages = 1;
+  int bk = 32;
 };
 
 struct NodeFunction {

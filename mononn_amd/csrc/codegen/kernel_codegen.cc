@@ -174,6 +174,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         g.warp_m = t.bm / t.wm;
         g.warp_n = t.bn / t.wn;
         g.warp_k = static_cast<int>(n.gemm.K / t.wk);
+        g.stages = t.stages;
+        g.tb_k = t.bk;
         if (!gemm_uses_mfma(n.gemm)) g.operator_class = "SIMT";
         auto bc = n.members[0]->attrs.find("backend_config");
         if (bc != n.members[0]->attrs.end()) g.backend_config = Json::parse(bc->second);
@@ -184,6 +186,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         t.wm = it->second.wave_m;
         t.wn = it->second.wave_n;
         t.wk = it->second.wave_k;
+        t.stages = it->second.stages;
+        t.bk = it->second.tb_k;
       }
       t.split_k = n.gemm.split_k;
       t.preload_b = spec.hip.operand_preload;
@@ -269,6 +273,12 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   if (spec.hip.barrier == "flags_allfence") pre << "#define MONONN_BARRIER_FENCE 1\n";
   else if (spec.hip.barrier == "flags_coherent") pre << "#define MONONN_BARRIER_FENCE 2\n#define MONONN_COHERENT_STORES 1\n";
   else MONONN_CHECK(spec.hip.barrier == "flags", kSpecError) << "unknown barrier flavour '" << spec.hip.barrier << "'";
+  {
+    // see mononn_dev::thread_id(): on in kernels that hold a stage with a large register tile (an LDS-staged GEMM)
+    bool opaque = spec.hip.opaque_thread_id;
+    for (auto& kv : spec.gemm_spec_list) opaque = opaque || kv.second.stages >= 2;
+    pre << "#define MONONN_OPAQUE_THREAD_ID " << (opaque ? 1 : 0) << "\n";
+  }
   pre << "#define MONONN_BARRIER_BUDGET_TICKS " << static_cast<long long>(spec.hip.barrier_timeout_ms) * 100000 << "ull   // wall clock: 100 MHz\n";
   pre << "#include \"headers.h\"\n\n";
   for (auto& c : hp.constants) {
@@ -294,7 +304,17 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   for (auto& g : globals) hp.global_decls.push_back(g);
   for (auto& g : hp.global_decls) glob << g << "\n";
   glob << "\n";
-  for (auto& d : fn_defs) src << d << "\n";
+  for (auto& d : fn_defs) {
+    // node functions read the thread index through mononn_dev::thread_id() (see there: keeps per-stage address
+    // arithmetic inside its stage)
+    std::string text = d;
+    size_t pos = 0;
+    while ((pos = text.find("threadIdx.x", pos)) != std::string::npos) {
+      text.replace(pos, 11, "mononn_dev::thread_id()");
+      pos += 23;
+    }
+    src << text << "\n";
+  }
 
   // The kernel is a small interpreter over the list of calls (node function + buffers), stage by stage.
   // Every distinct node function is inlined exactly once, in one case of the dispatch switch: calling

@@ -46,13 +46,39 @@ typedef int int4_t __attribute__((ext_vector_type(4)));
 #define MONONN_WAVES_PER_SIMD 1
 #endif
 
+// an empty statement after which the compiler knows nothing about the value of `v` (a vector register)
+#ifndef MONONN_OPAQUE_VALUE
+#define MONONN_OPAQUE_VALUE(v) asm volatile("" : "+v"(v))
+#endif
+// an empty statement that requires `v` in accumulation registers at this point of the program
+#ifndef MONONN_PIN_ACC
+#define MONONN_PIN_ACC(v) asm volatile("" : "+a"(v))
+#endif
+
 namespace mononn_dev {
 
 constexpr int kWaveSize = 64;
 constexpr int kFlagStride = 64;   // 256 bytes between workgroup flags: measured fastest among 64 B .. 4 KiB
 
-__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWaveSize - 1); }
-__device__ __forceinline__ int wave_id() { return threadIdx.x / kWaveSize; }
+// The thread's index in its workgroup, opaque to the compiler (MONONN_OPAQUE_THREAD_ID, the default): the kernel is
+// one function holding every stage, and whatever the compiler can derive from threadIdx.x once -- lane and wave
+// numbers, address parts of every stage -- it computes ahead of the stage loop and keeps in registers through all
+// stages.  A stage with a large register tile then pushes those values out to scratch, and the stages that use
+// them reload them in their inner loops (measured on a 12-layer decoder: one 256-register GEMM tile in the kernel
+// made the attention stages 29 -> 65 us and the row programs 14 -> 24 us; with the index re-read per use the same
+// kernel runs faster than without the tile).
+#ifndef MONONN_OPAQUE_THREAD_ID
+#define MONONN_OPAQUE_THREAD_ID 1
+#endif
+__device__ __forceinline__ int thread_id() {
+  int t = threadIdx.x;
+#if MONONN_OPAQUE_THREAD_ID
+  MONONN_OPAQUE_VALUE(t);
+#endif
+  return t;
+}
+__device__ __forceinline__ int lane_id() { return thread_id() & (kWaveSize - 1); }
+__device__ __forceinline__ int wave_id() { return thread_id() / kWaveSize; }
 
 // ---------------------------------------------------------------------------------------------
 // grid-wide barrier
@@ -606,6 +632,280 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         if (m < M && n < N) {
           float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
           epi(batch, m, n, v, pre[i * TN + j]);
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// GEMM for large problems: operand tiles staged through LDS, once per workgroup
+// ---------------------------------------------------------------------------------------------
+// gemm_tile above has every wave fetch its own fragments from global memory; with many rows the same fragment is
+// wanted by all waves (and all workgroups) of a tile row / column and the vector L1 becomes the limit.  Here a
+// workgroup of WM x WN waves owns a BM x BN tile, every k tile of BK is brought into LDS once, by all waves
+// together, and each wave reads the fragments of its (BM / WM) x (BN / WN) block from there.
+//
+// The MFMA is v_mfma_f32_32x32x16_f16: measured on this part it retires 32 clocks apart at twice the work of the
+// 16x16x32 form, which retires 27 clocks apart (2.2 against 1.4 PFLOP/s with every SIMD busy).  An operand fragment
+// is 32 rows x 16 k: lane l holds row l % 32, k piece l / 32 (8 halves).  LDS holds fragments in exactly that
+// order, block (row block of 32, k step of 16) = 1 KiB with lane l's piece at byte 16 * l, so that a fragment
+// read is ds_read_b128 at 16 * lane and a copy is ds_write_b128 at 16 * lane (no bank conflicts).  Memory keeps
+// the layouts of the rest of the kernel (row-major k-contiguous, or the 16-row x 32-k fragment order of packed
+// weights and in-kernel operands): each lane simply loads the 16 bytes that belong in its slot; from
+// fragment-order memory the 64 pieces of a block are four runs of 256 contiguous bytes.
+//
+// Pipeline, in k tiles: tile t is multiplied out of LDS buffer t % 2 while tile t + 1 is written from registers into
+// the other buffer and tile t + 3 is requested from memory into the registers that this frees; tile t + 2 is on
+// its way in a second set of registers.  A wave alone on its SIMD has nobody to hide its memory instructions
+// behind, and it issues in order: fragment reads, LDS writes and global loads are placed between the MFMAs by
+// hand, one MFMA at a time, each slot fenced from the instruction scheduler.  (The direct global-to-LDS load was
+// tried first: on this part one such load keeps the memory pipeline busy for hundreds of clocks, copies alone took
+// as long as the MFMAs alone, and in-order issue adds the two up.)
+//
+// One workgroup barrier per k tile, before its last step: "every wave has written its share of tile t + 1" and
+// "every wave has the last fragments of tile t in registers", so buffer t % 2 may be written during tile t + 1.
+
+// A buffer descriptor over `base` (byte offsets of up to 4 GiB): loads address memory as descriptor + 32-bit lane
+// offset + wave-uniform offset, which keeps one register per copy alive across the k loop.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t whole_buffer(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
+}
+__device__ __forceinline__ half8_t buffer_load_16(__amdgpu_buffer_rsrc_t buffer, unsigned lane_offset, unsigned wave_offset) {
+  typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+  // the wave-uniform offset is named as such: where the compiler cannot prove it, it wraps the load into a loop
+  // over the distinct values
+  const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, __builtin_amdgcn_readfirstlane(wave_offset), 0);
+  half8_t h;
+  __builtin_memcpy(&h, &v, 16);
+  return h;
+}
+
+template <bool B>
+struct BoolConstant {
+  static constexpr bool value = B;
+};
+
+constexpr int gemm_lds_bytes(int BM, int BN, int BK) { return 2 * (BM + BN) * BK * 2; }
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// BK: k extent of one LDS buffer (a multiple of 32); K a multiple of 32.
+template <int BM, int BN, int WM, int WN, int K, int KTOTAL, bool PACKED_A, bool PACKED_B, bool D_ALONG_M, int BK, class Epi,
+          class AMap = RowMajorA>
+__device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, int M, int N, int lda, int ldb, int batch, int tile_m,
+                                              int tile_n, Epi& epi, char* smem, const AMap& amap = AMap()) {
+  constexpr int NW = WM * WN;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;             // 32 x 32 fragments per wave
+  constexpr int KSTP = BK / 16;                                    // MFMA steps per k tile
+  constexpr int ABLK = BM / 32 * KSTP, BBLK = BN / 32 * KSTP;      // 1 KiB blocks of one k tile
+  constexpr int STAGE_BYTES = (ABLK + BBLK) * 1024;
+  constexpr int KSTEPS = K / 16;
+  constexpr int KT = (KSTEPS + KSTP - 1) / KSTP;                   // k tiles; the last one may hold fewer steps
+  constexpr bool SHORT_LAST = KSTEPS % KSTP != 0;
+  static_assert(K % 32 == 0 && BK % 32 == 0, "the LDS-staged tile takes k extents that are multiples of 32");
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile/wave mismatch");
+  static_assert(ABLK % NW == 0 && BBLK % NW == 0, "the waves share the copy of a k tile evenly");
+  static_assert(!PACKED_A || AMap::kRowMajor, "a fragment-order left operand takes no row map");
+  constexpr int ACPY = ABLK / NW, BCPY = BBLK / NW;                // copies per lane and k tile
+  constexpr int CPY = ACPY + BCPY;
+  const int lane = lane_id();
+  const int wave = wave_id();
+  const int wn = wave % WN;
+  const int wm = wave / WN;
+  const int r32 = lane & 31;
+  const int kq = (lane >> 5) * 8;   // this lane's k piece inside a step of 16
+
+  // Byte offset from the operand's base of the piece this lane copies for block (row block, step 0 of k tile 0).
+  // Fragment-order memory: [row / 16][k / 32][(k % 32 / 8) * 16 + row % 16][8 halves]; a step of 16 k is half such
+  // a block, 512 bytes on.
+  auto piece_offset = [&](bool packed, int row, int ld) -> unsigned {
+    if (packed) return (((unsigned)(row >> 4) * (KTOTAL / 32)) * 512u + ((kq >> 3) * 16 + (row & 15)) * 8) * 2u;
+    return ((unsigned)row * (unsigned)ld + kq) * 2u;
+  };
+  constexpr unsigned A_STEP = PACKED_A ? 512u : 32u;   // bytes between consecutive steps of 16 k
+  constexpr unsigned B_STEP = PACKED_B ? 512u : 32u;
+  const __amdgpu_buffer_rsrc_t a_buf = whole_buffer(A), b_buf = whole_buffer(B);
+  unsigned a_off[ACPY], b_off[BCPY];
+  int a_row[ACPY];
+#pragma unroll
+  for (int j = 0; j < ACPY; ++j) {
+    const int blk = wave + j * NW, rb = blk / KSTP;
+    int m = tile_m * BM + rb * 32 + r32;
+    m = m < M ? m : M - 1;
+    a_row[j] = m;
+    a_off[j] = piece_offset(PACKED_A, m, lda);
+  }
+#pragma unroll
+  for (int j = 0; j < BCPY; ++j) {
+    const int blk = wave + j * NW, rb = blk / KSTP;
+    int n = tile_n * BN + rb * 32 + r32;
+    const int n_max = PACKED_B ? (N + 15) / 16 * 16 - 1 : N - 1;   // packed weights are padded to whole blocks of 16 columns
+    n = n < n_max ? n : n_max;
+    b_off[j] = piece_offset(PACKED_B, n, ldb);
+  }
+
+  // c-th of the CPY pieces this lane moves per k tile (the left operand's first): memory -> register, register ->
+  // LDS.  Tiles past the end are the last tile once more (a redundant copy into a buffer nobody reads any more,
+  // which keeps the loop body free of branches); the steps of the last tile that lie past the end of k re-read
+  // its first step and are not multiplied.
+  half8_t staged[2][CPY];
+  auto load_one = [&](int t, int set, int c) {
+    t = t < KT ? t : KT - 1;
+    if (c < ACPY) {
+      const int blk = wave + c * NW, ks = blk % KSTP;
+      const bool past = SHORT_LAST && t * KSTP + ks >= KSTEPS;
+      if constexpr (AMap::kRowMajor) {
+        staged[set][c] = buffer_load_16(a_buf, a_off[c], (unsigned)(t * KSTP + (past ? 0 : ks)) * A_STEP);
+      } else {
+        const half_t* src = amap(A, a_row[c], (t * KSTP + (past ? 0 : ks)) * 16 + kq, lda);
+        staged[set][c] = buffer_load_16(a_buf, (unsigned)(reinterpret_cast<const char*>(src) - reinterpret_cast<const char*>(A)), 0u);
+      }
+    } else {
+      const int blk = wave + (c - ACPY) * NW, ks = blk % KSTP;
+      const bool past = SHORT_LAST && t * KSTP + ks >= KSTEPS;
+      staged[set][c] = buffer_load_16(b_buf, b_off[c - ACPY], (unsigned)(t * KSTP + (past ? 0 : ks)) * B_STEP);
+    }
+  };
+  // LDS is named outright (a generic pointer would turn the accesses into flat ones wherever the compiler cannot
+  // see where `smem` comes from)
+  typedef __attribute__((address_space(3))) char lds_char_t;
+  typedef __attribute__((address_space(3))) half8_t lds_half8_t;
+  lds_char_t* const lds = (lds_char_t*)smem;
+  auto store_one = [&](int buf, int set, int c) {
+    const int blk = c < ACPY ? wave + c * NW : ABLK + wave + (c - ACPY) * NW;
+    *reinterpret_cast<lds_half8_t*>(lds + buf * STAGE_BYTES + blk * 1024 + lane * 16) = staged[set][c];
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // A lane's part of a 32 x 32 fragment: four groups g of four consecutive positions along one dimension (offset
+  // 8 * g + 4 * (lane / 32)), at position lane % 32 of the other.  Along n unless D_ALONG_M.
+  const int m_base = tile_m * BM + wm * (TM * 32);
+  const int n_base = tile_n * BN + wn * (TN * 32);
+  const int lane_m = D_ALONG_M ? (lane >> 5) * 4 : r32;
+  const int lane_n = D_ALONG_M ? r32 : (lane >> 5) * 4;
+  // Operands of the epilogue (bias, residual) are requested one row of fragments ahead of their use: the first row
+  // now, row i + 1 while row i is finalised (all of them at once would cost more registers than the tile has left).
+  typename Epi::Pre pre[2][TN * 4];
+  auto preload_row = [&](int i, typename Epi::Pre (&dst)[TN * 4]) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int m = m_base + i * 32 + lane_m + (D_ALONG_M ? 8 * g : 0);
+        int n = n_base + j * 32 + lane_n + (D_ALONG_M ? 0 : 8 * g);
+        if (D_ALONG_M) {
+          m = m < M ? m : (M >= 4 ? M - 4 : 0);
+          n = n < N ? n : N - 1;
+        } else {
+          m = m < M ? m : M - 1;
+          n = n < N ? n : (N >= 4 ? N - 4 : 0);
+        }
+        epi.preload(batch, m, n, dst[j * 4 + g]);
+      }
+  };
+  preload_row(0, pre[0]);
+
+  // tiles 0 and 1 on their way; tile 0 into LDS (the previous unit of this workgroup may still be reading its last
+  // tiles there: barrier first); tile 2 requested into the registers tile 0 has left
+#pragma unroll
+  for (int c = 0; c < CPY; ++c) load_one(0, 0, c);
+#pragma unroll
+  for (int c = 0; c < CPY; ++c) load_one(1, 1, c);
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < CPY; ++c) store_one(0, 0, c);
+#pragma unroll
+  for (int c = 0; c < CPY; ++c) load_one(2, 0, c);
+  __syncthreads();
+
+  const lds_char_t* a_frag = lds + (wm * TM * KSTP) * 1024 + lane * 16;
+  const lds_char_t* b_frag = lds + (ABLK + wn * TN * KSTP) * 1024 + lane * 16;
+  half8_t fa[2][TM], fb[2][TN];
+  auto read_one = [&](int buf, int ks, int rb, int r) {
+    if (r < TM) fa[rb][r] = *reinterpret_cast<const lds_half8_t*>(a_frag + buf * STAGE_BYTES + (r * KSTP + ks) * 1024);
+    else fb[rb][r - TM] = *reinterpret_cast<const lds_half8_t*>(b_frag + buf * STAGE_BYTES + ((r - TM) * KSTP + ks) * 1024);
+  };
+  constexpr int R = TM + TN, Q = TM * TN;
+#pragma unroll
+  for (int r = 0; r < R; ++r) read_one(0, 0, 0, r);
+
+  // One step: the MFMAs of fragment set rb; between them the fragment reads of (read_buf, read_ks) into the other
+  // set, pieces [c0, c1) of tile t + 1 from register set `set` into LDS buffer `write_buf` and pieces [l0, l1) of
+  // tile t + 3 from memory into the same registers.
+  auto step = [&](int rb, bool reads, int read_buf, int read_ks, int t, int set, int write_buf, int c0, int c1, int l0, int l1) {
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      if (reads) {
+#pragma unroll
+        for (int r = (R * q) / Q; r < (R * (q + 1)) / Q; ++r) read_one(read_buf, read_ks, rb ^ 1, r);
+      }
+#pragma unroll
+      for (int c = c0 + ((c1 - c0) * q) / Q; c < c0 + ((c1 - c0) * (q + 1)) / Q; ++c) store_one(write_buf, set, c);
+#pragma unroll
+      for (int c = l0 + ((l1 - l0) * q) / Q; c < l0 + ((l1 - l0) * (q + 1)) / Q; ++c) load_one(t + 3, set, c);
+      const int i = q / TN, j = q % TN;
+      acc[i][j] = D_ALONG_M ? __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[rb][i], fb[rb][j], acc[i][j], 0, 0, 0)
+                            : __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[rb][j], fa[rb][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // Tile t: all steps but the last write tile t + 1 into the other buffer; before the last step the hand-over (this
+  // wave's LDS writes and fragment reads have completed, then the bare barrier instruction: __syncthreads() would
+  // also wait for the loads in flight); the last step reads the first fragments of tile t + 1 and requests tile
+  // t + 3.  The register set (t + 1) % 2 is a compile-time argument: registers cannot be indexed at run time.
+  auto run_tile = [&](int t, auto set_c, auto last_c) {
+    constexpr int SET = decltype(set_c)::value ? 1 : 0;
+    constexpr bool LAST = decltype(last_c)::value;        // the last tile: LAST_STEPS steps, nothing behind it
+    constexpr int STEPS = LAST ? KSTEPS - (KT - 1) * KSTP : KSTP;
+    const int buf = t & 1;
+#pragma unroll
+    for (int ks = 0; ks < STEPS; ++ks) {
+      if (ks + 1 < STEPS) {
+        step(ks & 1, true, buf, ks + 1, t, SET, buf ^ 1, LAST ? 0 : (CPY * ks) / (KSTP - 1), LAST ? 0 : (CPY * (ks + 1)) / (KSTP - 1), 0, 0);
+      } else if (!LAST) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): LDS writes and reads of this wave are done
+        __builtin_amdgcn_s_barrier();
+        step(ks & 1, true, buf ^ 1, 0, t, SET, 0, 0, 0, 0, CPY);
+      } else {
+        step(ks & 1, false, 0, 0, t, SET, 0, 0, 0, 0, 0);
+      }
+    }
+  };
+  for (int t = 0; t + 1 < KT; t += 2) {
+    run_tile(t, BoolConstant<true>(), BoolConstant<false>());
+    if (t + 2 < KT) run_tile(t + 1, BoolConstant<false>(), BoolConstant<false>());
+  }
+  if constexpr ((KT - 1) % 2 == 0) run_tile(KT - 1, BoolConstant<true>(), BoolConstant<true>());
+  else run_tile(KT - 1, BoolConstant<false>(), BoolConstant<true>());
+
+  // One row of fragments at a time.  The accumulators sit in the accumulation registers (a0..a255); the epilogue
+  // needs its operands in ordinary vector registers, and left alone the compiler moves the whole tile over when the
+  // k loop ends: as many registers again as the tile itself, paid for by spilling everything else that is live in
+  // the loop.  Pinning the rows that are not yet due (an empty statement that wants them in accumulation
+  // registers) keeps the move to one row at a time.
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = i + 1; r < TM; ++r)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) MONONN_PIN_ACC(acc[r][j]);
+    if (i + 1 < TM) preload_row(i + 1, pre[(i + 1) & 1]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int m = m_base + i * 32 + lane_m + (D_ALONG_M ? 8 * g : 0);
+        const int n = n_base + j * 32 + lane_n + (D_ALONG_M ? 0 : 8 * g);
+        if (m < M && n < N) {
+          float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          epi(batch, m, n, v, pre[i & 1][j * 4 + g]);
         }
       }
   }

@@ -137,6 +137,7 @@ Json GraphSpecification::to_json() const {
   h["profile_stages"] = hip.profile_stages;
   h["cooperative_launch"] = hip.cooperative_launch;
   h["barrier_timeout_ms"] = hip.barrier_timeout_ms;
+  h["opaque_thread_id"] = hip.opaque_thread_id;
   h["operand_preload"] = hip.operand_preload;
   h["pack_left_operands"] = hip.pack_left_operands;
   h["attention_out_proj_fusion"] = hip.attention_out_proj_fusion;
@@ -227,7 +228,7 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
   s.codegen_reject_list = strings_from(j, "codegen_reject_list");
   if (j.contains("mononn_hip")) {
     const Json& h = j.at("mononn_hip");
-    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "barrier", "profile_stages", "cooperative_launch", "operand_preload", "pack_left_operands", "attention_out_proj_fusion", "stage_rotation", "barrier_timeout_ms"}, "mononn_hip");
+    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "barrier", "profile_stages", "cooperative_launch", "operand_preload", "pack_left_operands", "attention_out_proj_fusion", "stage_rotation", "barrier_timeout_ms", "opaque_thread_id"}, "mononn_hip");
     s.hip.merge_dependent = getb(h, "merge_dependent", true);
     s.hip.gemm_epilogue_fusion = getb(h, "gemm_epilogue_fusion", true);
     s.hip.transpose_constant_b = getb(h, "transpose_constant_b", true);
@@ -238,6 +239,7 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
     s.hip.profile_stages = getb(h, "profile_stages", false);
     s.hip.cooperative_launch = getb(h, "cooperative_launch", false);
     s.hip.barrier_timeout_ms = geti(h, "barrier_timeout_ms", 10000);
+    s.hip.opaque_thread_id = getb(h, "opaque_thread_id", false);
     MONONN_CHECK(s.hip.barrier_timeout_ms >= 1 && s.hip.barrier_timeout_ms <= 3600000, kSpecError) << "barrier_timeout_ms must lie in [1, 3600000]";
     s.hip.operand_preload = getb(h, "operand_preload", true);
     s.hip.pack_left_operands = getb(h, "pack_left_operands", true);

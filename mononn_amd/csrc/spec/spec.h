@@ -90,6 +90,10 @@ struct HipOptions {       // "mononn_hip" section
   // A grid-barrier wait that is still polling this long after the kernel started gives up (the kernel then runs to
   // its end and the host finds an error word): what stands between a grid that is not wholly resident and a hang.
   int barrier_timeout_ms = 10000;
+  // Node functions re-read the thread index where they use it instead of letting the compiler derive lane numbers and
+  // address parts of all stages once, ahead of the stage loop (values that then live through every stage).  Always
+  // on in kernels with an LDS-staged GEMM, whose register tile would push those values out to scratch.
+  bool opaque_thread_id = false;
   // GEMM stages request their packed weights between announcing the end of the previous stage and waiting for the
   // other workgroups (the wait moves behind the requests; idle workgroups skip it)
   bool operand_preload = true;

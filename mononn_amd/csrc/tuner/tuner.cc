@@ -114,6 +114,25 @@ std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int w
     }
     out = kept;
   }
+  // large problems: operand tiles staged through LDS once per workgroup (the reference's tiles with shared-memory
+  // stages, tile_description.cc:84-258); four waves as 2 x 2, per-wave blocks of up to 128 x 128
+  if (waves == 4 && g.K % 32 == 0 && g.K >= 128 && g.split_k <= 1 && g.M >= 128 && g.N >= 128) {
+    struct Shape { int bm, bn, bk; };
+    for (const Shape& sh : {Shape{256, 256, 32}, Shape{192, 256, 32}, Shape{256, 192, 32}, Shape{256, 128, 64}, Shape{128, 256, 64}, Shape{192, 128, 64},
+                            Shape{128, 192, 64}, Shape{128, 128, 64}}) {
+      if (sh.bm > g.M || sh.bn > g.N) continue;
+      if (budget >= 2 && sh.bm * sh.bn < 192 * 128) continue;
+      codegen::GemmTuning t;
+      t.bm = sh.bm;
+      t.bn = sh.bn;
+      t.wm = 2;
+      t.wn = 2;
+      t.wk = 1;
+      t.stages = 2;
+      t.bk = sh.bk;
+      out.push_back(t);
+    }
+  }
   return out;
 }
 
@@ -143,6 +162,8 @@ void apply_gemm(GraphSpecification& s, const std::string& node, const codegen::G
   g.warp_m = t.bm / t.wm;
   g.warp_n = t.bn / t.wn;
   g.warp_k = static_cast<int>(K / t.wk);
+  g.stages = t.stages;
+  g.tb_k = t.bk;
 }
 
 double time_module(MonoNNModule& m, int device, DeviceBuffers& bufs, int warmup, int iters) {
@@ -296,7 +317,8 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           GraphSpecification s = filled;
           for (auto& n : c.nodes) apply_gemm(s, n, t, c.sample->gemm.K);
           char lbl[96];
-          std::snprintf(lbl, sizeof lbl, "tile%dx%d_waves%dx%dx%d", t.bm, t.bn, t.wm, t.wn, t.wk);
+          if (t.stages >= 2) std::snprintf(lbl, sizeof lbl, "tile%dx%dx%d_lds_waves%dx%d", t.bm, t.bn, t.bk, t.wm, t.wn);
+          else std::snprintf(lbl, sizeof lbl, "tile%dx%d_waves%dx%dx%d", t.bm, t.bn, t.wm, t.wn, t.wk);
           add(lbl, s);
         }
       } else if (c.kind == "attention") {

@@ -20,8 +20,22 @@
 #define __hip_atomic_load(p, order, scope) (*(p))
 #define __builtin_amdgcn_s_sleep(x) break /* the only use is the body of a spin on a flag */
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_sched_group_barrier(mask, size, sync) ((void)0)
 #define __builtin_amdgcn_s_waitcnt(x) ((void)0)
 #define __hip_atomic_compare_exchange_strong(p, expected, v, ok, fail, scope) (*(p) == *(expected) ? (*(p) = (v), true) : false)
+#define __builtin_amdgcn_s_barrier() ((void)0)
+#define __builtin_amdgcn_readfirstlane(x) (x)
+#define MONONN_PIN_ACC(v) ((void)0) /* register placement only */
+#define MONONN_OPAQUE_VALUE(v) ((void)0) /* an empty asm with a GPU register constraint */
+/* buffer descriptor + 16-byte load at descriptor base + lane offset + wave offset */
+typedef const char* __amdgpu_buffer_rsrc_t;
+#define __builtin_amdgcn_make_buffer_rsrc(p, stride, records, flags) ((const char*)(p))
+typedef unsigned host_uint4 __attribute__((ext_vector_type(4)));
+inline host_uint4 __builtin_amdgcn_raw_buffer_load_b128(const char* rsrc, unsigned voffset, unsigned soffset, int) {
+  host_uint4 v;
+  std::memcpy(&v, rsrc + (size_t)voffset + (size_t)soffset, 16);
+  return v;
+}
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) (src)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __shfl_xor(v, ...) (v)
@@ -39,6 +53,11 @@ inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
 inline unsigned long long wall_clock64() { return 1; }
 typedef _Float16 host_half8 __attribute__((ext_vector_type(8)));
 typedef float host_float4 __attribute__((ext_vector_type(4)));
+typedef float host_float16 __attribute__((ext_vector_type(16)));
+inline host_float16 __builtin_amdgcn_mfma_f32_32x32x16_f16(host_half8 a, host_half8 b, host_float16 c, int, int, int) {
+  c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
+  return c;
+}
 inline host_float4 __builtin_amdgcn_mfma_f32_16x16x32_f16(host_half8 a, host_half8 b, host_float4 c, int, int, int) {
   c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
   return c;

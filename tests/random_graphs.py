@@ -154,3 +154,31 @@ def random_gemm_cases(seed: int, count: int):
             c["warpshape"] = {"m": 16 * tm, "n": 16 * tn, "k": c["warpshape"]["k"]}
             c["wave_arrangement"] = {"m": wm, "n": wn, "k": wk}
         yield case, text, json.dumps(spec)
+
+
+LDS_TILES = [(128, 128, 64), (128, 128, 32), (256, 128, 64), (128, 256, 32), (192, 128, 64), (192, 256, 32), (256, 256, 32), (128, 128, 128)]
+
+
+def random_lds_gemm_cases(seed: int, count: int):
+    """Seeded GEMM modules for the LDS-staged tile (k a multiple of 32, both operands k-contiguous or the right one a
+    packed constant), ragged M / N, with and without batch dimensions: yields (case, hlo_text, specification json)."""
+    import json
+    from mononn_amd import MonoNNModule
+    import test_gpu_parity as parity
+    rng = np.random.default_rng(seed)
+    for _ in range(count):
+        batch = [(), (), (2,), (2, 2)][int(rng.integers(0, 4))]
+        r = len(batch) + 2
+        case = dict(M=int(rng.integers(1, 600)), N=int(rng.integers(1, 600)), K=int(rng.choice([32, 64, 96, 128, 160, 256, 320])),
+                    batch=batch, lhs_c=r - 1, rhs_c=r - 1)
+        if not batch and rng.random() < 0.5:
+            case.update(b_const=True, rhs_c=r - 2)
+        text = parity.gemm_module(**case)[0].text()
+        spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+        bm, bn, bk = LDS_TILES[int(rng.integers(0, len(LDS_TILES)))]
+        c = next(iter(spec["gemm_spec_list"].values()))["cutlass_config"]
+        c["threadblockshape"] = {"m": bm, "n": bn, "k": bk}
+        c["warpshape"] = {"m": bm // 2, "n": bn // 2, "k": case["K"]}
+        c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+        c["stages"] = 2
+        yield case, text, json.dumps(spec)

@@ -39,6 +39,14 @@ def test_random_gemm_shapes_layouts_and_tiles():
         assert ok, f"{case}: {msg}"
 
 
+def test_random_gemms_on_lds_staged_tiles():
+    from random_graphs import random_lds_gemm_cases
+    for case, text, spec in random_lds_gemm_cases(6, 12):
+        assert "gemm_tile_lds<" in MonoNNModule.compile(text, spec, build=False).get_source("main.hip"), case
+        ok, msg = check_module(text, spec, opt="-O1")
+        assert ok, f"{case}: {msg}"
+
+
 def test_encoder_variants():
     fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
     variants = {

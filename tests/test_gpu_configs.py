@@ -40,6 +40,35 @@ def test_bert_large_shapes_with_padding_masks(gpu_device):
     _check(got, want, "bert-large shapes, L=2 B=2 S=384")
 
 
+def test_encoder_on_lds_staged_gemm_tiles(gpu_device):
+    """Every projection / feed-forward GEMM of an encoder on the LDS-staged tile (fragment-order and row-major left
+    operands, packed weights, bias / GELU / residual / head-split epilogues in both accumulator orientations)."""
+    import json
+    from mononn_amd import MonoNNModule
+    fx = models.bert_encoder(L=2, B=4, S=128, H=256, NH=4, F=1024, vocab=300, max_pos=128, mask_kind="length_mask")
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    staged = 0
+    for name, g in spec["gemm_spec_list"].items():
+        if not name.startswith("cublas_gemm_"):
+            continue
+        c = g["cutlass_config"]
+        bm, bn, bk = [(128, 128, 64), (128, 256, 32), (192, 128, 64), (256, 128, 64)][staged % 4]
+        c["threadblockshape"] = {"m": bm, "n": bn, "k": bk}
+        c["warpshape"]["m"], c["warpshape"]["n"] = bm // 2, bn // 2
+        c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+        c["stages"] = 2
+        c["split_k"] = 1
+        staged += 1
+    assert staged >= 8
+    consts = fx.make_constants(1241, "random")
+    inputs = fx.make_inputs(1241)
+    m, got = _run(fx, consts, inputs, gpu_device, json.dumps(spec))
+    assert m.get_source("main.hip").count("gemm_tile_lds<") >= 4
+    m.close()
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _check(got, want, "encoder L=2 B=4 S=128 H=256 on LDS-staged tiles")
+
+
 @pytest.mark.parametrize("shape", [dict(L=2, B=2, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64),     # fused causal attention
                                    dict(L=2, B=2, S=32, H=64, NH=4, F=256, vocab=131, max_pos=64)])     # head dim 16: fallback GEMMs
 def test_gpt2_decoder_parity(gpu_device, shape):

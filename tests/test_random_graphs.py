@@ -132,3 +132,27 @@ def test_random_gemms_match_the_oracle(gpu_device):
         want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
         scale = np.abs(want).max()
         assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * scale + 1e-3, case
+
+
+@pytest.mark.gpu
+def test_random_gemms_on_lds_staged_tiles_match_the_oracle(gpu_device):
+    # the cases whose addresses tests/test_cpu_bounds.py checks on the CPU, here for their values
+    import test_gpu_parity as parity
+    from random_graphs import random_lds_gemm_cases
+    rng = np.random.default_rng(10)
+    for case, text, spec in random_lds_gemm_cases(6, 24):
+        mb, a_dims, b_dims, d_dims = parity.gemm_module(**case)
+        a = rng.normal(0, 1, a_dims).astype(np.float16)
+        b = rng.normal(0, 1, b_dims).astype(np.float16)
+        consts = {n: b for n in mb.constants}
+        inputs = [a] if case.get("b_const") else [a, b]
+        m = MonoNNModule.compile(text, spec)
+        assert "gemm_tile_lds<" in m.get_source("main.hip"), case
+        m.set_constants(consts)
+        m.load(gpu_device)
+        print(case, flush=True)
+        (got,) = m.run(inputs, [{"dtype": "f16", "dims": d_dims}])
+        m.close()
+        want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
+        scale = np.abs(want).max()
+        assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * scale + 1e-3, case
