@@ -1,5 +1,6 @@
 """Headline benchmark: full BERT-base encoder (12 layers + embeddings, batch 1, seq 128, fp16) as ONE
-monolithic cooperative kernel launch on one MI355X.
+launch of the monolithic persistent kernel on one MI355X (an ordinary launch; the grid is checked against the
+co-resident capacity when the module is loaded).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
@@ -7,7 +8,9 @@ One "step" is one forward pass = one launch of the generated kernel, inputs and 
 HBM.  Prints one JSON line: throughput (seq/s) as `value`, latency in `ms_per_step` / `latency_us`,
 the HBM roofline of the kernel (algorithmic bytes = weights + gathered rows + ids + output, read or
 written once) with the launch duration measured by HIP events on the launch stream, and the NumPy
-oracle timed on the host cores as `cpu_baseline`.
+oracle timed on the host cores as `cpu_baseline`.  `other_configs` carries the three batched configurations
+(BERT-large b16 s384, GPT-2 b4 s512 with the LM head, ViT-B/16 b8) with their shipped specifications: kernel
+latency, fraction of the dense fp16 MFMA peak, and a property check of the output (a few seconds each).
 """
 from __future__ import annotations
 
@@ -119,6 +122,78 @@ def torch_baseline(fx, consts, inputs, got):
             "max_abs_diff_vs_kernel": diff, "note": "torch.nn.functional fp16 on the same GPU; scale only"}
 
 
+def barrier_time(module, fx, consts, inputs, launches=10):
+    """Stage count and total time spent in grid barriers (last workgroup done -> first workgroup in the next stage),
+    from the in-kernel clocks of the same specification rebuilt with per-stage stamps."""
+    from mononn_amd import MonoNNModule
+    spec = json.loads(module.get_tuning_spec())
+    spec["mononn_hip"]["profile_stages"] = True
+    prof_mod = MonoNNModule.compile(fx.hlo_text, json.dumps(spec))
+    prof_mod.set_constants(consts)
+    prof_mod.load(0)
+    for _ in range(3):
+        prof_mod.run(inputs, fx.outputs)
+    total = 0.0
+    for _ in range(launches):
+        prof_mod.run(inputs, fx.outputs)
+        p = prof_mod.stage_profile()
+        total += sum(a["barrier_us"] for a in p)
+    n = len(p)
+    prof_mod.close()
+    return n, total / launches
+
+
+def other_configs():
+    """The batched configurations (parity cases of the path, not the headline): shipped specification, kernel latency
+    by HIP events, GEMM FLOPs / latency against the dense fp16 MFMA peak, and a property of the output that needs no
+    oracle (the parity tests hold the oracle comparisons)."""
+    import torch
+    from mononn_amd import MonoNNModule
+    from mononn_amd.hlo import models
+    out = {}
+    for key, make, spec_name, seed in (("bert_large_b16_s384", models.bert_large, "bert_large_b16_s384", 1236),
+                                       ("gpt2_b4_s512", models.gpt2, "gpt2_b4_s512", 1237),
+                                       ("vit_b16_b8", models.vit, "vit_b16_b8", 1238)):
+        fx = make()
+        cfg = fx.config
+        spec_dir = os.path.join(ROOT, "mononn_amd", "specs", spec_name)
+        used = "default"
+        m = None
+        if os.path.isdir(spec_dir):
+            try:
+                m = MonoNNModule.from_spec_dir(fx.hlo_text, spec_dir)
+                used = os.path.relpath(spec_dir, ROOT)
+            except Exception as e:
+                print(f"bench.py: {spec_dir} unusable ({e}); default specification", file=sys.stderr)
+        if m is None:
+            m = MonoNNModule.compile(fx.hlo_text)
+        m.set_constants(fx.make_constants(seed, "baseline"))
+        m.load(0)
+        inputs = fx.make_inputs(seed)
+        y = m.run(inputs, fx.outputs)[0]
+        avg_ms, _ = m.time_raw(m.buffer_pointers(), torch.cuda.current_stream().cuda_stream, warmup=3, iters=15)
+        flops = gemm_flops(cfg)
+        if fx.name.startswith("gpt2"):
+            flops += 2 * cfg["B"] * cfg["S"] * cfg["H"] * cfg["vocab"]
+        if fx.name.startswith("vit"):
+            flops += 2 * cfg["B"] * (cfg["S"] - 1) * cfg["H"] * (3 * cfg["patch"] ** 2)      # patch embedding as a GEMM
+        x = y.astype(np.float64)
+        if fx.name.startswith("gpt2"):
+            again = m.run(inputs, fx.outputs)[0]
+            prop = {"check": "finite logits, bit-identical on a second launch", "ok": bool(np.isfinite(x).all() and np.array_equal(again, y))}
+        else:   # the output is a LayerNorm with gamma 1 / beta 0 ("baseline" constants): rows of mean 0, variance 1
+            prop = {"check": "rows of the final LayerNorm: |mean| < 5e-3, |var - 1| < 2e-2",
+                    "ok": bool(np.isfinite(x).all() and np.abs(x.mean(-1)).max() < 5e-3 and np.abs(x.var(-1) - 1.0).max() < 2e-2)}
+        tflops = flops / (avg_ms * 1e-3) / 1e12
+        out[key] = {"latency_us": round(avg_ms * 1e3, 1), "tuning_spec": used, "grid_barriers": m.launch_dims()["barriers"],
+                    "mfma": {"achieved_tflops": round(tflops, 1), "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "gemm_flops": flops},
+                    "property": prop}
+        m.close()
+        del m
+        torch.cuda.empty_cache()
+    return out
+
+
 def stage_profile(module, fx, consts, inputs, args):
     """Per-stage clocks of the benchmark's own specification (stamped by every workgroup at stage entry / exit)."""
     from mononn_amd import MonoNNModule
@@ -160,6 +235,7 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the three batched configurations")
     ap.add_argument("--spec-dir", default=SPEC_DIR)
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof counters)")
@@ -272,8 +348,15 @@ def main():
                  "frac": round(achieved_tflops / MFMA_F16_PEAK_TFLOPS, 5), "gemm_flops": flops},
     }
 
+    n_stages, barrier_us = barrier_time(module, fx, consts, inputs)
+    result["config"]["stages"] = n_stages
+    result["config"]["barrier_us_total"] = round(barrier_us, 1)
+
     if args.torch_baseline:
         result["torch_baseline"] = torch_baseline(fx, consts, inputs, got)
+    if not args.no_other_configs:
+        module.close()
+        result["other_configs"] = other_configs()
 
     if not args.no_cpu_baseline:
         from oracle import hlo_interp

@@ -559,11 +559,16 @@ bool can_merge_clusters(const Program& prog, const std::vector<const Instr*>& pr
 // GEMM
 // ------------------------------------------------------------------------------------------
 bool gemm_uses_mfma(const graph::GemmDesc& g) {
+  if (g.f32) return !g.is_conv && g.a_k_contig;   // f32 tiles take any k extent and either right-operand layout
   if (g.is_conv && !g.conv_fragment_loads()) return false;
-  if (!g.a_k_contig || !(g.b_k_contig || g.b_packed)) return false;
+  // the left operand k-contiguous; the right one k-contiguous, packed, or a plain [K, N] matrix (gathered per lane)
+  if (!g.a_k_contig) return false;
   // a k extent that is not a multiple of 32 is zero-filled in the last step, from plain row-major operands only
   return g.K % 32 == 0 || (!g.is_conv && !g.b_packed && !g.a_packed && g.split_k <= 1);
 }
+
+// the LDS-staged tile copies k-contiguous or fragment-order operands
+static bool gemm_lds_capable(const graph::GemmDesc& g) { return !g.f32 && gemm_uses_mfma(g) && (g.b_k_contig || g.b_packed) && g.K % 32 == 0; }
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus) {
   GemmTuning t;
@@ -581,7 +586,7 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
   // units x tile area / throughput of a compute unit that is busy with such a tile, relative to 256 x 256 (measured
   // on [6144, 1024] x [1024, 4096] with both operands in fragment order: 1.0 PFLOP/s-equivalent for 256 x 256,
   // which fills the chip only 1.5 times there; 0.87 for 192 x 256, which fills it twice).
-  if (gemm_uses_mfma(g) && g.K % 32 == 0 && g.K >= 128 && waves == 4 && ls.waves_per_simd == 1 && g.split_k <= 1) {
+  if (gemm_lds_capable(g) && g.K >= 128 && waves == 4 && ls.waves_per_simd == 1 && g.split_k <= 1) {
     struct Cand { int bm, bn, bk; double eff; };
     double best = 0;
     const int cus = std::max(num_cus, 1);
@@ -610,6 +615,7 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
     }
   }
   for (int per_wave : {64, 32}) {
+    if (g.f32 && per_wave > 32) continue;   // 16 fragments of a 64 x 64 block leave no room for a chunk in flight
     int wm = 1, wn = waves;
     while (wn > wm) {
       wn /= 2;
@@ -627,7 +633,7 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
     }
   }
   int wk = 1;
-  while (wk * 2 <= waves && g.K / 32 >= wk * 2 * 2 && g.K >= 256 * wk) wk *= 2;
+  while (!g.f32 && wk * 2 <= waves && g.K / 32 >= wk * 2 * 2 && g.K >= 256 * wk) wk *= 2;
   t.wk = wk;
   int rest = waves / wk;
   t.wm = 1;
@@ -642,6 +648,11 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
 }
 
 void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t, bool has_prologue) {
+  if (g.f32) {
+    MONONN_CHECK(!has_prologue && t.wk == 1 && t.stages < 2 && t.split_k <= 1, kSpecError)
+        << "an f32 GEMM tile takes no row-program prologue, no k split (over waves or workgroups) and no LDS staging";
+    MONONN_CHECK((t.bm / std::max(t.wm, 1) / 16) * (t.bn / std::max(t.wn, 1) / 16) <= 16, kSpecError) << "f32 GEMM tile " << t.bm << "x" << t.bn << ": more than 16 fragments per wave";
+  }
   if (has_prologue) {
     const int tm = t.bm / std::max(t.wm, 1) / 16, tn = t.bn / std::max(t.wn, 1) / 16;
     const int64_t ksteps = g.K / 32;
@@ -657,6 +668,7 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)
       << "GEMM tile " << t.bm << "x" << t.bn << " is not a multiple of 16 per wave";
   if (t.stages >= 2) {
+    MONONN_CHECK(g.b_k_contig || g.b_packed, kSpecError) << "an LDS-staged GEMM tile takes a k-contiguous or packed right operand";
     MONONN_CHECK(!has_prologue && t.wk == 1 && g.K % 32 == 0, kSpecError) << "an LDS-staged GEMM tile takes no row-program prologue, no k split over waves and a k extent that is a multiple of 32";
     MONONN_CHECK(t.stages == 2 && t.bk >= 32 && t.bk % 32 == 0 && t.bk <= 128, kSpecError)
         << "LDS-staged GEMM tile: " << t.stages << " stages of " << t.bk << " k: two LDS buffers of 32, 64, 96 or 128 k";
@@ -840,7 +852,8 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
       expr = "(" + expr + " + " + beta_lit + "f * (float)" + c + ")";
     }
     std::string gv = em.fresh("g");
-    cb.line("const _Float16 " + gv + " = (_Float16)" + expr + ";");
+    const std::string gt = hlo::dtype_ctype(gi->shape.dtype);   // the GEMM's value as the HLO defines it: rounded to its result type
+    cb.line("const " + gt + " " + gv + " = (" + gt + ")" + expr + ";");
     em.bind(gi, gidx, gv);
     for (auto& out : outs) {
       if (out.o == gi) {
@@ -1249,9 +1262,14 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
              << ", bidx, tile_m, tile_n, epi, smem, mononn_dev::NoPrologue(), @NAME@_amap());";
     } else {
       std::ostringstream b_expr;
-      b_expr << pb << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : KS);
+      const bool b_along_n = !g.b_k_contig && !g.b_packed;
+      b_expr << pb << " + (long)bidx * " << g.b_batch_stride << " + ksplit * " << (g.b_packed ? KS / 32 * 512 : b_along_n ? KS * g.N : KS);
       preload = t.preload_b && g.b_packed && t.stages < 2;
-      if (t.stages >= 2)
+      if (g.f32)
+        call << "mononn_dev::gemm_tile_f32<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << g.K << ", " << (b_along_n ? "true" : "false") << ", "
+             << (epi.along_m ? "true" : "false") << ", @NAME@_epi>(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * " << g.b_batch_stride
+             << ", " << g.M << ", " << g.N << ", " << g.K << ", " << (b_along_n ? g.N : g.K) << ", bidx, tile_m, tile_n, epi";
+      else if (t.stages >= 2)
         call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", "
              << (g.a_packed ? "true" : "false") << ", " << (g.b_packed ? "true" : "false") << ", " << (epi.along_m ? "true" : "false") << ", " << t.bk
              << ", @NAME@_epi>(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
@@ -1260,9 +1278,9 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
              << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
              << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
-             << (epi.along_m ? "true" : "false") << ">("
+             << (epi.along_m ? "true" : "false") << ", " << (b_along_n ? "true" : "false") << ">("
              << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
-             << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
+             << ", " << g.N << ", " << g.K << ", " << (b_along_n ? g.N : g.K) << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
              << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");
       call << ");";
       if (preload) {
@@ -1381,17 +1399,27 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
-  MONONN_CHECK(K1 % 32 == 0 && N1 % 32 == 0 && N2 % 16 == 0, kUnsupported) << "attention fusion: extents must be MFMA multiples";
+  MONONN_CHECK(K1 % 32 == 0 && N2 % 16 == 0, kUnsupported) << "attention fusion: head size must be an MFMA multiple";
+  // A key count off the MFMA step (ViT: 197): every wave's slice is rounded up to whole steps of 32 keys; the keys
+  // past the end are read from the last valid key (finite values, in range), take no part in the row reductions
+  // and get probability zero.  Plain k-contiguous K and V only (fragment-order operands have whole blocks).
+  const bool ragged = N1 % 32 != 0;
+  MONONN_CHECK(!ragged || (!d1.b_tiled && !d2.b_tiled && !g3), kUnsupported) << "attention fusion: a key count off the MFMA step needs plain k-contiguous keys and values";
   int KW = 1;
-  while (KW * 2 <= NW && N1 % (32 * KW * 2) == 0 && N1 / (KW * 2) >= 32) KW *= 2;
+  if (ragged) {
+    while (KW * 2 <= NW && (N1 + KW * 2 - 1) / (KW * 2) >= 32) KW *= 2;
+  } else {
+    while (KW * 2 <= NW && N1 % (32 * KW * 2) == 0 && N1 / (KW * 2) >= 32) KW *= 2;
+  }
   if (key_waves > 0) {
     // tuning knob: fewer key slices per row block mean fewer exchanges through LDS but fewer, longer units
-    MONONN_CHECK(NW % key_waves == 0 && N1 % (32 * key_waves) == 0, kSpecError)
+    MONONN_CHECK(NW % key_waves == 0 && (ragged || N1 % (32 * key_waves) == 0), kSpecError)
         << "attention: " << key_waves << " key waves do not divide " << NW << " waves / " << N1 << " keys";
     KW = key_waves;
   }
   const int RW = NW / KW;
-  const int64_t NKW = N1 / KW;   // keys per wave
+  const int64_t NKW = ragged ? ((N1 + KW - 1) / KW + 31) / 32 * 32 : N1 / KW;   // keys per wave
+  MONONN_CHECK(!ragged || (KW - 1) * NKW < N1, kUnsupported) << "attention fusion: " << KW << " key waves leave a wave without keys";
   const int KS1 = static_cast<int>(K1 / 32), NT1 = static_cast<int>(NKW / 16), KS2 = static_cast<int>(NKW / 32), NT2 = static_cast<int>(N2 / 16);
   RowInfo info = analyze_rows(row_members);
   MONONN_CHECK(info.row_program && info.rows == d1.batch * M1 && info.row_len == N1, kUnsupported)
@@ -1419,7 +1447,9 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   auto elem_index = [&](int j, int r) {
     Index idx = delinearize(LinExpr::variable(vb, d1.batch), batch_dims, vars);
     idx.push_back(LinExpr::variable(vm, M1));
-    idx.push_back(LinExpr::variable(vkw, KW).scaled(NKW).plus(LinExpr::variable(vg, 4).scaled(4)).plus_const(j * 16 + r));
+    // ragged key count: the column comes from a run-time value clamped to the last key (colc[j][r], set up below)
+    if (ragged) idx.push_back(LinExpr::opaque("colc[" + S(j) + "][" + S(r) + "]", N1));
+    else idx.push_back(LinExpr::variable(vkw, KW).scaled(NKW).plus(LinExpr::variable(vg, 4).scaled(4)).plus_const(j * 16 + r));
     return idx;
   };
   Index row_index = delinearize(LinExpr::variable(vb, d1.batch), batch_dims, vars);
@@ -1465,9 +1495,25 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.line("const _Float16* qp = " + pq + " + (long)bidx * " + S(d1.a_batch_stride) + " + m * " + S(K1) + " + g * 8;");
   }
   if (d1.b_tiled) cb.line("const _Float16* kp = " + pk + " + (((long)bidx * " + S(N1 / 16) + " + kw * " + S(NKW / 16) + ") * " + S(KS1 * 64) + " + lane) * 8;");
+  else if (ragged) cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + g * 8;   // + key * " + S(K1));
   else cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + (kw * " + S(NKW) + " + r16) * " + S(K1) + " + g * 8;");
   if (d2.b_tiled) cb.line("const _Float16* vp = " + pv + " + (((long)bidx * " + S(N2 / 16) + ") * " + S(N1 / 32) + " + kw * " + S(NKW / 32) + ") * 512 + lane * 8;");
+  else if (ragged) cb.line("const _Float16* vp = " + pv + " + (long)bidx * " + S(d2.b_batch_stride) + " + r16 * " + S(N1) + ";   // row r16 of V^T; + t * 16 rows + key");
   else cb.line("const _Float16* vp = " + pv + " + (long)bidx * " + S(d2.b_batch_stride) + " + r16 * " + S(N1) + " + kw * " + S(NKW) + " + g * 4;");
+  if (ragged) {
+    // this lane's score columns: key kw * NKW + 16 j + 4 g + r; colc = the key it reads instead when that one is past the end
+    cb.line("int colc[" + S(NT1) + "][4];");
+    cb.line("bool colv[" + S(NT1) + "][4];");
+    cb.line("#pragma unroll");
+    cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
+    cb.line("#pragma unroll");
+    cb.open("for (int r = 0; r < 4; ++r)");
+    cb.line("const int col = kw * " + S(NKW) + " + j * 16 + g * 4 + r;");
+    cb.line("colv[j][r] = col < " + S(N1) + ";");
+    cb.line("colc[j][r] = colv[j][r] ? col : " + S(N1 - 1) + ";");
+    cb.close();
+    cb.close();
+  }
   // ---- absorbed output projection: this head's K3 slice of the packed weights, all N3 columns split over the KW waves
   std::string pw, po, preload_body;
   int NT3 = 0, NJ = 0, KS3 = 0;
@@ -1506,8 +1552,17 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.line("#pragma unroll");
   cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
   cb.line("#pragma unroll");
-  if (d1.b_tiled) cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + (j * " + S(KS1) + " + ks) * 512);");
-  else cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + j * " + S(16 * K1) + " + ks * 32);");
+  if (d1.b_tiled) {
+    cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + (j * " + S(KS1) + " + ks) * 512);");
+  } else if (ragged) {
+    cb.open("for (int ks = 0; ks < " + S(KS1) + "; ++ks)");
+    cb.line("int key = kw * " + S(NKW) + " + j * 16 + r16;");
+    cb.line("key = key < " + S(N1) + " ? key : " + S(N1 - 1) + ";");
+    cb.line("kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + key * " + S(K1) + " + ks * 32);");
+    cb.close();
+  } else {
+    cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) kf[j][ks] = *reinterpret_cast<const half8_t*>(kp + j * " + S(16 * K1) + " + ks * 32);");
+  }
   cb.close();
   cb.line("#pragma unroll");
   cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
@@ -1515,6 +1570,10 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.open("for (int ks = 0; ks < " + S(KS2) + "; ++ks)");
   if (d2.b_tiled) {
     cb.line("vf[t][ks] = *reinterpret_cast<const half8_t*>(vp + (t * " + S(N1 / 32) + " + ks) * 512);");
+  } else if (ragged) {
+    // rows of an odd length start at odd element offsets: no alignment promise, and the keys past the end read the
+    // row's last element (their probabilities are zero)
+    cb.line("vf[t][ks] = mononn_dev::load_key_run(vp + t * " + S(16 * N1) + ", kw * " + S(NKW) + " + ks * 32 + g * 4, " + S(N1) + ");");
   } else {
     cb.line("const half4_t lo = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32);");
     cb.line("const half4_t hi = *reinterpret_cast<const half4_t*>(vp + t * " + S(16 * N1) + " + ks * 32 + 16);");
@@ -1548,6 +1607,8 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
       for (int r = 0; r < 4; ++r) {
         bind_elem(j, r);
         std::string val = em.value(red->operands[0], elem_index(j, r));
+        // a key past the end contributes the reduction's init value (its identity)
+        if (ragged) val = "(colv[" + S(j) + "][" + S(r) + "] ? (" + Tn + ")(" + val + ") : (" + Tn + ")(" + em.value(red->operands[1], {}) + "))";
         cb.line(acc + " = (" + Tn + ")" + Emitter::reducer_expr(red, acc, val) + ";");
       }
     for (int off : {16, 32}) {
@@ -1567,7 +1628,8 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   for (int j = 0; j < NT1; ++j)
     for (int r = 0; r < 4; ++r) {
       bind_elem(j, r);
-      cb.line("pr[" + S(j) + "][" + S(r) + "] = " + em.value(em.resolve_output(P), elem_index(j, r)) + ";");
+      if (ragged) cb.line("pr[" + S(j) + "][" + S(r) + "] = colv[" + S(j) + "][" + S(r) + "] ? (_Float16)(" + em.value(em.resolve_output(P), elem_index(j, r)) + ") : (_Float16)0;");
+      else cb.line("pr[" + S(j) + "][" + S(r) + "] = " + em.value(em.resolve_output(P), elem_index(j, r)) + ";");
     }
   em.unbind(g1);
   // ---- second contraction ---------------------------------------------------------------------------

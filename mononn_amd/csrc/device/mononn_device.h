@@ -341,6 +341,24 @@ __device__ __forceinline__ T sign_of(T x) {
   return (T)((x > (T)0) - (x < (T)0));
 }
 
+// The right operand of P.V in the fused attention when the key count n is off the MFMA step: elements k .. k + 3 and
+// k + 16 .. k + 19 of a row of V^T, without an alignment promise; positions past the end read the last element.
+__device__ __forceinline__ half8_t load_key_run(const half_t* row, int k, int n) {
+  half8_t v;
+  if (k + 20 <= n) {
+    __builtin_memcpy(&v, row + k, 8);
+    __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, row + k + 16, 8);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int lo = k + e, hi = k + 16 + e;
+      v[e] = row[lo < n ? lo : n - 1];
+      v[4 + e] = row[hi < n ? hi : n - 1];
+    }
+  }
+  return v;
+}
+
 // ---------------------------------------------------------------------------------------------
 // GEMM:  D[m][n] = sum_k A[m][k] * B[k][n]      A contiguous along k
 // ---------------------------------------------------------------------------------------------
@@ -445,8 +463,11 @@ __device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_
 // K is the k extent this call contracts over; KTOTAL the k extent of the operands in memory (they differ
 // when the k range is split over workgroups: the caller then offsets A and B to the start of its slice).
 // PRE_B: the right operand's first chunk was requested by gemm_b_preload with the same parameters and comes in `pb`.
+// B_ALONG_N: the right operand is stored [K, ldb] with n contiguous (a run-time [K, N] matrix, weights passed as
+// kernel parameters): a lane gathers its eight k values of one column with eight 2-byte loads.  Slower per byte
+// than the k-contiguous layouts, but the contraction stays on the MFMAs.
 template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA,
-          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false>
+          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false, bool B_ALONG_N = false>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
                                           int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
                                           const AMap& amap = AMap(), const Pre* pb = nullptr) {
@@ -462,6 +483,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
   static_assert(!RAGGED_K || (!PACKED_A && !PACKED_B && !PRE_B && AMap::kRowMajor && K == KTOTAL && !Pro::enabled),
                 "a k extent that is not a multiple of 32 is taken from plain k-contiguous operands only");
+  static_assert(!B_ALONG_N || (!PACKED_B && !PRE_B), "an n-contiguous right operand is neither packed nor requested ahead");
   const int lane = lane_id();
   const int wave = wave_id();
   const int wk = wave % WK;
@@ -501,10 +523,17 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     } else {
       int n = n_base + j * 16 + r16;
       n = n < N ? n : N - 1;
-      b_ptr[j] = B + (long)n * ldb + kq;
+      b_ptr[j] = B_ALONG_N ? B + n + (long)kq * ldb : B + (long)n * ldb + kq;
     }
   }
-  constexpr int B_STEP = PACKED_B ? 64 * 8 : 32;   // halves between consecutive k steps
+  constexpr int B_STEP = PACKED_B ? 64 * 8 : 32;   // halves between consecutive k steps (k-contiguous layouts)
+  // eight k values of one column of an n-contiguous operand, zero past the end of k
+  auto load_along_n = [&](const half_t* p, int k0) {
+    half8_t v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (!RAGGED_K || k0 + e < K) ? p[(long)e * ldb] : half_t(0);
+    return v;
+  };
 
   half8_t a[2][CH][TM], b[2][CH][TN];
   // Rows whose k extent is not a multiple of 32 start at odd element offsets, so their fragments are read
@@ -527,6 +556,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         if (PRE_B && c == 0) b[buf][s][j] = pb->v[s * TN + j];
+        else if constexpr (B_ALONG_N) b[buf][s][j] = load_along_n(b_ptr[j] + (long)ks * 32 * ldb, ks * 32 + kq);
         else if constexpr (RAGGED_K) b[buf][s][j] = load_ragged(b_ptr[j] + (long)ks * B_STEP, ks * 32 + kq);
         else b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
       }
@@ -635,6 +665,124 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         }
       }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// f32 GEMM:  D[m][n] = sum_k A[m][k] * B[k][n], all f32, on v_mfma_f32_16x16x4_f32
+// ---------------------------------------------------------------------------------------------
+// A workgroup of WM x WN waves owns a BM x BN tile; each wave keeps (BM / WM / 16) x (BN / WN / 16) accumulator
+// fragments and walks the whole k range in chunks of 16: a lane loads four consecutive k of its row (one 16-byte
+// load when the operand is k-contiguous) and the chunk is four MFMAs, the s-th of which contracts the s-th
+// element of every lane (k = 4 * (lane / 16) + s within the chunk: any split of the 16 k over the four MFMAs is
+// as good as any other, as long as both operands use the same one).  A is row-major [M, lda]; B is [N, ldb]
+// (k-contiguous) or, with B_ALONG_N, [K, ldb].  The last chunk of a k extent that is not a multiple of 16 is
+// zero-filled.  Rows / columns beyond M / N are clamped on load and skipped on store.  Epilogue functor and lane
+// layout of the result as in gemm_tile.
+template <int BM, int BN, int WM, int WN, int K, bool B_ALONG_N, bool D_ALONG_M, class Epi>
+__device__ __forceinline__ void gemm_tile_f32(const float* A, const float* B, int M, int N, int lda, int ldb, int batch, int tile_m, int tile_n,
+                                              Epi& epi) {
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
+  constexpr int CHUNKS = (K + 15) / 16;
+  static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "tile/wave mismatch");
+  const int lane = lane_id();
+  const int wave = wave_id();
+  const int wn = wave % WN, wm = wave / WN;
+  const int m_base = tile_m * BM + wm * (TM * 16);
+  const int n_base = tile_n * BN + wn * (TN * 16);
+  const int r16 = lane & 15;
+  const int kq = (lane >> 4) * 4;
+  const float* a_ptr[TM];
+  const float* b_ptr[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int m = m_base + i * 16 + r16;
+    m = m < M ? m : M - 1;
+    a_ptr[i] = A + (long)m * lda + kq;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int n = n_base + j * 16 + r16;
+    n = n < N ? n : N - 1;
+    b_ptr[j] = B_ALONG_N ? B + n + (long)kq * ldb : B + (long)n * ldb + kq;
+  }
+  // four consecutive k from a k-contiguous row (no alignment promise: rows of an odd length start anywhere)
+  auto load_k4 = [&](const float* p, int k0) {
+    float4_t v;
+    if ((K % 16 == 0) || k0 + 4 <= K) {
+      __builtin_memcpy(&v, p, 16);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = k0 + e < K ? p[e] : 0.f;
+    }
+    return v;
+  };
+  auto load_n4 = [&](const float* p, int k0) {
+    float4_t v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = ((K % 16 == 0) || k0 + e < K) ? p[(long)e * ldb] : 0.f;
+    return v;
+  };
+  float4_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+  typename Epi::Pre pre[TM * TN];
+#pragma unroll
+  for (int f = 0; f < TM * TN; ++f) {
+    int m = m_base + (f / TN) * 16 + (D_ALONG_M ? (lane >> 4) * 4 : r16);
+    int n = n_base + (f % TN) * 16 + (D_ALONG_M ? r16 : (lane >> 4) * 4);
+    if (D_ALONG_M) {
+      m = m < M ? m : (M >= 4 ? M - 4 : 0);
+      n = n < N ? n : N - 1;
+    } else {
+      m = m < M ? m : M - 1;
+      n = n < N ? n : (N >= 4 ? N - 4 : 0);
+    }
+    epi.preload(batch, m, n, pre[f]);
+  }
+  float4_t a[2][TM], b[2][TN];
+  auto load_chunk = [&](int c, int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a[buf][i] = load_k4(a_ptr[i] + c * 16, c * 16 + kq);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b[buf][j] = B_ALONG_N ? load_n4(b_ptr[j] + (long)c * 16 * ldb, c * 16 + kq) : load_k4(b_ptr[j] + c * 16, c * 16 + kq);
+  };
+  load_chunk(0, 0);
+  for (int c = 0; c < CHUNKS; c += 2) {
+    // two chunks per trip so that the register set a chunk is loaded into is known at compile time
+    if (c + 1 < CHUNKS) load_chunk(c + 1, 1);
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = D_ALONG_M ? __builtin_amdgcn_mfma_f32_16x16x4f32(a[0][i][s], b[0][j][s], acc[i][j], 0, 0, 0)
+                                : __builtin_amdgcn_mfma_f32_16x16x4f32(b[0][j][s], a[0][i][s], acc[i][j], 0, 0, 0);
+    if (c + 1 < CHUNKS) {
+      if (c + 2 < CHUNKS) load_chunk(c + 2, 0);
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = D_ALONG_M ? __builtin_amdgcn_mfma_f32_16x16x4f32(a[1][i][s], b[1][j][s], acc[i][j], 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_16x16x4f32(b[1][j][s], a[1][i][s], acc[i][j], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int m = m_base + i * 16 + (D_ALONG_M ? (lane >> 4) * 4 : r16);
+      const int n = n_base + j * 16 + (D_ALONG_M ? r16 : (lane >> 4) * 4);
+      if (m < M && n < N) {
+        float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+        epi(batch, m, n, v, pre[i * TN + j]);
+      }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -915,12 +1063,12 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
 // contiguous along k, K not a multiple of 32): one thread per output element, fp32 accumulation.
 // Strides are in elements.  Epilogue functor as above but with a single value:
 //   void operator()(int batch, int m, int n, float v)
-template <class Epi>
-__device__ __forceinline__ void gemm_naive_element(const half_t* A, const half_t* B, int K, long a_sm, long a_sk,
+template <class T, class Epi>
+__device__ __forceinline__ void gemm_naive_element(const T* A, const T* B, int K, long a_sm, long a_sk,
                                                    long b_sk, long b_sn, int batch, int m, int n, Epi& epi) {
   float acc = 0.f;
-  const half_t* a = A + m * a_sm;
-  const half_t* b = B + n * b_sn;
+  const T* a = A + m * a_sm;
+  const T* b = B + n * b_sn;
   for (int k = 0; k < K; ++k) acc += (float)a[k * a_sk] * (float)b[k * b_sk];
   epi(batch, m, n, acc);
 }

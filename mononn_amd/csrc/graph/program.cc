@@ -28,7 +28,7 @@ const Node* Program::node_of(const Instr* member) const {
 
 std::string GemmDesc::problem_hash() const {
   std::ostringstream os;
-  os << "f16_b" << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_packed ? "_bp" : (b_k_contig ? "_bk" : "_bn"));
+  os << (f32 ? "f32_b" : "f16_b") << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_packed ? "_bp" : (b_k_contig ? "_bk" : "_bn"));
   if (is_conv) os << "_conv" << conv.R << "x" << conv.S << "s" << conv.stride_h << "x" << conv.stride_w << "p" << conv.pad_h << "x" << conv.pad_w;
   return os.str();
 }
@@ -69,11 +69,16 @@ struct Builder {
     MONONN_CHECK(g->operands.size() == 2 || g->operands.size() == 3, kUnsupported) << g->hlo_name << ": GEMM takes 2 or 3 operands";
     const hlo::Shape &A = g->operands[0]->shape, &B = g->operands[1]->shape, &D = g->shape;
     MONONN_CHECK(A.rank() == B.rank() && A.rank() == D.rank() && A.rank() >= 2, kUnsupported) << g->hlo_name << ": A, B and D must have equal rank >= 2";
-    MONONN_CHECK(A.dtype == hlo::DType::kF16 && B.dtype == hlo::DType::kF16 && D.dtype == hlo::DType::kF16, kUnsupported)
-        << g->hlo_name << ": only f16 GEMMs are supported";
+    // f16 x f16 -> f16 and f32 x f32 -> f32, both with fp32 accumulation (the reference: half and float / TF32,
+    // gemm_impl.cc:56, :229)
+    const bool all_f16 = A.dtype == hlo::DType::kF16 && B.dtype == hlo::DType::kF16 && D.dtype == hlo::DType::kF16;
+    const bool all_f32 = A.dtype == hlo::DType::kF32 && B.dtype == hlo::DType::kF32 && D.dtype == hlo::DType::kF32;
+    MONONN_CHECK(all_f16 || all_f32, kUnsupported) << g->hlo_name << ": GEMM operands and result must all be f16 or all be f32";
+    MONONN_CHECK(g->operands.size() == 2 || g->operands[2]->shape.dtype == D.dtype, kUnsupported) << g->hlo_name << ": addend type differs from the result type";
     const int r = A.rank();
     const hlo::GemmConfig& c = g->gemm;
     GemmDesc d;
+    d.f32 = all_f32;
     MONONN_CHECK(c.lhs_contracting == r - 1 || c.lhs_contracting == r - 2, kUnsupported) << g->hlo_name << ": lhs contracting dim must be one of the two minor dims";
     MONONN_CHECK(c.rhs_contracting == r - 1 || c.rhs_contracting == r - 2, kUnsupported) << g->hlo_name << ": rhs contracting dim must be one of the two minor dims";
     d.a_k_contig = c.lhs_contracting == r - 1;
@@ -299,7 +304,7 @@ struct Builder {
       std::vector<int> takers;
       for (int ci : succ[ri]) {
         Node& c = nodes[ci];
-        if (c.kind != NodeKind::kGemm || !c.prologue.empty() || c.gemm.is_conv) continue;
+        if (c.kind != NodeKind::kGemm || !c.prologue.empty() || c.gemm.is_conv || c.gemm.f32) continue;
         const Instr* g = c.members[0];
         if (p.storage_root(g->operands[0]) != h || p.storage_root(g->operands[1]) == h) continue;
         if (g->operands.size() > 2 && p.storage_root(g->operands[2]) == h) continue;
@@ -367,9 +372,10 @@ struct Builder {
         if (reaches_via_outside(g1i, static_cast<int>(ri), succ) || reaches_via_outside(static_cast<int>(ri), g2i, succ)) continue;
         // the other producers of gemm2 (V) must not depend on gemm1 / the row program
         const GemmDesc &d1 = g1.gemm, &d2 = g2.gemm;
-        if (!d1.a_k_contig || !d1.b_k_contig || !d2.a_k_contig || d2.has_addend || d1.has_addend || d1.is_conv || d2.is_conv) continue;
+        if (!d1.a_k_contig || !d1.b_k_contig || !d2.a_k_contig || d2.has_addend || d1.has_addend || d1.is_conv || d2.is_conv || d1.f32 || d2.f32) continue;
         if (d2.batch != d1.batch || d2.M != d1.M || d2.K != d1.N) continue;
-        if (d1.K % 32 != 0 || d1.N % 32 != 0 || d2.N % 16 != 0 || d1.N > 512 || d2.N > 256 || d1.K > 256) continue;
+        // key counts off the MFMA step are taken (rounded up per wave, masked); head sizes are not
+        if (d1.K % 32 != 0 || d1.N < 32 || d2.N % 16 != 0 || d1.N > 512 || d2.N > 256 || d1.K > 256) continue;
         const Instr* vroot = p.storage_root(gi2->operands[1]);
         if (!d2.b_k_contig && !(opt.assign_operand_layouts && enabled("OperandLayoutPass") && can_store_k_contig(vroot, gi2->operands[1], gi2->gemm.rhs_contracting)))
           continue;
@@ -400,7 +406,7 @@ struct Builder {
     auto succ = successors();
     for (size_t ai = 0; ai < nodes.size(); ++ai) {
       const Node& a = nodes[ai];
-      if (a.members.empty() || a.kind != NodeKind::kAttention || a.gemm3_index != 0) continue;
+      if (a.members.empty() || a.kind != NodeKind::kAttention || a.gemm3_index != 0 || a.gemm.N % 32 != 0) continue;
       auto outs = codegen::external_outputs(p, a.members);
       if (outs.size() != 1 || succ[ai].size() != 1) continue;
       const Node& g = nodes[succ[ai][0]];
@@ -549,7 +555,7 @@ struct Builder {
       if (c->opcode != "constant" || c->is_scalar_constant() || c->shape.rank() != 2) continue;
       bool all = !c->users.empty();
       for (auto* u : c->users) {
-        bool good = u->is_gemm() && u->operands.size() >= 2 &&
+        bool good = u->is_gemm() && u->operands.size() >= 2 && c->shape.dtype == hlo::DType::kF16 &&
                     u->operands[1] == c && u->operands[0] != c && u->gemm.rhs_contracting == 0 && c->shape.dims[0] % 32 == 0 &&
                     u->gemm.lhs_contracting == u->operands[0]->shape.rank() - 1 && (u->operands.size() < 3 || u->operands[2] != c);
         if (!good) all = false;
@@ -631,9 +637,12 @@ struct Builder {
         const bool dense = d1.a_k_contig && d1.b_k_contig && d2.b_k_contig && d1.a_batch_stride == d1.M * d1.K && d1.b_batch_stride == d1.N * d1.K &&
                            d2.b_batch_stride == d2.N * d2.K && d1.M % 16 == 0 && d1.N % 16 == 0 && d2.N % 16 == 0;
         use(g1->operands[0], dense, d1.batch * d1.M, d1.K, Order::kRunsOf8, false);
-        use(g1->operands[1], dense, d1.batch * d1.N, d1.K, Order::kRunsOf8, false);
+        // a key count off the MFMA step leaves the last fragments partly empty: keys and values are then read in
+        // place, row by row, with the rows past the end clamped
+        const bool whole_steps = d1.N % 32 == 0;
+        use(g1->operands[1], dense && whole_steps, d1.batch * d1.N, d1.K, Order::kRunsOf8, false);
         // values: stored [.., N2, keys] (transposed by the operand layout pass), contracted over the keys
-        use(g2->operands[1], dense && p.physical_perm.count(p.storage_root(g2->operands[1])), d2.batch * d2.N, d2.K, Order::kPairsOf4, true);
+        use(g2->operands[1], dense && whole_steps && p.physical_perm.count(p.storage_root(g2->operands[1])), d2.batch * d2.N, d2.K, Order::kPairsOf4, true);
         continue;
       }
       if (n.kind != NodeKind::kGemm) continue;
@@ -686,8 +695,8 @@ struct Builder {
         if (n.kind == NodeKind::kGemm && n.members[0]->name == kv.first) node = &n;
       MONONN_CHECK(node != nullptr, kSpecError) << "split_k names GEMM '" << kv.first << "' which is not a GEMM node of the graph";
       const Instr* g = node->members[0];
-      MONONN_CHECK(node->members.size() == 1 && node->prologue.empty() && !node->gemm.has_addend && !node->gemm.is_conv, kSpecError)
-          << "split_k: GEMM " << kv.first << " has a fused epilogue / prologue / addend or is a convolution";
+      MONONN_CHECK(node->members.size() == 1 && node->prologue.empty() && !node->gemm.has_addend && !node->gemm.is_conv && !node->gemm.f32, kSpecError)
+          << "split_k: GEMM " << kv.first << " has a fused epilogue / prologue / addend, is a convolution or an f32 GEMM";
       MONONN_CHECK(node->gemm.K % (32 * kv.second) == 0, kSpecError) << "split_k: K of " << kv.first << " is not a multiple of 32 * " << kv.second;
       for (auto* lo : p.live_outs) MONONN_CHECK(lo != g, kSpecError) << "split_k: the result of " << kv.first << " is a module output";
       for (auto& n : p.nodes)

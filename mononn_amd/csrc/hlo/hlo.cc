@@ -277,9 +277,11 @@ Shape parse_shape(Lexer& lx) {
     if (lay.find(':') != std::string::npos) MONONN_FAIL(kUnsupported) << "line " << lx.line << ": tiled or annotated layouts are not supported: " << lay;
     for (auto v : ints_of(lay)) sh.minor_to_major.push_back(static_cast<int>(v));
     MONONN_CHECK(sh.minor_to_major.size() == sh.dims.size(), kParseError) << "layout rank mismatch in " << lay;
-    for (size_t i = 0; i < sh.dims.size(); ++i)
-      if (sh.minor_to_major[i] != static_cast<int>(sh.dims.size() - 1 - i))
-        MONONN_FAIL(kUnsupported) << "line " << lx.line << ": only descending minor-to-major layouts are supported, got " << lay;
+    std::vector<bool> seen(sh.dims.size(), false);
+    for (int d : sh.minor_to_major) {
+      MONONN_CHECK(d >= 0 && d < static_cast<int>(sh.dims.size()) && !seen[d], kParseError) << "line " << lx.line << ": layout " << lay << " is not a permutation of the dimensions";
+      seen[d] = true;
+    }
   } else {
     for (int i = static_cast<int>(sh.dims.size()) - 1; i >= 0; --i) sh.minor_to_major.push_back(i);
   }
@@ -700,6 +702,246 @@ void decode_attrs(Instr* ins, Module* mod) {
   validate_shapes(ins);
 }
 
+// ---- layouts --------------------------------------------------------------------------------------------------------
+// Every operation of the dialect is defined on logical indices, so a value's minor-to-major order matters only where
+// memory is handed over or reinterpreted: entry parameters, constants whose bytes the host supplies, the results, and
+// `bitcast` (same bytes, another shape).  A value with dims L and order m lies in memory as the row-major array
+// transpose(value, perm) with perm[i] = m[rank-1-i]; the reference turns the same list into per-dimension positions
+// (ir_parser_fused.cc:132-152) and carries them through its index arithmetic.  Here the four places get explicit
+// transposes instead, and every instruction leaves with the descending order the rest of the compiler assumes.
+bool is_descending(const std::vector<int>& m) {
+  for (size_t i = 0; i < m.size(); ++i)
+    if (m[i] != static_cast<int>(m.size() - 1 - i)) return false;
+  return true;
+}
+
+void reset_layout(Shape& s) {
+  s.minor_to_major.clear();
+  for (int i = s.rank() - 1; i >= 0; --i) s.minor_to_major.push_back(i);
+  for (auto& t : s.tuple) reset_layout(t);
+}
+
+std::vector<int64_t> major_to_minor(const std::vector<int>& m) { return std::vector<int64_t>(m.rbegin(), m.rend()); }
+
+std::vector<int64_t> inverse_permutation(const std::vector<int64_t>& p) {
+  std::vector<int64_t> inv(p.size());
+  for (size_t i = 0; i < p.size(); ++i) inv[p[i]] = static_cast<int64_t>(i);
+  return inv;
+}
+
+std::vector<int64_t> permuted(const std::vector<int64_t>& dims, const std::vector<int64_t>& p) {
+  std::vector<int64_t> out(p.size());
+  for (size_t i = 0; i < p.size(); ++i) out[i] = dims[p[i]];
+  return out;
+}
+
+void unlink_user(Instr* operand, const Instr* user) {
+  auto& u = operand->users;
+  u.erase(std::remove(u.begin(), u.end(), user), u.end());
+}
+
+// transposes that exchange the two minor dimensions and keep the leading (batch) ones
+bool swaps_minor_pair(const Instr* t) {
+  const int r = static_cast<int>(t->dimensions.size());
+  if (t->opcode != "transpose" || r < 2 || t->dimensions[r - 1] != r - 2 || t->dimensions[r - 2] != r - 1) return false;
+  for (int i = 0; i < r - 2; ++i)
+    if (t->dimensions[i] != i) return false;
+  return true;
+}
+
+void renumber(Computation* comp) {
+  for (size_t i = 0; i < comp->instrs.size(); ++i) comp->instrs[i]->index_in_comp = static_cast<int>(i);
+}
+
+void normalize_layouts(Computation* comp, std::set<const Instr*>* made) {
+  std::map<const Instr*, std::vector<int>> order;   // as written, non-tuple values only
+  bool any = false;
+  for (auto& up : comp->instrs) {
+    if (!up->shape.is_tuple()) {
+      order[up.get()] = up->shape.minor_to_major;
+      any = any || !is_descending(up->shape.minor_to_major);
+    }
+    reset_layout(up->shape);
+  }
+  if (!any) return;
+  std::set<std::string> names;
+  for (auto& up : comp->instrs) names.insert(up->name);
+  auto fresh = [&](const std::string& base) {
+    std::string n = base;
+    for (int k = 1; names.count(n); ++k) n = base + "_" + std::to_string(k);
+    names.insert(n);
+    return n;
+  };
+  std::vector<std::unique_ptr<Instr>> old = std::move(comp->instrs), out;
+  // a new one-operand instruction, appended to `out`
+  auto make = [&](const std::string& base, const char* opcode, std::vector<int64_t> dims, std::vector<int64_t> dimensions, Instr* operand) {
+    auto ins = std::make_unique<Instr>();
+    ins->name = ins->hlo_name = fresh(base);
+    ins->opcode = opcode;
+    ins->shape.dtype = operand->shape.dtype;
+    ins->shape.dims = std::move(dims);
+    reset_layout(ins->shape);
+    ins->dimensions = std::move(dimensions);
+    ins->operands = {operand};
+    ins->parent = comp;
+    operand->users.push_back(ins.get());
+    if (ins->opcode == "transpose") made->insert(ins.get());
+    out.push_back(std::move(ins));
+    return out.back().get();
+  };
+  std::map<const Instr*, Instr*> memory_of;   // logical value -> an instruction whose row-major array is its memory image
+  // the memory image of `x` as a row-major value; appended to `out` when it has to be computed
+  auto image = [&](Instr* x, const std::string& base) -> Instr* {
+    auto it = order.find(x);
+    if (it == order.end() || is_descending(it->second)) return x;
+    auto mo = memory_of.find(x);
+    if (mo != memory_of.end()) return mo->second;
+    const auto p = major_to_minor(it->second);
+    return memory_of[x] = make(base, "transpose", permuted(x->shape.dims, p), p, x);
+  };
+  Instr* old_root = comp->root;
+  for (auto& up : old) {
+    Instr* ins = up.get();
+    auto it = order.find(ins);
+    const bool plain = it == order.end() || is_descending(it->second);
+    const std::vector<int64_t> p = plain ? std::vector<int64_t>() : major_to_minor(it->second);
+    if (comp->is_entry && ins == old_root) {
+      // results leave as memory images
+      if (ins->opcode == "tuple") {
+        for (size_t i = 0; i < ins->operands.size(); ++i) {
+          Instr* x = ins->operands[i];
+          Instr* y = image(x, x->name + "_memory");
+          if (y == x) continue;
+          unlink_user(x, ins);   // every position that holds x gets the same image
+          ins->operands[i] = y;
+          if (std::find(y->users.begin(), y->users.end(), ins) == y->users.end()) y->users.push_back(ins);
+          ins->shape.tuple[i].dims = y->shape.dims;
+        }
+      }
+    }
+    if (ins->opcode == "bitcast") {
+      Instr* x = ins->operands[0];
+      Instr* in = image(x, ins->name + "_operand_memory");
+      if (in != x) {
+        unlink_user(x, ins);
+        ins->operands[0] = in;
+        in->users.push_back(ins);
+      }
+      if (!plain) {
+        // the instruction keeps its name and its users and becomes the way back from the new bitcast's row-major
+        // array to logical order
+        Instr* raw = make(ins->name + "_memory", "bitcast", permuted(ins->shape.dims, p), {}, in);
+        unlink_user(in, ins);
+        ins->opcode = "transpose";
+        ins->operands = {raw};
+        raw->users.push_back(ins);
+        ins->dimensions = inverse_permutation(p);
+        memory_of[ins] = raw;
+        made->insert(ins);
+      }
+      out.push_back(std::move(up));
+      continue;
+    }
+    const bool buffer = (ins->opcode == "parameter" && comp->is_entry) || (ins->opcode == "constant" && ins->literal_elided);
+    out.push_back(std::move(up));
+    if (buffer && !plain) {
+      // the host hands over the memory image: that is what this instruction now is, and its users read the
+      // transpose back to logical order
+      const std::vector<int64_t> logical = ins->shape.dims;
+      std::vector<Instr*> users = ins->users;
+      ins->users.clear();
+      ins->shape.dims = permuted(logical, p);
+      Instr* t = make(ins->name + "_logical", "transpose", logical, inverse_permutation(p), ins);
+      for (Instr* u : users) {
+        for (auto& o : u->operands)
+          if (o == ins) o = t;
+        t->users.push_back(u);
+      }
+      order[t] = it->second;
+      memory_of[t] = ins;
+      order.erase(ins);
+    }
+  }
+  if (comp->is_entry && old_root->opcode != "tuple") {
+    Instr* y = image(old_root, old_root->name + "_memory");
+    if (y != old_root) {
+      old_root->is_root = false;
+      y->is_root = true;
+      comp->root = y;
+    }
+  }
+  comp->instrs = std::move(out);
+  renumber(comp);
+}
+
+void erase_instr(Computation* comp, Instr* dead) {
+  for (Instr* o : dead->operands) unlink_user(o, dead);
+  auto& v = comp->instrs;
+  v.erase(std::remove_if(v.begin(), v.end(), [&](const std::unique_ptr<Instr>& u) { return u.get() == dead; }), v.end());
+}
+
+// The transposes above next to a GEMM go into the call itself, as the reference's GEMM takes either order of each
+// operand and a column-major result by exchanging the operands (gemm_impl.cc:345-351, :408-469):
+//   gemm(transpose(X), B) = gemm(X, B) contracting X's other minor dimension (same for the right operand);
+//   transpose(gemm(A, B)) = gemm(B, A) with the roles of the contracting and batch dimensions exchanged, taken only
+//   when that leaves the new left operand contiguous along k (the order the MFMA tiles read).
+void fold_layout_transposes_into_gemms(Computation* comp, std::set<const Instr*>* made) {
+  for (auto& up : comp->instrs) {
+    Instr* g = up.get();
+    if (!g->is_gemm() || g->operands.size() < 2) continue;
+    const int r = g->shape.rank();
+    for (int side = 0; side < 2; ++side) {
+      Instr* t = g->operands[side];
+      if (!made->count(t) || !swaps_minor_pair(t) || t->shape.rank() != r) continue;
+      Instr* x = t->operands[0];
+      unlink_user(t, g);
+      g->operands[side] = x;
+      x->users.push_back(g);
+      if (g->operands[0] == t || g->operands[1] == t) t->users.push_back(g);   // still read by the other side
+      int& c = side == 0 ? g->gemm.lhs_contracting : g->gemm.rhs_contracting;
+      c = c == r - 1 ? r - 2 : (c == r - 2 ? r - 1 : c);
+    }
+  }
+  for (auto& up : comp->instrs) {
+    Instr* t = up.get();
+    if (!made->count(t) || !swaps_minor_pair(t)) continue;
+    Instr* g = t->operands[0];
+    const int r = g->shape.rank();
+    if (!g->is_gemm() || g->operands.size() != 2 || g->users.size() != 1 || g == comp->root || g->gemm.rhs_contracting != r - 1) continue;
+    Instr *a = g->operands[0], *b = g->operands[1];
+    unlink_user(g, t);
+    unlink_user(a, g);
+    unlink_user(b, g);
+    g->operands.clear();
+    t->opcode = g->opcode;
+    t->custom_call_target = g->custom_call_target;
+    t->attrs = g->attrs;
+    t->dimensions.clear();
+    t->gemm = g->gemm;
+    std::swap(t->gemm.lhs_contracting, t->gemm.rhs_contracting);
+    std::swap(t->gemm.lhs_batch, t->gemm.rhs_batch);
+    std::swap(t->gemm.lhs_stride, t->gemm.rhs_stride);
+    t->operands = {b, a};
+    b->users.push_back(t);
+    a->users.push_back(t);
+    made->erase(t);
+  }
+  // what the rewrites left without a reader
+  for (bool again = true; again;) {
+    again = false;
+    for (auto& up : comp->instrs) {
+      Instr* d = up.get();
+      const bool candidate = made->count(d) || (d->is_gemm() && d->operands.empty());
+      if (!candidate || !d->users.empty() || d == comp->root) continue;
+      made->erase(d);
+      erase_instr(comp, d);
+      again = true;
+      break;
+    }
+  }
+  renumber(comp);
+}
+
 }  // namespace
 
 std::unique_ptr<Module> parse_module(const std::string& text) {
@@ -824,6 +1066,11 @@ std::unique_ptr<Module> parse_module(const std::string& text) {
     mod->computations.push_back(std::move(comp));
   }
   MONONN_CHECK(mod->entry != nullptr, kParseError) << "module has no ENTRY computation";
+  std::set<const Instr*> layout_transposes;
+  for (auto& comp : mod->computations) {
+    normalize_layouts(comp.get(), &layout_transposes);
+    if (!layout_transposes.empty()) fold_layout_transposes_into_gemms(comp.get(), &layout_transposes);
+  }
   return mod;
 }
 

@@ -27,7 +27,7 @@ inline bool is_float(DType t) { return t == DType::kF16 || t == DType::kF32 || t
 struct Shape {
   DType dtype = DType::kInvalid;
   std::vector<int64_t> dims;
-  std::vector<int> minor_to_major;   // always descending (row-major) after validation
+  std::vector<int> minor_to_major;   // as written while parsing; descending (row-major) on everything parse_module returns
   std::vector<Shape> tuple;          // when dtype == kTuple
 
   bool is_tuple() const { return dtype == DType::kTuple; }
@@ -119,6 +119,10 @@ struct Module {
 
 // Parse HLO text.  Throws Error(kParseError) on malformed text and Error(kUnsupported) on
 // constructs outside the dialect (unknown opcode, dynamic dimension, tiled layout ...).
+// Minor-to-major orders other than the descending one are taken out of the module: entry parameters, host-supplied
+// constants and results become the row-major arrays their memory holds (dims listed slowest first), with
+// transposes to and from logical order next to them and around `bitcast`; those next to a GEMM are folded into
+// its contracting dimensions or an exchange of its operands.
 std::unique_ptr<Module> parse_module(const std::string& text);
 
 // '.' and '-' -> '_'  (mononn_engine/helpers/string_helpers.cc:22-32)

@@ -227,6 +227,13 @@ void MonoNNModule::load(int device) {
   runtime::DeviceProperties props = runtime::query_device(device);
   MONONN_CHECK(props.arch == spec_.device.cuda_arch, kRuntimeError)
       << "code object was built for " << spec_.device.cuda_arch << " but device " << device << " is " << props.arch;
+  // Known defect, fenced off: a process that used the cooperative launch entry point under rocprofv3 died with a
+  // segmentation fault in an exit handler, after the profiler had written its output (five runs; no frame of this
+  // library on the stack: the fault lies in the teardown of the runtime's cooperative queue after the tool has
+  // finalised).  The ordinary launch under the same profiler exits cleanly.
+  MONONN_CHECK(!(hip_.cooperative && runtime::profiler_tool_attached()), kRuntimeError)
+      << "cooperative_launch is refused while a profiler tool library is attached to the process (the combination crashes at process exit); "
+         "profile the ordinary launch: \"cooperative_launch\": false in the specification's mononn_hip section";
   dev_.load(device, code_object_, kernel_name_);
   dev_.set_dynamic_smem(hip_.smem);
   // The grid barrier needs every workgroup resident at once.  The reference's barrier would

@@ -2,6 +2,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <dlfcn.h>
+
 #include <cstdlib>
 
 #include <algorithm>
@@ -25,6 +27,21 @@ int device_count() {
     return 0;
   }
   return n;
+}
+
+bool profiler_tool_attached() {
+  // rocprofv3 starts its target with the tool library named in ROCP_TOOL_LIBRARIES and mapped into the process
+  for (const char* var : {"ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB"}) {
+    const char* v = std::getenv(var);
+    if (v && *v) return true;
+  }
+  for (const char* lib : {"librocprofiler-sdk-tool.so", "librocprofiler-sdk-tool.so.1", "librocprofiler64.so.2"}) {
+    if (void* h = dlopen(lib, RTLD_NOLOAD | RTLD_LAZY)) {
+      dlclose(h);
+      return true;
+    }
+  }
+  return false;
 }
 
 DeviceProperties query_device(int device) {

@@ -27,6 +27,8 @@ struct DeviceProperties {
 };
 
 int device_count();                           // 0 when no GPU is visible (never throws)
+// a profiler tool library (rocprofv3 and its predecessors) is mapped into this process or named in its environment
+bool profiler_tool_attached();
 DeviceProperties query_device(int device);    // throws Error(kRuntimeError) without a GPU
 
 class DeviceModule {

@@ -116,7 +116,7 @@ std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int w
   }
   // large problems: operand tiles staged through LDS once per workgroup (the reference's tiles with shared-memory
   // stages, tile_description.cc:84-258); four waves as 2 x 2, per-wave blocks of up to 128 x 128
-  if (waves == 4 && g.K % 32 == 0 && g.K >= 128 && g.split_k <= 1 && g.M >= 128 && g.N >= 128) {
+  if (waves == 4 && g.K % 32 == 0 && g.K >= 128 && g.split_k <= 1 && g.M >= 128 && g.N >= 128 && (g.b_k_contig || g.b_packed)) {
     struct Shape { int bm, bn, bk; };
     for (const Shape& sh : {Shape{256, 256, 32}, Shape{192, 256, 32}, Shape{256, 192, 32}, Shape{256, 128, 64}, Shape{128, 256, 64}, Shape{192, 128, 64},
                             Shape{128, 192, 64}, Shape{128, 128, 64}}) {

@@ -10,6 +10,9 @@ reference attaches to each instruction when it lowers it:
 
   * opcode set ......................... mononn_engine/core/op/op_type.h:20-65
   * dtype / layout rules ............... mononn_engine/parser/ir_parser_fused.cc:68-152
+    (a value with minor_to_major m lies in memory with dimension m[0] varying fastest; entry
+    parameters, constant payloads and results are such memory images, `bitcast` keeps the bytes,
+    every other instruction is defined on logical indices)
   * fusion -> called computation ....... ir_parser_fused.cc:490-539, :866-1019
   * reduce (one reduced dim, constant
     init, reducer = called computation)  ir_parser_fused.cc:1169-1213,
@@ -29,7 +32,9 @@ reference attaches to each instruction when it lowers it:
 The parser below is written independently of the product's C++ parser so that a parsing bug is
 not shared between the thing under test and its checker.
 
-Pinning (what fixes these functions besides the formulae above): tests/test_oracle_pinning.py
+Pinning (what fixes these functions besides the formulae above): tests/test_layouts.py checks the
+layout handling against element offsets computed from strides by brute force, np.transpose and
+np.einsum; tests/test_oracle_pinning.py
 checks the evaluator against closed forms and library routines -- fp64 triple-loop GEMM on tiny
 shapes, the two worked backend_config examples of gemm_impl.cc:290-316 against numpy einsum,
 torch.nn.functional soft-max / layer_norm / gelu(tanh), brute-force gather, torch max/avg
@@ -69,10 +74,29 @@ _NP = {"pred": np.bool_, "s8": np.int8, "u8": np.uint8, "s16": np.int16, "u16": 
 
 
 class Shape:
-    __slots__ = ("dtype", "dims", "tuple_shapes")
+    __slots__ = ("dtype", "dims", "tuple_shapes", "layout")
 
-    def __init__(self, dtype=None, dims=(), tuple_shapes=None):
+    def __init__(self, dtype=None, dims=(), tuple_shapes=None, layout=None):
         self.dtype, self.dims, self.tuple_shapes = dtype, tuple(dims), tuple_shapes
+        self.layout = layout     # minor-to-major list as written, None when descending (row-major)
+
+    def major_to_minor(self):
+        """Logical dimension numbers from the slowest-varying to the fastest-varying one in memory."""
+        return list(range(len(self.dims))) if self.layout is None else list(reversed(self.layout))
+
+    def memory_dims(self):
+        return tuple(self.dims[d] for d in self.major_to_minor())
+
+
+def _memory_image(a: np.ndarray, shape: "Shape") -> np.ndarray:
+    """The value's elements in the order they lie in memory, as a row-major array of shape.memory_dims()."""
+    return np.ascontiguousarray(np.transpose(a, shape.major_to_minor()))
+
+
+def _from_memory(buf: np.ndarray, shape: "Shape") -> np.ndarray:
+    """Inverse of _memory_image: logical array from its memory image (any shape with the right element count)."""
+    order = shape.major_to_minor()
+    return np.transpose(np.ascontiguousarray(buf).reshape(shape.memory_dims()), np.argsort(order))
 
 
 class Instr:
@@ -131,11 +155,16 @@ def _parse_shape(s: str) -> Shape:
     if not m:
         raise ValueError(f"bad shape: {s!r}")
     dims = [int(d) for d in m.group(2).split(",") if d.strip()]
+    layout = None
     if m.group(3):
+        if ":" in m.group(3):
+            raise ValueError(f"tiled or annotated layouts are not supported: {s}")
         lay = [int(x) for x in m.group(3)[1:-1].split(",") if x.strip()]
+        if sorted(lay) != list(range(len(dims))):
+            raise ValueError(f"layout is not a permutation of the dimensions: {s}")
         if lay != list(reversed(range(len(dims)))):
-            raise ValueError(f"only descending minor-to-major layouts are supported: {s}")
-    return Shape(m.group(1), dims)
+            layout = lay
+    return Shape(m.group(1), dims, layout=layout)
 
 
 def _match_paren(s: str, start: int) -> int:
@@ -285,18 +314,28 @@ class Evaluator:
         return list(res) if isinstance(res, tuple) else [res]
 
     def _cast_in(self, a: np.ndarray, shape: Shape) -> np.ndarray:
+        """A buffer handed in by the host (entry parameter, constant payload): its memory image, dims listed from the
+        slowest-varying one; with the default layout that is the logical array itself."""
         a = np.asarray(a)
-        if tuple(a.shape) != tuple(shape.dims):
-            raise ValueError(f"shape mismatch: got {a.shape}, HLO says {shape.dims}")
-        return a.astype(self.np_dtype(shape.dtype), copy=False)
+        if tuple(a.shape) != tuple(shape.memory_dims()):
+            raise ValueError(f"shape mismatch: got {a.shape}, HLO says {shape.dims} laid out as {shape.memory_dims()}")
+        return _from_memory(a, shape).astype(self.np_dtype(shape.dtype), copy=False)
 
     def _run_comp(self, comp: Comp, args: List[np.ndarray], top: bool = False):
         env: Dict[str, object] = {}
+        shapes = {i.name: i.shape for i in comp.instrs}
         for ins in comp.instrs:
+            self._top, self._shapes = top, shapes
             env[ins.name] = self._eval(ins, env, args)
             if top and self._keep and isinstance(env[ins.name], np.ndarray):
                 self.trace[ins.name] = env[ins.name]
-        return env[comp.root.name]
+        res = env[comp.root.name]
+        if top:     # results leave as memory images, like the parameters came in
+            if isinstance(res, tuple):
+                res = tuple(_memory_image(r, shapes[o]) for r, o in zip(res, comp.root.operands))
+            else:
+                res = _memory_image(res, comp.root.shape)
+        return res
 
     def _eval(self, ins: Instr, env, args):
         op = ins.opcode
@@ -306,6 +345,11 @@ class Evaluator:
         if op == "parameter":
             if self._vector_depth:   # a reducer body applied to whole arrays at once: its scalar shapes are not checked
                 return np.asarray(args[int(ins.literal)]).astype(self.np_dtype(sh.dtype), copy=False)
+            if not self._top:        # a called computation receives values, not buffers
+                a = np.asarray(args[int(ins.literal)])
+                if tuple(a.shape) != tuple(sh.dims):
+                    raise ValueError(f"shape mismatch: got {a.shape}, HLO says {sh.dims}")
+                return a.astype(self.np_dtype(sh.dtype), copy=False)
             return self._cast_in(args[int(ins.literal)], sh)
         if op == "constant":
             if ins.literal.replace(" ", "") == "{...}":
@@ -317,8 +361,10 @@ class Evaluator:
             return tuple(x)
         if op == "get-tuple-element":
             return x[0][int(ins.attrs["index"])]
-        if op in ("bitcast", "reshape"):
+        if op == "reshape":      # defined on logical row-major order whatever the layouts
             return np.ascontiguousarray(x[0]).reshape(sh.dims)
+        if op == "bitcast":      # the same bytes under another shape and layout
+            return _from_memory(_memory_image(x[0], self._shapes[ins.operands[0]]), sh)
         if op == "fusion" or op == "call":
             key = "calls" if "calls" in ins.attrs else "to_apply"
             return self._run_comp(self.mod["comps"][ins.attrs[key].lstrip("%")], x)

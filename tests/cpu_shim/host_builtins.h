@@ -58,6 +58,10 @@ inline host_float16 __builtin_amdgcn_mfma_f32_32x32x16_f16(host_half8 a, host_ha
   c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
   return c;
 }
+inline host_float4 __builtin_amdgcn_mfma_f32_16x16x4f32(float a, float b, host_float4 c, int, int, int) {
+  c[0] += a * b;
+  return c;
+}
 inline host_float4 __builtin_amdgcn_mfma_f32_16x16x32_f16(host_half8 a, host_half8 b, host_float4 c, int, int, int) {
   c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
   return c;

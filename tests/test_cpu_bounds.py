@@ -39,6 +39,18 @@ def test_random_gemm_shapes_layouts_and_tiles():
         assert ok, f"{case}: {msg}"
 
 
+def test_fused_attention_with_key_counts_off_the_mfma_step():
+    for kw in (dict(L=1, B=2, image=96, patch=16, H=128, NH=2, F=256), dict(L=1, B=1, image=224, patch=16, H=128, NH=2, F=256)):
+        fx = models.vit(**kw)
+        assert "colv[" in MonoNNModule.compile(fx.hlo_text, build=False).get_source("main.hip")
+        ok, msg = check_module(fx.hlo_text, opt="-O1")
+        assert ok, f"{kw}: {msg}"
+    fx = models.bert_encoder(L=1, B=2, S=100, H=128, NH=2, F=256, vocab=97, max_pos=128, mask_kind="length_mask")
+    assert "colv[" in MonoNNModule.compile(fx.hlo_text, build=False).get_source("main.hip")
+    ok, msg = check_module(fx.hlo_text, opt="-O1")
+    assert ok, msg
+
+
 def test_random_gemms_on_lds_staged_tiles():
     from random_graphs import random_lds_gemm_cases
     for case, text, spec in random_lds_gemm_cases(6, 12):

@@ -185,6 +185,19 @@ def test_vit_encoder_parity(gpu_device):
     _check(got, want, "vit L=2 B=2 64x64/16")
 
 
+@pytest.mark.parametrize("image,B", [(96, 3), (224, 2)])   # 37 and 197 tokens: one stage per attention, keys masked past the end
+def test_vit_attention_with_key_counts_off_the_mfma_step(gpu_device, image, B):
+    fx = models.vit(L=2, B=B, image=image, patch=16, H=128, NH=2, F=256)
+    consts = fx.make_constants(1242, "random")
+    inputs = fx.make_inputs(1242)
+    m, got = _run(fx, consts, inputs, gpu_device)
+    src = m.get_source("main.hip")
+    assert "colv[" in src and "load_key_run" in src
+    m.close()
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _check(got, want, f"vit image {image}: fused attention over {(image // 16) ** 2 + 1} keys")
+
+
 def test_vit_full_size_properties(gpu_device):
     """ViT-B/16, 12 layers, batch 8, 224x224 pixels, 197 tokens per image."""
     fx = models.vit()
@@ -220,6 +233,8 @@ def test_encoders_with_sizes_off_the_mfma_steps(gpu_device, shape):
     consts = fx.make_constants(1240, "random")
     inputs = fx.make_inputs(1240)
     m, got = _run(fx, consts, inputs, gpu_device)
+    # key counts of 32 and more that are off the MFMA step take the fused attention with masked key slices
+    assert ("colv[" in m.get_source("main.hip")) == (shape["S"] >= 32 and shape["S"] % 32 != 0 and shape["H"] // shape["NH"] % 32 == 0), shape
     want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
     _check(got, want, f"encoder {shape}")
     m.close()

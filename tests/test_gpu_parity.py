@@ -30,7 +30,7 @@ def check_close(got, want32, atol=2e-2, cos_min=0.9999):
     return err, cos
 
 
-def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=False, as_dot=False):
+def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=False, as_dot=False, dtype="f16"):
     mb = HloModuleBuilder("cluster_7__gemm_test.1")
     e = mb.entry
     r = len(batch) + 2
@@ -38,8 +38,8 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
     rhs_c = r - 2 if rhs_c is None else rhs_c
     a_dims = list(batch) + ([M, K] if lhs_c == r - 1 else [K, M])
     b_dims = list(batch) + ([K, N] if rhs_c == r - 2 else [N, K])
-    a = e.parameter("f16", a_dims, "a")
-    b = e.elided_constant("f16", b_dims, "w/kernel") if b_const else e.parameter("f16", b_dims, "b")
+    a = e.parameter(dtype, a_dims, "a")
+    b = e.elided_constant(dtype, b_dims, "w/kernel") if b_const else e.parameter(dtype, b_dims, "b")
     if as_dot:
         d = e.dot(a, b, lhs_c, rhs_c, batch_dims=tuple(range(len(batch))))
     else:
@@ -50,31 +50,69 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
 
 @pytest.mark.parametrize("case", [
     dict(M=128, N=768, K=768, b_const=True),                      # weight GEMM, constant transposed at upload
-    dict(M=128, N=96, K=64),                                      # [K,N] parameter operand -> fallback path
+    dict(M=128, N=96, K=64),                                      # [K,N] parameter operand: gathered per lane, still on the MFMAs
     dict(M=128, N=128, K=64, batch=(1, 12), rhs_c=3, alpha=0.125),  # scores: both operands k-contiguous
     dict(M=128, N=64, K=128, batch=(2, 3)),                       # context: B stored [K,N]
     dict(M=100, N=52, K=96, rhs_c=1),                             # ragged M / N on the MFMA path
     dict(M=64, N=48, K=40, rhs_c=1),                              # K not a multiple of 32: zero-filled last MFMA step
     dict(M=197, N=64, K=197, batch=(2, 3), rhs_c=3),              # odd row length: fragments start at unaligned addresses
     dict(M=33, N=20, K=17, rhs_c=1),                              # K below one MFMA step
-    dict(M=64, N=48, K=40),                                       # K not a multiple of 32 and B stored [K,N] -> fallback path
+    dict(M=64, N=48, K=40),                                       # K not a multiple of 32 and B stored [K,N]: zero-filled gather
     dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                     # A stored [K,M]
     dict(M=128, N=256, K=256, b_const=True, as_dot=True),         # plain `dot` with a constant right operand
     dict(M=48, N=80, K=64, batch=(3,), rhs_c=2, as_dot=True),     # batched `dot`, both operands k-contiguous
+    dict(M=200, N=136, K=256, dtype="f32", rhs_c=1),              # f32 on v_mfma_f32_16x16x4_f32, both operands k-contiguous
+    dict(M=128, N=96, K=100, dtype="f32"),                        # f32, B stored [K,N], k extent off the chunk of 16
+    dict(M=77, N=50, K=33, batch=(2,), dtype="f32", rhs_c=2),     # f32, batched, everything ragged
+    dict(M=128, N=256, K=128, dtype="f32", b_const=True),         # f32 constant weights (not packed)
+    dict(M=40, N=24, K=64, dtype="f32", lhs_c=0, rhs_c=1),        # f32 with A stored [K,M]: per-element fallback
 ])
 def test_gemm_cases(gpu_device, case):
     mb, a_dims, b_dims, d_dims = gemm_module(**case)
     rng = np.random.default_rng(3)
-    a = rng.normal(0, 1, a_dims).astype(np.float16)
-    b = rng.normal(0, 1, b_dims).astype(np.float16)
+    dtype = case.get("dtype", "f16")
+    npdt = np.float32 if dtype == "f32" else np.float16
+    a = rng.normal(0, 1, a_dims).astype(npdt)
+    b = rng.normal(0, 1, b_dims).astype(npdt)
     text = mb.text()
     consts = {n: b for n in mb.constants}
     inputs = [a] if case.get("b_const") else [a, b]
-    (got,), _ = run_module(text, inputs, consts, [{"dtype": "f16", "dims": d_dims}])
+    (got,), _ = run_module(text, inputs, consts, [{"dtype": dtype, "dims": d_dims}])
     want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
-    # fp16 output rounding of values up to ~sqrt(K): relative tolerance
     scale = np.abs(want).max()
-    assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * scale + 1e-3
+    if dtype == "f32":
+        # f32 inputs and accumulation: only the summation order differs from the oracle's
+        assert got.dtype == np.float32 and np.abs(got - want).max() <= 2e-5 * scale
+    else:
+        # fp16 output rounding of values up to ~sqrt(K): relative tolerance
+        assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * scale + 1e-3
+
+
+def test_f32_gemm_with_fused_epilogue(gpu_device):
+    # f32 [M,K] x constant [K,N] with bias add and ReLU fused onto the accumulator tile
+    M, N, K = 150, 200, 96
+    mb = HloModuleBuilder("cluster_8__gemm_f32_epilogue.1")
+    e = mb.entry
+    a = e.parameter("f32", (M, K), "a")
+    w = e.elided_constant("f32", (K, N), "w/kernel")
+    bias = e.elided_constant("f32", (N,), "w/bias")
+    d = e.gemm(a, w, 1, 0)
+
+    def body(f, pd, pb):
+        return f.maximum(f.add(pd, f.broadcast(pb, pd.dims, [1])), f.splat("f32", 0.0, pd.dims))
+    y = e.fusion("kLoop", [d, bias], body)
+    e.set_tuple_root([y])
+    rng = np.random.default_rng(12)
+    av = rng.normal(0, 1, (M, K)).astype(np.float32)
+    consts = {}
+    for name, meta in mb.constants.items():
+        consts[name] = rng.normal(0, 1, meta["dims"]).astype(np.float32)
+    (got,), m = run_module(mb.text(), [av], consts, [{"dtype": "f32", "dims": [M, N]}])
+    src = m.get_source("main.hip")
+    assert "gemm_tile_f32<" in src and m.launch_dims()["barriers"] == 0      # one stage: the epilogue is fused
+    want = hlo_interp.evaluate(mb.text(), [av], consts, "fp32")[0]
+    assert (want == 0).any() and (want > 0).any()
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
 
 
 def test_bert_layer_parity(gpu_device):

@@ -161,7 +161,7 @@ HEAD = "HloModule cluster_9__t.1\n\n"
     (HEAD + "ENTRY %main {\n  %p = f32[4]{0} parameter(0)\n  ROOT %r = f32[4]{0} cosine(f32[4]{0} %p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f32[<=4]{0} parameter(0)\n  ROOT %r = f32[<=4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f32[4,4]{1,0:T(2,2)} parameter(0)\n  ROOT %r = f32[4,4]{1,0} negate(%p)\n}\n", "UNSUPPORTED"),
-    (HEAD + "ENTRY %main {\n  %p = f32[4,4]{0,1} parameter(0)\n  ROOT %r = f32[4,4]{0,1} negate(%p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f32[4,4]{0,1:T(2,128)} parameter(0)\n  ROOT %r = f32[4,4]{0,1} negate(%p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = bf16[4]{0} parameter(0)\n  ROOT %r = bf16[4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f32[1,4,4,1]{3,2,1,0} parameter(0)\n  %w = f32[1,1,1,1]{3,2,1,0} parameter(1)\n"
             "  ROOT %r = f32[1,4,4,1]{3,2,1,0} convolution(%p, %w), window={size=1x1}, dim_labels=b01f_01io->b01f\n}\n", "UNSUPPORTED"),
@@ -275,13 +275,18 @@ def test_convolution_call_is_lowered_as_implicit_gemm():
 def test_contraction_length_off_the_mfma_step_still_takes_mfma_tiles():
     # ViT's P.V product contracts over 197 keys: the tile zero-fills the last step instead of falling back to one
     # thread per element; V is stored transposed by the stage that writes it, so both operands are k-contiguous
+    # (with the attention left as separate stages; fused, the product never is a GEMM stage of its own)
     fx = models.vit(L=1, B=1)
-    src = MonoNNModule.compile(fx.hlo_text, build=False).get_source("main.hip")
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    spec["mononn_hip"]["fuse_attention"] = False
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}, {}
+    src = MonoNNModule.compile(fx.hlo_text, json.dumps(spec), build=False).get_source("main.hip")
     assert "gemm_naive_element" not in src
     assert re.search(r"gemm_tile<\d+, \d+, \d+, \d+, \d+, 197, false, 197,", src)
 
 
-SHIPPED_SPECS = {"bert_base_b1_s128": models.bert_base, "vit_b16_b8": models.vit, "gpt2_b4_s512": models.gpt2}
+SHIPPED_SPECS = {"bert_base_b1_s128": models.bert_base, "vit_b16_b8": models.vit, "gpt2_b4_s512": models.gpt2,
+                 "bert_large_b16_s384": models.bert_large}
 
 
 def test_results_only_the_host_reads_are_stored_through_the_cache():

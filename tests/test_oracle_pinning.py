@@ -42,6 +42,24 @@ def test_gemm_brute_force_fp64_tiny():
     assert np.abs(got - want).max() < 1e-5
 
 
+def test_f32_gemm_against_fp64_brute_force():
+    # all-f32 GEMM (gemm_impl.cc:56, :229): no rounding to half anywhere, both right-operand layouts
+    from test_gpu_parity import gemm_module
+    rng = np.random.default_rng(21)
+    for case in (dict(M=9, N=7, K=13, dtype="f32"), dict(M=6, N=5, K=11, dtype="f32", rhs_c=1), dict(M=4, N=3, K=5, batch=(2,), dtype="f32", rhs_c=2)):
+        mb, a_dims, b_dims, d_dims = gemm_module(**case)
+        a = rng.normal(size=a_dims).astype(np.float32) * 1000.0      # values a half would overflow or round visibly
+        b = rng.normal(size=b_dims).astype(np.float32) + 1e-4
+        for mode in ("fp32", "as_written"):
+            got = hlo_interp.evaluate(mb.text(), [a, b], precision=mode)[0]
+            bt = np.swapaxes(b, -1, -2) if case.get("rhs_c") == len(b_dims) - 1 else b
+            want = np.zeros(d_dims)
+            for idx in np.ndindex(*d_dims):
+                lead, i, j = idx[:-2], idx[-2], idx[-1]
+                want[idx] = sum(float(a[lead + (i, k)]) * float(bt[lead + (k, j)]) for k in range(case["K"]))
+            assert got.dtype == np.float32 and np.abs(got - want).max() <= 1e-5 * np.abs(want).max(), (case, mode)
+
+
 def test_gemm_row_major_example_shapes():
     # shapes / strides of the row-major worked example in the reference (gemm_impl.cc:290-303):
     # f16[512,384] = f16[512,128] x f16[128,384], contracting lhs 1 / rhs 0, lhs_stride 65536, rhs_stride 49152
