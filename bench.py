@@ -194,6 +194,56 @@ def other_configs():
     return out
 
 
+# configurations bench.py can run: name -> (fixture in mononn_amd.hlo.models, seed)
+WORKLOADS = {"bert_base_b1_s128": ("bert_base", 1235), "bert_large_b16_s384": ("bert_large", 1236), "gpt2_b4_s512": ("gpt2", 1237),
+             "vit_b16_b8": ("vit", 1238), "gemm_stage_6144x4096x1024": ("gemm_stage", 1239)}
+
+
+def single_workload(args):
+    """One configuration other than the benchmark's: its launches and one line with its latency (not the metric)."""
+    import torch
+    from mononn_amd import MonoNNModule
+    from mononn_amd.hlo import models
+    make, seed = WORKLOADS[args.workload]
+    fx = getattr(models, make)()
+    spec_dir = os.path.join(ROOT, "mononn_amd", "specs", args.workload)
+    used = "default"
+    if os.path.isdir(spec_dir):
+        module = MonoNNModule.from_spec_dir(fx.hlo_text, spec_dir)
+        used = os.path.relpath(spec_dir, ROOT)
+    else:
+        module = MonoNNModule.compile(fx.hlo_text)
+    consts, inputs = fx.make_constants(seed, "baseline"), fx.make_inputs(seed)
+    module.set_constants(consts)
+    module.load(0)
+    if args.stage_profile:
+        stage_profile(module, fx, consts, inputs, args)
+        return
+    module.run(inputs, fx.outputs)
+    avg_ms, _ = module.time_raw(module.buffer_pointers(), torch.cuda.current_stream().cuda_stream, warmup=args.warmup, iters=args.steps)
+    line = {"workload": args.workload, "not_the_benchmark_metric": True, "kernel": module.kernel_name, "kernel_avg_us": round(avg_ms * 1e3, 2),
+            "steps": args.steps, "warmup": args.warmup, "tuning_spec": used, **module.launch_dims()}
+    if make == "gemm_stage" and not args.launches_only:
+        # the GEMM stage alone, by the in-kernel clocks of the same specification
+        spec = json.loads(module.get_tuning_spec())
+        spec["mononn_hip"]["profile_stages"] = True
+        prof = MonoNNModule.compile(fx.hlo_text, json.dumps(spec))
+        prof.set_constants(consts)
+        prof.load(0)
+        us = []
+        for i in range(8):
+            prof.run(inputs, fx.outputs)
+            if i >= 3:
+                us.append(prof.stage_profile()[1]["busy_us"])
+        c = fx.config
+        flops = 2 * c["M"] * c["N"] * c["K"]
+        line["gemm_stage"] = {"busy_us": round(float(np.mean(us)), 2), "tflops": round(flops / np.mean(us) / 1e6, 1),
+                              "frac_of_dense_f16_mfma_peak": round(flops / np.mean(us) / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)}
+        prof.close()
+    print(json.dumps(line))
+    module.close()
+
+
 def stage_profile(module, fx, consts, inputs, args):
     """Per-stage clocks of the benchmark's own specification (stamped by every workgroup at stage entry / exit)."""
     from mononn_amd import MonoNNModule
@@ -242,6 +292,13 @@ def main():
     ap.add_argument("--torch-baseline", action="store_true",
                     help="also time the same model written with torch.nn.functional in fp16 on this GPU (eager and "
                          "captured in a HIP graph), reported under \"torch_baseline\"")
+    ap.add_argument("--workload", default="bert_base_b1_s128", choices=sorted(WORKLOADS),
+                    help="bert_base_b1_s128 is the benchmark; any other name runs that configuration alone (shipped "
+                         "specification where there is one) for --warmup + --steps launches and prints its latency: "
+                         "the command profilers are pointed at.  With --stage-profile: its stage clocks")
+    ap.add_argument("--launches-only", action="store_true",
+                    help="with --workload: nothing but the configuration's own launches (for counter collection, where "
+                         "every kernel of the process is profiled)")
     ap.add_argument("--stage-profile", action="store_true",
                     help="instead of the benchmark: rebuild the same specification with per-stage clocks and print, "
                          "per stage, busy time / barrier time averaged over --steps launches")
@@ -256,6 +313,9 @@ def main():
     from mononn_amd.hlo import models
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.workload != "bert_base_b1_s128":
+        single_workload(args)
+        return
     fx = models.bert_base(B=1, S=128)
     consts = fx.make_constants(1235, "baseline")
     inputs = fx.make_inputs(1235)

@@ -198,7 +198,10 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
   if (info.row_program) {
     const int64_t ROWS = info.rows, R = info.row_len;
     const bool block_tier = t.locality_tier == 2;
-    const int stride = block_tier ? ls.block_size : 64;
+    // 8 rows per wave, 8 lanes per row, 16-byte runs per lane: rows of whole runs that fit the registers
+    const int group_run = 16 / hlo::dtype_bytes(outputs[0]->shape.dtype);
+    const bool row_groups = !block_tier && t.reduce_implementation == 1 && R % group_run == 0 && R / group_run >= 8 && (R / group_run + 7) / 8 * group_run <= 160;
+    const int stride = block_tier ? ls.block_size : row_groups ? 8 : 64;
     int row = vars.add("row", ROWS);
     std::vector<const Instr*> row_outs, full_outs;
     for (auto* o : outputs) {
@@ -208,10 +211,13 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       else MONONN_FAIL(kUnsupported) << o->hlo_name << ": output with " << n << " elements does not fit a " << ROWS << " x " << R << " row space";
     }
     cb.line("const int lane = mononn_dev::lane_id();");
-    cb.line(std::string("const int tid = ") + (block_tier ? "(int)threadIdx.x;" : "lane;"));
+    cb.line(std::string("const int tid = ") + (block_tier ? "(int)threadIdx.x;" : row_groups ? "lane >> 3;" : "lane;"));
     if (block_tier) {
       cb.line("const int row = unit;");
       cb.open("");
+    } else if (row_groups) {
+      cb.line("const int row = (unit * " + S(NW) + " + mononn_dev::wave_id()) * 8 + (lane & 7);");
+      cb.open("if (row < " + S(ROWS) + ")");   // the 8 lanes of a row agree
     } else {
       cb.line("const int row = unit * " + S(NW) + " + mononn_dev::wave_id();");
       cb.open("if (row < " + S(ROWS) + ")");
@@ -219,6 +225,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     auto all_reduce = [&](const Instr* r, const std::string& acc) {
       std::string T = hlo::dtype_ctype(r->shape.dtype);
       if (block_tier) cb.line(acc + " = mononn_dev::block_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ", reinterpret_cast<" + T + "*>(smem));");
+      else if (row_groups) cb.line(acc + " = mononn_dev::lane_group8_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
       else cb.line(acc + " = mononn_dev::wave_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
     };
     // Tuple-valued reductions: N accumulators, the reducer computation inlined for every element and, as a local
@@ -276,7 +283,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
         return comb + "(" + args + ");";
       };
       cb.line("#pragma unroll");
-      cb.open("for (int off = 32; off >= 1; off >>= 1)");
+      cb.open("for (int off = 32; off >= " + S(row_groups ? 8 : 1) + "; off >>= 1)");
       cb.line(call([&](size_t i) { return "mononn_dev::lane_xor(" + ta.acc[i] + ", off)"; }));
       cb.close();
       if (!block_tier) return;
@@ -323,10 +330,10 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     // Register-resident form: a thread owns T chunks of V consecutive columns, the whole row program
     // is straight-line code, so a value loaded for the first reduction is still in a register when
     // the later phases need it (one trip to memory per row instead of one per phase).
-    const int V = t.ilp_factor > 1 && R % t.ilp_factor == 0 ? t.ilp_factor : pick_vector_width(R, stride);
+    const int V = row_groups ? group_run : t.ilp_factor > 1 && R % t.ilp_factor == 0 ? t.ilp_factor : pick_vector_width(R, stride);
     const int64_t NQ = R / V;
     const int64_t T = (NQ + stride - 1) / stride;
-    if (T * V <= 32) {
+    if (T * V <= 32 || row_groups) {
       std::vector<int> qvar(T);
       std::vector<bool> partial(T);
       for (int64_t k = 0; k < T; ++k) {
@@ -444,8 +451,8 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       }
     }
     cb.close();
-    int64_t units = block_tier ? ROWS : (ROWS + NW - 1) / NW;
-    return finish(T * V <= 32 ? hoist_row_loads(cb.text()) : cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 * static_cast<int>(max_tuple) : 0);
+    int64_t units = block_tier ? ROWS : row_groups ? (ROWS + 8 * NW - 1) / (8 * NW) : (ROWS + NW - 1) / NW;
+    return finish(T * V <= 32 || row_groups ? hoist_row_loads(cb.text()) : cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 * static_cast<int>(max_tuple) : 0);
   }
 
   // element-wise loop(s); outputs of equal element count share one loop.  A thread owns V consecutive
@@ -738,6 +745,11 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   }
   MONONN_CHECK(!along_m || (mfma && g.M % 4 == 0 && !g.is_conv), kUnsupported) << gi->hlo_name << ": rows cannot be taken four at a time";
   const bool vec4 = mfma && (along_m || g.N % 4 == 0);
+  // N off the lane's run of 4 columns (an LM head over 50257 tokens): the rows start at addresses that are only
+  // 2-byte aligned.  A single f16 result that only the host reads is still written four columns at a time, through
+  // a copy without an alignment promise, wherever the whole run lies inside the row (decided further down).
+  bool ragged4 = false;
+  std::string ragged4_offset;
   CodeBuffer cb;   // epilogue body
   VarTable vars;
   Emitter em(prog, cluster_members, cb, vars, ptrs);
@@ -892,7 +904,30 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
         if (out.vector_store) cb.line(out.stage + "[r] = " + v + ";");
         else store(prog, cb, ptrs, vars, out.o, out.idx, v);
       } else {
-        store(prog, cb, ptrs, vars, out.o, out.idx, v);
+        if (mfma && !along_m && !g.is_conv && outs.size() == 1 && out.o->shape.dtype == DType::kF16 && host_only_output(prog, out.o) && g.N >= 4) {
+          Index at0 = out.idx;
+          // the same element with column 0: the offset must be that plus the column
+          Index probe_idx = delinearize(linearize([&] {
+            Index z = delinearize(LinExpr::variable(vb, g.batch), batch_dims, vars);
+            z.push_back(LinExpr::variable(vm, g.M));
+            z.push_back(LinExpr::constant(0));
+            return z;
+          }(), D.dims), out.o->shape.dims, vars);
+          if (out.o == gi) probe_idx = [&] {
+            Index z = delinearize(LinExpr::variable(vb, g.batch), batch_dims, vars);
+            z.push_back(LinExpr::variable(vm, g.M));
+            z.push_back(LinExpr::constant(0));
+            return z;
+          }();
+          LinExpr full = physical_offset(prog, out.o, out.idx, &vars);
+          LinExpr base = physical_offset(prog, out.o, probe_idx, &vars);
+          if (full.equals(base.plus(LinExpr::variable(vnn, g.N)))) {
+            ragged4 = true;
+            ragged4_offset = ptrs.output(out.o) + " + " + base.str(vars);   // (registers the pointer as a member of the functor)
+          }
+        }
+        if (ragged4) cb.line("return " + v + ";");
+        else store(prog, cb, ptrs, vars, out.o, out.idx, v);
       }
     }
   }
@@ -946,8 +981,19 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   else if (vec4) pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&acc)[4], const Pre& pre) const {\n";
   else if (mfma) {
     pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&accv)[4], const Pre&) const {\n";
-    pre += "    for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") { const float acc = accv[r]; one(bidx, m, nn, acc); } }\n  }\n";
-    pre += "  __device__ __forceinline__ void one(int bidx, int m, int nn, float acc) const {\n";
+    if (ragged4) {
+      pre += "    _Float16* row = " + ragged4_offset + ";\n";
+      pre += "    if (n0 + 3 < " + S(g.N) + ") {\n";
+      pre += "      const _Float16 st[4] = {one(bidx, m, n0, accv[0]), one(bidx, m, n0 + 1, accv[1]), one(bidx, m, n0 + 2, accv[2]), one(bidx, m, n0 + 3, accv[3])};\n";
+      pre += "      mononn_dev::stN_plain_unaligned<_Float16, 4>(row + n0, st);\n";
+      pre += "    } else {\n";
+      pre += "      for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") mononn_dev::st1_plain(row + nn, one(bidx, m, nn, accv[r])); }\n";
+      pre += "    }\n  }\n";
+      pre += "  __device__ __forceinline__ _Float16 one(int bidx, int m, int nn, float acc) const {\n";
+    } else {
+      pre += "    for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") { const float acc = accv[r]; one(bidx, m, nn, acc); } }\n  }\n";
+      pre += "  __device__ __forceinline__ void one(int bidx, int m, int nn, float acc) const {\n";
+    }
   } else {
     pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int nn, float acc) const {\n";
   }

@@ -201,11 +201,18 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
           r.name = n.name;
           // long rows get a whole workgroup, short ones a wave (tiers 2 / 1 of schedule_factory.cc:42-79)
           r.locality_tier = (n.row_program && n.row_len >= 512) ? 2 : 1;
+          // many rows: a wave takes 8 of them at once, which keeps 8 rows' worth of bytes in flight per wave and
+          // fills whole lines with every store (the generator falls back when the row length does not fit)
+          if (n.row_program && n.rows >= 4096 && n.row_len >= 64 && n.row_len <= 1280 && n.row_len % 8 == 0) {
+            r.locality_tier = 1;
+            r.reduce_implementation = 1;
+          }
           spec.cluster_reduce_spec[n.name] = r;
           it = spec.cluster_reduce_spec.find(n.name);
         }
         t.ilp_factor = it->second.ilp_factor;
         t.locality_tier = it->second.locality_tier;
+        t.reduce_implementation = it->second.reduce_implementation;
       } else {
         auto it = spec.cluster_elewise_spec.find(n.name);
         if (it == spec.cluster_elewise_spec.end()) {

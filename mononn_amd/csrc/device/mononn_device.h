@@ -50,6 +50,16 @@ typedef int int4_t __attribute__((ext_vector_type(4)));
 #ifndef MONONN_OPAQUE_VALUE
 #define MONONN_OPAQUE_VALUE(v) asm volatile("" : "+v"(v))
 #endif
+// 16 bytes written through to the memory side with one instruction.  Agent-scope atomic stores stop at 8 bytes (two
+// instructions, two requests per lane); the cache policy bit they carry (sc1) is available on a plain 16-byte store
+// as well.  The store counts in vmcnt like any other, which is what the grid barrier's arrive() waits on.
+#ifndef MONONN_STORE16_AGENT
+// The compiler does not look inside an asm statement, so it places none of the wait states it would put between a
+// vector-ALU write of the data registers and a store that reads them, nor behind a store of more than 8 bytes whose
+// registers are overwritten next.  Without the idle cycles in front the first dword of some lanes arrived as garbage
+// (measured; identical on every run), with them no wrong value was seen.
+#define MONONN_STORE16_AGENT(p, v) asm volatile("s_nop 7\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory")
+#endif
 // an empty statement that requires `v` in accumulation registers at this point of the program
 #ifndef MONONN_PIN_ACC
 #define MONONN_PIN_ACC(v) asm volatile("" : "+a"(v))
@@ -219,10 +229,17 @@ __device__ __forceinline__ void stN(T* p, const T (&v)[N]) {
     __builtin_memcpy(&b, v, 8);
     st1(reinterpret_cast<unsigned long long*>(p), b);
   } else {
+#if MONONN_COHERENT_STORES
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    v4u b;
+    __builtin_memcpy(&b, v, 16);
+    MONONN_STORE16_AGENT(p, b);
+#else
     unsigned long long b[2];
     __builtin_memcpy(b, v, 16);
     st1(reinterpret_cast<unsigned long long*>(p), b[0]);
     st1(reinterpret_cast<unsigned long long*>(p) + 1, b[1]);
+#endif
   }
 }
 
@@ -248,6 +265,13 @@ __device__ __forceinline__ void stN_plain(T* p, const T (&v)[N]) {
     __builtin_memcpy(&b, v, 16);
     *reinterpret_cast<v4u*>(p) = b;
   }
+}
+
+// N consecutive elements at an address that is only known to be aligned to one element: a copy without an alignment
+// promise, for which the compiler picks whatever store width the target's unaligned-access rules allow
+template <class T, int N>
+__device__ __forceinline__ void stN_plain_unaligned(T* p, const T (&v)[N]) {
+  __builtin_memcpy(p, v, N * sizeof(T));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -282,6 +306,17 @@ __device__ __forceinline__ T wave_all_reduce(T v, Op op) {
     for (int off = kWaveSize / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWaveSize));
     return v;
   }
+}
+
+// Reduction over the 8 lanes that share (lane % 8): a wave that works on 8 rows at once keeps row r in lanes r, r + 8,
+// ..., r + 56.  One rotation by 8 inside the row of 16 lanes on the vector ALU, two LDS-crossbar permutes.
+template <class T, class Op>
+__device__ __forceinline__ T lane_group8_all_reduce(T v, Op op) {
+  if constexpr (sizeof(T) == 4) v = op(v, dpp_move<0x128>(v));   // row_ror:8
+  else v = op(v, __shfl_xor(v, 8, kWaveSize));
+  v = op(v, __shfl_xor(v, 16, kWaveSize));
+  v = op(v, __shfl_xor(v, 32, kWaveSize));
+  return v;
 }
 
 // value of `v` in lane (own lane ^ mask), for any type of up to 8 bytes (tuple reductions exchange every member)

@@ -343,9 +343,20 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             for (auto& n : c.nodes) {
               s.cluster_reduce_spec[n].locality_tier = tier;
               s.cluster_reduce_spec[n].ilp_factor = ilp;
+              s.cluster_reduce_spec[n].reduce_implementation = 0;
             }
             add("tier" + std::to_string(tier) + "_ilp" + std::to_string(ilp), s);
           }
+        {
+          // a wave on 8 rows at once (rows of whole 16-byte runs; other rows fall back to one row per wave)
+          GraphSpecification s = filled;
+          for (auto& n : c.nodes) {
+            s.cluster_reduce_spec[n].locality_tier = 1;
+            s.cluster_reduce_spec[n].ilp_factor = 1;
+            s.cluster_reduce_spec[n].reduce_implementation = 1;
+          }
+          add("tier1_rows8", s);
+        }
       } else if (c.kind == "cluster_elewise") {
         for (int ilp : {2, 4, 8}) {
           GraphSpecification s = filled;

@@ -300,6 +300,25 @@ def bert_large(B=16, S=384) -> ModelFixture:
     return bert_encoder(L=24, B=B, S=S, H=1024, NH=16, F=4096, mask_kind="length_mask")
 
 
+def gemm_stage(M=6144, N=4096, K=1024) -> ModelFixture:
+    """One weight GEMM at the shape of BERT-large's first feed-forward projection (16 x 384 rows), fed by an
+    element-wise stage the way every GEMM inside an encoder is fed by the stage before it: f16[M,K] activations,
+    constant f16[K,N] weights, f16[M,N] result.  Two stages, one grid barrier."""
+    mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
+    e = mb.entry
+    x = e.parameter("f16", (M, K), "activations")
+
+    def body(f, p):
+        return f.convert(f.mul(f.convert(p, "f32"), f.splat("f32", 0.5, p.dims)), "f16")
+    a = e.fusion("kLoop", [x], body)
+    w = e.elided_constant("f16", (K, N), "gemm_stage/kernel")
+    e.set_tuple_root([e.gemm(a, w, 1, 0)])
+    return ModelFixture(
+        f"gemm_stage_{M}x{N}x{K}", mb.text(),
+        [{"name": "activations", "dtype": "f16", "dims": [M, K], "kind": "normal"}],
+        mb.constants, [{"dtype": "f16", "dims": [M, N]}], dict(M=M, N=N, K=K))
+
+
 def gpt2(L=12, B=4, S=512, H=768, NH=12, F=3072, vocab=50257, max_pos=1024, eps=1e-5) -> ModelFixture:
     """GPT-2 style decoder prefill: token + learned position embeddings, L pre-LayerNorm layers with causal
     self-attention and tanh-GELU MLP, final LayerNorm, LM head tied to the token embedding

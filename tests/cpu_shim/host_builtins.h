@@ -26,6 +26,7 @@
 #define __builtin_amdgcn_s_barrier() ((void)0)
 #define __builtin_amdgcn_readfirstlane(x) (x)
 #define MONONN_PIN_ACC(v) ((void)0) /* register placement only */
+#define MONONN_STORE16_AGENT(p, v) std::memcpy((void*)(p), &(v), 16) /* a GPU store instruction written in assembly */
 #define MONONN_OPAQUE_VALUE(v) ((void)0) /* an empty asm with a GPU register constraint */
 /* buffer descriptor + 16-byte load at descriptor base + lane offset + wave offset */
 typedef const char* __amdgpu_buffer_rsrc_t;

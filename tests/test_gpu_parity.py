@@ -66,6 +66,8 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
     dict(M=77, N=50, K=33, batch=(2,), dtype="f32", rhs_c=2),     # f32, batched, everything ragged
     dict(M=128, N=256, K=128, dtype="f32", b_const=True),         # f32 constant weights (not packed)
     dict(M=40, N=24, K=64, dtype="f32", lhs_c=0, rhs_c=1),        # f32 with A stored [K,M]: per-element fallback
+    dict(M=256, N=1001, K=128, rhs_c=1, b_const=True),            # odd N: rows at 2-byte aligned addresses, 4 columns per store where they fit
+    dict(M=70, N=50, K=64, batch=(2,), rhs_c=2),                  # N off the run of 4, batched
 ])
 def test_gemm_cases(gpu_device, case):
     mb, a_dims, b_dims, d_dims = gemm_module(**case)
