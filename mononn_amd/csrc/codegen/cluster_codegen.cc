@@ -471,28 +471,77 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
   int64_t unit_base = 0;
   for (size_t gi = 0; gi < groups.size(); ++gi) {
     const int64_t N = groups[gi].first;
-    const int V = (t.ilp_factor > 1 && N % t.ilp_factor == 0 && t.ilp_factor <= 16) ? t.ilp_factor : 1;
+    // A thread owns V consecutive elements (one 16-byte run of the first output unless the specification names a
+    // width) and, where the stage is long enough to come round several times, U such runs a workgroup apart: all
+    // U * V values are computed before the first store, so the loads of a unit are in flight together and the
+    // stores, whose acknowledgements a later load would otherwise wait for, come last.
+    const int auto_v = std::min<int>(8, 16 / hlo::dtype_bytes(groups[gi].second[0]->shape.dtype));
+    int V = 1;
+    if (t.ilp_factor > 1 && N % t.ilp_factor == 0 && t.ilp_factor <= 16) V = t.ilp_factor;
+    else if (t.ilp_factor <= 1 && N % auto_v == 0) V = auto_v;
     const int64_t NQ = N / V;
-    const int64_t units = (NQ + ls.block_size - 1) / ls.block_size;
+    const int U = NQ >= 4 * static_cast<int64_t>(ls.block_size) * 256 ? 4 : 1;
+    const int64_t units = (NQ + static_cast<int64_t>(ls.block_size) * U - 1) / (static_cast<int64_t>(ls.block_size) * U);
     std::string u = "unit";
     if (groups.size() > 1) {
       cb.open(std::string(gi ? "else " : "") + "if (unit < " + S(unit_base + units) + ")");
       u = "(unit - " + S(unit_base) + ")";
+    } else {
+      cb.open("");
     }
-    std::string qv = "q" + S(gi);
-    int var = vars.add(qv, NQ);
-    cb.line("const int " + qv + " = " + u + " * " + S(ls.block_size) + " + (int)threadIdx.x;");
-    cb.open("if (" + qv + " < " + S(NQ) + ")");
     em.push_scope();
-    for (int v = 0; v < V; ++v)
-      for (auto* o : groups[gi].second) {
-        LinExpr lin = LinExpr::variable(var, NQ).scaled(V).plus_const(v);
-        Index oi = delinearize(lin, o->shape.dims, vars);
-        store(prog, cb, ptrs, vars, o, oi, em.value(em.resolve_output(o), oi));
+    struct Pending {
+      std::string guard;
+      std::vector<std::string> lines;
+    };
+    std::vector<Pending> stores;
+    for (int uu = 0; uu < U; ++uu) {
+      const std::string qv = "q" + S(static_cast<int64_t>(gi)) + "_" + S(uu);
+      const std::string act = "act" + S(static_cast<int64_t>(gi)) + "_" + S(uu);
+      int var = vars.add(qv, NQ);
+      const std::string raw = u + " * " + S(static_cast<int64_t>(ls.block_size) * U) + " + " + S(static_cast<int64_t>(uu) * ls.block_size) + " + (int)mononn_dev::thread_id()";
+      const bool exact = NQ % (static_cast<int64_t>(ls.block_size) * U) == 0;
+      if (exact) {
+        cb.line("const int " + qv + " = " + raw + ";");
+      } else {
+        // past the end: values are computed for the last run (in range), nothing is stored
+        cb.line("const bool " + act + " = " + raw + " < " + S(NQ) + ";");
+        cb.line("const int " + qv + " = " + act + " ? " + raw + " : " + S(NQ - 1) + ";");
       }
+      Pending pend;
+      pend.guard = exact ? "" : act;
+      for (auto* o : groups[gi].second) {
+        std::vector<std::string> vals;
+        std::vector<LinExpr> offs;
+        for (int v = 0; v < V; ++v) {
+          LinExpr lin = LinExpr::variable(var, NQ).scaled(V).plus_const(v);
+          Index oi = delinearize(lin, o->shape.dims, vars);
+          vals.push_back(em.value(em.resolve_output(o), oi));
+          offs.push_back(physical_offset(prog, o, oi, &vars));
+        }
+        const int bytes = V * hlo::dtype_bytes(o->shape.dtype);
+        bool adjacent = V > 1 && (bytes == 4 || bytes == 8 || bytes == 16);
+        for (int v = 1; adjacent && v < V; ++v) adjacent = offs[v].equals(offs[0].plus_const(v));
+        if (adjacent) {
+          std::string T = hlo::dtype_ctype(o->shape.dtype);
+          std::string arr = em.fresh("pk");
+          std::string init;
+          for (int v = 0; v < V; ++v) init += (v ? ", " : "") + vals[v];
+          pend.lines.push_back("const " + T + " " + arr + "[" + S(V) + "] = {" + init + "};");
+          pend.lines.push_back(stN_of(prog, o) + T + ", " + S(V) + ">(" + ptrs.output(o) + " + " + offs[0].str(vars) + ", " + arr + ");");
+        } else {
+          for (int v = 0; v < V; ++v) pend.lines.push_back(st1_of(prog, o) + ptrs.output(o) + " + " + offs[v].str(vars) + ", " + vals[v] + ");");
+        }
+      }
+      stores.push_back(std::move(pend));
+    }
+    for (auto& pend : stores) {
+      if (!pend.guard.empty()) cb.open("if (" + pend.guard + ")");
+      for (auto& l : pend.lines) cb.line(l);
+      if (!pend.guard.empty()) cb.close();
+    }
     em.pop_scope();
     cb.close();
-    if (groups.size() > 1) cb.close();
     unit_base += units;
   }
   return finish(cb.text(), ptrs, tables_of(em), unit_base, 0);

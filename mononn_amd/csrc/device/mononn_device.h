@@ -973,9 +973,13 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   const int n_base = tile_n * BN + wn * (TN * 32);
   const int lane_m = D_ALONG_M ? (lane >> 5) * 4 : r32;
   const int lane_n = D_ALONG_M ? r32 : (lane >> 5) * 4;
-  // Operands of the epilogue (bias, residual) are requested one row of fragments ahead of their use: the first row
-  // now, row i + 1 while row i is finalised (all of them at once would cost more registers than the tile has left).
-  typename Epi::Pre pre[2][TN * 4];
+  // Operands of the epilogue (bias, residual).  When those of the whole tile fit in 128 registers, the first row is
+  // requested now and the others three k tiles before the end, so that their latency passes under the last
+  // MFMAs (after the k loop a wave has nothing left to wait behind: a row requested only while the row before
+  // it is finalised costs a full trip to memory).  Larger tiles keep that row-ahead scheme.
+  constexpr int PRE_REGS = (int)(sizeof(typename Epi::Pre) + 3) / 4 * TN * 4 * TM;
+  constexpr bool PRE_ALL = sizeof(typename Epi::Pre) > 1 && PRE_REGS <= 128 && TM > 1;
+  typename Epi::Pre pre[PRE_ALL ? TM : 2][TN * 4];
   auto preload_row = [&](int i, typename Epi::Pre (&dst)[TN * 4]) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -1061,10 +1065,24 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
       }
     }
   };
+  constexpr int PRE_AT = KT >= 3 ? KT - 3 : 0;   // the k tile in front of which the other rows' operands are requested
+  auto preload_rest = [&](int t) {
+    if constexpr (PRE_ALL) {
+      if (t == PRE_AT) {
+#pragma unroll
+        for (int i = 1; i < TM; ++i) preload_row(i, pre[i]);
+      }
+    }
+  };
   for (int t = 0; t + 1 < KT; t += 2) {
+    preload_rest(t);
     run_tile(t, BoolConstant<true>(), BoolConstant<false>());
-    if (t + 2 < KT) run_tile(t + 1, BoolConstant<false>(), BoolConstant<false>());
+    if (t + 2 < KT) {
+      preload_rest(t + 1);
+      run_tile(t + 1, BoolConstant<false>(), BoolConstant<false>());
+    }
   }
+  preload_rest(KT - 1);
   if constexpr ((KT - 1) % 2 == 0) run_tile(KT - 1, BoolConstant<true>(), BoolConstant<true>());
   else run_tile(KT - 1, BoolConstant<false>(), BoolConstant<true>());
 
@@ -1079,7 +1097,7 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
     for (int r = i + 1; r < TM; ++r)
 #pragma unroll
       for (int j = 0; j < TN; ++j) MONONN_PIN_ACC(acc[r][j]);
-    if (i + 1 < TM) preload_row(i + 1, pre[(i + 1) & 1]);
+    if (!PRE_ALL && i + 1 < TM) preload_row(i + 1, pre[(i + 1) & 1]);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -1088,7 +1106,7 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
         const int n = n_base + j * 32 + lane_n + (D_ALONG_M ? 0 : 8 * g);
         if (m < M && n < N) {
           float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-          epi(batch, m, n, v, pre[i & 1][j * 4 + g]);
+          epi(batch, m, n, v, pre[PRE_ALL ? i : (i & 1)][j * 4 + g]);
         }
       }
   }
