@@ -189,7 +189,12 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     int per_cu, block;
   };
   std::vector<Ctx> contexts = {{1, 256}, {1, 512}};
-  if (budget == 0) contexts.push_back({2, 256});
+  if (budget == 0) {
+    // the reference's space also holds more workgroups per SM and smaller workgroups (tuning_space_generator.cc:65-66)
+    contexts.push_back({2, 256});
+    contexts.push_back({3, 256});
+    contexts.push_back({1, 128});
+  }
   if (budget >= 2) contexts = {{1, 256}};
   // MONONN_TUNER_LAUNCH_CONTEXTS="1x256,2x256": workgroups per CU x threads, instead of the list above (large models:
   // one context of a full search takes minutes)

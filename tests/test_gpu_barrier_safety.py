@@ -106,3 +106,32 @@ def test_stage_outputs_are_complete_when_the_flag_is_seen(gpu_device):
         want = (((xv.T * 3 + 1).T * 5 - 7).T * 7 + 11).astype(np.int32)
         assert np.array_equal(got, want), f"launch {launch}: {(got != want).sum()} wrong words"
     m.close()
+
+
+@pytest.mark.gpu
+def test_cooperative_launch_is_refused_while_a_profiler_tool_is_attached(gpu_device):
+    """A process that used the cooperative launch entry point under a profiler tool died in an exit handler; the
+    combination is refused at load time with a message that names the way out, and the ordinary launch is not
+    affected.  (The tool is only named in the environment here: nothing is loaded.)"""
+    import os
+    import test_gpu_parity as parity
+    from mononn_amd import MonoNNError, MonoNNModule
+    mb, a_dims, b_dims, d_dims = parity.gemm_module(M=64, N=64, K=64)
+    rng = np.random.default_rng(3)
+    a, b = rng.normal(size=a_dims).astype(np.float16), rng.normal(size=b_dims).astype(np.float16)
+    coop = MonoNNModule.compile(mb.text(), parity._spec_with(mb.text(), hip={"cooperative_launch": True}))
+    plain = MonoNNModule.compile(mb.text())
+    assert "HSA_TOOLS_LIB" not in os.environ and "ROCP_TOOL_LIBRARIES" not in os.environ
+    os.environ["HSA_TOOLS_LIB"] = "libsome-profiler-tool.so"
+    try:
+        with pytest.raises(MonoNNError, match="cooperative_launch is refused while a profiler tool"):
+            coop.load(gpu_device)
+        plain.load(gpu_device)
+        want = plain.run([a, b], [{"dtype": "f16", "dims": d_dims}])[0]
+    finally:
+        del os.environ["HSA_TOOLS_LIB"]
+    coop.load(gpu_device)          # without the tool the cooperative launch loads and agrees
+    got = coop.run([a, b], [{"dtype": "f16", "dims": d_dims}])[0]
+    assert np.array_equal(got, want)
+    coop.close()
+    plain.close()
