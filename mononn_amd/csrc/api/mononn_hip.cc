@@ -97,8 +97,13 @@ int mononn_compile_from_spec_dir(const char* hlo_text, size_t hlo_len, const cha
     auto h = std::make_unique<mononn_module>();
     h->impl = std::make_unique<MonoNNModule>(text, spec, "");
     h->impl->generate_code();
-    std::string co;
-    if (!mononn::env::is_true("TF_MONONN_NO_USE_PTX_CACHE") && mononn::module::read_file(cdir + "/best_tuning_spec.hsaco", &co) && !co.empty())
+    // The cached code object is used only when it was built from exactly the sources just generated (same HLO, same
+    // specification, same device prelude, same compiler options): grid, LDS size, argument order, constant packing
+    // and the number of barrier flags on the host side come from the fresh code, and a kernel that disagrees with
+    // them computes garbage or never passes its first barrier.
+    std::string co, key;
+    if (!mononn::env::is_true("TF_MONONN_NO_USE_PTX_CACHE") && mononn::module::read_file(cdir + "/best_tuning_spec.hsaco", &co) && !co.empty() &&
+        mononn::module::read_file(cdir + "/best_tuning_spec.hsaco.key", &key) && key == h->impl->source_key())
       h->impl->set_code_object(std::vector<char>(co.begin(), co.end()));
     else
       h->impl->build_assembly();

@@ -366,6 +366,27 @@ std::string MonoNNModule::cluster_dir(const std::string& dump_dir) const {
   return dump_dir + "/" + shortn;
 }
 
+std::string MonoNNModule::source_key() const {
+  // FNV-1a over file names and contents in name order, then the extra compiler options of the environment
+  unsigned long long h = 1469598103934665603ull;
+  auto mix = [&](const std::string& t) {
+    for (unsigned char c : t) {
+      h ^= c;
+      h *= 1099511628211ull;
+    }
+    h ^= 0xff;
+    h *= 1099511628211ull;
+  };
+  for (auto& kv : hip_.files) {
+    mix(kv.first);
+    mix(kv.second);
+  }
+  mix(env::get("MONONN_HIPRTC_FLAGS"));
+  char buf[40];
+  std::snprintf(buf, sizeof buf, "fnv1a64:%016llx", h);
+  return buf;
+}
+
 void MonoNNModule::dump_candidate(const std::string& dump_dir) const {
   std::string dir = cluster_dir(dump_dir);
   std::string ctx = spec_.context_string();
@@ -379,7 +400,10 @@ void MonoNNModule::dump_best(const std::string& dump_dir) const {
   std::string dir = cluster_dir(dump_dir);
   make_dirs(dir);
   write_file(dir + "/best_tuning_spec.json", tuning_spec_json());
-  if (has_code_object()) write_file(dir + "/best_tuning_spec.hsaco", code_object_);
+  if (has_code_object()) {
+    write_file(dir + "/best_tuning_spec.hsaco", code_object_);
+    write_file(dir + "/best_tuning_spec.hsaco.key", source_key());
+  }
   // source of the kernel and of the standalone driver (host_main.cpp), and what that driver feeds the module
   // globals with: literal constants always, elided ones when the host has supplied them and the module has not
   // been loaded yet (payloads are handed to the device at load time)

@@ -32,6 +32,9 @@ class MonoNNModule {
   void build_assembly();                      // hipRTC -> code object (needs generate_code)
   bool has_code_object() const { return !code_object_.empty(); }
   void set_code_object(const std::vector<char>& co) { code_object_ = co; }   // cached build (best_tuning_spec.hsaco)
+  // Key of what a code object of this module is built from: the generated sources (kernel, device prelude) and the
+  // compiler options.  Written beside a cached code object, compared before that cache is used.
+  std::string source_key() const;
 
   const std::string& kernel_name() const { return kernel_name_; }
   const std::string& module_name() const { return module_name_; }

@@ -371,6 +371,8 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       }
     }
     // ---- code generation in the pool; one hipRTC compilation and one module load per class -----------
+    const bool progress = env::is_true("TF_MONONN_ENABLE_WORKER_THRAED_LOGGING") || env::is_true("MONONN_TUNER_VERBOSE");
+    std::atomic<size_t> generated{0};
     parallel_for(trials.size(), threads, [&](size_t i) {
       Trial& t = trials[i];
       try {
@@ -380,6 +382,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         t.error = e.what();
         t.mod.reset();
       }
+      const size_t done = ++generated;
+      if (progress && (done % 16 == 0 || done == trials.size()))
+        std::fprintf(stderr, "[mononn tuner] %s code generated for %zu of %zu candidates\n", ctx_str.c_str(), done, trials.size());
     });
     GraphSpecification stitched = filled;
     // runners-up of every class by the isolated stage clocks, for the whole-kernel refinement below
@@ -548,8 +553,11 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         m.generate_code();
         m.build_assembly();
         bufs.ensure_temp(static_cast<size_t>(m.hip_program().temp_bytes));
-        return time_module(m, params.device, bufs, 5, 40);
-      } catch (const Error&) {
+        const double us = time_module(m, params.device, bufs, 5, 40);
+        if (verbose) std::fprintf(stderr, "[mononn tuner] %s   a whole kernel built and timed: %.2f us\n", ctx_str.c_str(), us);
+        return us;
+      } catch (const Error& e) {
+        if (verbose) std::fprintf(stderr, "[mononn tuner] %s   a whole kernel was not built: %.200s\n", ctx_str.c_str(), e.what());
         return -1;
       }
     };

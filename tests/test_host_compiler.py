@@ -115,6 +115,19 @@ def test_spec_round_trip_and_reload(layer, tmp_path):
         assert (d / f).exists(), f
     m3 = MonoNNModule.from_spec_dir(layer.hlo_text, str(tmp_path))
     assert m3.get_code_object() == mb.get_code_object()      # cached code object was picked up
+    # ... because it was built from the sources this load generates: the key beside it says so.  A cache whose key
+    # does not match (another specification, HLO, prelude or compiler options) is left alone and the kernel rebuilt
+    assert (d / "best_tuning_spec.hsaco.key").read_text().startswith("fnv1a64:")
+    good = (d / "best_tuning_spec.hsaco").read_bytes()
+    (d / "best_tuning_spec.hsaco").write_bytes(b"stale code object")
+    assert bytes(MonoNNModule.from_spec_dir(layer.hlo_text, str(tmp_path)).get_code_object()) == b"stale code object"    # the key still matches
+    edited = json.loads((d / "best_tuning_spec.json").read_text())
+    edited["mononn_hip"]["barrier_timeout_ms"] = 2000          # changes the generated preamble, hence the key
+    (d / "best_tuning_spec.json").write_text(json.dumps(edited))
+    rebuilt = bytes(MonoNNModule.from_spec_dir(layer.hlo_text, str(tmp_path)).get_code_object())
+    assert rebuilt != b"stale code object" and rebuilt[:4] == b"\x7fELF"
+    (d / "best_tuning_spec.json").write_text(json.dumps(spec if False else json.loads(mb.get_tuning_spec())))
+    (d / "best_tuning_spec.hsaco").write_bytes(good)
     os.environ["TF_MONONN_EXISTING_TUNING_SPEC_DIR"] = str(tmp_path)
     try:
         m4 = MonoNNModule.from_spec_dir(layer.hlo_text, None)
