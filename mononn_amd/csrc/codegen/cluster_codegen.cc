@@ -3,7 +3,10 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <functional>
+#include <map>
+#include <memory>
 #include <set>
 #include <regex>
 #include <sstream>
@@ -1096,6 +1099,206 @@ const Instr* prologue_primary(const Program& prog, const std::vector<const Instr
 
 namespace {
 
+// ---- LayerNorm recogniser -------------------------------------------------------------------------------------------
+// A row program in front of a GEMM is generated element by element from whatever the HLO says.  For the one program
+// that matters there (LayerNorm: y = (x - mean(x)) * rsqrt(var(x) + eps) * gamma + beta over the last dimension) a
+// hand-laid-out form is an order of magnitude cheaper, so the program's expression is rebuilt symbolically from the
+// member fusions and compared with that formula (operand order of + and * free).  Anything else keeps the generic form.
+struct Sym {
+  enum Kind { kX, kCol, kConst, kRowSum, kOp };
+  enum Class { kScalar, kRow, kColumn, kFull };
+  Kind kind = kOp;
+  Class cls = kScalar;
+  std::string op;              // kOp: add subtract multiply divide rsqrt
+  double c = 0;                // kConst
+  const Instr* col = nullptr;  // kCol: a [K] vector read from outside the program
+  std::vector<std::shared_ptr<Sym>> kids;
+};
+using SymP = std::shared_ptr<Sym>;
+
+struct LayerNormMatch {
+  const Instr* gamma = nullptr;
+  const Instr* beta = nullptr;
+  double eps = 0;
+};
+
+struct SymBuilder {
+  const Program& prog;
+  std::set<const Instr*> members;
+  const Instr* primary;
+  int64_t K;
+  bool failed = false;
+
+  SymP fail() {
+    failed = true;
+    return nullptr;
+  }
+  static SymP make(Sym::Kind k, Sym::Class c) {
+    auto s = std::make_shared<Sym>();
+    s->kind = k;
+    s->cls = c;
+    return s;
+  }
+  // value of an instruction of the entry computation
+  SymP entry(const Instr* ins) {
+    if (failed) return nullptr;
+    if (members.count(ins)) {
+      if (ins->opcode != "fusion" || ins->shape.is_tuple()) return fail();
+      std::map<const Instr*, SymP> env;
+      for (size_t i = 0; i < ins->operands.size(); ++i) {
+        SymP v = entry(ins->operands[i]);
+        if (!v) return fail();
+        env[ins->called->params[i]] = v;
+      }
+      return inner(ins->called->root, env);
+    }
+    if (prog.storage_root(ins) == primary) return make(Sym::kX, Sym::kFull);
+    if (ins->opcode == "constant") {
+      if (ins->is_scalar_constant()) {
+        auto s = make(Sym::kConst, Sym::kScalar);
+        s->c = std::strtod(ins->literal.c_str(), nullptr);
+        return s;
+      }
+      if (ins->shape.rank() == 1 && ins->shape.dims[0] == K) {
+        auto s = make(Sym::kCol, Sym::kColumn);
+        s->col = ins;
+        return s;
+      }
+    }
+    return fail();
+  }
+  SymP inner(const Instr* ins, std::map<const Instr*, SymP>& env) {
+    if (failed) return nullptr;
+    auto it = env.find(ins);
+    if (it != env.end()) return it->second;
+    const std::string& op = ins->opcode;
+    SymP r;
+    if (op == "parameter") return fail();   // every parameter is bound above
+    if (op == "constant") {
+      if (!ins->is_scalar_constant()) return fail();
+      r = make(Sym::kConst, Sym::kScalar);
+      r->c = std::strtod(ins->literal.c_str(), nullptr);
+    } else if (op == "convert" || op == "bitcast" || op == "reshape" || op == "copy") {
+      r = inner(ins->operands[0], env);
+    } else if (op == "broadcast") {
+      SymP k = inner(ins->operands[0], env);
+      if (!k) return fail();
+      const int rank_in = ins->operands[0]->shape.rank();
+      if (rank_in == 0) r = k;
+      else if (rank_in == 1 && ins->shape.rank() == 1 && k->cls != Sym::kFull) r = k;   // a splat written as [M] -> [M]
+      else if (rank_in == 1 && ins->shape.rank() == 2 && ins->dimensions.size() == 1 &&
+               ((k->cls == Sym::kRow && ins->dimensions[0] == 0) || (k->cls == Sym::kColumn && ins->dimensions[0] == 1) || k->cls == Sym::kScalar))
+        r = k;
+      else return fail();
+    } else if (op == "reduce") {
+      if (ins->operands.size() != 2 || ins->dimensions.size() != 1 || ins->operands[0]->shape.rank() != 2 || ins->dimensions[0] != 1) return fail();
+      if (!ins->called || ins->called->root->opcode != "add") return fail();
+      SymP init = inner(ins->operands[1], env);
+      SymP x = inner(ins->operands[0], env);
+      if (!init || !x || init->kind != Sym::kConst || init->c != 0.0) return fail();
+      r = make(Sym::kRowSum, Sym::kRow);
+      r->kids = {x};
+    } else if (op == "add" || op == "subtract" || op == "multiply" || op == "divide") {
+      SymP a = inner(ins->operands[0], env), b = inner(ins->operands[1], env);
+      if (!a || !b) return fail();
+      r = make(Sym::kOp, Sym::kScalar);
+      r->op = op;
+      r->kids = {a, b};
+      if (a->cls == b->cls) r->cls = a->cls;
+      else if (a->cls == Sym::kScalar) r->cls = b->cls;
+      else if (b->cls == Sym::kScalar) r->cls = a->cls;
+      else r->cls = Sym::kFull;
+    } else if (op == "rsqrt") {
+      SymP a = inner(ins->operands[0], env);
+      if (!a) return fail();
+      r = make(Sym::kOp, a->cls);
+      r->op = op;
+      r->kids = {a};
+    } else {
+      return fail();
+    }
+    if (r) env[ins] = r;
+    return r;
+  }
+};
+
+bool sym_equal(const SymP& a, const SymP& b) {
+  if (a->kind != b->kind) return false;
+  switch (a->kind) {
+    case Sym::kX: return true;
+    case Sym::kCol: return a->col == b->col;
+    case Sym::kConst: return a->c == b->c;
+    case Sym::kRowSum: return sym_equal(a->kids[0], b->kids[0]);
+    case Sym::kOp:
+      if (a->op != b->op || a->kids.size() != b->kids.size()) return false;
+      if (a->kids.size() == 1) return sym_equal(a->kids[0], b->kids[0]);
+      if (sym_equal(a->kids[0], b->kids[0]) && sym_equal(a->kids[1], b->kids[1])) return true;
+      return (a->op == "add" || a->op == "multiply") && sym_equal(a->kids[0], b->kids[1]) && sym_equal(a->kids[1], b->kids[0]);
+  }
+  return false;
+}
+
+// s = op(p, q) with p satisfying `first` (either operand order when the operation commutes); p and q are returned
+bool sym_split(const SymP& s, const char* op, const std::function<bool(const SymP&)>& first, SymP* p, SymP* q) {
+  if (s->kind != Sym::kOp || s->op != op || s->kids.size() != 2) return false;
+  const bool commutes = s->op == "add" || s->op == "multiply";
+  for (int order = 0; order < (commutes ? 2 : 1); ++order) {
+    const SymP& a = s->kids[order];
+    const SymP& b = s->kids[1 - order];
+    if (first(a)) {
+      *p = a;
+      *q = b;
+      return true;
+    }
+  }
+  return false;
+}
+
+// sum / K written as a product with 1/K or a quotient by K
+bool sym_is_mean_of(const SymP& s, int64_t K, SymP* summed) {
+  SymP c, rest;
+  auto is_const = [](const SymP& v) { return v->kind == Sym::kConst; };
+  if (sym_split(s, "multiply", is_const, &c, &rest) && std::fabs(c->c * static_cast<double>(K) - 1.0) < 1e-5 && rest->kind == Sym::kRowSum) {
+    *summed = rest->kids[0];
+    return true;
+  }
+  if (s->kind == Sym::kOp && s->op == "divide" && s->kids[1]->kind == Sym::kConst && s->kids[1]->c == static_cast<double>(K) && s->kids[0]->kind == Sym::kRowSum) {
+    *summed = s->kids[0]->kids[0];
+    return true;
+  }
+  return false;
+}
+
+bool match_layer_norm(const Program& prog, const std::vector<const Instr*>& row_members, const Instr* primary, const Instr* H, int64_t K, LayerNormMatch* out) {
+  SymBuilder b{prog, std::set<const Instr*>(row_members.begin(), row_members.end()), primary, K};
+  SymP y = b.entry(H);
+  if (!y || b.failed) return false;
+  auto is_col = [](const SymP& v) { return v->kind == Sym::kCol; };
+  auto is_row = [](const SymP& v) { return v->cls == Sym::kRow; };
+  auto is_const = [](const SymP& v) { return v->kind == Sym::kConst; };
+  SymP beta, t, gamma, u, r, d;
+  if (!sym_split(y, "add", is_col, &beta, &t)) return false;
+  if (!sym_split(t, "multiply", is_col, &gamma, &u)) return false;
+  if (!sym_split(u, "multiply", is_row, &r, &d)) return false;
+  // d = x - mean(x)
+  auto is_centred = [&](const SymP& v) {
+    SymP summed;
+    return v->kind == Sym::kOp && v->op == "subtract" && v->kids[0]->kind == Sym::kX && sym_is_mean_of(v->kids[1], K, &summed) && summed->kind == Sym::kX;
+  };
+  if (!is_centred(d)) return false;
+  // r = rsqrt(mean(d * d) + eps)
+  if (r->kind != Sym::kOp || r->op != "rsqrt") return false;
+  SymP eps, var, sq;
+  if (!sym_split(r->kids[0], "add", is_const, &eps, &var)) return false;
+  if (!sym_is_mean_of(var, K, &sq)) return false;
+  if (sq->kind != Sym::kOp || sq->op != "multiply" || !is_centred(sq->kids[0]) || !sym_equal(sq->kids[0], sq->kids[1]) || !sym_equal(sq->kids[0], d)) return false;
+  if (!(eps->c > 0)) return false;
+  out->gamma = gamma->col;
+  out->beta = beta->col;
+  out->eps = eps->c;
+  return out->gamma->shape.dtype == DType::kF16 && out->beta->shape.dtype == DType::kF16;
+}
+
 Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& row_members, const Instr* gi, const graph::GemmDesc& g,
                         const GemmTuning& t, const LaunchShape& ls, bool stores, PointerTable& ptrs) {
   (void)ls;
@@ -1144,6 +1347,100 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
     cb.line("const int m" + S(i) + " = mv" + S(i) + " ? m_base + " + S(i * 16) + " + r16 : " + S(g.M - 1) + ";");
   }
   auto bind_elem = [&](int i, int s, int e) { em.bind(primary, primary_index(i, s, e), "a[" + S(s) + "][" + S(i) + "][" + S(e) + "]"); };
+  auto finish_struct = [&](const std::string& body, int smem_bytes) {
+    out.smem = smem_bytes;
+    for (auto& kv : em.literal_tables()) out.globals.push_back(kv.second);
+    std::string st = "struct @NAME@_pro {\n  static constexpr bool enabled = true;\n";
+    for (size_t i = first; i < ptrs.entries.size(); ++i) {
+      auto& e = ptrs.entries[i];
+      st += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
+    }
+    st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, char* smem) const {\n";
+    std::istringstream is(body);
+    std::string l;
+    while (std::getline(is, l)) st += "  " + l + "\n";
+    st += "  }\n};\n";
+    out.struct_text = st;
+    std::string init = "@NAME@_pro pro{";
+    for (size_t i = first; i < ptrs.entries.size(); ++i) init += (i > first ? ", " : "") + ptrs.entries[i].name;
+    init += "};";
+    out.init_line = init;
+  };
+  // LayerNorm, laid out by hand: gamma / beta of the lane's columns requested first (16 bytes per k step each), the
+  // sums of x and x * x in one pass over the fragments, one exchange across the 4 lanes of a row and (WK > 1) one
+  // through LDS for both sums, then ((x - mean) * r) * gamma + beta as two fused multiply-adds per element.  The variance is
+  // E[x^2] - mean^2 in fp32 (one exchange instead of two); the generic form computes the centred sum of squares.
+  LayerNormMatch ln;
+  if (match_layer_norm(prog, row_members, primary, H, g.K, &ln)) {
+    const std::string pg = ptrs.input(ln.gamma), pb = ptrs.input(ln.beta);
+    char num[64];
+    for (int s = 0; s < CH; ++s) {
+      const std::string col = "(wk * 32 + g * 8 + " + S(static_cast<int64_t>(s) * WK * 32) + ")";
+      cb.line("const half8_t gam" + S(s) + " = *reinterpret_cast<const half8_t*>(" + pg + " + " + col + ");");
+      cb.line("const half8_t bet" + S(s) + " = *reinterpret_cast<const half8_t*>(" + pb + " + " + col + ");");
+    }
+    for (int i = 0; i < TM; ++i) {
+      // two elements per instruction and sum: v_dot2_f32_f16 (products and sums in fp32)
+      cb.line("float s1_" + S(i) + " = 0.f, s2_" + S(i) + " = 0.f;");
+      for (int s = 0; s < CH; ++s)
+        for (int p2 = 0; p2 < 4; ++p2) {
+          const std::string h = "__builtin_shufflevector(a[" + S(s) + "][" + S(i) + "], a[" + S(s) + "][" + S(i) + "], " + S(2 * p2) + ", " + S(2 * p2 + 1) + ")";
+          cb.line("s1_" + S(i) + " = __builtin_amdgcn_fdot2(" + h + ", half2_t{(_Float16)1, (_Float16)1}, s1_" + S(i) + ", false);");
+          cb.line("s2_" + S(i) + " = __builtin_amdgcn_fdot2(" + h + ", " + h + ", s2_" + S(i) + ", false);");
+        }
+      for (int off : {16, 32}) {
+        cb.line("s1_" + S(i) + " += __shfl_xor(s1_" + S(i) + ", " + S(off) + ", 64);");
+        cb.line("s2_" + S(i) + " += __shfl_xor(s2_" + S(i) + ", " + S(off) + ", 64);");
+      }
+    }
+    int smem_ln = 0;
+    if (WK > 1) {
+      // [mn wave][row fragment][wk][16 rows][2 sums]
+      cb.line("float* rb = reinterpret_cast<float*>(smem) + mn_wave * " + S(TM * WK * 32) + ";");
+      smem_ln = t.wm * t.wn * TM * WK * 32 * 4;
+      cb.open("if (g == 0)");
+      for (int i = 0; i < TM; ++i) {
+        cb.line("rb[" + S(i * WK * 32) + " + wk * 32 + r16 * 2] = s1_" + S(i) + ";");
+        cb.line("rb[" + S(i * WK * 32) + " + wk * 32 + r16 * 2 + 1] = s2_" + S(i) + ";");
+      }
+      cb.close();
+      cb.line("__syncthreads();");
+      for (int i = 0; i < TM; ++i) {
+        cb.line("s1_" + S(i) + " = rb[" + S(i * WK * 32) + " + r16 * 2];");
+        cb.line("s2_" + S(i) + " = rb[" + S(i * WK * 32) + " + r16 * 2 + 1];");
+        for (int w = 1; w < WK; ++w) {
+          cb.line("s1_" + S(i) + " += rb[" + S(i * WK * 32 + w * 32) + " + r16 * 2];");
+          cb.line("s2_" + S(i) + " += rb[" + S(i * WK * 32 + w * 32) + " + r16 * 2 + 1];");
+        }
+      }
+    }
+    std::snprintf(num, sizeof num, "%.9g", 1.0 / static_cast<double>(g.K));
+    const std::string inv_k = std::string(num) + "f";
+    std::snprintf(num, sizeof num, "%.9g", ln.eps);
+    std::string eps_lit = num;
+    if (eps_lit.find_first_of(".e") == std::string::npos) eps_lit += ".0";
+    eps_lit += "f";
+    for (int i = 0; i < TM; ++i) {
+      cb.line("const float mean" + S(i) + " = s1_" + S(i) + " * " + inv_k + ";");
+      cb.line("const float rs" + S(i) + " = rsqrtf(fmaxf(s2_" + S(i) + " * " + inv_k + " - mean" + S(i) + " * mean" + S(i) + ", 0.f) + " + eps_lit + ");");
+      cb.line("const float nmr" + S(i) + " = -mean" + S(i) + " * rs" + S(i) + ";   // (x - mean) * r as one fused multiply-add");
+      for (int s = 0; s < CH; ++s) {
+        std::string arr = em.fresh("hn");
+        cb.line("_Float16 " + arr + "[8];");
+        cb.line("#pragma unroll");
+        cb.open("for (int e = 0; e < 8; ++e)");
+        cb.line(arr + "[e] = (_Float16)fmaf(fmaf((float)a[" + S(s) + "][" + S(i) + "][e], rs" + S(i) + ", nmr" + S(i) + "), (float)gam" + S(s) + "[e], (float)bet" + S(s) + "[e]);");
+        cb.close();
+        cb.line("a[" + S(s) + "][" + S(i) + "] = half8_t{" + arr + "[0], " + arr + "[1], " + arr + "[2], " + arr + "[3], " + arr + "[4], " + arr + "[5], " + arr + "[6], " + arr + "[7]};");
+        if (stores) {
+          LinExpr off = physical_offset(prog, H, primary_index(i, s, 0), &vars);
+          cb.line("if (store && mv" + S(i) + ") mononn_dev::stN<_Float16, 8>(" + ptrs.output(H) + " + " + off.str(vars) + ", " + arr + ");");
+        }
+      }
+    }
+    finish_struct(cb.text(), smem_ln);
+    return out;
+  }
   auto reduces = em.collect_reduces();
   std::vector<std::vector<std::string>> reduce_accs_;   // [reduce][row fragment]
   int smem = 0;

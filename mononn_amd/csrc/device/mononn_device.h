@@ -611,10 +611,6 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     for (int j = 0; j < TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   load_chunk(0, 0);
-  if constexpr (Pro::enabled) {
-    static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
-    pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, smem);
-  }
   // The epilogue's operands (bias, residual) of the fragments this wave finalises are requested now and used
   // after the main loop, so that their latency overlaps it.  Slot q belongs to fragment q * WK + wk; the
   // addresses are clamped instead of guarded so that the loads stay in this basic block (a load under a
@@ -635,6 +631,12 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       n = n < N ? n : (N >= 4 ? N - 4 : 0);
     }
     epi.preload(batch, m, n, pre[q]);
+  }
+  // (a row program in front of the MFMAs runs after those requests: it waits for the left operand and, with the
+  // k range split over waves, at a workgroup barrier)
+  if constexpr (Pro::enabled) {
+    static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
+    pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, smem);
   }
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {

@@ -52,6 +52,8 @@ using std::max;
 using std::min;
 inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
 inline unsigned long long wall_clock64() { return 1; }
+typedef _Float16 host_half2 __attribute__((ext_vector_type(2)));
+inline float __builtin_amdgcn_fdot2(host_half2 a, host_half2 b, float c, bool) { return (float)a[0] * (float)b[0] + (float)a[1] * (float)b[1] + c; }
 typedef _Float16 host_half8 __attribute__((ext_vector_type(8)));
 typedef float host_float4 __attribute__((ext_vector_type(4)));
 typedef float host_float16 __attribute__((ext_vector_type(16)));

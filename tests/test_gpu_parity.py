@@ -117,6 +117,27 @@ def test_f32_gemm_with_fused_epilogue(gpu_device):
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("with_beta", [True, False])
+def test_row_program_in_front_of_a_gemm(gpu_device, with_beta):
+    # LayerNorm inside the GEMM in its hand-laid-out form (with_beta) and a row program that is not LayerNorm in the
+    # generic form, both against the oracle
+    import json
+    from test_host_compiler import norm_gemm_module
+    text, constants = norm_gemm_module(with_beta)
+    spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+    spec["mononn_hip"]["gemm_prologue_fusion"] = True
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"] = {}, {}
+    rng = np.random.default_rng(31)
+    x = rng.normal(0.7, 2.0, (64, 256)).astype(np.float16)          # a mean well away from zero
+    consts = {name: (rng.normal(1.0, 0.2, meta["dims"]) if len(meta["dims"]) == 1 else rng.normal(0, 0.05, meta["dims"])).astype(np.float16)
+              for name, meta in constants.items()}
+    want = hlo_interp.evaluate(text, [x], consts, "fp32")[0]
+    (got,), m = run_module(text, [x], consts, [{"dtype": "f16", "dims": [64, 128]}], json.dumps(spec))
+    assert ("__builtin_amdgcn_fdot2" in m.get_source("main.hip")) == with_beta
+    m.close()
+    check_close(got, want, atol=2e-2)
+
+
 def test_bert_layer_parity(gpu_device):
     fx = models.bert_layer()
     consts = fx.make_constants(1234, "random")

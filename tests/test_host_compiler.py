@@ -558,3 +558,52 @@ def test_layernorm_in_gemm_over_split_k_partial_sums():
     src = fused.get_source()
     # the partial sums of the split GEMMs are stored in fragment order for the row program in front of the next GEMM
     assert re.search(r"stN<float, 4>\(out \+ \(long\)ksplit \* \d+ \+ \(m % 16\) \* 8", src)
+
+
+def norm_gemm_module(with_beta):
+    """Mean / variance normalisation with a scale (and, with_beta, a shift: LayerNorm) feeding a weight GEMM."""
+    mb = HloModuleBuilder("cluster_3__norm_gemm.1")
+    e = mb.entry
+    M, K, N = 64, 256, 128
+    x = e.parameter("f16", (M, K), "x")
+    gamma = e.elided_constant("f16", (K,), "ln/gamma")
+    beta = e.elided_constant("f16", (K,), "ln/beta")
+    add = mb.reducer("add", "f32")
+
+    def sum_body(f, px):
+        return f.reduce(f.convert(px, "f32"), f.scalar("f32", 0.0), 1, add)
+    s = e.fusion("kInput", [x], sum_body)
+
+    def centred(f, px, ps):
+        return f.sub(f.convert(px, "f32"), f.broadcast(f.mul(ps, f.splat("f32", 1.0 / K, (M,))), (M, K), [0]))
+
+    def var_body(f, px, ps):
+        d = centred(f, px, ps)
+        return f.reduce(f.mul(d, d), f.scalar("f32", 0.0), 1, add)
+    v = e.fusion("kInput", [x, s], var_body)
+
+    def norm_body(f, px, ps, pv, pg, pb):
+        r = f.rsqrt(f.add(f.mul(pv, f.splat("f32", 1.0 / K, (M,))), f.splat("f32", 1e-5, (M,))))
+        y = f.mul(f.broadcast(f.convert(pg, "f32"), (M, K), [1]), f.mul(f.broadcast(r, (M, K), [0]), centred(f, px, ps)))   # operands the other way round
+        if with_beta:
+            y = f.add(f.broadcast(f.convert(pb, "f32"), (M, K), [1]), y)
+        return f.convert(y, "f16")
+    h = e.fusion("kLoop", [x, s, v, gamma, beta], norm_body)
+    w = e.elided_constant("f16", (K, N), "w/kernel")
+    e.set_tuple_root([e.gemm(h, w, 1, 0)])
+    return mb.text(), mb.constants
+
+
+def test_layer_norm_in_front_of_a_gemm_is_recognised_and_other_row_programs_are_not():
+    # with the prologue fusion on, a row program that is exactly LayerNorm takes the hand-laid-out form (sums by
+    # v_dot2_f32_f16, one exchange); anything else - here the same normalisation without the shift - is generated
+    # element by element from the HLO as before
+    for with_beta in (True, False):
+        text, _ = norm_gemm_module(with_beta)
+        spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+        spec["mononn_hip"]["gemm_prologue_fusion"] = True
+        spec["gemm_spec_list"], spec["cluster_reduce_spec"] = {}, {}
+        m = MonoNNModule.compile(text, json.dumps(spec), build=False)
+        src = m.get_source("main.hip")
+        assert m.launch_dims()["barriers"] == 0 and "_pro {" in src          # one stage: the row program runs inside the GEMM
+        assert ("__builtin_amdgcn_fdot2" in src) == with_beta
