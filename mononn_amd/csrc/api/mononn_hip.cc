@@ -189,7 +189,7 @@ int mononn_module_constant_info(const mononn_module* m, int index, const char** 
     if (hlo_name) *hlo_name = cs[index].hlo_name.c_str();
     if (role) *role = cs[index].role.c_str();
     if (bytes) *bytes = cs[index].bytes;
-    if (needs_payload) *needs_payload = cs[index].literal.empty() ? 1 : 0;
+    if (needs_payload) *needs_payload = cs[index].literal.empty() && !cs[index].derived() ? 1 : 0;   // derived: built by the module from other payloads
   });
 }
 

@@ -759,9 +759,12 @@ struct Epilogue {
 // along_m: the MFMA is issued with the operands swapped, so that a lane holds four consecutive rows m of one
 // column n; outputs that are stored with m as the fast dimension (a transposed result) then take one packed
 // store instead of four scattered ones.
+// fold / fold_bm: the left operand's LayerNorm is folded (graph::LayerNormFold); the accumulator then holds
+// x . (gamma o W) and becomes the GEMM value as r[m] * (acc - mean[m] * colsum_gamma[n]) + colsum_beta[n], with mean and
+// r of the workgroup's fold_bm rows read from LDS (`ln_stats`, written by the statistics functor in front of the MFMAs).
 Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<const Instr*>& cluster_members,
                         const std::vector<const Instr*>& outputs, const graph::GemmDesc& g, bool mfma, PointerTable& ptrs,
-                        size_t first_epi, bool along_m = false) {
+                        size_t first_epi, bool along_m = false, const graph::LayerNormFold* fold = nullptr, int fold_bm = 0) {
   if (g.split_k > 1) {
     // fp32 partial sums [split][batch][M][N]; the consumers add them up and apply the rounding
     MONONN_CHECK(mfma && g.N % 4 == 0 && cluster_members.empty() && outputs.size() == 1 && outputs[0] == gi && !g.has_addend, kSpecError)
@@ -802,6 +805,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   // a copy without an alignment promise, wherever the whole run lies inside the row (decided further down).
   bool ragged4 = false;
   std::string ragged4_offset;
+  std::vector<std::pair<std::string, std::string>> fold_loads;   // (expression, type) of the folded LayerNorm's column sums
   CodeBuffer cb;   // epilogue body
   VarTable vars;
   Emitter em(prog, cluster_members, cb, vars, ptrs);
@@ -905,6 +909,16 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   {
     Index gidx = gemm_index(true);
     std::string accv = vec4 ? "acc[r]" : "acc";
+    if (fold) {
+      MONONN_CHECK(mfma && vec4 && alpha == 1.0 && !g.has_addend && fold_bm > 0, kInternal) << gi->hlo_name << ": folded LayerNorm outside its preconditions";
+      const std::string pc1 = ptrs.input(fold->colsum_gamma), pc2 = ptrs.input(fold->colsum_beta);
+      const std::string row = along_m ? "((m0 + r) % " + S(fold_bm) + ")" : "(m % " + S(fold_bm) + ")";
+      const std::string col = along_m ? "nn" : "n4 * 4 + r";
+      // the two column sums are requested with the other operands of the epilogue, ahead of the main loop
+      fold_loads = {{pc1 + "[" + col + "]", "float"}, {pc2 + "[" + col + "]", "float"}};
+      cb.line("const float ln_acc = ln_stats[" + row + " * 2 + 1] * (" + accv + " - ln_stats[" + row + " * 2] * " + fold_loads[0].first + ") + " + fold_loads[1].first + ";");
+      accv = "ln_acc";
+    }
     std::string expr = alpha == 1.0 ? accv : "(" + accv + " * " + alpha_lit + ")";
     if (g.has_addend) {
       std::ostringstream beta_s;
@@ -999,6 +1013,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     auto& e = ptrs.entries[i];
     pre += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
   }
+  if (fold) pre += "  const float* ln_stats = nullptr;   // LDS: (mean, rsqrt(var + eps)) of the workgroup's rows\n";
   // Operands of the epilogue (bias, residual) whose address depends on (bidx, m, n) only are loaded into
   // registers ahead of the GEMM main loop, so their latency overlaps it; the body then reads the registers.
   std::vector<std::pair<std::string, std::string>> preloads;
@@ -1011,6 +1026,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
         for (auto& q : preloads) seen = seen || q.first == l.first;
         if (!seen) preloads.push_back(l);
       }
+      for (auto& l : fold_loads) preloads.push_back(l);
       for (size_t i = 0; i < preloads.size(); ++i) pre += "    " + preloads[i].second + " v" + S(i) + "[4];\n";
     }
     pre += "  };\n";
@@ -1299,8 +1315,25 @@ bool match_layer_norm(const Program& prog, const std::vector<const Instr*>& row_
   return out->gamma->shape.dtype == DType::kF16 && out->beta->shape.dtype == DType::kF16;
 }
 
+}  // namespace
+
+bool match_prologue_layer_norm(const Program& prog, const std::vector<const Instr*>& row_members, const Instr* H, int64_t M, int64_t K,
+                               const Instr** gamma, const Instr** beta, double* eps) {
+  const Instr* primary = prologue_primary(prog, row_members, M, K);
+  if (!primary) return false;
+  LayerNormMatch ln;
+  if (!match_layer_norm(prog, row_members, primary, H, K, &ln)) return false;
+  *gamma = ln.gamma;
+  *beta = ln.beta;
+  *eps = ln.eps;
+  return true;
+}
+
+namespace {
+
 Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& row_members, const Instr* gi, const graph::GemmDesc& g,
-                        const GemmTuning& t, const LaunchShape& ls, bool stores, PointerTable& ptrs) {
+                        const GemmTuning& t, const LaunchShape& ls, bool stores, PointerTable& ptrs, const graph::LayerNormFold* fold = nullptr,
+                        int fold_stats_offset = 0, int fold_exchange_offset = 0) {
   (void)ls;
   RowInfo info = analyze_rows(row_members);
   MONONN_CHECK(info.row_program && info.rows == g.M && info.row_len == g.K && g.batch == 1, kUnsupported)
@@ -1350,12 +1383,12 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
   auto finish_struct = [&](const std::string& body, int smem_bytes) {
     out.smem = smem_bytes;
     for (auto& kv : em.literal_tables()) out.globals.push_back(kv.second);
-    std::string st = "struct @NAME@_pro {\n  static constexpr bool enabled = true;\n";
+    std::string st = std::string("struct @NAME@_pro {\n  static constexpr bool enabled = true;\n  static constexpr bool after_mfma = ") + (fold ? "true" : "false") + ";\n";
     for (size_t i = first; i < ptrs.entries.size(); ++i) {
       auto& e = ptrs.entries[i];
       st += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
     }
-    st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, char* smem) const {\n";
+    st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, int store_slot, char* smem) const {\n";
     std::istringstream is(body);
     std::string l;
     while (std::getline(is, l)) st += "  " + l + "\n";
@@ -1371,6 +1404,101 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
   // through LDS for both sums, then ((x - mean) * r) * gamma + beta as two fused multiply-adds per element.  The variance is
   // E[x^2] - mean^2 in fp32 (one exchange instead of two); the generic form computes the centred sum of squares.
   LayerNormMatch ln;
+  if (fold) {
+    // Folded LayerNorm: the fragments go into the MFMAs as they are.  This functor only computes the statistics of the
+    // wave's rows (nothing after it waits for them before the epilogue, so they overlap the MFMAs), leaves them in LDS
+    // for the epilogue, and - in the one GEMM that also owes the normalised rows to later stages - stores them, each
+    // column tile taking the k steps s with s % tiles == its own number so that no workgroup carries all of it.
+    char num[64];
+    const int64_t tiles_n = (g.N + t.bn - 1) / t.bn;
+    const int64_t ksteps = g.K / 32;
+    const int64_t owners = std::min<int64_t>(tiles_n, ksteps);
+    std::string pg, pb;
+    if (stores) {
+      pg = ptrs.input(fold->gamma);
+      pb = ptrs.input(fold->beta);
+      for (int s = 0; s < CH; ++s) {
+        const std::string col = "(wk * 32 + g * 8 + " + S(static_cast<int64_t>(s) * WK * 32) + ")";
+        cb.line("const bool own" + S(s) + " = store_slot >= 0 && (" + S(s * WK) + " + wk) % " + S(owners) + " == store_slot;");
+        cb.line("half8_t gam" + S(s) + " = {}, bet" + S(s) + " = {};");
+        cb.open("if (own" + S(s) + ")");
+        cb.line("gam" + S(s) + " = *reinterpret_cast<const half8_t*>(" + pg + " + " + col + ");");
+        cb.line("bet" + S(s) + " = *reinterpret_cast<const half8_t*>(" + pb + " + " + col + ");");
+        cb.close();
+      }
+    }
+    for (int i = 0; i < TM; ++i) {
+      cb.line("float s1_" + S(i) + " = 0.f, s2_" + S(i) + " = 0.f;");
+      for (int s = 0; s < CH; ++s)
+        for (int p2 = 0; p2 < 4; ++p2) {
+          const std::string h = "__builtin_shufflevector(a[" + S(s) + "][" + S(i) + "], a[" + S(s) + "][" + S(i) + "], " + S(2 * p2) + ", " + S(2 * p2 + 1) + ")";
+          cb.line("s1_" + S(i) + " = __builtin_amdgcn_fdot2(" + h + ", half2_t{(_Float16)1, (_Float16)1}, s1_" + S(i) + ", false);");
+          cb.line("s2_" + S(i) + " = __builtin_amdgcn_fdot2(" + h + ", " + h + ", s2_" + S(i) + ", false);");
+        }
+      for (int off : {16, 32}) {
+        cb.line("s1_" + S(i) + " += __shfl_xor(s1_" + S(i) + ", " + S(off) + ", 64);");
+        cb.line("s2_" + S(i) + " += __shfl_xor(s2_" + S(i) + ", " + S(off) + ", 64);");
+      }
+    }
+    int smem_ln = 0;
+    if (WK > 1) {
+      cb.line("float* rb = reinterpret_cast<float*>(smem + " + S(fold_exchange_offset) + ") + mn_wave * " + S(TM * WK * 32) + ";");
+      smem_ln = fold_exchange_offset + t.wm * t.wn * TM * WK * 32 * 4;
+      cb.open("if (g == 0)");
+      for (int i = 0; i < TM; ++i) {
+        cb.line("rb[" + S(i * WK * 32) + " + wk * 32 + r16 * 2] = s1_" + S(i) + ";");
+        cb.line("rb[" + S(i * WK * 32) + " + wk * 32 + r16 * 2 + 1] = s2_" + S(i) + ";");
+      }
+      cb.close();
+      cb.line("__syncthreads();");
+      for (int i = 0; i < TM; ++i) {
+        cb.line("s1_" + S(i) + " = rb[" + S(i * WK * 32) + " + r16 * 2];");
+        cb.line("s2_" + S(i) + " = rb[" + S(i * WK * 32) + " + r16 * 2 + 1];");
+        for (int w = 1; w < WK; ++w) {
+          cb.line("s1_" + S(i) + " += rb[" + S(i * WK * 32 + w * 32) + " + r16 * 2];");
+          cb.line("s2_" + S(i) + " += rb[" + S(i * WK * 32 + w * 32) + " + r16 * 2 + 1];");
+        }
+      }
+    } else {
+      cb.line("__syncthreads();   // the previous unit's epilogue may still be reading the statistics");
+    }
+    MONONN_CHECK(fold_stats_offset >= smem_ln, kInternal) << "statistics of a folded LayerNorm overlap the exchange buffer";
+    std::snprintf(num, sizeof num, "%.9g", 1.0 / static_cast<double>(g.K));
+    const std::string inv_k = std::string(num) + "f";
+    std::snprintf(num, sizeof num, "%.9g", fold->eps);
+    std::string eps_lit = num;
+    if (eps_lit.find_first_of(".e") == std::string::npos) eps_lit += ".0";
+    eps_lit += "f";
+    cb.line("float* ln_stats = reinterpret_cast<float*>(smem + " + S(fold_stats_offset) + ");");
+    for (int i = 0; i < TM; ++i) {
+      cb.line("const float mean" + S(i) + " = s1_" + S(i) + " * " + inv_k + ";");
+      cb.line("const float rs" + S(i) + " = rsqrtf(fmaxf(s2_" + S(i) + " * " + inv_k + " - mean" + S(i) + " * mean" + S(i) + ", 0.f) + " + eps_lit + ");");
+      cb.open("if (g == 0 && wk == 0)");
+      cb.line("ln_stats[(m_base % " + S(t.bm) + " + " + S(i * 16) + " + r16) * 2] = mean" + S(i) + ";");
+      cb.line("ln_stats[(m_base % " + S(t.bm) + " + " + S(i * 16) + " + r16) * 2 + 1] = rs" + S(i) + ";");
+      cb.close();
+    }
+    cb.line("__syncthreads();");
+    if (stores) {
+      for (int i = 0; i < TM; ++i) {
+        cb.line("const float nmr" + S(i) + " = -mean" + S(i) + " * rs" + S(i) + ";");
+        for (int s = 0; s < CH; ++s) {
+          LinExpr off = physical_offset(prog, H, primary_index(i, s, 0), &vars);
+          cb.open("if (own" + S(s) + " && mv" + S(i) + ")");
+          std::string arr = em.fresh("hn");
+          cb.line("_Float16 " + arr + "[8];");
+          cb.line("#pragma unroll");
+          cb.open("for (int e = 0; e < 8; ++e)");
+          cb.line(arr + "[e] = (_Float16)fmaf(fmaf((float)a[" + S(s) + "][" + S(i) + "][e], rs" + S(i) + ", nmr" + S(i) + "), (float)gam" + S(s) + "[e], (float)bet" + S(s) + "[e]);");
+          cb.close();
+          cb.line("mononn_dev::stN<_Float16, 8>(" + ptrs.output(H) + " + " + off.str(vars) + ", " + arr + ");");
+          cb.close();
+        }
+      }
+    }
+    finish_struct(cb.text(), std::max(smem_ln, fold_stats_offset + t.bm * 8));
+    return out;
+  }
   if (match_layer_norm(prog, row_members, primary, H, g.K, &ln)) {
     const std::string pg = ptrs.input(ln.gamma), pb = ptrs.input(ln.beta);
     char num[64];
@@ -1510,12 +1638,12 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
   em.unbind(primary);
   out.smem = smem;
   for (auto& kv : em.literal_tables()) out.globals.push_back(kv.second);
-  std::string st = "struct @NAME@_pro {\n  static constexpr bool enabled = true;\n";
+  std::string st = "struct @NAME@_pro {\n  static constexpr bool enabled = true;\n  static constexpr bool after_mfma = false;\n";
   for (size_t i = first; i < ptrs.entries.size(); ++i) {
     auto& e = ptrs.entries[i];
     st += std::string("  ") + (e.is_output ? "" : "const ") + hlo::dtype_ctype(e.dtype) + "* " + e.name + ";\n";
   }
-  st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, char* smem) const {\n";
+  st += "  __device__ __forceinline__ void operator()(half8_t (&a)[" + S(CH) + "][" + S(TM) + "], int m_base, int wk, int mn_wave, bool store, int store_slot, char* smem) const {\n";
   {
     // every operand of the row program is requested before the first of them is used: one trip to memory
     std::istringstream is(hoist_row_loads(cb.text(), true));
@@ -1533,8 +1661,20 @@ Prologue build_prologue(const Program& prog, const std::vector<const Instr*>& ro
 
 NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& members, const std::vector<const Instr*>& outputs,
                       const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t,
-                      const std::vector<const Instr*>& prologue = {}, bool prologue_stores = false) {
+                      const std::vector<const Instr*>& prologue = {}, bool prologue_stores = false, const graph::LayerNormFold* fold = nullptr) {
   const Instr* gi = members[0];
+  if (fold && !fold->on()) fold = nullptr;
+  // LDS of a folded LayerNorm: the statistics of the workgroup's rows live behind the slabs of the k-slice reduction
+  // and behind the exchange of the sums, which itself sits behind the slabs: a wave that is first into the next unit
+  // writes its sums while slower waves still read the slabs of this one
+  int fold_stats_offset = 0, fold_exchange_offset = 0;
+  if (fold) {
+    const int tm16 = t.bm / t.wm / 16, tn16 = t.bn / t.wn / 16;
+    const int red = t.wk > 1 ? ls.waves() * tm16 * tn16 * 64 * 16 : 0;
+    const int rb = t.wk > 1 ? t.wm * t.wn * tm16 * t.wk * 32 * 4 : 0;
+    fold_exchange_offset = (red + 15) / 16 * 16;
+    fold_stats_offset = (fold_exchange_offset + rb + 15) / 16 * 16;
+  }
   const bool mfma = gemm_uses_mfma(g);
   const bool has_pro = !prologue.empty();
   MONONN_CHECK(!has_pro || mfma, kUnsupported) << gi->hlo_name << ": a row-program prologue needs the MFMA path";
@@ -1548,10 +1688,10 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   if (has_pro) {
     // find the primary input first (the pointer order must start with the operand the GEMM loads)
     PointerTable probe_ptrs;
-    Prologue probe = build_prologue(prog, prologue, gi, g, t, ls, false, probe_ptrs);
+    Prologue probe = build_prologue(prog, prologue, gi, g, t, ls, false, probe_ptrs, fold, fold_stats_offset, fold_exchange_offset);
     pa = ptrs.input(probe.primary);
     pb = ptrs.input(prog.storage_root(gi->operands[1]));
-    pro = build_prologue(prog, prologue, gi, g, t, ls, prologue_stores, ptrs);
+    pro = build_prologue(prog, prologue, gi, g, t, ls, prologue_stores, ptrs, fold, fold_stats_offset, fold_exchange_offset);
     auto pouts = external_outputs(prog, prologue);
     epi_outputs.clear();
     for (auto* o : outputs)
@@ -1566,12 +1706,12 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   {
     // both orientations of the accumulator tile are generated; rows-per-lane wins when it packs more stores
     PointerTable p_n = ptrs;
-    epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, p_n, first_epi);
+    epi = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, p_n, first_epi, false, fold, t.bm);
     bool use_m = false;
     if (mfma && g.split_k <= 1 && !g.is_conv && g.M % 4 == 0) {
       try {
         PointerTable p_m = ptrs;
-        Epilogue e_m = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, p_m, first_epi, true);
+        Epilogue e_m = build_epilogue(prog, gi, cluster_members, epi_outputs, g, mfma, p_m, first_epi, true, fold, t.bm);
         if (e_m.vector_stores > epi.vector_stores) {
           epi = std::move(e_m);
           ptrs = std::move(p_m);
@@ -1588,6 +1728,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   bool preload = false;
   int preload_regs = 0;
   if (g.split_k <= 1) fb.line(epi.init_line);
+  if (fold) fb.line("epi.ln_stats = reinterpret_cast<const float*>(smem + " + S(fold_stats_offset) + ");");
   if (has_pro) fb.line(pro.init_line);
   int64_t units = 0;
   int smem = 0;
@@ -2154,7 +2295,7 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
 }  // namespace
 
 NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchShape& ls, const GemmTuning& t) {
-  return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores);
+  return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores, &node.ln_fold);
 }
 
 NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves, bool preload_weights) {

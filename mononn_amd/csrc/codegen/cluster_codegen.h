@@ -93,6 +93,10 @@ bool can_merge_clusters(const graph::Program& prog, const std::vector<const hlo:
 bool can_fuse_epilogue(const graph::Program& prog, const std::vector<const hlo::Instr*>& gemm_members,
                        const std::vector<const hlo::Instr*>& cluster_members);
 
+// true when the row program `row_members`, whose product `H` is the [M,K] left operand of a GEMM, is exactly
+// LayerNorm over the last dimension of its primary input: (x - mean) * rsqrt(var + eps) * gamma + beta
+bool match_prologue_layer_norm(const graph::Program& prog, const std::vector<const hlo::Instr*>& row_members, const hlo::Instr* H, int64_t M,
+                               int64_t K, const hlo::Instr** gamma, const hlo::Instr** beta, double* eps);
 bool can_fuse_prologue(const graph::Program& prog, const std::vector<const hlo::Instr*>& row_members,
                        const std::vector<const hlo::Instr*>& gemm_members, const graph::GemmDesc& g);
 

@@ -27,6 +27,7 @@ graph::BuildOptions build_options_from(const spec::GraphSpecification& s) {
   o.assign_operand_layouts = s.hip.assign_operand_layouts;
   o.fuse_attention = s.hip.fuse_attention;
   o.fuse_gemm_prologue = s.hip.gemm_prologue_fusion;
+  o.fold_layer_norm = s.hip.layer_norm_folding;
   o.pack_left_operands = s.hip.pack_left_operands;
   o.fuse_attention_out_proj = s.hip.attention_out_proj_fusion;
   o.reuse_temp_slots = s.hip.barrier != "flags_coherent";   // the fence-free barrier needs write-once addresses
@@ -109,6 +110,14 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     ci.device_bytes = ci.bytes;
     if (ci.transform == graph::ConstantTransform::kPackMfmaB) ci.device_bytes = (ci.dims[1] + 15) / 16 * 16 * ci.dims[0] * hlo::dtype_bytes(ci.dtype);
     if (!c->literal_elided) ci.literal = c->literal;
+    auto rs = prog.constant_row_scale.find(c);
+    if (rs != prog.constant_row_scale.end()) ci.row_scale_by = rs->second->name;
+    auto dc = prog.derived_constants.find(c);
+    if (dc != prog.derived_constants.end()) {
+      ci.sums_weight = dc->second.weight->name;
+      ci.sums_vector = dc->second.vector->name;
+      ci.role = "derived: column sums of " + dc->second.weight->hlo_name + " weighted by " + dc->second.vector->hlo_name;
+    }
     auto md = c->attrs.find("metadata");
     if (md != c->attrs.end()) {
       size_t p = md->second.find("op_name=\"");

@@ -31,6 +31,12 @@ struct ConstantInfo {
   std::vector<int64_t> dims;
   graph::ConstantTransform transform = graph::ConstantTransform::kNone;
   std::string literal;     // payload text when the HLO carries it (not elided)
+  // folded LayerNorms (graph::LayerNormFold): a weight matrix whose row k is multiplied by element k of the named
+  // [K] constant before it is laid out for the device ...
+  std::string row_scale_by;
+  // ... and a constant the host never supplies: f32[N] = sum_k vector[k] * weight[k, n] of two named constants
+  std::string sums_weight, sums_vector;
+  bool derived() const { return !sums_weight.empty(); }
 };
 
 struct NodeReport {

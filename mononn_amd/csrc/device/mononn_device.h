@@ -435,6 +435,7 @@ __device__ __forceinline__ half8_t load_key_run(const half_t* row, int k, int n)
 // rows to memory for later consumers.
 struct NoPrologue {
   static constexpr bool enabled = false;
+  static constexpr bool after_mfma = false;
 };
 
 // Where row m, column k of the left operand lives.  The default is a row-major [M, lda] matrix; an implicit-GEMM
@@ -634,9 +635,9 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   }
   // (a row program in front of the MFMAs runs after those requests: it waits for the left operand and, with the
   // k range split over waves, at a workgroup barrier)
-  if constexpr (Pro::enabled) {
+  if constexpr (Pro::enabled && !Pro::after_mfma) {
     static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
-    pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, smem);
+    pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, wn == 0 ? tile_n : -1, smem);
   }
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
@@ -656,6 +657,12 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
     }
   }
 
+  // A functor that only derives something from the left operand's fragments for the epilogue (row statistics of a
+  // folded LayerNorm) runs here, behind the issued MFMAs: its vector-ALU work passes while the matrix pipe drains.
+  if constexpr (Pro::enabled && Pro::after_mfma) {
+    static_assert(NCHUNK == 1, "a GEMM prologue needs the whole k range of a wave in registers");
+    pro(a[0], m_base, wk, wave / WK, tile_n == 0 && wn == 0, wn == 0 ? tile_n : -1, smem);
+  }
   if (WK > 1) {
     // [wk][wm*wn][frag][lane] float4 : each wave writes its own slab, then every wave finalises the
     // fragments f with f % WK == wk from all WK slabs.

@@ -294,8 +294,11 @@ struct Builder {
       // a row program that adds up the partial sums of a split-K GEMM stays a stage of its own
       bool reads_split = false;
       for (auto* in : external_inputs(r.members)) {
+        // partial sums of a split GEMM reach the row program through the element emitter, fused or not; with
+        // LayerNorm folding on, a row program that adds them up stays a stage (the fold needs the finished rows, and
+        // the split is worth more than the stage: every column tile would re-read all partial sums)
         auto sk = opt.gemm_split_k.find(in->name);
-        (void)sk;   // partial sums of a split GEMM reach the row program through the element emitter, fused or not
+        if (opt.fold_layer_norm && sk != opt.gemm_split_k.end() && sk->second > 1) reads_split = true;
         reads_split = reads_split || absorbed.count(in->name);
       }
       if (reads_split) continue;
@@ -684,6 +687,40 @@ struct Builder {
     }
   }
 
+  // LayerNorm prologues of GEMMs with constant, packed weights that nothing else reads: folded (program.h).
+  void fold_layer_norms() {
+    if (!opt.fold_layer_norm || !enabled("LayerNormFoldingPass")) return;
+    for (auto& n : p.nodes) {
+      if (n.kind != NodeKind::kGemm || n.prologue.empty() || !n.gemm.b_packed || n.gemm.batch != 1 || n.gemm.alpha != 1.0 || n.gemm.has_addend) continue;
+      const Instr* g = n.members[0];
+      const Instr* w = p.storage_root(g->operands[1]);
+      if (w->opcode != "constant" || w->shape.dtype != hlo::DType::kF16 || w->shape.dims != std::vector<int64_t>({n.gemm.K, n.gemm.N})) continue;
+      if (w->users.size() != 1 || p.constant_row_scale.count(w)) continue;
+      LayerNormFold f;
+      if (!codegen::match_prologue_layer_norm(p, n.prologue, p.storage_root(g->operands[0]), n.gemm.M, n.gemm.K, &f.gamma, &f.beta, &f.eps)) continue;
+      auto column_sums = [&](const char* suffix, const Instr* vec) {
+        auto c = std::make_unique<hlo::Instr>();
+        c->name = w->name + suffix;
+        c->hlo_name = w->hlo_name + suffix;
+        c->opcode = "constant";
+        c->shape.dtype = hlo::DType::kF32;
+        c->shape.dims = {n.gemm.N};
+        c->shape.minor_to_major = {0};
+        c->literal = "{...}";
+        c->literal_elided = true;
+        c->parent = const_cast<hlo::Computation*>(w->parent);
+        const Instr* raw = c.get();
+        p.derived_constants[raw] = {w, vec};
+        p.synthetic.push_back(std::move(c));
+        return raw;
+      };
+      f.colsum_gamma = column_sums("_ln_gamma_sums", f.gamma);
+      f.colsum_beta = column_sums("_ln_beta_sums", f.beta);
+      p.constant_row_scale[w] = f.gamma;
+      n.ln_fold = f;
+    }
+  }
+
   void apply_split_k() {
     // a projection absorbed by an attention node leaves it as one partial sum per head
     for (auto& n : p.nodes)
@@ -734,6 +771,14 @@ struct Builder {
       b.bytes = c->shape.byte_size();
       p.constants.push_back(c);
       p.buffers[c] = b;
+    }
+    for (auto& up : p.synthetic) {
+      Buffer b;
+      b.kind = Buffer::kConstant;
+      b.index = static_cast<int>(p.constants.size());
+      b.bytes = up->shape.byte_size();
+      p.constants.push_back(up.get());
+      p.buffers[up.get()] = b;
     }
     std::map<const Instr*, int> live_index;
     for (size_t i = 0; i < p.live_outs.size(); ++i) live_index[p.live_outs[i]] = static_cast<int>(i);
@@ -825,6 +870,7 @@ std::unique_ptr<Program> build_program(std::unique_ptr<hlo::Module> module, cons
   if (opt.fuse_gemm_prologue && b.enabled("GemmPrologueFusionPass")) b.fuse_gemm_prologues();
   b.finalize();
   b.decide_constant_layouts();
+  b.fold_layer_norms();
   b.apply_split_k();
   b.assign_operand_layouts();
   for (auto& n : prog->nodes)

@@ -50,6 +50,19 @@ struct GemmDesc {
   std::string problem_hash() const;   // dtype+shape key, cf. mononn_module_tuner.cc:386-408
 };
 
+// LayerNorm in front of a constant-weight GEMM, folded: with h = (x - mean) * r * gamma + beta per row,
+//   h . W = r * (x . (gamma o W) - mean * (gamma^T W)) + beta^T W,
+// so the MFMAs run on the raw rows x against weights scaled by gamma once on the host, and the row statistics enter
+// in the epilogue as a rank-1 correction with two constant column-sum vectors.
+struct LayerNormFold {
+  const hlo::Instr* gamma = nullptr;
+  const hlo::Instr* beta = nullptr;
+  double eps = 0;
+  const hlo::Instr* colsum_gamma = nullptr;   // f32[N]: sum over k of gamma[k] * W[k, n], a constant built on the host
+  const hlo::Instr* colsum_beta = nullptr;    // f32[N]: sum over k of beta[k] * W[k, n]
+  bool on() const { return gamma != nullptr; }
+};
+
 struct Node {
   int id = -1;
   std::string name;
@@ -70,6 +83,7 @@ struct Node {
   // with prologue_stores also writes the row program's result for consumers in later stages
   std::vector<const hlo::Instr*> prologue;
   bool prologue_stores = false;
+  LayerNormFold ln_fold;          // the prologue is a LayerNorm and is folded into weights and epilogue
   // kAttention: second GEMM and where it sits in `members`
   GemmDesc gemm2;
   size_t gemm2_index = 0;
@@ -101,6 +115,16 @@ struct Program {
   std::vector<const hlo::Instr*> parameters;                       // entry parameters in order
   std::vector<const hlo::Instr*> constants;                        // non-scalar entry constants (device buffers)
   std::map<const hlo::Instr*, ConstantTransform> constant_transform;
+  // Constants of folded LayerNorms.  A weight matrix [K,N] whose rows are multiplied by a [K] vector before it is laid
+  // out for the device, and column-sum vectors f32[N] = sum_k vector[k] * weight[k,n] that exist only as module
+  // globals: the host builds them from the payloads of their sources (instructions owned by `synthetic`).
+  std::map<const hlo::Instr*, const hlo::Instr*> constant_row_scale;
+  struct ColumnSums {
+    const hlo::Instr* weight = nullptr;
+    const hlo::Instr* vector = nullptr;
+  };
+  std::map<const hlo::Instr*, ColumnSums> derived_constants;
+  std::vector<std::unique_ptr<hlo::Instr>> synthetic;
   // storage roots kept in a permuted physical order: physical dim i = logical dim perm[i]
   // (right-hand GEMM operands produced inside the kernel are stored with k minor-most)
   std::map<const hlo::Instr*, std::vector<int>> physical_perm;
@@ -136,6 +160,7 @@ struct BuildOptions {
   bool fuse_gemm_epilogue = true;       // element-wise consumers of a GEMM run in its epilogue
   bool transpose_constant_b = true;     // store constant [K,N] GEMM operands in MFMA fragment order
   bool fuse_gemm_prologue = false;      // row programs feeding a GEMM's left operand run inside that GEMM
+  bool fold_layer_norm = false;         // ... and when that row program is a LayerNorm and the weights are constant: folded
   bool fuse_attention = true;           // GEMM -> soft-max style row program -> GEMM in one stage
   bool assign_operand_layouts = true;   // store in-kernel right-hand GEMM operands k-contiguous
   bool pack_left_operands = true;       // store in-kernel left-hand GEMM operands in MFMA fragment order

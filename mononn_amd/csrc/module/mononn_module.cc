@@ -126,18 +126,113 @@ static const codegen::ConstantInfo* find_constant(const codegen::HipProgram& hp,
   return nullptr;
 }
 
+static std::vector<char> device_payload(const codegen::ConstantInfo& ci, const std::vector<char>& payload);
+static std::vector<char> literal_payload(const codegen::ConstantInfo& ci);
+
 void MonoNNModule::set_constant(const std::string& name, const void* host_data, size_t bytes) {
   MONONN_CHECK(program_ != nullptr, kInvalidArgument) << "set_constant called before generate_code";
   const codegen::ConstantInfo* ci = find_constant(hip_, name);
   MONONN_CHECK(ci != nullptr, kNotFound) << "the module has no constant named '" << name << "'";
   MONONN_CHECK(static_cast<int64_t>(bytes) == ci->bytes, kInvalidArgument)
       << "constant '" << name << "' needs " << ci->bytes << " bytes, got " << bytes;
+  MONONN_CHECK(!ci->derived(), kInvalidArgument) << "constant '" << name << "' is built by the module from " << ci->sums_weight << " and " << ci->sums_vector;
   std::vector<char> payload(static_cast<const char*>(host_data), static_cast<const char*>(host_data) + bytes);
-  if (dev_.loaded()) {
-    upload_constant(*ci, payload);
-  } else {
+  if (!dev_.loaded()) {
     host_constants_[ci->name] = std::move(payload);
+    return;
   }
+  if (!is_fold_source(ci->name)) {
+    upload_constant(*ci, payload);
+    return;
+  }
+  // a source of a folded LayerNorm supplied after load: everything built from it is built and sent again
+  fold_sources_[ci->name] = std::move(payload);
+  for (auto& c : hip_.constants)
+    if (c.name == ci->name || c.row_scale_by == ci->name || c.sums_weight == ci->name || c.sums_vector == ci->name) upload_resolved(c);
+}
+
+bool MonoNNModule::is_fold_source(const std::string& name) const {
+  for (auto& c : hip_.constants)
+    if (c.row_scale_by == name || c.sums_weight == name || c.sums_vector == name || (c.name == name && !c.row_scale_by.empty())) return true;
+  return false;
+}
+
+const std::vector<char>* MonoNNModule::raw_payload(const std::string& name, std::vector<char>* scratch) const {
+  auto f = fold_sources_.find(name);
+  if (f != fold_sources_.end()) return &f->second;
+  auto h = host_constants_.find(name);
+  if (h != host_constants_.end()) return &h->second;
+  for (auto& c : hip_.constants)
+    if (c.name == name && !c.literal.empty()) {
+      *scratch = literal_payload(c);
+      return scratch;
+    }
+  return nullptr;
+}
+
+static float half_bits_to_float(uint16_t b) {
+  _Float16 h;
+  std::memcpy(&h, &b, 2);
+  return static_cast<float>(h);
+}
+
+bool MonoNNModule::resolve_device_bytes(const codegen::ConstantInfo& ci, std::vector<char>* out) const {
+  std::vector<char> s0, s1;
+  if (ci.derived()) {
+    // f32[N]: sum over k of vector[k] * weight[k, n], accumulated in double (the weights as the host gave them,
+    // before any scaling)
+    const std::vector<char>* w = raw_payload(ci.sums_weight, &s0);
+    const std::vector<char>* v = raw_payload(ci.sums_vector, &s1);
+    if (!w || !v) return false;
+    const int64_t N = ci.dims[0], K = static_cast<int64_t>(v->size() / 2);
+    MONONN_CHECK(static_cast<int64_t>(w->size()) == K * N * 2, kInternal) << "sources of " << ci.name << " do not match";
+    const uint16_t* wp = reinterpret_cast<const uint16_t*>(w->data());
+    const uint16_t* vp = reinterpret_cast<const uint16_t*>(v->data());
+    std::vector<double> acc(static_cast<size_t>(N), 0.0);
+    for (int64_t k = 0; k < K; ++k) {
+      const double vk = half_bits_to_float(vp[k]);
+      for (int64_t n = 0; n < N; ++n) acc[n] += vk * half_bits_to_float(wp[k * N + n]);
+    }
+    out->assign(static_cast<size_t>(N) * 4, 0);
+    for (int64_t n = 0; n < N; ++n) {
+      const float f = static_cast<float>(acc[n]);
+      std::memcpy(out->data() + n * 4, &f, 4);
+    }
+    return true;
+  }
+  const std::vector<char>* raw = raw_payload(ci.name, &s0);
+  if (!raw) return false;
+  if (ci.row_scale_by.empty()) {
+    *out = device_payload(ci, *raw);
+    return true;
+  }
+  // weight[k, n] * vector[k], rounded to half once, then laid out like any other weight matrix
+  const std::vector<char>* v = raw_payload(ci.row_scale_by, &s1);
+  if (!v) return false;
+  const int64_t K = ci.dims[0], N = ci.dims[1];
+  MONONN_CHECK(static_cast<int64_t>(v->size()) == K * 2 && static_cast<int64_t>(raw->size()) == K * N * 2, kInternal) << "sources of " << ci.name << " do not match";
+  std::vector<char> scaled(raw->size());
+  const uint16_t* wp = reinterpret_cast<const uint16_t*>(raw->data());
+  const uint16_t* vp = reinterpret_cast<const uint16_t*>(v->data());
+  for (int64_t k = 0; k < K; ++k) {
+    const float vk = half_bits_to_float(vp[k]);
+    for (int64_t n = 0; n < N; ++n) {
+      const _Float16 h = static_cast<_Float16>(vk * half_bits_to_float(wp[k * N + n]));
+      std::memcpy(scaled.data() + (k * N + n) * 2, &h, 2);
+    }
+  }
+  *out = device_payload(ci, scaled);
+  return true;
+}
+
+void MonoNNModule::upload_resolved(const codegen::ConstantInfo& ci) {
+  std::vector<char> bytes;
+  if (!resolve_device_bytes(ci, &bytes)) return;
+  size_t n = 0;
+  void* dst = dev_.global(ci.symbol, &n);
+  MONONN_CHECK(n >= bytes.size(), kRuntimeError) << "global " << ci.symbol << " is smaller than its constant in device layout";
+  dev_.upload(dst, bytes.data(), bytes.size());
+  uploaded_[ci.name] = true;
 }
 
 // bytes of the module global for a payload given in the HLO's layout
@@ -176,7 +271,7 @@ void MonoNNModule::upload_constant(const codegen::ConstantInfo& ci, const std::v
 std::vector<std::string> MonoNNModule::missing_constants() const {
   std::vector<std::string> out;
   for (auto& c : hip_.constants)
-    if (c.literal.empty() && !uploaded_.count(c.name) && !host_constants_.count(c.name)) out.push_back(c.hlo_name);
+    if (!c.derived() && c.literal.empty() && !uploaded_.count(c.name) && !host_constants_.count(c.name) && !fold_sources_.count(c.name)) out.push_back(c.hlo_name);
   return out;
 }
 
@@ -254,7 +349,15 @@ void MonoNNModule::load(int device) {
   void* err = dev_.global("mononn_barrier_error", &err_bytes);
   dev_.zero(err, err_bytes);
   uploaded_.clear();
+  // the sources of folded LayerNorms stay on the host: scaled weights and column sums are built from them, now and
+  // whenever one of them is supplied again
+  for (auto& kv : host_constants_)
+    if (is_fold_source(kv.first)) fold_sources_[kv.first] = kv.second;
   for (auto& ci : hip_.constants) {
+    if (ci.derived() || !ci.row_scale_by.empty() || is_fold_source(ci.name)) {
+      upload_resolved(ci);
+      continue;
+    }
     if (!ci.literal.empty()) {
       upload_constant(ci, literal_payload(ci));
       continue;
@@ -412,10 +515,7 @@ void MonoNNModule::dump_best(const std::string& dump_dir) const {
   bool any = false;
   for (auto& c : hip_.constants) {
     std::vector<char> bytes;
-    auto it = host_constants_.find(c.name);
-    if (!c.literal.empty()) bytes = device_payload(c, literal_payload(c));
-    else if (it != host_constants_.end()) bytes = device_payload(c, it->second);
-    else continue;
+    if (!resolve_device_bytes(c, &bytes)) continue;
     if (!any) make_dirs(dir + "/constants");
     any = true;
     write_file(dir + "/constants/" + c.symbol + ".bin", bytes);

@@ -93,6 +93,14 @@ class MonoNNModule {
   int grid_ = 0;
   std::map<std::string, std::vector<char>> host_constants_;   // canonical name -> payload as given
   std::map<std::string, bool> uploaded_;
+  // payloads that outlive load(): the sources of folded LayerNorms (weights, gamma, beta), from which scaled weights
+  // and column sums are rebuilt whenever one of them is supplied again
+  std::map<std::string, std::vector<char>> fold_sources_;
+  bool is_fold_source(const std::string& name) const;
+  const std::vector<char>* raw_payload(const std::string& name, std::vector<char>* scratch) const;
+  // bytes of the module global of `ci`, built from whatever payloads are at hand; false while a source is missing
+  bool resolve_device_bytes(const codegen::ConstantInfo& ci, std::vector<char>* out) const;
+  void upload_resolved(const codegen::ConstantInfo& ci);
   std::string static_scratch_error_;   // why the static temp arena has no address on this device ("" when it has)
 };
 

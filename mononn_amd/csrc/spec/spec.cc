@@ -133,6 +133,7 @@ Json GraphSpecification::to_json() const {
   h["assign_operand_layouts"] = hip.assign_operand_layouts;
   h["fuse_attention"] = hip.fuse_attention;
   h["gemm_prologue_fusion"] = hip.gemm_prologue_fusion;
+  h["layer_norm_folding"] = hip.layer_norm_folding;
   h["barrier"] = hip.barrier;
   h["profile_stages"] = hip.profile_stages;
   h["cooperative_launch"] = hip.cooperative_launch;
@@ -229,13 +230,14 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
   s.codegen_reject_list = strings_from(j, "codegen_reject_list");
   if (j.contains("mononn_hip")) {
     const Json& h = j.at("mononn_hip");
-    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "barrier", "profile_stages", "cooperative_launch", "operand_preload", "pack_left_operands", "attention_out_proj_fusion", "stage_rotation", "barrier_timeout_ms", "opaque_thread_id"}, "mononn_hip");
+    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "layer_norm_folding", "barrier", "profile_stages", "cooperative_launch", "operand_preload", "pack_left_operands", "attention_out_proj_fusion", "stage_rotation", "barrier_timeout_ms", "opaque_thread_id"}, "mononn_hip");
     s.hip.merge_dependent = getb(h, "merge_dependent", true);
     s.hip.gemm_epilogue_fusion = getb(h, "gemm_epilogue_fusion", true);
     s.hip.transpose_constant_b = getb(h, "transpose_constant_b", true);
     s.hip.assign_operand_layouts = getb(h, "assign_operand_layouts", true);
     s.hip.fuse_attention = getb(h, "fuse_attention", true);
     s.hip.gemm_prologue_fusion = getb(h, "gemm_prologue_fusion", false);
+    s.hip.layer_norm_folding = getb(h, "layer_norm_folding", false);
     s.hip.barrier = gets(h, "barrier", "flags_coherent");
     s.hip.profile_stages = getb(h, "profile_stages", false);
     s.hip.cooperative_launch = getb(h, "cooperative_launch", false);

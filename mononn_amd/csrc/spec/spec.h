@@ -76,6 +76,7 @@ struct HipOptions {       // "mononn_hip" section
   // LayerNorm inside the consuming GEMM: removes a stage and a barrier but every column tile repeats the
   // row program on its rows, which only pays off when a GEMM has few column tiles; off unless tuned on
   bool gemm_prologue_fusion = false;
+  bool layer_norm_folding = false;   // with gemm_prologue_fusion: a LayerNorm in front of a constant-weight GEMM is folded into weights and epilogue
   // "flags_coherent": fence-free flag barrier; stage outputs are written with agent-scope write-through
   // stores to temp addresses that are used once per launch, readers use cached loads.
   // "flags": the same barrier with agent-scope release/acquire (L2 write-back + invalidate) around it,

@@ -229,12 +229,12 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     base.runtime.grid_dim.x = props.compute_units * cx.per_cu;
     base.runtime.block_dim.x = cx.block;
     if (env::is_true("MONONN_TUNER_GEMM_PROLOGUE")) base.hip.gemm_prologue_fusion = true;
+    if (env::is_true("MONONN_TUNER_LAYER_NORM_FOLDING")) base.hip.gemm_prologue_fusion = base.hip.layer_norm_folding = true;
     const std::string ctx_str = base.context_string();
 
     // default module of this context: classes of identical node functions
-    MonoNNModule def(params.hlo_text, base.to_json().dump(0), params.kernel_name);
-    def.generate_code();
-    GraphSpecification filled = def.tuning_spec();
+    auto def_holder = std::make_unique<MonoNNModule>(params.hlo_text, base.to_json().dump(0), params.kernel_name);
+    def_holder->generate_code();
     // MONONN_TUNER_SEED_SPEC_DIR: a dump directory of an earlier tuning run of the same module.  Its entries join
     // the candidates that are tried in the whole kernel, so a new run ends no worse than the one it starts from
     // (the stage clocks are noisy, and the order in which classes are decided matters).
@@ -244,7 +244,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       if (sd && *sd) {
         try {
           std::string text;
-          MONONN_CHECK(module::read_file(def.cluster_dir(sd) + "/best_tuning_spec.json", &text), kInvalidArgument) << "no best_tuning_spec.json";
+          MONONN_CHECK(module::read_file(def_holder->cluster_dir(sd) + "/best_tuning_spec.json", &text), kInvalidArgument) << "no best_tuning_spec.json";
           auto sp = std::make_unique<GraphSpecification>(GraphSpecification::from_json(Json::parse(text)));
           if (sp->context_string() == ctx_str) seed = std::move(sp);
         } catch (const Error& e) {
@@ -252,6 +252,34 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         }
       }
     }
+    // MONONN_TUNER_KEEP_SEED_SPLIT_K=<F>: the seed's k splits by at least F are in place from the start.  With
+    // LayerNorm folding a split and a fold exclude each other at one LayerNorm (the row program that adds the partial
+    // sums up stays a stage), and the split-K search below only compares a GEMM and its consumer, so which of the
+    // two a LayerNorm gets is decided here: deep splits (BERT's second feed-forward GEMM, K 3072 by 8) are worth more
+    // than the stage they keep, shallow ones (K 768 by 2) less.
+    if (seed) {
+      const int keep_from = std::atoi(env::get("MONONN_TUNER_KEEP_SEED_SPLIT_K", "0").c_str());
+      int kept = 0;
+      if (keep_from >= 2)
+        for (auto& kv : seed->gemm_spec_list)
+          if (kv.second.split_k >= keep_from) {
+            base.gemm_spec_list[kv.first] = kv.second;
+            ++kept;
+          }
+      if (kept) {
+        try {
+          auto again = std::make_unique<MonoNNModule>(params.hlo_text, base.to_json().dump(0), params.kernel_name);
+          again->generate_code();
+          def_holder = std::move(again);
+          log << "  [" << ctx_str << "] " << kept << " k splits of the seed specification kept from the start\n";
+        } catch (const Error& e) {
+          log << "  [" << ctx_str << "] the seed's k splits do not apply here: " << e.what() << "\n";
+          base.gemm_spec_list.clear();
+        }
+      }
+    }
+    MonoNNModule& def = *def_holder;
+    GraphSpecification filled = def.tuning_spec();
     if (bufs.ptrs.empty()) {
       hipError_t e = hipSetDevice(params.device);
       if (e != hipSuccess) MONONN_FAIL(kRuntimeError) << "hipSetDevice: " << hipGetErrorString(e);

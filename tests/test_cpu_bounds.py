@@ -66,6 +66,7 @@ def test_encoder_variants():
         "8 workgroups": parity._spec_with(fx.hlo_text, grid=8),
         "2 workgroups per compute unit": parity._spec_with(fx.hlo_text, grid=512),
         "LayerNorm inside the GEMM": parity._spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}),
+        "LayerNorm folded into the GEMM": parity._spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True, "layer_norm_folding": True}),
         "output projection inside the attention": parity._spec_with(fx.hlo_text, hip={"attention_out_proj_fusion": True}),
         "no attention fusion": parity._spec_with(fx.hlo_text, hip={"fuse_attention": False}),
         "no epilogue fusion": parity._spec_with(fx.hlo_text, hip={"gemm_epilogue_fusion": False}),

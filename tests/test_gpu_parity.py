@@ -208,6 +208,10 @@ def test_fusion_variants_agree(gpu_device):
         "no epilogue fusion": _spec_with(fx.hlo_text, hip={"gemm_epilogue_fusion": False}),
         "LayerNorm as GEMM prologue": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}),
         "LayerNorm as GEMM prologue over split-K partial sums": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True}, gemm_overrides=split),
+        "LayerNorm folded into weights and epilogue": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True, "layer_norm_folding": True}),
+        # a LayerNorm fed by a k-split GEMM stays a stage that adds the partial sums up; the others are folded
+        "LayerNorm folded where no k split feeds it": _spec_with(fx.hlo_text, hip={"gemm_prologue_fusion": True, "layer_norm_folding": True},
+                                                              gemm_overrides={k: v for k, v in split.items() if v["split_k"] == 4}),
         "plain weight layout": _spec_with(fx.hlo_text, hip={"transpose_constant_b": False, "assign_operand_layouts": False}),
         "split-K": _spec_with(fx.hlo_text, gemm_overrides=split),
         "cooperative launch": _spec_with(fx.hlo_text, hip={"cooperative_launch": True}),

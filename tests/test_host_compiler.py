@@ -607,3 +607,31 @@ def test_layer_norm_in_front_of_a_gemm_is_recognised_and_other_row_programs_are_
         src = m.get_source("main.hip")
         assert m.launch_dims()["barriers"] == 0 and "_pro {" in src          # one stage: the row program runs inside the GEMM
         assert ("__builtin_amdgcn_fdot2" in src) == with_beta
+
+
+def test_layer_norm_folding_moves_the_scale_into_the_weights_and_the_rest_into_the_epilogue():
+    # h = ((x - mean) * r) * gamma + beta in front of h @ W becomes r * (x @ (gamma o W) - mean * (gamma^T W)) + beta^T W:
+    # the MFMAs read x as stored, the functor in front of them only computes (mean, r), the epilogue applies the
+    # rank-1 correction, and the host derives the scaled weights and the two column sums when the payloads arrive
+    text, _ = norm_gemm_module(True)
+    spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+    spec["mononn_hip"]["gemm_prologue_fusion"] = True
+    spec["mononn_hip"]["layer_norm_folding"] = True
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"] = {}, {}
+    m = MonoNNModule.compile(text, json.dumps(spec), build=False)
+    src = m.get_source("main.hip")
+    assert m.launch_dims()["barriers"] == 0
+    assert "after_mfma = true" in src and "ln_stats[" in src and "__builtin_amdgcn_fdot2" in src
+    consts = {c["name"]: c for c in m.constants()}
+    derived = [n for n in consts if n.endswith("_ln_gamma_sums") or n.endswith("_ln_beta_sums")]
+    assert len(derived) == 2 and all(consts[n]["bytes"] == 128 * 4 and not consts[n]["needs_payload"] for n in derived)
+    # gamma and beta themselves are still asked of the caller: the column sums are computed from them
+    assert sum(c["needs_payload"] for c in consts.values()) == 3
+    # without the shift it is not LayerNorm: the fold stays away and the generic prologue is generated
+    text, _ = norm_gemm_module(False)
+    m = MonoNNModule.compile(text, json.dumps(spec), build=False)
+    assert "ln_stats[" not in m.get_source("main.hip") and "_pro {" in m.get_source("main.hip")
+    # a spec that asks for the fold without the prologue fusion has nothing to fold
+    spec["mononn_hip"]["gemm_prologue_fusion"] = False
+    m = MonoNNModule.compile(norm_gemm_module(True)[0], json.dumps(spec), build=False)
+    assert "ln_stats[" not in m.get_source("main.hip") and m.launch_dims()["barriers"] >= 1
