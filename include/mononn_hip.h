@@ -84,7 +84,10 @@ int mononn_module_owns_temp(const mononn_module* m);
 int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int* smem, int* barriers);
 
 /* Non-scalar constants of the module ("buffer_for_<node>" globals that the host fills before
- * launch: mononn_engine/codegen/graph_codegen.cc:71-86, :448-459). */
+ * launch: mononn_engine/codegen/graph_codegen.cc:71-86, :448-459).  needs_payload is 1 for a constant the
+ * HLO text elides ("{...}") and the caller has to set, 0 for one whose literal is in the text and for one the
+ * module builds itself from other constants' payloads (the column sums of a folded LayerNorm); the latter
+ * cannot be set (MONONN_INVALID_ARGUMENT). */
 int mononn_module_num_constants(const mononn_module* m);
 int mononn_module_constant_info(const mononn_module* m, int index, const char** hlo_name, const char** role,
                                 int64_t* bytes, int* needs_payload);
