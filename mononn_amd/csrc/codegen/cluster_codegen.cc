@@ -1911,6 +1911,59 @@ void check_out_proj_mapping(const Program& prog, const Instr* g2, const graph::G
   MONONN_CHECK(v == "GV", kUnsupported) << g3->hlo_name << ": the clusters between the attention and the projection do more than move data";
 }
 
+// The row program between the two contractions of an attention node is straight-line code per query row block.  What
+// does not depend on the query row - a padding mask read per key column and everything computed from it alone - is
+// moved to the line `marker`, which sits with the operand loads in front of the first MFMA (and, with several row
+// blocks per wave, in front of their loop): definitions `const T vN = <expression>;` at the indentation of the
+// straight-line part whose identifiers are parameters, lane coordinates of the key column, the batch index, pure
+// functions and earlier moved values.
+std::string hoist_row_invariant_values(const std::string& text, const std::string& marker) {
+  std::vector<std::string> lines;
+  {
+    std::istringstream is(text);
+    std::string l;
+    while (std::getline(is, l)) lines.push_back(l);
+  }
+  size_t at = lines.size();
+  for (size_t i = 0; i < lines.size(); ++i)
+    if (lines[i].find(marker) != std::string::npos) at = i;
+  if (at == lines.size()) return text;
+  static const std::regex v_def(R"(^(\s*)const ([A-Za-z_]\w*) (v\d+) = (.*);$)");
+  static const std::regex ident(R"((^|[^\w.])([A-Za-z_]\w*))");
+  static const std::regex allowed(
+      R"(^(in\d+|bidx|g|kw|r16|lane|colc|colv|float|double|_Float16|int|long|unsigned|short|char|bool|int8_t|uint8_t|int16_t|uint16_t|int32_t|uint32_t|int64_t|uint64_t|fmaxf|fminf|fabsf|__expf|__logf|tanhf|sqrtf|rsqrtf|__builtin_amdgcn_rcpf|__builtin_inff)$)");
+  // the straight-line part: the indentation of the first value definition behind the marker
+  size_t body_indent = std::string::npos;
+  std::set<std::string> moved_names;
+  std::vector<std::string> moved, rest;
+  const std::string pad(lines[at].find_first_not_of(' ') == std::string::npos ? 0 : lines[at].find_first_not_of(' '), ' ');
+  for (size_t i = at + 1; i < lines.size(); ++i) {
+    std::smatch m;
+    bool move = false;
+    if (std::regex_match(lines[i], m, v_def)) {
+      if (body_indent == std::string::npos) body_indent = m[1].length();
+      if (static_cast<size_t>(m[1].length()) == body_indent) {
+        move = true;
+        const std::string rhs = m[4].str();
+        for (auto it = std::sregex_iterator(rhs.begin(), rhs.end(), ident); move && it != std::sregex_iterator(); ++it) {
+          const std::string id = (*it)[2].str();
+          move = std::regex_match(id, allowed) || moved_names.count(id) || (id.size() > 1 && id.back() == 'f' && std::isdigit(static_cast<unsigned char>(id[0])));
+        }
+        if (move) {
+          moved_names.insert(m[3].str());
+          moved.push_back(pad + "const " + m[2].str() + " " + m[3].str() + " = " + rhs + ";");
+        }
+      }
+    }
+    if (!move) rest.push_back(lines[i]);
+  }
+  std::string out;
+  for (size_t i = 0; i < at; ++i) out += lines[i] + "\n";
+  for (auto& l : moved) out += l + "\n";
+  for (auto& l : rest) out += l + "\n";
+  return out;
+}
+
 // GEMM -> row program -> GEMM with everything between the two contractions on chip.
 //
 // A workgroup owns RW blocks of 16 rows m of one batch element; the KW waves of a block split the
@@ -1928,7 +1981,7 @@ void check_out_proj_mapping(const Program& prog, const Instr* g2, const graph::G
 NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,
                            const Instr* g2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epi_members,
                            const std::vector<const Instr*>& outputs, const LaunchShape& ls, int key_waves,
-                           const Instr* g3 = nullptr, const graph::GemmDesc* d3p = nullptr, int heads = 0, bool preload_w = false) {
+                           const Instr* g3 = nullptr, const graph::GemmDesc* d3p = nullptr, int heads = 0, bool preload_w = false, int row_blocks = 1) {
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
@@ -1951,6 +2004,10 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     KW = key_waves;
   }
   const int RW = NW / KW;
+  // Row blocks a wave takes one after the other with the keys and values it loaded once (many rows per batch element:
+  // the operand traffic of a unit is the whole K and V of the head, whatever the number of rows it serves).
+  const int RB = std::max(1, row_blocks);
+  MONONN_CHECK(RB <= 32 && (RB == 1 || !g3), kSpecError) << "attention: " << RB << " row blocks per wave (at most 32, and one with the projection inside)";
   const int64_t NKW = ragged ? ((N1 + KW - 1) / KW + 31) / 32 * 32 : N1 / KW;   // keys per wave
   MONONN_CHECK(!ragged || (KW - 1) * NKW < N1, kUnsupported) << "attention fusion: " << KW << " key waves leave a wave without keys";
   const int KS1 = static_cast<int>(K1 / 32), NT1 = static_cast<int>(NKW / 16), KS2 = static_cast<int>(NKW / 32), NT2 = static_cast<int>(N2 / 16);
@@ -1971,6 +2028,7 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   CodeBuffer cb;
   VarTable vars;
   Emitter em(prog, row_members, cb, vars, ptrs);
+  em.set_fast_divide(true);
   const hlo::Shape& D1 = g1->shape;
   std::vector<int64_t> batch_dims(D1.dims.begin(), D1.dims.end() - 2);
   int vb = vars.add("bidx", d1.batch);
@@ -2009,24 +2067,44 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   // absorbed projection: the context rows of a row block as f16 left-operand fragments [N2 / 32][64 lanes][8]
   const int cx_off = smem;
   if (g3) smem += RW * static_cast<int>(N2) * 16 * 2;
+  // Several row blocks per wave over keys and values in fragment order: the workgroup copies the head's K and V into
+  // LDS once (a straight copy: fragment order is the order the MFMAs read) and every wave takes its fragments from
+  // there, row block after row block.  Holding them in registers across the rounds instead (what the other layouts
+  // do) leaves the soft-max no registers at 384 keys per wave.
+  const bool kv_lds = RB > 1 && d1.b_tiled && d2.b_tiled && !ragged && !g3 && (N1 * K1) % 8 == 0 && (N2 * N1) % 8 == 0;
+  const int kv_off = (smem + 15) / 16 * 16;
+  if (kv_lds) smem = kv_off + static_cast<int>((N1 * K1 + N2 * N1) * 2);
 
   cb.line("const int lane = mononn_dev::lane_id();");
   cb.line("const int r16 = lane & 15, g = lane >> 4;");
   cb.line("const int kw = mononn_dev::wave_id() % " + S(KW) + ", rw = mononn_dev::wave_id() / " + S(KW) + ";");
-  const int64_t blocks = (M1 + 16 * RW - 1) / (16 * RW);
+  const int64_t blocks = (M1 + 16 * RW * RB - 1) / (16 * RW * RB);
   cb.line("const int bidx = unit / " + S(blocks) + ";");
-  cb.line("const int mt = (unit % " + S(blocks) + ") * " + S(RW) + " + rw;");
-  cb.line("const bool m_valid = mt * 16 + r16 < " + S(M1) + ";");
-  cb.line("const int m = m_valid ? mt * 16 + r16 : " + S(M1 - 1) + ";");
+  // row block of this wave in round rb of the unit: mt0 + rb * RW
+  cb.line("const int mt0 = (unit % " + S(blocks) + ") * " + S(RW * RB) + " + rw;");
+  auto row_block_head = [&](const std::string& mt_expr) {
+    cb.line("const int mt = " + mt_expr + ";");
+    cb.line("const bool m_valid = mt * 16 + r16 < " + S(M1) + ";");
+    cb.line("const int m = m_valid ? mt * 16 + r16 : " + S(M1 - 1) + ";");
+  };
   // Operands in fragment order (stored so by the stage that produced them) are one contiguous KiB per MFMA step;
   // row-major ones cost a lane's 16 rows x 16 bytes = 16 cache lines per quarter wave.
   MONONN_CHECK(!d1.a_packed || M1 % 16 == 0, kInternal) << "fragment-order queries need whole row blocks";
-  if (d1.a_packed) {
-    cb.line("const int mt_c = mt < " + S(M1 / 16) + " ? mt : " + S(M1 / 16 - 1) + ";");
-    cb.line("const _Float16* qp = " + pq + " + (((long)bidx * " + S(M1 / 16) + " + mt_c) * " + S(KS1 * 64) + " + lane) * 8;");
-  } else {
-    cb.line("const _Float16* qp = " + pq + " + (long)bidx * " + S(d1.a_batch_stride) + " + m * " + S(K1) + " + g * 8;");
-  }
+  // the query fragments of row block `mt_expr` (clamped into the matrix) into `dst`
+  auto load_queries = [&](const std::string& dst, const std::string& mt_expr) {
+    cb.open("");
+    if (d1.a_packed) {
+      cb.line("const int mt_q = " + mt_expr + " < " + S(M1 / 16) + " ? " + mt_expr + " : " + S(M1 / 16 - 1) + ";");
+      cb.line("const _Float16* qp = " + pq + " + (((long)bidx * " + S(M1 / 16) + " + mt_q) * " + S(KS1 * 64) + " + lane) * 8;");
+    } else {
+      cb.line("const int m_q = (" + mt_expr + ") * 16 + r16 < " + S(M1) + " ? (" + mt_expr + ") * 16 + r16 : " + S(M1 - 1) + ";");
+      cb.line("const _Float16* qp = " + pq + " + (long)bidx * " + S(d1.a_batch_stride) + " + m_q * " + S(K1) + " + g * 8;");
+    }
+    cb.line("#pragma unroll");
+    cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) " + dst + "[ks] = *reinterpret_cast<const half8_t*>(qp + ks * " + S(d1.a_packed ? 512 : 32) + ");");
+    cb.close();
+  };
+  if (RB == 1) row_block_head("mt0");
   if (d1.b_tiled) cb.line("const _Float16* kp = " + pk + " + (((long)bidx * " + S(N1 / 16) + " + kw * " + S(NKW / 16) + ") * " + S(KS1 * 64) + " + lane) * 8;");
   else if (ragged) cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + g * 8;   // + key * " + S(K1));
   else cb.line("const _Float16* kp = " + pk + " + (long)bidx * " + S(d1.b_batch_stride) + " + (kw * " + S(NKW) + " + r16) * " + S(K1) + " + g * 8;");
@@ -2078,10 +2156,40 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     }
   }
   // all operand loads up front: one exposed memory latency for the whole unit
-  cb.line("half8_t qf[" + S(KS1) + "], kf[" + S(NT1) + "][" + S(KS1) + "];");
+  cb.line("half8_t qf[" + S(KS1) + "];");
+  load_queries("qf", "mt0");
+  std::string kfrag = "kf[j][ks]", vfrag = "vf[t][ks]";
+  if (kv_lds) {
+    const int64_t kc = N1 * K1 / 8, vc = N2 * N1 / 8;   // 16-byte pieces of the head's K and V
+    const int block = NW * 64;
+    const int per_thread = static_cast<int>((kc + vc + block - 1) / block);
+    MONONN_CHECK(per_thread <= 64, kSpecError) << "attention: keys and values of a head do not go through the workgroup's registers in one pass";
+    cb.line("half8_t* lk = reinterpret_cast<half8_t*>(smem + " + S(kv_off) + ");");
+    cb.line("half8_t* lv = lk + " + S(kc) + ";");
+    cb.open("");
+    cb.line("const half8_t* gk = reinterpret_cast<const half8_t*>(" + pk + " + (long)bidx * " + S(N1 * K1) + ");");
+    cb.line("const half8_t* gv = reinterpret_cast<const half8_t*>(" + pv + " + (long)bidx * " + S(N2 * N1) + ");");
+    cb.line("const int tid = mononn_dev::wave_id() * 64 + lane;");
+    cb.line("half8_t stg[" + S(per_thread) + "];");
+    cb.line("#pragma unroll");
+    cb.open("for (int c = 0; c < " + S(per_thread) + "; ++c)");
+    cb.line("const int i = c * " + S(block) + " + tid;");
+    cb.line("if (i < " + S(kc) + ") stg[c] = gk[i];");
+    cb.line("else if (i < " + S(kc + vc) + ") stg[c] = gv[i - " + S(kc) + "];");
+    cb.close();
+    cb.line("__syncthreads();   // the previous unit's readers are done with its keys and values");
+    cb.line("#pragma unroll");
+    cb.open("for (int c = 0; c < " + S(per_thread) + "; ++c)");
+    cb.line("const int i = c * " + S(block) + " + tid;");
+    cb.line("if (i < " + S(kc + vc) + ") lk[i] = stg[c];");
+    cb.close();
+    cb.line("__syncthreads();");
+    cb.close();
+    kfrag = "lk[((kw * " + S(NKW / 16) + " + j) * " + S(KS1) + " + ks) * 64 + lane]";
+    vfrag = "lv[(t * " + S(N1 / 32) + " + kw * " + S(NKW / 32) + " + ks) * 64 + lane]";
+  } else {
+  cb.line("half8_t kf[" + S(NT1) + "][" + S(KS1) + "];");
   cb.line("half8_t vf[" + S(NT2) + "][" + S(KS2) + "];");
-  cb.line("#pragma unroll");
-  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qp + ks * " + S(d1.a_packed ? 512 : 32) + ");");
   cb.line("#pragma unroll");
   cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
   cb.line("#pragma unroll");
@@ -2114,13 +2222,50 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   }
   cb.close();
   cb.close();
+  }
+  cb.line("// @ROW_INVARIANT@");
+  if (RB > 1) {
+    // one round per row block: the next block's queries are requested before this one's arithmetic
+    cb.line("#pragma unroll 1");
+    cb.open("for (int rb = 0; rb < " + S(RB) + "; ++rb)");
+    row_block_head("mt0 + rb * " + S(RW));
+    cb.line("half8_t qn[" + S(KS1) + "];");
+    load_queries("qn", "(mt + " + S(RW) + ")");
+  }
   cb.line("float4_t sacc[" + S(NT1) + "];");
+  if (kv_lds) {
+    // A wave alone on its SIMD has nobody to hide an LDS read behind: the fragments come in groups, the next group
+    // requested before the MFMAs of the current one, with the scheduler kept from sinking the reads to their uses.
+    int G = 1;
+    for (int c : {4, 3, 2})
+      if (NT1 % c == 0) { G = c; break; }
+    const int per = G * KS1;
+    cb.line("half8_t kb[2][" + S(per) + "];");
+    cb.line("#pragma unroll");
+    cb.line("for (int x = 0; x < " + S(per) + "; ++x) kb[0][x] = lk[((kw * " + S(NKW / 16) + " + x / " + S(KS1) + ") * " + S(KS1) + " + x % " + S(KS1) + ") * 64 + lane];");
+    cb.line("#pragma unroll");
+    cb.open("for (int jg = 0; jg < " + S(NT1 / G) + "; ++jg)");
+    cb.open("if (jg + 1 < " + S(NT1 / G) + ")");
+    cb.line("#pragma unroll");
+    cb.line("for (int x = 0; x < " + S(per) + "; ++x) kb[(jg + 1) & 1][x] = lk[((kw * " + S(NKW / 16) + " + (jg + 1) * " + S(G) + " + x / " + S(KS1) + ") * " + S(KS1) + " + x % " + S(KS1) + ") * 64 + lane];");
+    cb.close();
+    cb.line("__builtin_amdgcn_sched_barrier(0);");
+    cb.line("#pragma unroll");
+    cb.open("for (int x = 0; x < " + S(per) + "; ++x)");
+    cb.line("const int j = jg * " + S(G) + " + x / " + S(KS1) + ";");
+    cb.line("if (x % " + S(KS1) + " == 0) sacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};");
+    cb.line("sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb[jg & 1][x], qf[x % " + S(KS1) + "], sacc[j], 0, 0, 0);");
+    cb.close();
+    cb.line("__builtin_amdgcn_sched_barrier(0);");
+    cb.close();
+  } else {
   cb.line("#pragma unroll");
   cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
   cb.line("sacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};");
   cb.line("#pragma unroll");
-  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[j][ks], qf[ks], sacc[j], 0, 0, 0);");
+  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(" + kfrag + ", qf[ks], sacc[j], 0, 0, 0);");
   cb.close();
+  }
   // the first GEMM's result as the HLO defines it: scaled, rounded to f16
   cb.line("_Float16 sv[" + S(NT1) + "][4], pr[" + S(NT1) + "][4];");
   cb.line("#pragma unroll");
@@ -2169,14 +2314,38 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.line("float4_t oacc[" + S(NT2) + "];");
   cb.line("#pragma unroll");
   cb.line("for (int t = 0; t < " + S(NT2) + "; ++t) oacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};");
+  if (kv_lds) {
+    const int G2 = KS2 % 2 == 0 ? 2 : 1;   // k steps per group
+    const int per = G2 * NT2;
+    cb.line("half8_t vb[2][" + S(per) + "];");
+    cb.line("#pragma unroll");
+    cb.line("for (int x = 0; x < " + S(per) + "; ++x) vb[0][x] = lv[((x % " + S(NT2) + ") * " + S(N1 / 32) + " + kw * " + S(NKW / 32) + " + x / " + S(NT2) + ") * 64 + lane];");
+    cb.line("#pragma unroll");
+    cb.open("for (int kg = 0; kg < " + S(KS2 / G2) + "; ++kg)");
+    cb.open("if (kg + 1 < " + S(KS2 / G2) + ")");
+    cb.line("#pragma unroll");
+    cb.line("for (int x = 0; x < " + S(per) + "; ++x) vb[(kg + 1) & 1][x] = lv[((x % " + S(NT2) + ") * " + S(N1 / 32) + " + kw * " + S(NKW / 32) + " + (kg + 1) * " + S(G2) + " + x / " + S(NT2) + ") * 64 + lane];");
+    cb.close();
+    cb.line("__builtin_amdgcn_sched_barrier(0);");
+    cb.line("#pragma unroll");
+    cb.open("for (int y = 0; y < " + S(G2) + "; ++y)");
+    cb.line("const int ks = kg * " + S(G2) + " + y;");
+    cb.line("const half8_t pf = {pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]};");
+    cb.line("#pragma unroll");
+    cb.line("for (int t = 0; t < " + S(NT2) + "; ++t) oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb[kg & 1][y * " + S(NT2) + " + t], pf, oacc[t], 0, 0, 0);");
+    cb.close();
+    cb.line("__builtin_amdgcn_sched_barrier(0);");
+    cb.close();
+  } else {
   cb.line("#pragma unroll");
   cb.open("for (int ks = 0; ks < " + S(KS2) + "; ++ks)");
   cb.line("const half8_t pf = {pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]};");
   cb.line("#pragma unroll");
   cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
-  cb.line("oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[t][ks], pf, oacc[t], 0, 0, 0);");
+  cb.line("oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(" + vfrag + ", pf, oacc[t], 0, 0, 0);");
   cb.close();
   cb.close();
+  }
 
   std::vector<std::string> globals = tables_of(em);
   if (g3) {
@@ -2238,7 +2407,8 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.close();
     cb.close();
     cb.line("__syncthreads();   // LDS is reused by the next unit");
-    NodeFunction f = finish(cb.text(), ptrs, globals, d1.batch * blocks, smem, "typedef mononn_dev::PreB<" + S(NJ * KS3) + "> @NAME@_preb;\n");
+    NodeFunction f = finish(hoist_row_invariant_values(cb.text(), "@ROW_INVARIANT@"), ptrs, globals, d1.batch * blocks, smem,
+                            "typedef mononn_dev::PreB<" + S(NJ * KS3) + "> @NAME@_preb;\n");
     if (preload_w) {
       const std::string tail = ", char* smem) {";
       size_t at = f.text.find(tail);
@@ -2289,7 +2459,12 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.close();
     cb.close();
   }
-  return finish(cb.text(), ptrs, globals, d1.batch * blocks, smem, epi.struct_text);
+  if (RB > 1) {
+    cb.line("#pragma unroll");
+    cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) qf[ks] = qn[ks];");
+    cb.close();
+  }
+  return finish(hoist_row_invariant_values(cb.text(), "@ROW_INVARIANT@"), ptrs, globals, d1.batch * blocks, smem, epi.struct_text);
 }
 
 }  // namespace
@@ -2298,7 +2473,7 @@ NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchSh
   return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores, &node.ln_fold);
 }
 
-NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves, bool preload_weights) {
+NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves, bool preload_weights, int row_blocks) {
   std::vector<const Instr*> row(node.members.begin() + 1, node.members.begin() + node.gemm2_index);
   if (node.gemm3_index != 0) {
     std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.begin() + node.gemm3_index);
@@ -2306,7 +2481,8 @@ NodeFunction generate_attention(const Program& prog, const Node& node, const Lau
                          node.members[node.gemm3_index], &node.gemm3, node.heads, preload_weights);
   }
   std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.end());
-  return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls, key_waves);
+  return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls, key_waves, nullptr, nullptr, 0,
+                       false, row_blocks);
 }
 
 bool can_fuse_out_proj(const Program& prog, const Instr* gemm2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epilogue_members,

@@ -72,8 +72,10 @@ NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, 
 // (0 = as many as the key count allows); the remaining factor of the workgroup's waves takes further row blocks
 // preload_weights: an absorbed output projection takes its weight fragments from a companion function
 // (NodeFunction::preload_text), as generate_gemm does under GemmTuning::preload_b
+// row_blocks: blocks of 16 query rows a wave works through, one after the other, with the keys and values it loaded
+// once (a unit then covers 16 * row_blocks * (waves / key_waves) rows of one batch element)
 NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls, int key_waves = 0,
-                                bool preload_weights = false);
+                                bool preload_weights = false, int row_blocks = 1);
 // the input of a row program fused in front of a GEMM whose rows the GEMM loads as its left-operand fragments
 const hlo::Instr* prologue_primary(const graph::Program& prog, const std::vector<const hlo::Instr*>& row_members, int64_t M, int64_t K);
 // the GEMM `gemm3` reads nothing but the heads that the attention's second GEMM produces, merged by pure data movement

@@ -638,7 +638,11 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
   if (op == "add") { need(2); return def(dt, dt == DType::kPred ? "(" + a[0] + " || " + a[1] + ")" : "(" + T + ")(" + a[0] + " + " + a[1] + ")"); }
   if (op == "subtract") { need(2); return def(dt, "(" + T + ")(" + a[0] + " - " + a[1] + ")"); }
   if (op == "multiply") { need(2); return def(dt, dt == DType::kPred ? "(" + a[0] + " && " + a[1] + ")" : "(" + T + ")(" + a[0] + " * " + a[1] + ")"); }
-  if (op == "divide") { need(2); return def(dt, "(" + T + ")(" + a[0] + " / " + a[1] + ")"); }
+  if (op == "divide") {
+    need(2);
+    if (f32 && fast_divide_) return def(dt, "(" + a[0] + " * __builtin_amdgcn_rcpf(" + a[1] + "))");
+    return def(dt, "(" + T + ")(" + a[0] + " / " + a[1] + ")");
+  }
   if (op == "maximum") { need(2); return def(dt, f32 ? "fmaxf(" + a[0] + ", " + a[1] + ")" : "(" + a[0] + " > " + a[1] + " ? " + a[0] + " : " + a[1] + ")"); }
   if (op == "minimum") { need(2); return def(dt, f32 ? "fminf(" + a[0] + ", " + a[1] + ")" : "(" + a[0] + " < " + a[1] + " ? " + a[0] + " : " + a[1] + ")"); }
   if (op == "power") { need(2); return def(dt, f64 ? "pow(" + a[0] + ", " + a[1] + ")" : "(" + T + ")powf((float)" + a[0] + ", (float)" + a[1] + ")"); }

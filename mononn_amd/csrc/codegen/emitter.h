@@ -81,6 +81,10 @@ class Emitter {
   // (the statements they need are written to the code buffer)
   std::vector<std::string> inline_scalar_computation(const hlo::Computation* c, const std::vector<std::string>& args);
 
+  // f32 divisions as a multiplication by v_rcp_f32 (1 ulp) instead of the correctly rounded expansion (10
+  // instructions per element): for soft-max normalisations, whose quotients are rounded to f16 right after
+  void set_fast_divide(bool on) { fast_divide_ = on; }
+
   static std::string literal(const hlo::Instr* c);                    // scalar constant as C literal
   static std::string literal_of(hlo::DType t, const std::string& text);
   static std::string reducer_expr(const hlo::Instr* reduce, const std::string& a, const std::string& b);
@@ -116,6 +120,7 @@ class Emitter {
   };
   std::map<const hlo::Instr*, Bound> bound_;
   std::map<std::string, std::string> literal_tables_;
+  bool fast_divide_ = false;
   std::vector<std::pair<std::string, std::string>> simple_loads_;
   int counter_ = 0;
   int guarded_ = 0;   // scopes (conditions, loops) this emitter has opened and not yet closed

@@ -152,7 +152,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   for (auto& n : prog.nodes) {
     NodeFunction f;
     if (n.kind == NodeKind::kAttention) {
-      // the fused node borrows a gemm_spec_list entry; of its fields only wave_arrangement.k (key waves) is used
+      // the fused node borrows a gemm_spec_list entry; of its fields wave_arrangement.k (key waves) and
+      // threadblockshape.m (query rows per unit: 16 per wave along m, times the row blocks a wave takes in turn) are used
       auto it = spec.gemm_spec_list.find(n.name);
       if (it == spec.gemm_spec_list.end()) {
         spec::GemmSpec g;
@@ -168,7 +169,16 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         if (bc != n.members[0]->attrs.end()) g.backend_config = Json::parse(bc->second);
         it = spec.gemm_spec_list.emplace(n.name, g).first;
       }
-      f = generate_attention(prog, n, ls, it->second.wave_k, spec.hip.operand_preload);
+      int row_blocks = 1;
+      {
+        const spec::GemmSpec& g = it->second;
+        const int kw = g.wave_k > 0 ? g.wave_k : default_attention_key_waves(n.gemm, ls);
+        const int rows_per_round = 16 * std::max(1, ls.waves() / std::max(1, kw));
+        MONONN_CHECK(g.tb_m >= rows_per_round && g.tb_m % rows_per_round == 0, kSpecError)
+            << "gemm_spec_list[" << n.name << "]: threadblockshape.m " << g.tb_m << " is not a multiple of the " << rows_per_round << " query rows the workgroup's waves take per round";
+        row_blocks = g.tb_m / rows_per_round;
+      }
+      f = generate_attention(prog, n, ls, it->second.wave_k, spec.hip.operand_preload, row_blocks);
     } else if (n.kind == NodeKind::kGemm) {
       auto it = spec.gemm_spec_list.find(n.name);
       GemmTuning t;

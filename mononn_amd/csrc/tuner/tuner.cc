@@ -356,17 +356,25 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         }
       } else if (c.kind == "attention") {
         // key waves per row block: 1 (no exchange through LDS, a wave owns whole rows) .. all waves
+        // and the blocks of 16 query rows a wave takes in turn with the keys and values it loaded once, as long as
+        // the units still cover the grid
         for (int kw = 1; kw <= cx.block / 64; kw *= 2) {
-          if (c.sample->gemm.N % (32 * kw) != 0) continue;
-          GraphSpecification s = filled;
-          for (auto& n : c.nodes) {
-            spec::GemmSpec& g = s.gemm_spec_list[n];
-            g.wave_k = kw;
-            g.wave_m = cx.block / 64 / kw;
-            g.tb_m = 16 * g.wave_m;
-            g.warp_n = static_cast<int>(c.sample->gemm.N / kw);
+          if (c.sample->gemm.N % 32 == 0 && c.sample->gemm.N % (32 * kw) != 0) continue;   // a ragged key count is rounded up per wave
+          for (int rb : {1, 2, 3, 4, 6, 8}) {
+            const int wave_m = cx.block / 64 / kw;
+            const int64_t rows = 16 * wave_m * rb;
+            const int64_t units = c.sample->gemm.batch * ((c.sample->gemm.M + rows - 1) / rows);
+            if (rb > 1 && (c.sample->gemm3_index != 0 || 2 * units < base.runtime.grid_dim.x || rows >= c.sample->gemm.M + 16 * wave_m)) continue;
+            GraphSpecification s = filled;
+            for (auto& n : c.nodes) {
+              spec::GemmSpec& g = s.gemm_spec_list[n];
+              g.wave_k = kw;
+              g.wave_m = wave_m;
+              g.tb_m = static_cast<int>(rows);
+              g.warp_n = static_cast<int>(c.sample->gemm.N / kw);
+            }
+            add("key_waves" + std::to_string(kw) + (rb > 1 ? "_rows" + std::to_string(rows) : ""), s);
           }
-          add("key_waves" + std::to_string(kw), s);
         }
       } else if (c.kind == "cluster_reduce") {
         for (int tier : {1, 2})
@@ -607,6 +615,8 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           << " us with the seed specification; the search goes on from the faster one\n";
       if (verbose) std::fprintf(stderr, "[mononn tuner] %s whole kernel %.2f us tuned, %.2f us seed\n", ctx_str.c_str(), stitched_us, seed_us);
       if (seed_us > 0 && (stitched_us < 0 || seed_us < 0.999 * stitched_us)) {
+        // the winners by the stage clocks get their turn against the seed, class by class
+        for (auto& kv : classes) runners_up[kv.second.function].insert(runners_up[kv.second.function].begin(), {"best_by_stage_clocks", -1.0, stitched});
         stitched = std::move(whole);
         stitched_us = seed_us;
       }

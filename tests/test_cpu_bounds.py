@@ -79,6 +79,25 @@ def test_encoder_variants():
         assert ok, f"{name}: {msg}"
 
 
+def test_attention_with_several_row_blocks_per_wave():
+    import json
+    cases = [(models.bert_encoder(L=1, B=2, S=128, H=128, NH=2, F=256, vocab=300, max_pos=128, mask_kind="length_mask"), 3, 4),
+             (models.gpt2(L=1, B=2, S=64, H=128, NH=2, F=256, vocab=300, max_pos=64), 4, 2),
+             (models.vit(L=1, B=2, image=96, patch=16, H=128, NH=2, F=256), 2, 1)]
+    for fx, row_blocks, key_waves in cases:
+        spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+        block = spec["cuda_context"]["cuda_runtime_context"]["block_dim"]["x"]
+        for name, entry in spec["gemm_spec_list"].items():
+            if name.count("batch_gemm") >= 2:
+                c = entry["cutlass_config"]
+                c["wave_arrangement"] = {"m": block // 64 // key_waves, "n": 1, "k": key_waves}
+                c["threadblockshape"]["m"] = 16 * c["wave_arrangement"]["m"] * row_blocks
+        text = json.dumps(spec)
+        assert "for (int rb = 0; rb < %d; ++rb)" % row_blocks in MonoNNModule.compile(fx.hlo_text, text, build=False).get_source("main.hip")
+        ok, msg = check_module(fx.hlo_text, text)
+        assert ok, f"{row_blocks} row blocks, {key_waves} key waves: {msg}"
+
+
 ODD_ENCODERS = [dict(B=1, S=17, H=64, NH=1, F=100), dict(B=3, S=50, H=96, NH=2, F=100), dict(B=1, S=100, H=120, NH=3, F=256),
                 dict(B=3, S=64, H=128, NH=4, F=100), dict(B=1, S=50, H=120, NH=3, F=100), dict(B=3, S=17, H=96, NH=2, F=256)]
 

@@ -238,3 +238,42 @@ def test_encoders_with_sizes_off_the_mfma_steps(gpu_device, shape):
     want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
     _check(got, want, f"encoder {shape}")
     m.close()
+
+
+def _spec_with_attention_rows(hlo_text, row_blocks, key_waves=None):
+    """The default specification with every fused attention taking `row_blocks` blocks of 16 query rows per wave
+    (threadblockshape.m = query rows per unit) and, if given, `key_waves` waves per row block."""
+    import json
+    from mononn_amd import MonoNNModule
+    spec = json.loads(MonoNNModule.compile(hlo_text, build=False).get_tuning_spec())
+    block = spec["cuda_context"]["cuda_runtime_context"]["block_dim"]["x"]
+    n = 0
+    for name, entry in spec["gemm_spec_list"].items():
+        if name.count("batch_gemm") < 2:
+            continue
+        c = entry["cutlass_config"]
+        if key_waves:
+            c["wave_arrangement"] = {"m": block // 64 // key_waves, "n": 1, "k": key_waves}
+        c["threadblockshape"]["m"] = 16 * c["wave_arrangement"]["m"] * row_blocks
+        n += 1
+    assert n >= 1
+    return json.dumps(spec)
+
+
+@pytest.mark.parametrize("what,make,row_blocks,key_waves", [
+    ("encoder, padding masks, 4 key waves x 3 row blocks (rows 128 = 2 units of 48 + 32 past the end)",
+     lambda: models.bert_encoder(L=2, B=2, S=128, H=256, NH=4, F=512, vocab=300, max_pos=128, mask_kind="length_mask"), 3, 4),
+    ("encoder, a wave per row block x 2 row blocks", lambda: models.bert_encoder(L=2, B=2, S=128, H=256, NH=4, F=512, vocab=300, max_pos=128), 2, 1),
+    ("causal decoder, 2 key waves x 4 row blocks", lambda: models.gpt2(L=2, B=2, S=128, H=256, NH=4, F=512, vocab=300, max_pos=128), 4, 2),
+    ("ViT, 37 keys, a wave per row block x 2 row blocks", lambda: models.vit(L=2, B=3, image=96, patch=16, H=128, NH=2, F=256), 2, 1),
+])
+def test_attention_with_several_row_blocks_per_wave(gpu_device, what, make, row_blocks, key_waves):
+    # a wave keeps the keys and values of its head in registers and works through several blocks of 16 query rows
+    fx = make()
+    consts = fx.make_constants(1243, "random")
+    inputs = fx.make_inputs(1243)
+    m, got = _run(fx, consts, inputs, gpu_device, _spec_with_attention_rows(fx.hlo_text, row_blocks, key_waves))
+    assert "for (int rb = 0; rb < %d; ++rb)" % row_blocks in m.get_source("main.hip")
+    m.close()
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _check(got, want, what)

@@ -276,6 +276,7 @@ def test_attention_key_wave_arrangements(gpu_device, key_waves):
     assert names, "the attention block did not fuse"
     for n in names:
         spec["gemm_spec_list"][n]["cutlass_config"]["wave_arrangement"].update(k=key_waves, m=4 // key_waves)
+        spec["gemm_spec_list"][n]["cutlass_config"]["threadblockshape"]["m"] = 16 * (4 // key_waves)   # query rows per unit
     (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs, json.dumps(spec))
     assert f"kw = mononn_dev::wave_id() % {key_waves}" in m.get_source("main.hip")
     check_close(got, want)

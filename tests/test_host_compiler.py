@@ -156,6 +156,8 @@ def test_spec_changes_generated_code(layer):
     (lambda s: s["mononn_hip"].update(barrier="semaphore"), "SPEC_ERROR"),
     (lambda s: next(v for k, v in s["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))["cutlass_config"]["wave_arrangement"].update(m=3), "SPEC_ERROR"),
     (lambda s: next(v for k, v in s["gemm_spec_list"].items() if k.startswith("cublas_batch_gemm_"))["cutlass_config"]["wave_arrangement"].update(k=3), "SPEC_ERROR"),
+    # query rows per attention unit: whole rounds of 16 rows per wave along m
+    (lambda s: next(v for k, v in s["gemm_spec_list"].items() if k.startswith("cublas_batch_gemm_"))["cutlass_config"]["threadblockshape"].update(m=24), "SPEC_ERROR"),
 ])
 def test_bad_specs_are_rejected(layer, mutate, status):
     spec = json.loads(MonoNNModule.compile(layer.hlo_text, build=False).get_tuning_spec())
