@@ -300,7 +300,8 @@ class MonoNNModule:
         self.launch_raw(self.buffer_pointers(), stream)
         self.synchronize(stream)
         outs = []
-        npdt = {"f16": np.float16, "f32": np.float32, "s32": np.int32, "pred": np.bool_, "s64": np.int64, "u8": np.uint8, "s8": np.int8}
+        # bf16 results come back as their uint16 bit patterns (NumPy has no bfloat16; mononn_amd.bf16 converts)
+        npdt = {"f16": np.float16, "bf16": np.uint16, "f32": np.float32, "s32": np.int32, "pred": np.bool_, "s64": np.int64, "u8": np.uint8, "s8": np.int8}
         for t, o in zip(b["liveouts"], out_dtypes_dims):
             outs.append(t.cpu().numpy().view(npdt[o["dtype"]]).reshape(o["dims"]).copy())
         return outs

@@ -804,7 +804,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   // 2-byte aligned.  A single f16 result that only the host reads is still written four columns at a time, through
   // a copy without an alignment promise, wherever the whole run lies inside the row (decided further down).
   bool ragged4 = false;
-  std::string ragged4_offset;
+  std::string ragged4_offset, ragged4_type = "_Float16";
   std::vector<std::pair<std::string, std::string>> fold_loads;   // (expression, type) of the folded LayerNorm's column sums
   CodeBuffer cb;   // epilogue body
   VarTable vars;
@@ -965,12 +965,13 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
       if (vec4) {
         LinExpr full = physical_offset(prog, out.o, out.idx, &vars);
         LinExpr base = physical_offset(prog, out.o, out.idx_base, &vars);
-        out.vector_store = full.equals(base.plus(LinExpr::variable(vr, 4))) && out.o->shape.dtype == DType::kF16;
+        out.vector_store = full.equals(base.plus(LinExpr::variable(vr, 4))) && hlo::is_half_float(out.o->shape.dtype);
         if (out.vector_store) ++n_vector_stores;
         if (out.vector_store) cb.line(out.stage + "[r] = " + v + ";");
         else store(prog, cb, ptrs, vars, out.o, out.idx, v);
       } else {
-        if (mfma && !along_m && !g.is_conv && outs.size() == 1 && out.o->shape.dtype == DType::kF16 && host_only_output(prog, out.o) && g.N >= 4) {
+        if (mfma && !along_m && !g.is_conv && outs.size() == 1 && hlo::is_half_float(out.o->shape.dtype) && host_only_output(prog, out.o) && g.N >= 4) {
+          ragged4_type = hlo::dtype_ctype(out.o->shape.dtype);
           Index at0 = out.idx;
           // the same element with column 0: the offset must be that plus the column
           Index probe_idx = delinearize(linearize([&] {
@@ -1003,7 +1004,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
     for (auto& out : outs)
       if (out.vector_store) {
         std::string lin = physical_offset(prog, out.o, out.idx_base, &vars).str(vars);
-        cb.line(stN_of(prog, out.o) + "_Float16, 4>(" + ptrs.output(out.o) + " + " + lin + ", " + out.stage + ");");
+        cb.line(stN_of(prog, out.o) + hlo::dtype_ctype(out.o->shape.dtype) + ", 4>(" + ptrs.output(out.o) + " + " + lin + ", " + out.stage + ");");
       }
   }
 
@@ -1050,14 +1051,14 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   else if (mfma) {
     pre += "  __device__ __forceinline__ void operator()(int bidx, int m, int n0, const float (&accv)[4], const Pre&) const {\n";
     if (ragged4) {
-      pre += "    _Float16* row = " + ragged4_offset + ";\n";
+      pre += "    " + ragged4_type + "* row = " + ragged4_offset + ";\n";
       pre += "    if (n0 + 3 < " + S(g.N) + ") {\n";
-      pre += "      const _Float16 st[4] = {one(bidx, m, n0, accv[0]), one(bidx, m, n0 + 1, accv[1]), one(bidx, m, n0 + 2, accv[2]), one(bidx, m, n0 + 3, accv[3])};\n";
-      pre += "      mononn_dev::stN_plain_unaligned<_Float16, 4>(row + n0, st);\n";
+      pre += "      const " + ragged4_type + " st[4] = {one(bidx, m, n0, accv[0]), one(bidx, m, n0 + 1, accv[1]), one(bidx, m, n0 + 2, accv[2]), one(bidx, m, n0 + 3, accv[3])};\n";
+      pre += "      mononn_dev::stN_plain_unaligned<" + ragged4_type + ", 4>(row + n0, st);\n";
       pre += "    } else {\n";
       pre += "      for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") mononn_dev::st1_plain(row + nn, one(bidx, m, nn, accv[r])); }\n";
       pre += "    }\n  }\n";
-      pre += "  __device__ __forceinline__ _Float16 one(int bidx, int m, int nn, float acc) const {\n";
+      pre += "  __device__ __forceinline__ " + ragged4_type + " one(int bidx, int m, int nn, float acc) const {\n";
     } else {
       pre += "    for (int r = 0; r < 4; ++r) { const int nn = n0 + r; if (nn < " + S(g.N) + ") { const float acc = accv[r]; one(bidx, m, nn, acc); } }\n  }\n";
       pre += "  __device__ __forceinline__ void one(int bidx, int m, int nn, float acc) const {\n";
@@ -1701,6 +1702,14 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     pb = ptrs.input(prog.storage_root(gi->operands[1]));
   }
   const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
+  if (g.bf16) {
+    // the tiles move operands as 16-byte pieces whatever the 2-byte type; only the MFMA differs (last template argument)
+    MONONN_CHECK(!has_pro && !g.is_conv && !fold, kUnsupported) << gi->hlo_name << ": bf16 GEMMs take neither a row-program prologue nor a convolution's operand map";
+    if (mfma) {
+      pa = "reinterpret_cast<const half_t*>(" + pa + ")";
+      pb = "reinterpret_cast<const half_t*>(" + pb + ")";
+    }
+  }
   std::vector<const Instr*> cluster_members(members.begin() + 1, members.end());
   Epilogue epi;
   {
@@ -1805,13 +1814,13 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
       else if (t.stages >= 2)
         call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", "
              << (g.a_packed ? "true" : "false") << ", " << (g.b_packed ? "true" : "false") << ", " << (epi.along_m ? "true" : "false") << ", " << t.bk
-             << ", @NAME@_epi>(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
+             << ", @NAME@_epi" << (g.bf16 ? ", mononn_dev::RowMajorA, true" : "") << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
              << b_expr.str() << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
       else
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
              << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
              << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
-             << (epi.along_m ? "true" : "false") << ", " << (b_along_n ? "true" : "false") << ">("
+             << (epi.along_m ? "true" : "false") << ", " << (b_along_n ? "true" : "false") << (g.bf16 ? ", true" : "") << ">("
              << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
              << ", " << g.N << ", " << g.K << ", " << (b_along_n ? g.N : g.K) << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
              << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");
@@ -1985,6 +1994,7 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
+  MONONN_CHECK(!d1.f32 && !d2.f32 && !d1.bf16 && !d2.bf16, kUnsupported) << "attention fusion is built for f16 (scores and probabilities are held as f16 between the two contractions)";
   MONONN_CHECK(K1 % 32 == 0 && N2 % 16 == 0, kUnsupported) << "attention fusion: head size must be an MFMA multiple";
   // A key count off the MFMA step (ViT: 197): every wave's slice is rounded up to whole steps of 32 keys; the keys
   // past the end are read from the last valid key (finite values, in range), take no part in the row reductions

@@ -178,6 +178,7 @@ std::string Emitter::literal_of(DType t, const std::string& text_in) {
       }
     }
     if (t == DType::kF16) return "((_Float16)" + body + ")";
+    if (t == DType::kBF16) return "((__bf16)" + body + ")";
     if (t == DType::kF64) return "((double)" + body + ")";
     return "(" + body + ")";
   }
@@ -632,7 +633,7 @@ std::string Emitter::emit(const Instr* ins, const Index& idx) {
   const bool f32 = dt == DType::kF32, f16 = dt == DType::kF16, f64 = dt == DType::kF64;
   auto via_f32 = [&](const std::string& fn) {   // unary math evaluated in fp32
     if (f32) return def(dt, fn + "(" + a[0] + ")");
-    if (f16) return def(dt, "(_Float16)" + fn + "((float)" + a[0] + ")");
+    if (f16 || dt == DType::kBF16) return def(dt, "(" + T + ")" + fn + "((float)" + a[0] + ")");
     MONONN_FAIL(kUnsupported) << ins->hlo_name << ": " << op << " on " << hlo::dtype_name(dt);
   };
   if (op == "add") { need(2); return def(dt, dt == DType::kPred ? "(" + a[0] + " || " + a[1] + ")" : "(" + T + ")(" + a[0] + " + " + a[1] + ")"); }

@@ -31,6 +31,7 @@ typedef _Float16 half_t;
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef int int4_t __attribute__((ext_vector_type(4)));
@@ -399,6 +400,14 @@ __device__ __forceinline__ half8_t load_key_run(const half_t* row, int k, int n)
 // ---------------------------------------------------------------------------------------------
 // One workgroup owns a BM x BN output tile.  Its waves are arranged WM x WN x WK: WM*WN waves split
 // the tile, WK waves split the k range of each sub-tile (k steps interleaved).  Every wave feeds
+// One 16x16x32 MFMA step on operands held as 16-byte pieces: the f16 form, or the bf16 form on the same bits (the
+// tiles move operands without looking at them, so bf16 GEMMs share every layout and every load with f16 ones).
+template <bool BF16>
+__device__ __forceinline__ float4_t mfma_16x16x32(half8_t a, half8_t b, float4_t c) {
+  if constexpr (BF16) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
 // v_mfma_f32_16x16x32_f16 directly from global memory: a lane's operand is 8 consecutive halves
 // along k, i.e. one 16-byte load, and because a weight element is only ever needed by the waves that
 // own its columns there is nothing to share through LDS in the main loop.  Partial sums of the WK
@@ -503,7 +512,7 @@ __device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_
 // kernel parameters): a lane gathers its eight k values of one column with eight 2-byte loads.  Slower per byte
 // than the k-contiguous layouts, but the contraction stays on the MFMAs.
 template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA,
-          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false, bool B_ALONG_N = false>
+          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false, bool B_ALONG_N = false, bool BF16 = false>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
                                           int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
                                           const AMap& amap = AMap(), const Pre* pb = nullptr) {
@@ -651,8 +660,8 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = D_ALONG_M ? __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c & 1][s][i], b[c & 1][s][j], acc[i][j], 0, 0, 0)
-                                  : __builtin_amdgcn_mfma_f32_16x16x32_f16(b[c & 1][s][j], a[c & 1][s][i], acc[i][j], 0, 0, 0);
+            acc[i][j] = D_ALONG_M ? mfma_16x16x32<BF16>(a[c & 1][s][i], b[c & 1][s][j], acc[i][j])
+                                  : mfma_16x16x32<BF16>(b[c & 1][s][j], a[c & 1][s][i], acc[i][j]);
       }
     }
   }
@@ -881,9 +890,15 @@ constexpr int gemm_lds_bytes(int BM, int BN, int BK) { return 2 * (BM + BN) * BK
 
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
+template <bool BF16>
+__device__ __forceinline__ float16_t mfma_32x32x16(half8_t a, half8_t b, float16_t c) {
+  if constexpr (BF16) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
 // BK: k extent of one LDS buffer (a multiple of 32); K a multiple of 32.
 template <int BM, int BN, int WM, int WN, int K, int KTOTAL, bool PACKED_A, bool PACKED_B, bool D_ALONG_M, int BK, class Epi,
-          class AMap = RowMajorA>
+          class AMap = RowMajorA, bool BF16 = false>
 __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, int M, int N, int lda, int ldb, int batch, int tile_m,
                                               int tile_n, Epi& epi, char* smem, const AMap& amap = AMap()) {
   constexpr int NW = WM * WN;
@@ -1047,8 +1062,7 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
 #pragma unroll
       for (int c = l0 + ((l1 - l0) * q) / Q; c < l0 + ((l1 - l0) * (q + 1)) / Q; ++c) load_one(t + 3, set, c);
       const int i = q / TN, j = q % TN;
-      acc[i][j] = D_ALONG_M ? __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[rb][i], fb[rb][j], acc[i][j], 0, 0, 0)
-                            : __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[rb][j], fa[rb][i], acc[i][j], 0, 0, 0);
+      acc[i][j] = D_ALONG_M ? mfma_32x32x16<BF16>(fa[rb][i], fb[rb][j], acc[i][j]) : mfma_32x32x16<BF16>(fb[rb][j], fa[rb][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };

@@ -73,12 +73,16 @@ struct Builder {
     // gemm_impl.cc:56, :229)
     const bool all_f16 = A.dtype == hlo::DType::kF16 && B.dtype == hlo::DType::kF16 && D.dtype == hlo::DType::kF16;
     const bool all_f32 = A.dtype == hlo::DType::kF32 && B.dtype == hlo::DType::kF32 && D.dtype == hlo::DType::kF32;
-    MONONN_CHECK(all_f16 || all_f32, kUnsupported) << g->hlo_name << ": GEMM operands and result must all be f16 or all be f32";
+    // bf16 x bf16 -> bf16 (not in the reference, whose CUTLASS instantiations are half and float): the same tiles on the
+    // bf16 forms of the MFMAs
+    const bool all_bf16 = A.dtype == hlo::DType::kBF16 && B.dtype == hlo::DType::kBF16 && D.dtype == hlo::DType::kBF16;
+    MONONN_CHECK(all_f16 || all_f32 || all_bf16, kUnsupported) << g->hlo_name << ": GEMM operands and result must all be f16, all be bf16 or all be f32";
     MONONN_CHECK(g->operands.size() == 2 || g->operands[2]->shape.dtype == D.dtype, kUnsupported) << g->hlo_name << ": addend type differs from the result type";
     const int r = A.rank();
     const hlo::GemmConfig& c = g->gemm;
     GemmDesc d;
     d.f32 = all_f32;
+    d.bf16 = all_bf16;
     MONONN_CHECK(c.lhs_contracting == r - 1 || c.lhs_contracting == r - 2, kUnsupported) << g->hlo_name << ": lhs contracting dim must be one of the two minor dims";
     MONONN_CHECK(c.rhs_contracting == r - 1 || c.rhs_contracting == r - 2, kUnsupported) << g->hlo_name << ": rhs contracting dim must be one of the two minor dims";
     d.a_k_contig = c.lhs_contracting == r - 1;
@@ -558,7 +562,7 @@ struct Builder {
       if (c->opcode != "constant" || c->is_scalar_constant() || c->shape.rank() != 2) continue;
       bool all = !c->users.empty();
       for (auto* u : c->users) {
-        bool good = u->is_gemm() && u->operands.size() >= 2 && c->shape.dtype == hlo::DType::kF16 &&
+        bool good = u->is_gemm() && u->operands.size() >= 2 && hlo::is_half_float(c->shape.dtype) &&
                     u->operands[1] == c && u->operands[0] != c && u->gemm.rhs_contracting == 0 && c->shape.dims[0] % 32 == 0 &&
                     u->gemm.lhs_contracting == u->operands[0]->shape.rank() - 1 && (u->operands.size() < 3 || u->operands[2] != c);
         if (!good) all = false;

@@ -26,7 +26,8 @@ enum class NodeKind { kCluster, kGemm, kAttention };
 
 struct GemmDesc {
   int64_t batch = 1, M = 0, N = 0, K = 0;
-  bool f32 = false;          // operands and result are f32 (v_mfma_f32_16x16x4_f32 tiles); otherwise f16
+  bool f32 = false;          // operands and result are f32 (v_mfma_f32_16x16x4_f32 tiles); otherwise f16 or bf16
+  bool bf16 = false;         // operands and result are bf16 (the bf16 forms of the f16 MFMAs; same tiles, same layouts)
   bool a_k_contig = true;    // A stored [.., M, K]; false: [.., K, M]
   bool b_k_contig = false;   // B stored [.., N, K]; false: [.., K, N]
   bool b_packed = false;     // B is a constant that the host stores in MFMA fragment order at upload

@@ -26,6 +26,7 @@ const DTypeInfo kDTypes[] = {
     {DType::kU16, "u16", 2, "uint16_t"},     {DType::kU32, "u32", 4, "uint32_t"},
     {DType::kU64, "u64", 8, "uint64_t"},     {DType::kF16, "f16", 2, "_Float16"},
     {DType::kF32, "f32", 4, "float"},        {DType::kF64, "f64", 8, "double"},
+    {DType::kBF16, "bf16", 2, "__bf16"},
 };
 
 // Opcode set of mononn_engine/core/op/op_type.h:20-58 plus `fusion`; everything else is rejected

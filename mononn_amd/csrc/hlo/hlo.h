@@ -16,13 +16,14 @@
 namespace mononn {
 namespace hlo {
 
-enum class DType { kPred, kS8, kS16, kS32, kS64, kU8, kU16, kU32, kU64, kF16, kF32, kF64, kTuple, kInvalid };
+enum class DType { kPred, kS8, kS16, kS32, kS64, kU8, kU16, kU32, kU64, kF16, kBF16, kF32, kF64, kTuple, kInvalid };
 
 const char* dtype_name(DType t);          // "f16"
 int dtype_bytes(DType t);                 // 2
 const char* dtype_ctype(DType t);         // device C type, e.g. "_Float16"
 DType dtype_from_name(const std::string& s);
-inline bool is_float(DType t) { return t == DType::kF16 || t == DType::kF32 || t == DType::kF64; }
+inline bool is_float(DType t) { return t == DType::kF16 || t == DType::kBF16 || t == DType::kF32 || t == DType::kF64; }
+inline bool is_half_float(DType t) { return t == DType::kF16 || t == DType::kBF16; }   // 2-byte MFMA operand types
 
 struct Shape {
   DType dtype = DType::kInvalid;

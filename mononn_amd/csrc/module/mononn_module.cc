@@ -298,6 +298,15 @@ static std::vector<char> literal_payload(const codegen::ConstantInfo& ci) {
     char* p = &out[static_cast<size_t>(i * es)];
     switch (ci.dtype) {
       case hlo::DType::kF16: { _Float16 v = static_cast<_Float16>(d); std::memcpy(p, &v, 2); break; }
+      case hlo::DType::kBF16: {
+        // round to nearest even on the upper 16 bits of the f32 pattern (NaN stays NaN)
+        float f = static_cast<float>(d);
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        uint16_t h = f != f ? static_cast<uint16_t>((u >> 16) | 0x40) : static_cast<uint16_t>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+        std::memcpy(p, &h, 2);
+        break;
+      }
       case hlo::DType::kF32: { float v = static_cast<float>(d); std::memcpy(p, &v, 4); break; }
       case hlo::DType::kF64: std::memcpy(p, &d, 8); break;
       case hlo::DType::kPred: case hlo::DType::kS8: case hlo::DType::kU8: { int8_t v = static_cast<int8_t>(ll); std::memcpy(p, &v, 1); break; }

@@ -21,6 +21,17 @@ from .builder import Computation, HloModuleBuilder, Value
 
 NP_DTYPE = {"f16": np.float16, "f32": np.float32, "s32": np.int32, "pred": np.bool_, "s64": np.int64}
 
+# storage type of activations and weights in the fixtures below: "f16", or "bf16" inside bert_encoder(ftype="bf16")
+_FT = "f16"
+
+
+def _host_array(values, dtype):
+    """values as the host buffer of HLO type `dtype` (bf16: uint16 bit patterns)."""
+    if dtype == "bf16":
+        from .. import bf16
+        return np.ascontiguousarray(bf16.to_bits(values))
+    return np.ascontiguousarray(np.asarray(values).astype(NP_DTYPE[dtype]))
+
 
 @dataclass
 class ModelFixture:
@@ -40,14 +51,13 @@ class ModelFixture:
         out = {}
         for name, meta in self.constants.items():
             role, dims = meta["role"], meta["dims"]
-            dt = NP_DTYPE[meta["dtype"]]
             if role.endswith("/bias") or role.endswith("/beta"):
                 a = rng.normal(0.0, 0.05, dims) if init == "random" else np.zeros(dims)
             elif role.endswith("/gamma"):
                 a = 1.0 + rng.normal(0.0, 0.1, dims) if init == "random" else np.ones(dims)
             else:
                 a = rng.normal(0.0, 0.02, dims)
-            out[name] = np.ascontiguousarray(a.astype(dt))
+            out[name] = _host_array(a, meta["dtype"])
         return out
 
     def make_inputs(self, seed: int) -> List[np.ndarray]:
@@ -63,11 +73,11 @@ class ModelFixture:
                 lens = rng.integers(p["min_len"], p["max_len"] + 1, dims[0])
                 a = (np.arange(dims[1])[None, :] < lens[:, None]).astype(np.int32)
             elif kind == "zeros":
-                a = np.zeros(dims, NP_DTYPE[p["dtype"]])
+                a = _host_array(np.zeros(dims), p["dtype"])
             elif kind == "normal":
-                a = rng.normal(0.0, 1.0, dims).astype(NP_DTYPE[p["dtype"]])
+                a = _host_array(rng.normal(0.0, 1.0, dims), p["dtype"])
             elif kind == "uniform_pm1":
-                a = rng.uniform(-1.0, 1.0, dims).astype(NP_DTYPE[p["dtype"]])
+                a = _host_array(rng.uniform(-1.0, 1.0, dims), p["dtype"])
             else:
                 raise ValueError(kind)
             arrs.append(np.ascontiguousarray(a))
@@ -80,7 +90,7 @@ class ModelFixture:
 def _bias_add_f16(f: Computation, g: Value, bias: Value) -> Value:
     rows, cols = g.dims
     x = f.add(f.convert(g, "f32"), f.broadcast(f.convert(bias, "f32"), (rows, cols), [1]))
-    return f.convert(x, "f16")
+    return f.convert(x, _FT)
 
 
 def _layer_norm(e: Computation, mb: HloModuleBuilder, x: Value, gamma: Value, beta: Value,
@@ -111,7 +121,7 @@ def _layer_norm(e: Computation, mb: HloModuleBuilder, x: Value, gamma: Value, be
         y = f.mul(d, f.broadcast(r, (M, H), [0]))
         y = f.mul(y, f.broadcast(f.convert(pg, "f32"), (M, H), [1]))
         y = f.add(y, f.broadcast(f.convert(pb, "f32"), (M, H), [1]))
-        return f.convert(y, "f16")
+        return f.convert(y, _FT)
     return e.fusion("kLoop", [x, s, v, gamma, beta], norm_body)
 
 
@@ -175,7 +185,7 @@ def _attention(e: Computation, mb: HloModuleBuilder, h: Value, mask_add: Optiona
     def prob_body(f, *p):
         ps, pm, (pmx, psm) = split(p)
         ex = f.exp(f.sub(logits(f, ps, pm), f.broadcast(pmx, full, [0, 1, 2])))
-        return f.convert(f.div(ex, f.broadcast(psm, full, [0, 1, 2])), "f16")
+        return f.convert(f.div(ex, f.broadcast(psm, full, [0, 1, 2])), _FT)
     probs = e.fusion("kLoop", ops + [mx, sm], prob_body)
     ctx = e.gemm(probs, v, 3, 2, batch_dims=(0, 1))
 
@@ -188,7 +198,7 @@ def _residual_f16(e: Computation, g: Value, bias: Value, res: Value) -> Value:
     def body(f, pg, pb, pr):
         rows, cols = pg.dims
         x = f.add(f.convert(pg, "f32"), f.broadcast(f.convert(pb, "f32"), (rows, cols), [1]))
-        return f.convert(f.add(x, f.convert(pr, "f32")), "f16")
+        return f.convert(f.add(x, f.convert(pr, "f32")), _FT)
     return e.fusion("kLoop", [g, bias, res], body)
 
 
@@ -196,12 +206,12 @@ def _ffn_act(e: Computation, g: Value, bias: Value) -> Value:
     def body(f, pg, pb):
         rows, cols = pg.dims
         x = f.add(f.convert(pg, "f32"), f.broadcast(f.convert(pb, "f32"), (rows, cols), [1]))
-        return f.convert(_gelu_tanh(f, x), "f16")
+        return f.convert(_gelu_tanh(f, x), _FT)
     return e.fusion("kLoop", [g, bias], body)
 
 
 def _layer_weights(e: Computation, prefix: str, H: int, F: int) -> dict:
-    c = lambda role, dims: e.elided_constant("f16", dims, f"{prefix}/{role}")
+    c = lambda role, dims: e.elided_constant(_FT, dims, f"{prefix}/{role}")
     return {
         "q_w": c("attention/query/kernel", (H, H)), "q_b": c("attention/query/bias", (H,)),
         "k_w": c("attention/key/kernel", (H, H)), "k_b": c("attention/key/bias", (H,)),
@@ -238,7 +248,7 @@ def bert_layer(B=1, S=128, H=768, NH=12, F=3072, eps=1e-12) -> ModelFixture:
     """One BERT encoder layer (post-LN, tanh-GELU) on a given hidden state."""
     mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
     e = mb.entry
-    hidden = e.parameter("f16", (B, S, H), "hidden_states")
+    hidden = e.parameter(_FT, (B, S, H), "hidden_states")
     mask = e.parameter("s32", (B, S), "attention_mask")
     W = _layer_weights(e, "bert/encoder/layer_0", H, F)
     h = e.bitcast(hidden, (B * S, H))
@@ -246,33 +256,44 @@ def bert_layer(B=1, S=128, H=768, NH=12, F=3072, eps=1e-12) -> ModelFixture:
     e.set_tuple_root([e.bitcast(out, (B, S, H))])
     return ModelFixture(
         "bert_layer", mb.text(),
-        [{"name": "hidden_states", "dtype": "f16", "dims": [B, S, H], "kind": "normal"},
+        [{"name": "hidden_states", "dtype": _FT, "dims": [B, S, H], "kind": "normal"},
          {"name": "attention_mask", "dtype": "s32", "dims": [B, S], "kind": "ones_mask"}],
-        mb.constants, [{"dtype": "f16", "dims": [B, S, H]}],
+        mb.constants, [{"dtype": _FT, "dims": [B, S, H]}],
         dict(B=B, S=S, H=H, NH=NH, F=F, L=1))
 
 
 def bert_encoder(L=12, B=1, S=128, H=768, NH=12, F=3072, vocab=30522, max_pos=512, types=2,
-                 eps=1e-12, mask_kind="ones_mask") -> ModelFixture:
+                 eps=1e-12, mask_kind="ones_mask", ftype="f16") -> ModelFixture:
     """Full BERT encoder: word + position + segment embedding gather, LayerNorm, L layers.
     Entry parameters are the three s32[B,S] tensors of the reference's example input
-    (examples/data/bert_bs1.npy; 512 B each at B=1,S=128, README.md:192-194)."""
+    (examples/data/bert_bs1.npy; 512 B each at B=1,S=128, README.md:192-194).
+    ftype: storage type of weights and activations, "f16" (the reference's) or "bf16"."""
+    global _FT
+    assert ftype in ("f16", "bf16")
+    saved, _FT = _FT, ftype
+    try:
+        return _bert_encoder(L, B, S, H, NH, F, vocab, max_pos, types, eps, mask_kind)
+    finally:
+        _FT = saved
+
+
+def _bert_encoder(L, B, S, H, NH, F, vocab, max_pos, types, eps, mask_kind) -> ModelFixture:
     mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
     e = mb.entry
     ids = e.parameter("s32", (B, S), "input_ids")
     mask = e.parameter("s32", (B, S), "attention_mask")
     tts = e.parameter("s32", (B, S), "token_type_ids")
-    word = e.elided_constant("f16", (vocab, H), "bert/embeddings/word_embeddings")
-    pos = e.elided_constant("f16", (max_pos, H), "bert/embeddings/position_embeddings")
-    typ = e.elided_constant("f16", (types, H), "bert/embeddings/token_type_embeddings")
-    emb_g = e.elided_constant("f16", (H,), "bert/embeddings/LayerNorm/gamma")
-    emb_b = e.elided_constant("f16", (H,), "bert/embeddings/LayerNorm/beta")
+    word = e.elided_constant(_FT, (vocab, H), "bert/embeddings/word_embeddings")
+    pos = e.elided_constant(_FT, (max_pos, H), "bert/embeddings/position_embeddings")
+    typ = e.elided_constant(_FT, (types, H), "bert/embeddings/token_type_embeddings")
+    emb_g = e.elided_constant(_FT, (H,), "bert/embeddings/LayerNorm/gamma")
+    emb_b = e.elided_constant(_FT, (H,), "bert/embeddings/LayerNorm/beta")
 
     def emb_body(f, pi, pt, pw, pp, pty):
         w = f.convert(f.gather_rows(pw, pi), "f32")
         t = f.convert(f.gather_rows(pty, pt), "f32")
         p = f.convert(f.broadcast(f.slice(pp, (0, 0), (S, H)), (B, S, H), [1, 2]), "f32")
-        return f.convert(f.add(f.add(w, p), t), "f16")
+        return f.convert(f.add(f.add(w, p), t), _FT)
     emb = e.fusion("kLoop", [ids, tts, word, pos, typ], emb_body)
     h = _layer_norm(e, mb, e.bitcast(emb, (B * S, H)), emb_g, emb_b, eps)
     mask_add = _additive_mask(e, mask)
@@ -288,7 +309,7 @@ def bert_encoder(L=12, B=1, S=128, H=768, NH=12, F=3072, vocab=30522, max_pos=51
         [{"name": "input_ids", "dtype": "s32", "dims": [B, S], "kind": "token_ids", "vocab": vocab},
          mparam,
          {"name": "token_type_ids", "dtype": "s32", "dims": [B, S], "kind": "zeros"}],
-        mb.constants, [{"dtype": "f16", "dims": [B, S, H]}],
+        mb.constants, [{"dtype": _FT, "dims": [B, S, H]}],
         dict(B=B, S=S, H=H, NH=NH, F=F, L=L, vocab=vocab))
 
 
@@ -306,17 +327,17 @@ def gemm_stage(M=6144, N=4096, K=1024) -> ModelFixture:
     constant f16[K,N] weights, f16[M,N] result.  Two stages, one grid barrier."""
     mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
     e = mb.entry
-    x = e.parameter("f16", (M, K), "activations")
+    x = e.parameter(_FT, (M, K), "activations")
 
     def body(f, p):
-        return f.convert(f.mul(f.convert(p, "f32"), f.splat("f32", 0.5, p.dims)), "f16")
+        return f.convert(f.mul(f.convert(p, "f32"), f.splat("f32", 0.5, p.dims)), _FT)
     a = e.fusion("kLoop", [x], body)
-    w = e.elided_constant("f16", (K, N), "gemm_stage/kernel")
+    w = e.elided_constant(_FT, (K, N), "gemm_stage/kernel")
     e.set_tuple_root([e.gemm(a, w, 1, 0)])
     return ModelFixture(
         f"gemm_stage_{M}x{N}x{K}", mb.text(),
-        [{"name": "activations", "dtype": "f16", "dims": [M, K], "kind": "normal"}],
-        mb.constants, [{"dtype": "f16", "dims": [M, N]}], dict(M=M, N=N, K=K))
+        [{"name": "activations", "dtype": _FT, "dims": [M, K], "kind": "normal"}],
+        mb.constants, [{"dtype": _FT, "dims": [M, N]}], dict(M=M, N=N, K=K))
 
 
 def gpt2(L=12, B=4, S=512, H=768, NH=12, F=3072, vocab=50257, max_pos=1024, eps=1e-5) -> ModelFixture:
@@ -326,13 +347,13 @@ def gpt2(L=12, B=4, S=512, H=768, NH=12, F=3072, vocab=50257, max_pos=1024, eps=
     mb = HloModuleBuilder("cluster_0__XlaCompiledKernel_true__XlaNumConstantArgs_0_.1")
     e = mb.entry
     ids = e.parameter("s32", (B, S), "input_ids")
-    wte = e.elided_constant("f16", (vocab, H), "gpt2/wte")
-    wpe = e.elided_constant("f16", (max_pos, H), "gpt2/wpe")
+    wte = e.elided_constant(_FT, (vocab, H), "gpt2/wte")
+    wpe = e.elided_constant(_FT, (max_pos, H), "gpt2/wpe")
 
     def emb_body(f, pi, pw, pp):
         w = f.convert(f.gather_rows(pw, pi), "f32")
         p = f.convert(f.broadcast(f.slice(pp, (0, 0), (S, H)), (B, S, H), [1, 2]), "f32")
-        return f.convert(f.add(w, p), "f16")
+        return f.convert(f.add(w, p), _FT)
     h = e.bitcast(e.fusion("kLoop", [ids, wte, wpe], emb_body), (B * S, H))
     D = H // NH
     for l in range(L):
@@ -343,15 +364,15 @@ def gpt2(L=12, B=4, S=512, H=768, NH=12, F=3072, vocab=50257, max_pos=1024, eps=
         m = _layer_norm(e, mb, h, W["ln2_g"], W["ln2_b"], eps)
         act = _ffn_act(e, e.gemm(m, W["f1_w"], 1, 0), W["f1_b"])
         h = _residual_f16(e, e.gemm(act, W["f2_w"], 1, 0), W["f2_b"], h)
-    lnf_g = e.elided_constant("f16", (H,), "gpt2/ln_f/gamma")
-    lnf_b = e.elided_constant("f16", (H,), "gpt2/ln_f/beta")
+    lnf_g = e.elided_constant(_FT, (H,), "gpt2/ln_f/gamma")
+    lnf_b = e.elided_constant(_FT, (H,), "gpt2/ln_f/beta")
     hf = _layer_norm(e, mb, h, lnf_g, lnf_b, eps)
     logits = e.gemm(hf, wte, 1, 1)
     e.set_tuple_root([e.bitcast(logits, (B, S, vocab))])
     return ModelFixture(
         f"gpt2_L{L}_H{H}", mb.text(),
         [{"name": "input_ids", "dtype": "s32", "dims": [B, S], "kind": "token_ids", "vocab": vocab}],
-        mb.constants, [{"dtype": "f16", "dims": [B, S, vocab]}],
+        mb.constants, [{"dtype": _FT, "dims": [B, S, vocab]}],
         dict(B=B, S=S, H=H, NH=NH, F=F, L=L, vocab=vocab, eps=eps))
 
 
@@ -363,23 +384,23 @@ def vit(L=12, B=8, image=224, patch=16, H=768, NH=12, F=3072, eps=1e-6) -> Model
     e = mb.entry
     G = image // patch
     S = G * G + 1
-    pixels = e.parameter("f16", (B, 3, image, image), "pixel_values")
-    filt = e.elided_constant("f16", (H, patch, patch, 3), "vit/embeddings/patch_embeddings/kernel")
-    pbias = e.elided_constant("f16", (H,), "vit/embeddings/patch_embeddings/bias")
-    cls = e.elided_constant("f16", (1, 1, H), "vit/embeddings/cls_token")
-    pos = e.elided_constant("f16", (S, H), "vit/embeddings/position_embeddings")
+    pixels = e.parameter(_FT, (B, 3, image, image), "pixel_values")
+    filt = e.elided_constant(_FT, (H, patch, patch, 3), "vit/embeddings/patch_embeddings/kernel")
+    pbias = e.elided_constant(_FT, (H,), "vit/embeddings/patch_embeddings/bias")
+    cls = e.elided_constant(_FT, (1, 1, H), "vit/embeddings/cls_token")
+    pos = e.elided_constant(_FT, (S, H), "vit/embeddings/position_embeddings")
     nhwc = e.fusion("kLoop", [pixels], lambda f, px: f.transpose(px, (0, 2, 3, 1)))
     conv = e.conv_forward(nhwc, filt, stride=(patch, patch))
 
     def bias_body(f, pc, pb):
         x = f.add(f.convert(pc, "f32"), f.broadcast(f.convert(pb, "f32"), pc.dims, [3]))
-        return f.convert(x, "f16")
+        return f.convert(x, _FT)
     patches = e.fusion("kLoop", [conv, pbias], bias_body)
 
     def emb_body(f, pp, pc, ppos):
         tok = f.concatenate([f.broadcast(f.reshape(pc, (H,)), (B, 1, H), [2]), f.reshape(pp, (B, G * G, H))], 1)
         x = f.add(f.convert(tok, "f32"), f.broadcast(f.convert(ppos, "f32"), (B, S, H), [1, 2]))
-        return f.convert(x, "f16")
+        return f.convert(x, _FT)
     h = e.bitcast(e.fusion("kLoop", [patches, cls, pos], emb_body), (B * S, H))
     D = H // NH
     for l in range(L):
@@ -390,14 +411,14 @@ def vit(L=12, B=8, image=224, patch=16, H=768, NH=12, F=3072, eps=1e-6) -> Model
         m = _layer_norm(e, mb, h, W["ln2_g"], W["ln2_b"], eps)
         act = _ffn_act(e, e.gemm(m, W["f1_w"], 1, 0), W["f1_b"])
         h = _residual_f16(e, e.gemm(act, W["f2_w"], 1, 0), W["f2_b"], h)
-    lnf_g = e.elided_constant("f16", (H,), "vit/layernorm/gamma")
-    lnf_b = e.elided_constant("f16", (H,), "vit/layernorm/beta")
+    lnf_g = e.elided_constant(_FT, (H,), "vit/layernorm/gamma")
+    lnf_b = e.elided_constant(_FT, (H,), "vit/layernorm/beta")
     out = _layer_norm(e, mb, h, lnf_g, lnf_b, eps)
     e.set_tuple_root([e.bitcast(out, (B, S, H))])
     return ModelFixture(
         f"vit_L{L}_H{H}", mb.text(),
-        [{"name": "pixel_values", "dtype": "f16", "dims": [B, 3, image, image], "kind": "uniform_pm1"}],
-        mb.constants, [{"dtype": "f16", "dims": [B, S, H]}],
+        [{"name": "pixel_values", "dtype": _FT, "dims": [B, 3, image, image], "kind": "uniform_pm1"}],
+        mb.constants, [{"dtype": _FT, "dims": [B, S, H]}],
         dict(B=B, S=S, H=H, NH=NH, F=F, L=L, image=image, patch=patch, eps=eps))
 
 

@@ -16,7 +16,7 @@ import torch
 
 from .binding import MonoNNModule
 
-_TORCH_DTYPE = {"f16": torch.float16, "f32": torch.float32, "s32": torch.int32, "s64": torch.int64, "pred": torch.bool,
+_TORCH_DTYPE = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32, "s32": torch.int32, "s64": torch.int64, "pred": torch.bool,
                 "u8": torch.uint8, "s8": torch.int8}
 _REGISTRY: Dict[int, "MonoNNFunction"] = {}
 

@@ -59,6 +59,12 @@ the HLO as written, like this file; tests/test_oracle_pinning_ops.py pins that c
 precision="as_written": every f16-typed instruction result is rounded to IEEE half (what the
 HLO says).  precision="fp32": f16 is carried as float32 without rounding (the "fp32 reference"
 the tolerance max-abs-err <= 2e-2 / cosine >= 0.9999 is stated against).
+
+bf16 (not a type of the reference; the HIP path adds it): carried as float32, rounded to nearest
+even on the upper 16 bits of the pattern after every bf16-typed instruction in as_written mode,
+handed in as uint16 bit patterns and returned as float32 values.  Pinned against torch.bfloat16
+(conversions bit for bit including ties, infinities and NaN; a GEMM + element-wise program) in
+tests/test_oracle_pinning.py.
 """
 from __future__ import annotations
 
@@ -70,7 +76,28 @@ import numpy as np
 
 _NP = {"pred": np.bool_, "s8": np.int8, "u8": np.uint8, "s16": np.int16, "u16": np.uint16,
        "s32": np.int32, "u32": np.uint32, "s64": np.int64, "u64": np.uint64,
-       "f16": np.float16, "f32": np.float32, "f64": np.float64}
+       "f16": np.float16, "f32": np.float32, "f64": np.float64,
+       # NumPy has no bfloat16: bf16 values are carried as float32 and rounded to bf16 after every bf16-typed
+       # instruction (round_to_bf16); host buffers of that type are uint16 bit patterns (bf16_from_bits)
+       "bf16": np.float32}
+
+
+def bf16_from_bits(bits) -> np.ndarray:
+    """bf16 bit patterns (uint16) -> their values as float32: bf16 is the upper half of the f32 pattern."""
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def bf16_to_bits(values) -> np.ndarray:
+    """float32 values -> bf16 bit patterns, round to nearest, ties to even, on the 16 bits that are dropped
+    (what v_cvt_pk_bf16_f32 and XLA's convert do); NaN stays a quiet NaN."""
+    u = np.ascontiguousarray(values, dtype=np.float32).view(np.uint32)
+    rounded = ((u + np.uint32(0x7FFF) + ((u >> 16) & np.uint32(1))) >> 16).astype(np.uint16)
+    nan = np.isnan(np.asarray(values, dtype=np.float32))
+    return np.where(nan, ((u >> 16) | np.uint32(0x40)).astype(np.uint16), rounded)
+
+
+def round_to_bf16(values) -> np.ndarray:
+    return bf16_from_bits(bf16_to_bits(values)).reshape(np.shape(values))
 
 
 class Shape:
@@ -317,6 +344,10 @@ class Evaluator:
         """A buffer handed in by the host (entry parameter, constant payload): its memory image, dims listed from the
         slowest-varying one; with the default layout that is the logical array itself."""
         a = np.asarray(a)
+        if shape.dtype == "bf16":
+            if a.dtype != np.uint16:
+                raise ValueError("a bf16 buffer is handed in as uint16 bit patterns")
+            a = bf16_from_bits(a)
         if tuple(a.shape) != tuple(shape.memory_dims()):
             raise ValueError(f"shape mismatch: got {a.shape}, HLO says {shape.dims} laid out as {shape.memory_dims()}")
         return _from_memory(a, shape).astype(self.np_dtype(shape.dtype), copy=False)
@@ -327,6 +358,8 @@ class Evaluator:
         for ins in comp.instrs:
             self._top, self._shapes = top, shapes
             env[ins.name] = self._eval(ins, env, args)
+            if not self.fp32 and ins.shape.tuple_shapes is None and ins.shape.dtype == "bf16" and isinstance(env[ins.name], np.ndarray):
+                env[ins.name] = round_to_bf16(env[ins.name])
             if top and self._keep and isinstance(env[ins.name], np.ndarray):
                 self.trace[ins.name] = env[ins.name]
         res = env[comp.root.name]

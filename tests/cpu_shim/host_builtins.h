@@ -69,3 +69,12 @@ inline host_float4 __builtin_amdgcn_mfma_f32_16x16x32_f16(host_half8 a, host_hal
   c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
   return c;
 }
+typedef __bf16 host_bf16x8 __attribute__((ext_vector_type(8)));
+inline host_float16 __builtin_amdgcn_mfma_f32_32x32x16_bf16(host_bf16x8 a, host_bf16x8 b, host_float16 c, int, int, int) {
+  c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];   // keeps the operand loads alive
+  return c;
+}
+inline host_float4 __builtin_amdgcn_mfma_f32_16x16x32_bf16(host_bf16x8 a, host_bf16x8 b, host_float4 c, int, int, int) {
+  c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];
+  return c;
+}

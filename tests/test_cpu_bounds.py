@@ -146,3 +146,19 @@ def test_whatever_specification_is_accepted_stays_inside_the_buffers():
         ok, msg = check_module(fx.hlo_text, t)
         assert ok, msg + "\n" + t
     assert accepted >= 20
+
+
+def test_bf16_encoder_and_gemms():
+    import json
+    fx = models.bert_encoder(L=1, B=2, S=64, H=128, NH=2, F=256, vocab=300, max_pos=64, ftype="bf16", mask_kind="length_mask")
+    ok, msg = check_module(fx.hlo_text)
+    assert ok, msg
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    for name, e in spec["gemm_spec_list"].items():
+        c = e["cutlass_config"]
+        if name.startswith("cublas_gemm_") and c["split_k"] == 1:
+            c["threadblockshape"].update(m=64, n=64, k=32)
+            c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+            c["stages"] = 2
+    ok, msg = check_module(fx.hlo_text, json.dumps(spec), opt="-O1")
+    assert ok, "LDS-staged tiles: " + msg

@@ -336,3 +336,89 @@ def test_variadic_reduce_bit_exact(gpu_device, rows, n, direction, axis):
     if n <= 1000:
         wv, wi = hlo_interp.evaluate(text, [x], {})
         assert np.array_equal(i, wi) and np.array_equal(v.view(np.uint16), wv.view(np.uint16))
+
+
+# ---- bf16 (not in the reference, whose tiles are half and float): the same kernels on the bf16 forms of the MFMAs ----
+def _bf16_check(got_bits, want32, what, steps=4.0, atol=2e-2):
+    """bf16 results against fp32 values: within `steps` bf16 spacings (2^-8 relative) of the value's magnitude, plus
+    `atol` for sums whose terms cancel."""
+    from mononn_amd import bf16
+    assert got_bits.dtype == np.uint16
+    g = bf16.from_bits(got_bits).astype(np.float64).ravel()
+    w = want32.astype(np.float64).ravel()
+    assert np.all(np.isfinite(g))
+    err = np.abs(g - w)
+    bound = steps * 2.0 ** -8 * np.abs(w) + atol
+    cos = float(g @ w / (np.linalg.norm(g) * np.linalg.norm(w) + 1e-30))
+    print(f"{what}: max_abs_err={err.max():.3e} cosine={cos:.6f}")
+    assert (err <= bound).all(), f"{what}: {err.max()} at magnitude {np.abs(w)[err.argmax()]}"
+    assert cos >= 0.9999
+
+
+@pytest.mark.parametrize("case", [
+    dict(M=128, N=768, K=768, b_const=True),                       # weight GEMM: constant packed in fragment order
+    dict(M=128, N=96, K=64),                                       # [K,N] parameter operand, gathered per lane
+    dict(M=128, N=128, K=64, batch=(2, 3), rhs_c=3, alpha=0.125),  # batched, both operands k-contiguous
+    dict(M=100, N=52, K=96, rhs_c=1),                              # ragged M / N
+    dict(M=64, N=48, K=40, rhs_c=1),                               # K off the MFMA step: zero-filled last step
+    dict(M=256, N=1001, K=128, rhs_c=1, b_const=True),             # odd N: four columns per store where they fit
+    dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                      # A stored [K,M]: per-element fallback
+])
+def test_bf16_gemm_cases(gpu_device, case):
+    from mononn_amd import bf16
+    mb, a_dims, b_dims, d_dims = gemm_module(dtype="bf16", **case)
+    rng = np.random.default_rng(5)
+    a = bf16.to_bits(rng.normal(0, 1, a_dims))
+    b = bf16.to_bits(rng.normal(0, 1, b_dims))
+    text = mb.text()
+    consts = {n: b for n in mb.constants}
+    inputs = [a] if case.get("b_const") else [a, b]
+    (got,), m = run_module(text, inputs, consts, [{"dtype": "bf16", "dims": d_dims}])
+    if not (case.get("lhs_c") == 0):
+        assert ", true>(reinterpret_cast<const half_t*>(" in m.get_source("main.hip")
+    want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
+    # one rounding of an exactly accumulated sum: half a bf16 spacing, a little more for the summation order
+    _bf16_check(got, want, f"bf16 gemm {case}", steps=1.0, atol=2e-3 * float(np.abs(want).max()))
+
+
+def test_bf16_gemm_on_lds_staged_tiles_with_split_k_neighbours(gpu_device):
+    import json
+    from mononn_amd import bf16
+    M, N, K = 512, 384, 512
+    mb, a_dims, b_dims, d_dims = gemm_module(M=M, N=N, K=K, b_const=True, dtype="bf16")
+    text = mb.text()
+    rng = np.random.default_rng(6)
+    a = bf16.to_bits(rng.normal(0, 1, a_dims))
+    consts = {n: bf16.to_bits(rng.normal(0, 1, b_dims)) for n in mb.constants}
+    want = hlo_interp.evaluate(text, [a], consts, "fp32")[0]
+    for tile in (dict(m=128, n=128, k=32), dict(m=64, n=192, k=64)):
+        spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+        for e in spec["gemm_spec_list"].values():
+            c = e["cutlass_config"]
+            c["threadblockshape"].update(tile)
+            c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+            c["stages"] = 2
+        (got,), m = run_module(text, [a], consts, [{"dtype": "bf16", "dims": d_dims}], json.dumps(spec))
+        assert "gemm_tile_lds<" in m.get_source("main.hip")
+        m.close()
+        _bf16_check(got, want, f"bf16 LDS tile {tile}", steps=1.0, atol=2e-3 * float(np.abs(want).max()))
+
+
+def test_bf16_encoder_parity(gpu_device):
+    # two BERT layers with embeddings and padding masks, stored and multiplied in bf16: against the oracle run as
+    # written (every bf16 instruction rounded, as the kernel does) and against the unrounded fp32 evaluation
+    import json
+    fx = models.bert_encoder(L=2, B=2, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64, mask_kind="length_mask", ftype="bf16")
+    consts = fx.make_constants(27, "random")
+    inputs = fx.make_inputs(27)
+    (got,), m = run_module(fx.hlo_text, inputs, consts, fx.outputs)
+    assert m.get_source("main.hip").count(", true>(reinterpret_cast<const half_t*>(") >= 6   # the layers share their node functions
+    written = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "as_written")[0]
+    _bf16_check(got, written, "bf16 encoder against the oracle as written", steps=4.0, atol=3e-2)
+    free = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _bf16_check(got, free, "bf16 encoder against the fp32 evaluation", steps=8.0, atol=6e-2)
+    # split-K on the second feed-forward GEMM: fp32 partial sums, added by the LayerNorm stage, rounded once
+    gemms = _gemm_instr_names(fx.hlo_text)
+    split = {gemms[l * 6 + 5]: {"split_k": 4} for l in range(2)}
+    (got2,), m2 = run_module(fx.hlo_text, inputs, consts, fx.outputs, _spec_with(fx.hlo_text, gemm_overrides=split))
+    _bf16_check(got2, written, "bf16 encoder with split-K", steps=4.0, atol=3e-2)

@@ -177,7 +177,7 @@ HEAD = "HloModule cluster_9__t.1\n\n"
     (HEAD + "ENTRY %main {\n  %p = f32[<=4]{0} parameter(0)\n  ROOT %r = f32[<=4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f32[4,4]{1,0:T(2,2)} parameter(0)\n  ROOT %r = f32[4,4]{1,0} negate(%p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f32[4,4]{0,1:T(2,128)} parameter(0)\n  ROOT %r = f32[4,4]{0,1} negate(%p)\n}\n", "UNSUPPORTED"),
-    (HEAD + "ENTRY %main {\n  %p = bf16[4]{0} parameter(0)\n  ROOT %r = bf16[4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
+    (HEAD + "ENTRY %main {\n  %p = f8e4m3fn[4]{0} parameter(0)\n  ROOT %r = f8e4m3fn[4]{0} negate(%p)\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f32[1,4,4,1]{3,2,1,0} parameter(0)\n  %w = f32[1,1,1,1]{3,2,1,0} parameter(1)\n"
             "  ROOT %r = f32[1,4,4,1]{3,2,1,0} convolution(%p, %w), window={size=1x1}, dim_labels=b01f_01io->b01f\n}\n", "UNSUPPORTED"),
     (HEAD + "ENTRY %main {\n  %p = f16[4,4]{1,0} parameter(0)\n  ROOT %r = f16[4,4]{1,0} custom-call(%p), custom_call_target=\"__my$thing\"\n}\n",
@@ -637,3 +637,37 @@ def test_layer_norm_folding_moves_the_scale_into_the_weights_and_the_rest_into_t
     spec["mononn_hip"]["gemm_prologue_fusion"] = False
     m = MonoNNModule.compile(norm_gemm_module(True)[0], json.dumps(spec), build=False)
     assert "ln_stats[" not in m.get_source("main.hip") and m.launch_dims()["barriers"] >= 1
+
+
+def test_bf16_modules_take_the_bf16_mfma_on_the_same_tiles():
+    # bf16 is parsed, element-wise code computes through float and rounds where the HLO says bf16, weight GEMMs run
+    # on the direct tile or the LDS-staged tile with the bf16 form of the MFMA (last template argument), constants
+    # are packed in fragment order like f16 ones, and the attention stays three stages (the fused form is f16)
+    fx = models.bert_encoder(L=1, B=2, S=64, H=128, NH=2, F=256, vocab=300, max_pos=64, ftype="bf16")
+    m = MonoNNModule.compile(fx.hlo_text)          # hipRTC build
+    src = m.get_source("main.hip")
+    assert "__bf16" in src and "_Float16" not in src.split("extern \"C\"")[1]
+    calls = src.count("mononn_dev::gemm_tile<")
+    assert calls >= 6 and src.count(", true>(reinterpret_cast<const half_t*>(") == calls
+    assert m.launch_dims()["barriers"] == 9        # embeddings, QKV, scores, soft-max, context, out, LN, FFN1, FFN2, LN
+    packed = [c for c in m.constants() if c["role"].endswith("/kernel")]
+    assert packed and all(c["needs_payload"] for c in packed)
+    # the LDS-staged tile
+    spec = json.loads(m.get_tuning_spec())
+    n = 0
+    for name, e in spec["gemm_spec_list"].items():
+        c = e["cutlass_config"]
+        if name.startswith("cublas_gemm_") and c["split_k"] == 1:
+            c["threadblockshape"].update(m=64, n=64, k=32)
+            c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+            c["stages"] = 2
+            n += 1
+    assert n >= 4
+    lds = MonoNNModule.compile(fx.hlo_text, json.dumps(spec)).get_source("main.hip")
+    assert lds.count("mononn_dev::RowMajorA, true>(reinterpret_cast<const half_t*>(") >= 4 and lds.count("gemm_tile_lds<") >= 4
+    # a mixed GEMM is refused
+    bad = fx.hlo_text.replace("bf16[128,128]{1,0} custom-call(", "f16[128,128]{1,0} custom-call(", 1)
+    if bad != fx.hlo_text:
+        with pytest.raises(MonoNNError) as ei:
+            MonoNNModule.compile(bad, build=False)
+        assert ei.value.status in ("UNSUPPORTED", "PARSE_ERROR", "INVALID_ARGUMENT")

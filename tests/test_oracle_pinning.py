@@ -389,3 +389,59 @@ def test_variadic_reduce_is_argmax_with_first_index_on_ties():
     assert np.array_equal(i, np.argmax(x, axis=1).astype(np.int32)) and np.array_equal(v, x.max(axis=1))
     v, i = hlo_interp.evaluate(arg_reduce_module(7, 50, "LT"), [x], {})
     assert np.array_equal(i, np.argmin(x, axis=1).astype(np.int32)) and np.array_equal(v, x.min(axis=1))
+
+
+def test_bf16_conversions_match_torch_bfloat16():
+    # bf16 has no NumPy type: the oracle and the product's boundary both carry it as uint16 bit patterns and convert by
+    # rounding the float32 pattern to nearest even on its upper half.  torch.bfloat16 is the independent statement.
+    from mononn_amd import bf16
+    rng = np.random.default_rng(71)
+    x = np.concatenate([rng.normal(0, 1, 4096), rng.normal(0, 1e-3, 1024), rng.normal(0, 1e4, 1024),
+                        [0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, 65504.0, 3.3895314e38, 1e-40, -1e-40],
+                        # exact ties between two bf16 neighbours: 1 + 2^-8 (down to even), 1 + 3 * 2^-8 (up to even)
+                        [1.00390625, 1.01171875, -1.00390625, 257.0, 259.0]]).astype(np.float32)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    for to_bits, from_bits in ((hlo_interp.bf16_to_bits, hlo_interp.bf16_from_bits), (bf16.to_bits, bf16.from_bits)):
+        got = to_bits(x)
+        assert got.dtype == np.uint16 and np.array_equal(got, want)
+        back = from_bits(got)
+        assert np.array_equal(back, torch.from_numpy(want.view(np.int16)).view(torch.bfloat16).to(torch.float32).numpy())
+    assert np.isnan(hlo_interp.bf16_from_bits(hlo_interp.bf16_to_bits(np.array([np.nan], np.float32))))[0]
+    assert np.isnan(bf16.from_bits(bf16.to_bits(np.array([np.nan], np.float32))))[0]
+
+
+def test_bf16_program_as_written_rounds_like_torch_bfloat16():
+    # convert, an element-wise chain and a GEMM in bf16: every bf16-typed instruction result is a bf16 value
+    M, K, N = 24, 40, 16
+    mb = HloModuleBuilder("cluster_5__bf16_pin.1")
+    e = mb.entry
+    a = e.parameter("bf16", (M, K), "a")
+    b = e.parameter("bf16", (K, N), "b")
+    bias = e.parameter("f32", (N,), "bias")
+    d = e.gemm(a, b, 1, 0)
+
+    def body(f, pd, pb):
+        y = f.add(f.convert(pd, "f32"), f.broadcast(pb, (M, N), [1]))
+        h = f.convert(y, "bf16")                       # rounded
+        return f.mul(h, h)                             # bf16 x bf16 -> bf16: the product rounded once
+    out = e.fusion("kLoop", [d, bias], body)
+    e.set_tuple_root([out])
+    rng = np.random.default_rng(72)
+    av, bv = rng.normal(0, 1, (M, K)).astype(np.float32), rng.normal(0, 1, (K, N)).astype(np.float32)
+    biasv = rng.normal(0, 1, N).astype(np.float32)
+    a_bits, b_bits = hlo_interp.bf16_to_bits(av), hlo_interp.bf16_to_bits(bv)
+    got = hlo_interp.evaluate(mb.text(), [a_bits, b_bits, biasv], {}, "as_written")[0]
+    ta = torch.from_numpy(av).to(torch.bfloat16).to(torch.float32)
+    tb = torch.from_numpy(bv).to(torch.bfloat16).to(torch.float32)
+    dd = (ta.double() @ tb.double()).to(torch.float32).to(torch.bfloat16)          # GEMM result stored as bf16
+    h = (dd.to(torch.float32) + torch.from_numpy(biasv)).to(torch.bfloat16)
+    want = (h.to(torch.float32) * h.to(torch.float32)).to(torch.bfloat16).to(torch.float32).numpy()
+    assert got.dtype == np.float32
+    # fp32 accumulation order may move a GEMM element by one bf16 step before the squaring
+    steps = np.abs(got - want) / np.maximum(np.abs(want) * 2.0 ** -7, 1e-30)
+    assert (steps <= 2.5).all() and (got == want).mean() > 0.97
+    assert np.array_equal(hlo_interp.round_to_bf16(got), got)          # results are bf16 values
+    # the fp32 mode carries the same program without intermediate rounding
+    free = hlo_interp.evaluate(mb.text(), [a_bits, b_bits, biasv], {}, "fp32")[0]
+    exact = ((ta.double() @ tb.double()).float() + torch.from_numpy(biasv)).numpy() ** 2
+    assert np.allclose(free, exact, rtol=1e-5, atol=1e-5)
