@@ -1994,7 +1994,13 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
-  MONONN_CHECK(!d1.f32 && !d2.f32 && !d1.bf16 && !d2.bf16, kUnsupported) << "attention fusion is built for f16 (scores and probabilities are held as f16 between the two contractions)";
+  MONONN_CHECK(!d1.f32 && !d2.f32 && d1.bf16 == d2.bf16, kUnsupported) << "attention fusion needs both contractions in the same 2-byte type";
+  // scores and probabilities are held between the two contractions in the type the HLO gives them: f16, or bf16 with
+  // the bf16 form of the MFMA on the same bits (operands move as 16-byte pieces either way)
+  const bool bf = d1.bf16;
+  const std::string ET = bf ? "__bf16" : "_Float16";
+  const std::string MFMA = std::string("mononn_dev::mfma_16x16x32<") + (bf ? "true" : "false") + ">(";
+  MONONN_CHECK(!bf || !g3, kUnsupported) << "the projection inside the attention node is built for f16";
   MONONN_CHECK(K1 % 32 == 0 && N2 % 16 == 0, kUnsupported) << "attention fusion: head size must be an MFMA multiple";
   // A key count off the MFMA step (ViT: 197): every wave's slice is rounded up to whole steps of 32 keys; the keys
   // past the end are read from the last valid key (finite values, in range), take no part in the row reductions
@@ -2025,14 +2031,19 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   MONONN_CHECK(info.row_program && info.rows == d1.batch * M1 && info.row_len == N1, kUnsupported)
       << "attention fusion: the cluster between the GEMMs is not a row program over the first GEMM's rows";
   auto row_outs = external_outputs(prog, row_members);
-  MONONN_CHECK(row_outs.size() == 1 && row_outs[0]->shape.num_elements() == d1.batch * M1 * N1 && row_outs[0]->shape.dtype == DType::kF16, kUnsupported)
-      << "attention fusion: the row program must produce exactly one f16 matrix";
+  MONONN_CHECK(row_outs.size() == 1 && row_outs[0]->shape.num_elements() == d1.batch * M1 * N1 && row_outs[0]->shape.dtype == (bf ? DType::kBF16 : DType::kF16), kUnsupported)
+      << "attention fusion: the row program must produce exactly one matrix of the operands' type";
   const Instr* P = row_outs[0];
 
   PointerTable ptrs;
   std::string pq = ptrs.input(prog.storage_root(g1->operands[0]));
   std::string pk = ptrs.input(prog.storage_root(g1->operands[1]));
   std::string pv = ptrs.input(prog.storage_root(g2->operands[1]));
+  if (bf) {
+    pq = "reinterpret_cast<const _Float16*>(" + pq + ")";
+    pk = "reinterpret_cast<const _Float16*>(" + pk + ")";
+    pv = "reinterpret_cast<const _Float16*>(" + pv + ")";
+  }
   const size_t first_epi = ptrs.entries.size();
 
   CodeBuffer cb;
@@ -2264,7 +2275,7 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.open("for (int x = 0; x < " + S(per) + "; ++x)");
     cb.line("const int j = jg * " + S(G) + " + x / " + S(KS1) + ";");
     cb.line("if (x % " + S(KS1) + " == 0) sacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};");
-    cb.line("sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb[jg & 1][x], qf[x % " + S(KS1) + "], sacc[j], 0, 0, 0);");
+    cb.line("sacc[j] = " + MFMA + "kb[jg & 1][x], qf[x % " + S(KS1) + "], sacc[j]);");
     cb.close();
     cb.line("__builtin_amdgcn_sched_barrier(0);");
     cb.close();
@@ -2273,15 +2284,15 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
   cb.line("sacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};");
   cb.line("#pragma unroll");
-  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(" + kfrag + ", qf[ks], sacc[j], 0, 0, 0);");
+  cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) sacc[j] = " + MFMA + "" + kfrag + ", qf[ks], sacc[j]);");
   cb.close();
   }
   // the first GEMM's result as the HLO defines it: scaled, rounded to f16
-  cb.line("_Float16 sv[" + S(NT1) + "][4], pr[" + S(NT1) + "][4];");
+  cb.line(ET + " sv[" + S(NT1) + "][4], pr[" + S(NT1) + "][4];");
   cb.line("#pragma unroll");
   cb.open("for (int j = 0; j < " + S(NT1) + "; ++j)");
   cb.line("#pragma unroll");
-  cb.line(std::string("for (int r = 0; r < 4; ++r) sv[j][r] = (_Float16)(sacc[j][r]") + (d1.alpha == 1.0 ? "" : " * " + alpha_lit + "f") + ");");
+  cb.line(std::string("for (int r = 0; r < 4; ++r) sv[j][r] = (" + ET + ")(sacc[j][r]") + (d1.alpha == 1.0 ? "" : " * " + alpha_lit + "f") + ");");
   cb.close();
   // ---- row program on the register-resident rows ------------------------------------------------
   auto bind_elem = [&](int j, int r) { em.bind(g1, elem_index(j, r), "sv[" + S(j) + "][" + S(r) + "]"); };
@@ -2316,11 +2327,14 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   for (int j = 0; j < NT1; ++j)
     for (int r = 0; r < 4; ++r) {
       bind_elem(j, r);
-      if (ragged) cb.line("pr[" + S(j) + "][" + S(r) + "] = colv[" + S(j) + "][" + S(r) + "] ? (_Float16)(" + em.value(em.resolve_output(P), elem_index(j, r)) + ") : (_Float16)0;");
+      if (ragged) cb.line("pr[" + S(j) + "][" + S(r) + "] = colv[" + S(j) + "][" + S(r) + "] ? (" + ET + ")(" + em.value(em.resolve_output(P), elem_index(j, r)) + ") : (" + ET + ")0;");
       else cb.line("pr[" + S(j) + "][" + S(r) + "] = " + em.value(em.resolve_output(P), elem_index(j, r)) + ";");
     }
   em.unbind(g1);
   // ---- second contraction ---------------------------------------------------------------------------
+  // the probabilities of one k step as an MFMA operand (bf16: the same 16 bytes under the f16 vector type)
+  const std::string pf_elems = "pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]";
+  const std::string pf_line = bf ? "const half8_t pf = __builtin_bit_cast(half8_t, bf16x8_t{" + pf_elems + "});" : "const half8_t pf = {" + pf_elems + "};";
   cb.line("float4_t oacc[" + S(NT2) + "];");
   cb.line("#pragma unroll");
   cb.line("for (int t = 0; t < " + S(NT2) + "; ++t) oacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};");
@@ -2340,19 +2354,19 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.line("#pragma unroll");
     cb.open("for (int y = 0; y < " + S(G2) + "; ++y)");
     cb.line("const int ks = kg * " + S(G2) + " + y;");
-    cb.line("const half8_t pf = {pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]};");
+    cb.line(pf_line);
     cb.line("#pragma unroll");
-    cb.line("for (int t = 0; t < " + S(NT2) + "; ++t) oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vb[kg & 1][y * " + S(NT2) + " + t], pf, oacc[t], 0, 0, 0);");
+    cb.line("for (int t = 0; t < " + S(NT2) + "; ++t) oacc[t] = " + MFMA + "vb[kg & 1][y * " + S(NT2) + " + t], pf, oacc[t]);");
     cb.close();
     cb.line("__builtin_amdgcn_sched_barrier(0);");
     cb.close();
   } else {
   cb.line("#pragma unroll");
   cb.open("for (int ks = 0; ks < " + S(KS2) + "; ++ks)");
-  cb.line("const half8_t pf = {pr[2 * ks][0], pr[2 * ks][1], pr[2 * ks][2], pr[2 * ks][3], pr[2 * ks + 1][0], pr[2 * ks + 1][1], pr[2 * ks + 1][2], pr[2 * ks + 1][3]};");
+  cb.line(pf_line);
   cb.line("#pragma unroll");
   cb.open("for (int t = 0; t < " + S(NT2) + "; ++t)");
-  cb.line("oacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(" + vfrag + ", pf, oacc[t], 0, 0, 0);");
+  cb.line("oacc[t] = " + MFMA + "" + vfrag + ", pf, oacc[t]);");
   cb.close();
   cb.close();
   }
@@ -2408,7 +2422,7 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.open("for (int jj = 0; jj < " + S(NJ) + "; ++jj)");
     cb.line("float4_t pacc = {0.f, 0.f, 0.f, 0.f};");
     cb.line("#pragma unroll");
-    cb.line("for (int s = 0; s < " + S(KS3) + "; ++s) pacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pre_w.v[jj * " + S(KS3) + " + s], af[s], pacc, 0, 0, 0);");
+    cb.line("for (int s = 0; s < " + S(KS3) + "; ++s) pacc = " + MFMA + "pre_w.v[jj * " + S(KS3) + " + s], af[s], pacc);");
     cb.line("const int nt = jj * " + S(KW) + " + kw;");
     cb.open("if (m_valid && nt < " + S(NT3) + ")");
     const std::string a3 = d3.alpha == 1.0 ? "" : " * " + lit(d3.alpha);

@@ -642,14 +642,15 @@ def test_layer_norm_folding_moves_the_scale_into_the_weights_and_the_rest_into_t
 def test_bf16_modules_take_the_bf16_mfma_on_the_same_tiles():
     # bf16 is parsed, element-wise code computes through float and rounds where the HLO says bf16, weight GEMMs run
     # on the direct tile or the LDS-staged tile with the bf16 form of the MFMA (last template argument), constants
-    # are packed in fragment order like f16 ones, and the attention stays three stages (the fused form is f16)
+    # are packed in fragment order like f16 ones, and the attention is one fused stage holding scores and
+    # probabilities as bf16 between its two contractions
     fx = models.bert_encoder(L=1, B=2, S=64, H=128, NH=2, F=256, vocab=300, max_pos=64, ftype="bf16")
     m = MonoNNModule.compile(fx.hlo_text)          # hipRTC build
     src = m.get_source("main.hip")
     assert "__bf16" in src and "_Float16" not in src.split("extern \"C\"")[1]
     calls = src.count("mononn_dev::gemm_tile<")
-    assert calls >= 6 and src.count(", true>(reinterpret_cast<const half_t*>(") == calls
-    assert m.launch_dims()["barriers"] == 9        # embeddings, QKV, scores, soft-max, context, out, LN, FFN1, FFN2, LN
+    assert calls >= 4 and src.count(", true>(reinterpret_cast<const half_t*>(") == calls
+    assert m.launch_dims()["barriers"] == 7 and "mononn_dev::mfma_16x16x32<true>(" in src   # as the f16 encoder
     packed = [c for c in m.constants() if c["role"].endswith("/kernel")]
     assert packed and all(c["needs_payload"] for c in packed)
     # the LDS-staged tile
