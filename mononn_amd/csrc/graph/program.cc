@@ -630,7 +630,7 @@ struct Builder {
     auto use = [&](const Instr* operand, bool fits, int64_t rows, int64_t k, Order order, bool perm_ok) {
       const Instr* root = p.storage_root(operand);
       fits = fits && rows % 16 == 0 && k % 32 == 0 && p.producer.count(root) && !live.count(root) && (perm_ok || !p.physical_perm.count(root)) &&
-             root->shape.dtype == hlo::DType::kF16 && root->shape.num_elements() == rows * k &&
+             hlo::is_half_float(root->shape.dtype) && root->shape.num_elements() == rows * k &&
              (!want.count(root) || (want[root].k == k && want[root].order == order));
       if (fits) want[root] = {k, order};
       else spoiled.insert(root);
