@@ -1734,7 +1734,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   }
   CodeBuffer fb;
   std::string conv_struct, preload_body;
-  bool preload = false;
+  bool preload = false, rows_lds = false;
   int preload_regs = 0;
   if (g.split_k <= 1) fb.line(epi.init_line);
   if (fold) fb.line("epi.ln_stats = reinterpret_cast<const float*>(smem + " + S(fold_stats_offset) + ");");
@@ -1811,12 +1811,19 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         call << "mononn_dev::gemm_tile_f32<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << g.K << ", " << (b_along_n ? "true" : "false") << ", "
              << (epi.along_m ? "true" : "false") << ", @NAME@_epi>(" << pa << " + (long)bidx * " << g.a_batch_stride << ", " << pb << " + (long)bidx * " << g.b_batch_stride
              << ", " << g.M << ", " << g.N << ", " << g.K << ", " << (b_along_n ? g.N : g.K) << ", bidx, tile_m, tile_n, epi";
-      else if (t.stages >= 2)
+      else if (t.stages >= 2) {
+        // results stored row-major go through LDS a fragment row at a time, so that the epilogue's stores and operand
+        // loads cover whole rows of the wave's tile (results in fragment order are written in 8-byte pieces of
+        // different 16-byte runs either way)
+        // (a result in fragment order is already written as runs of 256 contiguous bytes per instruction; dealt out in
+        // that order through LDS it came out slower)
+        rows_lds = !epi.along_m && !epi_outputs.empty();
+        for (auto* o : epi_outputs) rows_lds = rows_lds && !prog.physical_tile.count(prog.storage_root(o)) && !prog.physical_perm.count(prog.storage_root(o));
         call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", "
              << (g.a_packed ? "true" : "false") << ", " << (g.b_packed ? "true" : "false") << ", " << (epi.along_m ? "true" : "false") << ", " << t.bk
-             << ", @NAME@_epi" << (g.bf16 ? ", mononn_dev::RowMajorA, true" : "") << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
+             << ", @NAME@_epi" << (g.bf16 || rows_lds ? std::string(", mononn_dev::RowMajorA, ") + (g.bf16 ? "true" : "false") + (rows_lds ? ", true" : "") : std::string()) << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
              << b_expr.str() << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
-      else
+      } else
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
              << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
              << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
@@ -1848,7 +1855,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     }
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
-    if (t.stages >= 2) smem = 2 * (t.bm + t.bn) * t.bk * 2;
+    if (t.stages >= 2) smem = std::max(2 * (t.bm + t.bn) * t.bk * 2, rows_lds ? ls.waves() * 32 * (t.bn / t.wn + 4) * 4 : 0);
     smem = std::max(smem, pro.smem);
   } else {
     const int64_t total = g.batch * g.M * g.N;

@@ -898,7 +898,7 @@ __device__ __forceinline__ float16_t mfma_32x32x16(half8_t a, half8_t b, float16
 
 // BK: k extent of one LDS buffer (a multiple of 32); K a multiple of 32.
 template <int BM, int BN, int WM, int WN, int K, int KTOTAL, bool PACKED_A, bool PACKED_B, bool D_ALONG_M, int BK, class Epi,
-          class AMap = RowMajorA, bool BF16 = false>
+          class AMap = RowMajorA, bool BF16 = false, bool ROWS_LDS = false>
 __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, int M, int N, int lda, int ldb, int batch, int tile_m,
                                               int tile_n, Epi& epi, char* smem, const AMap& amap = AMap()) {
   constexpr int NW = WM * WN;
@@ -1004,13 +1004,24 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   constexpr int PRE_REGS = (int)(sizeof(typename Epi::Pre) + 3) / 4 * TN * 4 * TM;
   constexpr bool PRE_ALL = sizeof(typename Epi::Pre) > 1 && PRE_REGS <= 128 && TM > 1;
   typename Epi::Pre pre[PRE_ALL ? TM : 2][TN * 4];
+  // ROWS_LDS: a finished row of fragments passes through LDS so that the epilogue takes its groups of four values
+  // (four consecutive columns of a row) in row-major order, group q * 64 + lane to a lane in its q-th turn (TN * 4
+  // turns): consecutive lanes then store consecutive 8-byte pieces of a row, and a store or operand load of the wave
+  // covers whole cache lines.  Straight from the accumulators an instruction touches 32 rows at 16 bytes each.  (For a
+  // result in fragment order that is already two runs of 256 contiguous bytes; nothing to gain there.)
+  constexpr int W4 = TN * 8;                 // groups per row of the wave's tile
+  constexpr int PITCH = TN * 32 + 4;         // floats between rows in LDS: 16 lanes of a write hit 64 different banks
+  static_assert(!ROWS_LDS || !D_ALONG_M, "the epilogue through LDS takes accumulators with four values per lane along n");
+  // (m, n) of the q-th group of four values a lane finalises in fragment row i
+  auto group_m = [&](int i, int q) { return ROWS_LDS ? m_base + i * 32 + (q * 64 + lane) / W4 : m_base + i * 32 + lane_m + (D_ALONG_M ? 8 * (q % 4) : 0); };
+  auto group_n = [&](int q) { return ROWS_LDS ? n_base + 4 * ((q * 64 + lane) % W4) : n_base + (q / 4) * 32 + lane_n + (D_ALONG_M ? 0 : 8 * (q % 4)); };
   auto preload_row = [&](int i, typename Epi::Pre (&dst)[TN * 4]) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        int m = m_base + i * 32 + lane_m + (D_ALONG_M ? 8 * g : 0);
-        int n = n_base + j * 32 + lane_n + (D_ALONG_M ? 0 : 8 * g);
+        int m = group_m(i, j * 4 + g);
+        int n = group_n(j * 4 + g);
         if (D_ALONG_M) {
           m = m < M ? m : (M >= 4 ? M - 4 : 0);
           n = n < N ? n : N - 1;
@@ -1114,6 +1125,9 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   // k loop ends: as many registers again as the tile itself, paid for by spilling everything else that is live in
   // the loop.  Pinning the rows that are not yet due (an empty statement that wants them in accumulation
   // registers) keeps the move to one row at a time.
+  typedef __attribute__((address_space(3))) float4_t lds_float4_t;
+  lds_char_t* const rows_lds = lds + wave * (32 * PITCH * 4);   // this wave's 32 rows
+  if constexpr (ROWS_LDS) __syncthreads();   // the other waves may still be reading the last operand tiles
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -1121,17 +1135,42 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
 #pragma unroll
       for (int j = 0; j < TN; ++j) MONONN_PIN_ACC(acc[r][j]);
     if (!PRE_ALL && i + 1 < TM) preload_row(i + 1, pre[(i + 1) & 1]);
+    if constexpr (ROWS_LDS) {
+      // LDS serves a wave's accesses in the order they were issued: the reads below see the writes above without a
+      // barrier (no other wave touches these rows); the fences keep the compiler from moving one past the other
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int m = m_base + i * 32 + lane_m + (D_ALONG_M ? 8 * g : 0);
-        const int n = n_base + j * 32 + lane_n + (D_ALONG_M ? 0 : 8 * g);
+        for (int g = 0; g < 4; ++g)
+          *reinterpret_cast<lds_float4_t*>(rows_lds + (r32 * PITCH + j * 32 + lane_n + 8 * g) * 4) =
+              float4_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int q = 0; q < TN * 4; ++q) {
+        const float4_t f = *reinterpret_cast<const lds_float4_t*>(rows_lds + (((q * 64 + lane) / W4) * PITCH + 4 * ((q * 64 + lane) % W4)) * 4);
+        const int m = group_m(i, q), n = group_n(q);
         if (m < M && n < N) {
-          float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-          epi(batch, m, n, v, pre[PRE_ALL ? i : (i & 1)][j * 4 + g]);
+          float v[4] = {f[0], f[1], f[2], f[3]};
+          epi(batch, m, n, v, pre[PRE_ALL ? i : (i & 1)][q]);
         }
       }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int m = group_m(i, j * 4 + g), n = group_n(j * 4 + g);
+          if (m < M && n < N) {
+            float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+            epi(batch, m, n, v, pre[PRE_ALL ? i : (i & 1)][j * 4 + g]);
+          }
+        }
+    }
   }
 }
 

@@ -78,3 +78,5 @@ inline host_float4 __builtin_amdgcn_mfma_f32_16x16x32_bf16(host_bf16x8 a, host_b
   c[0] += (float)a[0] * (float)b[0] + (float)a[7] * (float)b[7];
   return c;
 }
+#define __builtin_amdgcn_fence(order, scope) ((void)0)
+#define __builtin_amdgcn_wave_barrier() ((void)0)

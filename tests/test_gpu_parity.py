@@ -1,6 +1,8 @@
 """GPU parity: the generated monolithic kernel against the NumPy oracle on the same seeded inputs.
 Tolerance (stated by the north star): max-abs-err <= 2e-2 and cosine >= 0.9999 against the fp32
 evaluation of the HLO; integer / gather work bit-exact."""
+import re
+
 import numpy as np
 import pytest
 
@@ -437,3 +439,48 @@ def test_bf16_attention_with_a_key_count_off_the_mfma_step(gpu_device):
     src = m.get_source("main.hip")
     assert "colv[" in src and "mononn_dev::mfma_16x16x32<true>(" in src
     _bf16_check(got, hlo_interp.evaluate(fx.hlo_text, inputs, consts, "as_written")[0], "bf16 encoder, 48 keys", steps=4.0, atol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,tile", [
+    (512, 384, 256, dict(m=128, n=128, k=64)),      # 64 columns per wave: 16 lanes per row
+    (500, 392, 128, dict(m=128, n=192, k=32)),      # 96 columns per wave (24 lanes per row), M and N off the tile
+    (300, 1001, 128, dict(m=64, n=256, k=32)),      # 128 columns per wave, odd N: rows at 2-byte aligned addresses
+    (256, 64, 512, dict(m=64, n=64, k=64)),         # 32 columns per wave
+])
+def test_lds_tile_epilogue_through_lds_by_rows(gpu_device, dtype, M, N, K, tile):
+    # a row-major result of the LDS-staged tile passes through LDS a fragment row at a time so that the epilogue
+    # (here: bias + residual) loads and stores whole rows of the wave's tile; against the oracle
+    import json
+    from mononn_amd import bf16
+    mb = HloModuleBuilder("cluster_9__gemm_rows.1")
+    e = mb.entry
+    a = e.parameter(dtype, (M, K), "a")
+    res = e.parameter(dtype, (M, N), "res")
+    w = e.elided_constant(dtype, (K, N), "w/kernel")
+    bias = e.elided_constant(dtype, (N,), "w/bias")
+    d = e.gemm(a, w, 1, 0)
+
+    def body(f, pd, pb, pr):
+        return f.convert(f.add(f.add(f.convert(pd, "f32"), f.broadcast(f.convert(pb, "f32"), (M, N), [1])), f.convert(pr, "f32")), dtype)
+    e.set_tuple_root([e.fusion("kLoop", [d, bias, res], body)])
+    text = mb.text()
+    rng = np.random.default_rng(9)
+    host = (lambda v: bf16.to_bits(v)) if dtype == "bf16" else (lambda v: v.astype(np.float16))
+    av, rv = host(rng.normal(0, 1, (M, K))), host(rng.normal(0, 1, (M, N)))
+    consts = {n: host(rng.normal(0, 0.1 if len(meta["dims"]) == 2 else 1.0, meta["dims"])) for n, meta in mb.constants.items()}
+    spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+    for g in spec["gemm_spec_list"].values():
+        c = g["cutlass_config"]
+        c["threadblockshape"].update(tile)
+        c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+        c["stages"] = 2
+    (got,), m = run_module(text, [av, rv], consts, [{"dtype": dtype, "dims": [M, N]}], json.dumps(spec))
+    src = m.get_source("main.hip")
+    assert "gemm_tile_lds<" in src and re.search(r"mononn_dev::RowMajorA, (true|false), true>\(", src)
+    m.close()
+    want = hlo_interp.evaluate(text, [av, rv], consts, "fp32")[0]
+    if dtype == "bf16":
+        _bf16_check(got, want, f"bf16 {M}x{N}x{K} {tile}", steps=1.0, atol=2e-3 * float(np.abs(want).max()))
+    else:
+        assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * np.abs(want).max() + 1e-3

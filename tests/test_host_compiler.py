@@ -665,7 +665,9 @@ def test_bf16_modules_take_the_bf16_mfma_on_the_same_tiles():
             n += 1
     assert n >= 4
     lds = MonoNNModule.compile(fx.hlo_text, json.dumps(spec)).get_source("main.hip")
-    assert lds.count("mononn_dev::RowMajorA, true>(reinterpret_cast<const half_t*>(") >= 4 and lds.count("gemm_tile_lds<") >= 4
+    staged = lds.count("gemm_tile_lds<")
+    # (a second `true`: the result is row-major and goes through LDS a fragment row at a time)
+    assert staged >= 4 and len(re.findall(r"mononn_dev::RowMajorA, true(?:, true)?>\(reinterpret_cast<const half_t\*>\(", lds)) == staged
     # a mixed GEMM is refused
     bad = fx.hlo_text.replace("bf16[128,128]{1,0} custom-call(", "f16[128,128]{1,0} custom-call(", 1)
     if bad != fx.hlo_text:
