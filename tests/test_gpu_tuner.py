@@ -98,3 +98,63 @@ def test_launch_contexts_can_be_named(gpu_device, encoder, tmp_path, monkeypatch
     with pytest.raises(MonoNNError) as ei:
         MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, None, budget=2)
     assert "MONONN_TUNER_LAUNCH_CONTEXTS" in str(ei.value)
+
+
+def test_attention_row_blocks_are_searched_on_many_rows(gpu_device, tmp_path, monkeypatch):
+    # with many query rows per head the tuner also tries several row blocks per wave on one set of keys and values
+    monkeypatch.setenv("MONONN_TUNER_LAUNCH_CONTEXTS", "1x256")
+    monkeypatch.setenv("MONONN_TUNER_NO_SPLIT_K", "1")
+    fx = models.bert_encoder(L=1, B=8, S=256, H=256, NH=4, F=512, vocab=300, max_pos=256, mask_kind="length_mask")
+    consts, inputs = fx.make_constants(33, "random"), fx.make_inputs(33)
+    out = str(tmp_path / "rows")
+    tuned = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, out, budget=2)
+    log = open(os.path.join(out, "cluster_0", "tuning_log.log")).read()
+    line = next(l for l in log.splitlines() if "attention x1" in l)
+    assert "_rows" in line, line                       # candidates like key_waves1_rows128 were timed
+    tuned.set_constants(consts)
+    tuned.load(gpu_device)
+    _check(tuned.run(inputs, fx.outputs)[0], hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0])
+
+
+def test_tuning_with_layer_norm_folding_and_the_seed_s_deep_splits(gpu_device, encoder, tmp_path, monkeypatch):
+    # MONONN_TUNER_LAYER_NORM_FOLDING tunes the folded form; with a seed, MONONN_TUNER_KEEP_SEED_SPLIT_K keeps its k
+    # splits of at least that factor from the start, and the LayerNorm behind such a GEMM stays a stage
+    fx, consts, inputs, want = encoder
+    monkeypatch.setenv("MONONN_TUNER_LAUNCH_CONTEXTS", "1x256")
+    monkeypatch.setenv("MONONN_TUNER_LAYER_NORM_FOLDING", "1")
+    folded_dir = str(tmp_path / "folded")
+    folded = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, folded_dir, budget=2)
+    spec = json.loads(folded.get_tuning_spec())
+    assert spec["mononn_hip"]["layer_norm_folding"] is True and spec["mononn_hip"]["gemm_prologue_fusion"] is True
+    assert "ln_stats[" in folded.get_source("main.hip")
+    folded.set_constants(consts)
+    folded.load(gpu_device)
+    _check(folded.run(inputs, fx.outputs)[0], want)
+    # a seed with FFN2 split by 4: kept from the start, so only the LayerNorm in front of FFN1 is folded
+    seed = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    import re
+    gemms = [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", fx.hlo_text)]
+    template = next(v for k, v in seed["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))
+    seed["gemm_spec_list"] = {k: v for k, v in seed["gemm_spec_list"].items() if not k.startswith("cublas_gemm_")}
+    seed["cluster_reduce_spec"], seed["cluster_elewise_spec"] = {}, {}
+    for layer in range(2):
+        e = json.loads(json.dumps(template))
+        e["cutlass_config"]["split_k"] = 4
+        seed["gemm_spec_list"][gemms[layer * 6 + 5]] = e
+    seed_dir = tmp_path / "seed" / "cluster_0"
+    seed_dir.mkdir(parents=True)
+    filled = MonoNNModule.compile(fx.hlo_text, json.dumps(seed), build=False).get_tuning_spec()
+    (seed_dir / "best_tuning_spec.json").write_text(filled)
+    monkeypatch.setenv("MONONN_TUNER_SEED_SPEC_DIR", str(tmp_path / "seed"))
+    monkeypatch.setenv("MONONN_TUNER_KEEP_SEED_SPLIT_K", "4")
+    monkeypatch.setenv("MONONN_TUNER_NO_SPLIT_K", "1")
+    mixed_dir = str(tmp_path / "mixed")
+    mixed = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, mixed_dir, budget=2)
+    log = open(os.path.join(mixed_dir, "cluster_0", "tuning_log.log")).read()
+    assert "2 k splits of the seed specification kept from the start" in log
+    mspec = json.loads(mixed.get_tuning_spec())
+    assert sum(1 for v in mspec["gemm_spec_list"].values() if v["cutlass_config"]["split_k"] == 4) == 2
+    assert folded.launch_dims()["barriers"] < mixed.launch_dims()["barriers"] < MonoNNModule.compile(fx.hlo_text, build=False).launch_dims()["barriers"] + 1
+    mixed.set_constants(consts)
+    mixed.load(gpu_device)
+    _check(mixed.run(inputs, fx.outputs)[0], want)
