@@ -1931,8 +1931,8 @@ void check_out_proj_mapping(const Program& prog, const Instr* g2, const graph::G
 // does not depend on the query row - a padding mask read per key column and everything computed from it alone - is
 // moved to the line `marker`, which sits with the operand loads in front of the first MFMA (and, with several row
 // blocks per wave, in front of their loop): definitions `const T vN = <expression>;` at the indentation of the
-// straight-line part whose identifiers are parameters, lane coordinates of the key column, the batch index, pure
-// functions and earlier moved values.
+// straight-line part whose identifiers are parameters, the lane's coordinates of the key column (g, kw; not r16 or
+// lane, which also say which row the lane holds), the batch index, pure functions and earlier moved values.
 std::string hoist_row_invariant_values(const std::string& text, const std::string& marker) {
   std::vector<std::string> lines;
   {
@@ -1947,7 +1947,7 @@ std::string hoist_row_invariant_values(const std::string& text, const std::strin
   static const std::regex v_def(R"(^(\s*)const ([A-Za-z_]\w*) (v\d+) = (.*);$)");
   static const std::regex ident(R"((^|[^\w.])([A-Za-z_]\w*))");
   static const std::regex allowed(
-      R"(^(in\d+|bidx|g|kw|r16|lane|colc|colv|float|double|_Float16|int|long|unsigned|short|char|bool|int8_t|uint8_t|int16_t|uint16_t|int32_t|uint32_t|int64_t|uint64_t|fmaxf|fminf|fabsf|__expf|__logf|tanhf|sqrtf|rsqrtf|__builtin_amdgcn_rcpf|__builtin_inff)$)");
+      R"(^(in\d+|bidx|g|kw|colc|colv|float|double|_Float16|int|long|unsigned|short|char|bool|int8_t|uint8_t|int16_t|uint16_t|int32_t|uint32_t|int64_t|uint64_t|fmaxf|fminf|fabsf|__expf|__logf|tanhf|sqrtf|rsqrtf|__builtin_amdgcn_rcpf|__builtin_inff)$)");
   // the straight-line part: the indentation of the first value definition behind the marker
   size_t body_indent = std::string::npos;
   std::set<std::string> moved_names;
