@@ -156,3 +156,46 @@ def test_random_gemms_on_lds_staged_tiles_match_the_oracle(gpu_device):
         want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
         scale = np.abs(want).max()
         assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * scale + 1e-3, case
+
+
+def _as_bf16(text, inputs, descs):
+    """The same module with every f16 replaced by bf16; f16 inputs become bf16 bit patterns of the same values."""
+    import re
+    from mononn_amd import bf16
+    text = re.sub(r"\bf16\b", "bf16", text)
+    inputs = [bf16.to_bits(a.astype(np.float32)) if a.dtype == np.float16 else a for a in inputs]
+    descs = [dict(d, dtype="bf16") if d["dtype"] == "f16" else d for d in descs]
+    return text, inputs, descs
+
+
+def test_random_graphs_in_bf16_are_lowered_and_stay_inside_their_buffers():
+    from cpu_bounds import check_module
+    for seed in SEEDS[:12]:
+        text, inputs, descs = _as_bf16(*random_module(seed))
+        want = hlo_interp.evaluate(text, inputs, {})
+        assert all(np.isfinite(w.astype(np.float64)).all() for w in want), seed
+        ok, msg = check_module(text)
+        assert ok, f"seed {seed} in bf16: {msg}"
+
+
+@pytest.mark.gpu
+def test_random_graphs_in_bf16_match_the_oracle(gpu_device):
+    from mononn_amd import bf16
+    worst = 0.0
+    for seed in SEEDS:
+        text, inputs, descs = _as_bf16(*random_module(seed))
+        want = hlo_interp.evaluate(text, inputs, {})          # as written: rounded to bf16 after every bf16 instruction
+        m = MonoNNModule.compile(text)
+        m.load(gpu_device)
+        got = m.run(inputs, descs)
+        m.close()
+        for g, w, d in zip(got, want, descs):
+            g64 = (bf16.from_bits(g) if d["dtype"] == "bf16" else g).astype(np.float64)
+            w64 = w.astype(np.float64)
+            assert np.isfinite(g64).all(), seed
+            # the same rounding points on both sides; a fast-math transcendental or another summation order moves a
+            # value by a bf16 spacing (2^-8 relative) here and there, and a few of those can meet in one result
+            err = np.abs(g64 - w64) / (1.0 + np.abs(w64))
+            worst = max(worst, float(err.max()))
+            assert err.max() <= 2e-2, f"seed {seed}: relative error {err.max()} at {np.unravel_index(err.argmax(), err.shape)}"
+    print(f"random graphs in bf16: worst relative error {worst:.3e} over {len(SEEDS)} modules")
