@@ -45,6 +45,48 @@ def test_custom_op_matches_the_ctypes_path_bit_for_bit(gpu_device):
     m.close()
 
 
+def test_custom_op_with_bfloat16_tensors(gpu_device):
+    # a bf16 module through the operator: torch.bfloat16 results, the same bits as the ctypes path hands back as uint16,
+    # and against torch's own bf16 GEMM + bias on the same operands
+    import torch
+    from mononn_amd import MonoNNModule, bf16, torch_op
+    from mononn_amd.hlo.builder import HloModuleBuilder
+    M, K, N = 256, 512, 384
+    mb = HloModuleBuilder("cluster_4__bf16_op.1")
+    e = mb.entry
+    a = e.parameter("bf16", (M, K), "a")
+    w = e.elided_constant("bf16", (K, N), "w/kernel")
+    bias = e.elided_constant("bf16", (N,), "w/bias")
+    d = e.gemm(a, w, 1, 0)
+
+    def body(f, pd, pb):
+        return f.convert(f.add(f.convert(pd, "f32"), f.broadcast(f.convert(pb, "f32"), (M, N), [1])), "bf16")
+    e.set_tuple_root([e.fusion("kLoop", [d, bias], body)])
+    rng = np.random.default_rng(41)
+    av = rng.normal(0, 1, (M, K)).astype(np.float32)
+    consts = {n: bf16.to_bits(rng.normal(0, 0.1 if len(meta["dims"]) == 2 else 1.0, meta["dims"])) for n, meta in mb.constants.items()}
+    outputs = [{"dtype": "bf16", "dims": [M, N]}]
+    m = MonoNNModule.compile(mb.text())
+    m.set_constants(consts)
+    m.load(gpu_device)
+    want_bits = m.run([bf16.to_bits(av)], outputs)[0]
+    fn = torch_op.MonoNNFunction(m, outputs, gpu_device)
+    dev = torch.device("cuda", gpu_device)
+    ta = torch.from_numpy(av).to(dev).to(torch.bfloat16)
+    (got,) = torch_op.forward(fn, ta)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (M, N)
+    assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want_bits)
+    by_name = {meta["role"]: torch.from_numpy(consts[n].view(np.int16)).view(torch.bfloat16).to(dev) for n, meta in mb.constants.items()}
+    # the HLO rounds twice: the GEMM's result is bf16, and so is the sum with the bias
+    d = (ta.float() @ by_name["w/kernel"].float()).to(torch.bfloat16).float()
+    ref = (d + by_name["w/bias"].float()).to(torch.bfloat16).float().cpu().numpy()
+    g = got.float().cpu().numpy()
+    spacing = 2.0 ** -7 * np.maximum(np.abs(ref), np.abs(d.cpu().numpy()))      # a bf16 step at the larger of the two magnitudes
+    assert (np.abs(g - ref) <= spacing + 1e-6).all() and (g == ref).mean() > 0.9
+    fn.close()
+    m.close()
+
+
 def test_perf_report_lists_every_stage(gpu_device, tmp_path):
     # the per-node report (perf dumper counterpart) of a small encoder: one row per stage, times positive
     import csv
