@@ -313,8 +313,8 @@ def _bert_encoder(L, B, S, H, NH, F, vocab, max_pos, types, eps, mask_kind) -> M
         dict(B=B, S=S, H=H, NH=NH, F=F, L=L, vocab=vocab))
 
 
-def bert_base(B=1, S=128) -> ModelFixture:
-    return bert_encoder(L=12, B=B, S=S)
+def bert_base(B=1, S=128, ftype="f16") -> ModelFixture:
+    return bert_encoder(L=12, B=B, S=S, ftype=ftype)
 
 
 def bert_large(B=16, S=384) -> ModelFixture:
