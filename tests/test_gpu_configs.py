@@ -277,3 +277,34 @@ def test_attention_with_several_row_blocks_per_wave(gpu_device, what, make, row_
     m.close()
     want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
     _check(got, want, what)
+
+
+def test_k_split_gemm_on_lds_staged_tiles(gpu_device):
+    """FFN2 and the output projection of an encoder on LDS-staged tiles with their k range split over workgroups: fp32
+    partial sums leave the tile row by row through LDS (16 bytes per lane) and are added up by the LayerNorm stage."""
+    import json
+    import re
+    from mononn_amd import MonoNNModule
+    fx = models.bert_encoder(L=2, B=4, S=128, H=256, NH=4, F=1024, vocab=300, max_pos=128, mask_kind="length_mask")
+    gemms = [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", fx.hlo_text)]
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    template = next(v for k, v in spec["gemm_spec_list"].items() if k.startswith("cublas_gemm_"))
+    spec["gemm_spec_list"] = {k: v for k, v in spec["gemm_spec_list"].items() if not k.startswith("cublas_gemm_")}
+    spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}
+    for layer in range(2):
+        for index, split in ((3, 2), (5, 4)):
+            e = json.loads(json.dumps(template))
+            c = e["cutlass_config"]
+            c["threadblockshape"] = {"m": 128, "n": 128, "k": 32}
+            c["wave_arrangement"] = {"m": 2, "n": 2, "k": 1}
+            c["stages"] = 2
+            c["split_k"] = split
+            spec["gemm_spec_list"][gemms[layer * 6 + index]] = e
+    consts = fx.make_constants(1244, "random")
+    inputs = fx.make_inputs(1244)
+    m, got = _run(fx, consts, inputs, gpu_device, json.dumps(spec))
+    src = m.get_source("main.hip")
+    assert len(re.findall(r"gemm_tile_lds<[^;]*mononn_dev::RowMajorA, false, true>\(", src)) >= 2 and "stN<float, 4>" in src
+    m.close()
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    _check(got, want, "encoder with k-split GEMMs on LDS-staged tiles")
