@@ -92,8 +92,11 @@ bool host_only_output(const Program& prog, const Instr* out) {
   auto it = prog.buffers.find(prog.storage_root(out));
   return it != prog.buffers.end() && it->second.kind == graph::Buffer::kLiveOut && it->second.last_use_stage == it->second.def_stage;
 }
-std::string st1_of(const Program& prog, const Instr* out) { return host_only_output(prog, out) ? "mononn_dev::st1_plain(" : "mononn_dev::st1("; }
-std::string stN_of(const Program& prog, const Instr* out) { return host_only_output(prog, out) ? "mononn_dev::stN_plain<" : "mononn_dev::stN<"; }
+// Likewise a result whose readers all sit on the XCD that wrote what they read (regional synchronisation): the
+// hand-over goes through that XCD's L2.
+bool plain_stored_output(const Program& prog, const Instr* out) { return host_only_output(prog, out) || prog.regional_roots.count(prog.storage_root(out)) > 0; }
+std::string st1_of(const Program& prog, const Instr* out) { return plain_stored_output(prog, out) ? "mononn_dev::st1_plain(" : "mononn_dev::st1("; }
+std::string stN_of(const Program& prog, const Instr* out) { return plain_stored_output(prog, out) ? "mononn_dev::stN_plain<" : "mononn_dev::stN<"; }
 
 void store(const Program& prog, CodeBuffer& cb, PointerTable& ptrs, const VarTable& vars, const Instr* out, const Index& idx, const std::string& v) {
   cb.line(st1_of(prog, out) + ptrs.output(out) + " + " + physical_offset(prog, out, idx, &vars).str(vars) + ", " + v + ");");
@@ -552,6 +555,37 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
 
 }  // namespace
 
+bool WriteMap::element_offset(int64_t bidx, int64_t m, int64_t n, int64_t* out) const {
+  std::vector<int64_t> v(num_vars, 0);
+  auto set = [&](int var, int64_t value) {
+    if (var >= 0 && static_cast<size_t>(var) < v.size()) v[var] = value;
+  };
+  set(vb, bidx);
+  if (vm4 >= 0) {   // four consecutive rows per call
+    set(vm4, m / 4);
+    set(vr, m % 4);
+    set(vnn, n);
+  } else {
+    set(vm, m);
+    if (vn4 >= 0) {
+      set(vn4, n / 4);
+      set(vr, n % 4);
+    } else {
+      set(vnn, n);
+    }
+  }
+  return offset.evaluate(v, out);
+}
+
+bool operand_offset_expr(const Program& prog, const Instr* operand, int64_t elements, LinExpr* out) {
+  const Instr* root = prog.storage_root(operand);
+  if (root->shape.num_elements() != elements) return false;
+  VarTable vars;
+  const int ve = vars.add("e", elements);
+  *out = physical_offset(prog, root, delinearize(LinExpr::variable(ve, elements), root->shape.dims, vars), &vars);
+  return true;
+}
+
 std::vector<const Instr*> external_outputs(const Program& prog, const std::vector<const Instr*>& members) {
   std::set<const Instr*> mem(members.begin(), members.end());
   const Instr* root = prog.module->entry->root;
@@ -754,6 +788,7 @@ struct Epilogue {
   int vector_stores = 0;     // outputs written with one 8-byte store per call
   std::string init_line;     // @NAME@_epi epi{...};
   std::vector<std::string> globals;
+  std::vector<WriteMap> writes;   // where each output's element (bidx, m, n) goes (not for split-K partial sums)
 };
 
 // along_m: the MFMA is issued with the operands swapped, so that a lane holds four consecutive rows m of one
@@ -1000,6 +1035,16 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   }
   em.pop_scope();
   cb.close();
+  std::vector<WriteMap> writes;
+  for (auto& out : outs) {
+    WriteMap w;
+    w.root = prog.storage_root(out.o);
+    w.offset = physical_offset(prog, out.o, out.idx, &vars);
+    w.vb = vb, w.vm = vm, w.vm4 = vm4, w.vn4 = vn4, w.vr = vr, w.vnn = vnn;
+    w.num_vars = vars.size();
+    w.batch = g.batch, w.M = g.M, w.N = g.N;
+    writes.push_back(w);
+  }
   if (vec4) {
     for (auto& out : outs)
       if (out.vector_store) {
@@ -1081,6 +1126,7 @@ Epilogue build_epilogue(const Program& prog, const Instr* gi, const std::vector<
   for (size_t i = first_epi; i < ptrs.entries.size(); ++i) init += (i > first_epi ? ", " : "") + ptrs.entries[i].name;
   init += "};";
   out_e.init_line = init;
+  out_e.writes = writes;
   for (auto& kv : em.literal_tables()) out_e.globals.push_back(kv.second);
   return out_e;
 }
@@ -1750,10 +1796,23 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     const int64_t KS = g.K / S_;   // k extent of one split
     const int64_t per_batch = tiles_n * tiles_m * S_;
     units = g.batch * per_batch;
+    // Regional synchronisation: unit 8 q + x belongs to XCD x, which takes its slice of the columns or its k slice
+    const Partition& part = t.part;
+    if (part.on()) {
+      MONONN_CHECK(g.batch == 1 && !g.is_conv && t.stages < 2 && part.parts <= 8, kInternal) << gi->hlo_name << ": GEMM cannot be dealt to the XCDs";
+      MONONN_CHECK(part.kind == Partition::kSplitK ? S_ == part.parts : (part.kind == Partition::kColumns && S_ == 1 && tiles_n % part.parts == 0 && g.N % t.bn == 0), kInternal)
+          << gi->hlo_name << ": partition does not fit the tile grid";
+      units = 8 * (part.kind == Partition::kSplitK ? tiles_n * tiles_m : tiles_n / part.parts * tiles_m);
+      fb.line("const int bidx = 0;");
+      fb.line("const int xcd = unit & 7;   // of " + S(part.parts) + " that take part");
+      fb.line(std::string("const int ksplit = ") + (part.kind == Partition::kSplitK ? "xcd" : "0") + ";");
+      fb.line("const int rem = unit >> 3;");
+    } else {
     fb.line("const int bidx = unit / " + S(per_batch) + ";");
     fb.line("const int rem0 = unit % " + S(per_batch) + ";");
     fb.line("const int ksplit = rem0 % " + S(S_) + ";");
     fb.line("const int rem = rem0 / " + S(S_) + ";");
+    }
     if (g.split_k > 1) fb.line(epi.init_line);
     // LDS-staged tiles (large problems): the 8 XCDs each take a rectangle of the tile grid, rm x rn tiles, walked
     // row by row, so that the tiles an XCD works on at one time share few operand panels: every panel an XCD
@@ -1770,7 +1829,10 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         if (best < 0 || cost < best) best = cost, gm = a, gn = b;
       }
     }
-    if (gm > 0) {
+    if (part.kind == Partition::kColumns) {
+      fb.line("const int tile_n = xcd * " + S(tiles_n / part.parts) + " + rem / " + S(tiles_m) + ";");
+      fb.line("const int tile_m = rem % " + S(tiles_m) + ";");
+    } else if (gm > 0) {
       const int64_t rn = tiles_n / gn, rm = tiles_m / gm;
       fb.line("const int xcd = rem & 7, q = rem >> 3;   // " + S(rm) + " x " + S(rn) + " tiles per XCD");
       fb.line("const int tile_n = (xcd / " + S(gm) + ") * " + S(rn) + " + q % " + S(rn) + ";");
@@ -1840,11 +1902,19 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         const int ch_max = chunk / (TM + TN) > 0 ? chunk / (TM + TN) : 1;   // mirrors mononn_dev::gemm_chunk_steps
         preload_regs = (my_steps * (TM + TN) <= ls.whole_range_fragments() ? my_steps : std::min(my_steps, ch_max)) * TN;
         CodeBuffer pf;
+        if (part.on()) {
+          pf.line("const int bidx = 0;");
+          pf.line("const int xcd = unit & 7;");
+          pf.line(std::string("const int ksplit = ") + (part.kind == Partition::kSplitK ? "xcd" : "0") + ";");
+          pf.line("const int rem = unit >> 3;");
+        } else {
         pf.line("const int bidx = unit / " + S(per_batch) + ";");
         pf.line("const int rem0 = unit % " + S(per_batch) + ";");
         pf.line("const int ksplit = rem0 % " + S(S_) + ";");
         pf.line("const int rem = rem0 / " + S(S_) + ";");
-        if (tiles_n % 8 == 0 && S_ == 1) pf.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
+        }
+        if (part.kind == Partition::kColumns) pf.line("const int tile_n = xcd * " + S(tiles_n / part.parts) + " + rem / " + S(tiles_m) + ";");
+        else if (tiles_n % 8 == 0 && S_ == 1) pf.line("const int tile_n = (rem >> 3) / " + S(tiles_m) + " * 8 + (rem & 7);");
         else pf.line("const int tile_n = rem / " + S(tiles_m) + ";");
         std::ostringstream pc;
         pc << "mononn_dev::gemm_b_preload<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", " << g.K << ">("
@@ -1881,6 +1951,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   std::vector<std::string> globals = epi.globals;
   for (auto& gl : pro.globals) globals.push_back(gl);
   NodeFunction f = finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text + conv_struct);
+  f.write_maps = epi.writes;
   if (preload) {
     const std::string tail = ", char* smem) {";
     size_t at = f.text.find(tail);
@@ -1997,7 +2068,8 @@ std::string hoist_row_invariant_values(const std::string& text, const std::strin
 NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::GemmDesc& d1, const std::vector<const Instr*>& row_members,
                            const Instr* g2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epi_members,
                            const std::vector<const Instr*>& outputs, const LaunchShape& ls, int key_waves,
-                           const Instr* g3 = nullptr, const graph::GemmDesc* d3p = nullptr, int heads = 0, bool preload_w = false, int row_blocks = 1) {
+                           const Instr* g3 = nullptr, const graph::GemmDesc* d3p = nullptr, int heads = 0, bool preload_w = false, int row_blocks = 1,
+                           Partition part = Partition()) {
   const int NW = ls.waves();
   const int64_t M1 = d1.M, N1 = d1.N, K1 = d1.K, N2 = d2.N;
   MONONN_CHECK(d1.a_k_contig && d1.b_k_contig && d2.a_k_contig, kUnsupported) << "attention fusion needs k-contiguous operands";
@@ -2107,9 +2179,18 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
   cb.line("const int r16 = lane & 15, g = lane >> 4;");
   cb.line("const int kw = mononn_dev::wave_id() % " + S(KW) + ", rw = mononn_dev::wave_id() / " + S(KW) + ";");
   const int64_t blocks = (M1 + 16 * RW * RB - 1) / (16 * RW * RB);
+  int64_t num_units = d1.batch * blocks;
+  if (part.on()) {
+    // regional synchronisation: unit 8 q + x belongs to XCD x, which takes a run of batch elements (heads)
+    MONONN_CHECK(part.kind == Partition::kHeads && !g3 && part.parts <= 8 && d1.batch % part.parts == 0, kInternal) << "attention node cannot be dealt to the XCDs";
+    num_units = 8 * (d1.batch / part.parts) * blocks;
+    cb.line("const int bidx = (unit & 7) * " + S(d1.batch / part.parts) + " + (unit >> 3) / " + S(blocks) + ";");
+    cb.line("const int mt0 = ((unit >> 3) % " + S(blocks) + ") * " + S(RW * RB) + " + rw;");
+  } else {
   cb.line("const int bidx = unit / " + S(blocks) + ";");
   // row block of this wave in round rb of the unit: mt0 + rb * RW
   cb.line("const int mt0 = (unit % " + S(blocks) + ") * " + S(RW * RB) + " + rw;");
+  }
   auto row_block_head = [&](const std::string& mt_expr) {
     cb.line("const int mt = " + mt_expr + ";");
     cb.line("const bool m_valid = mt * 16 + r16 < " + S(M1) + ";");
@@ -2495,7 +2576,9 @@ NodeFunction gen_attention(const Program& prog, const Instr* g1, const graph::Ge
     cb.line("for (int ks = 0; ks < " + S(KS1) + "; ++ks) qf[ks] = qn[ks];");
     cb.close();
   }
-  return finish(hoist_row_invariant_values(cb.text(), "@ROW_INVARIANT@"), ptrs, globals, d1.batch * blocks, smem, epi.struct_text);
+  NodeFunction f = finish(hoist_row_invariant_values(cb.text(), "@ROW_INVARIANT@"), ptrs, globals, num_units, smem, epi.struct_text);
+  f.write_maps = epi.writes;
+  return f;
 }
 
 }  // namespace
@@ -2504,7 +2587,7 @@ NodeFunction generate_gemm(const Program& prog, const Node& node, const LaunchSh
   return gen_gemm(prog, node.members, node.outputs, node.gemm, ls, t, node.prologue, node.prologue_stores, &node.ln_fold);
 }
 
-NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves, bool preload_weights, int row_blocks) {
+NodeFunction generate_attention(const Program& prog, const Node& node, const LaunchShape& ls, int key_waves, bool preload_weights, int row_blocks, Partition part) {
   std::vector<const Instr*> row(node.members.begin() + 1, node.members.begin() + node.gemm2_index);
   if (node.gemm3_index != 0) {
     std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.begin() + node.gemm3_index);
@@ -2513,7 +2596,7 @@ NodeFunction generate_attention(const Program& prog, const Node& node, const Lau
   }
   std::vector<const Instr*> epi(node.members.begin() + node.gemm2_index + 1, node.members.end());
   return gen_attention(prog, node.members[0], node.gemm, row, node.members[node.gemm2_index], node.gemm2, epi, node.outputs, ls, key_waves, nullptr, nullptr, 0,
-                       false, row_blocks);
+                       false, row_blocks, part);
 }
 
 bool can_fuse_out_proj(const Program& prog, const Instr* gemm2, const graph::GemmDesc& d2, const std::vector<const Instr*>& epilogue_members,

@@ -35,7 +35,33 @@ struct ClusterTuning {
   int reduce_implementation = 0;
 };
 
+// Regional synchronisation: how the units of a node are dealt to the XCDs.  With parts > 0 unit u belongs to XCD
+// u % 8 (units are dealt to the workgroups round-robin and a workgroup's XCD is its index modulo 8); XCD x < parts
+// takes partition x of the node's work, XCDs from `parts` on have empty units:
+//   kColumns  a GEMM's result columns in `parts` equal slices (all rows, whole k range)
+//   kSplitK   the k slices of a GEMM that is split `parts` ways over workgroups
+//   kHeads    the batch elements of an attention node in `parts` equal runs
+struct Partition {
+  enum Kind { kNone, kColumns, kSplitK, kHeads };
+  Kind kind = kNone;
+  int parts = 0;
+  bool on() const { return kind != kNone && parts > 0; }
+};
+
+// Where a node writes element (bidx, m, n) of its GEMM-shaped result: the element offset inside the buffer of
+// `root`, as the epilogue computes it (through reshapes, transposes and fragment-order layouts)
+struct WriteMap {
+  const hlo::Instr* root = nullptr;
+  LinExpr offset;
+  int vb = -1, vm = -1, vm4 = -1, vn4 = -1, vr = -1, vnn = -1;   // variables of `offset`; -1 = not used
+  size_t num_vars = 0;
+  int64_t batch = 1, M = 0, N = 0;
+  // false when the offset has run-time terms
+  bool element_offset(int64_t bidx, int64_t m, int64_t n, int64_t* out) const;
+};
+
 struct GemmTuning {
+  Partition part;            // set by the regional synchronisation plan, not by the specification
   int bm = 32, bn = 32;      // workgroup tile
   int wm = 1, wn = 1, wk = 4;   // wave arrangement; wm*wn*wk == waves per workgroup
   int split_k = 1;              // k range also split over workgroups (fp32 partial sums to memory)
@@ -58,6 +84,7 @@ struct NodeFunction {
   // the previous stage.  When present, `text` defines the register block type `@NAME@_preb` and takes a trailing
   // `const @NAME@_preb&` after `smem`.
   std::string preload_text;
+  std::vector<WriteMap> write_maps;            // GEMM and attention nodes: one entry per result written by the epilogue
 };
 
 // fills has_reduce / row_program / rows / row_len
@@ -75,7 +102,11 @@ NodeFunction generate_gemm(const graph::Program& prog, const graph::Node& node, 
 // row_blocks: blocks of 16 query rows a wave works through, one after the other, with the keys and values it loaded
 // once (a unit then covers 16 * row_blocks * (waves / key_waves) rows of one batch element)
 NodeFunction generate_attention(const graph::Program& prog, const graph::Node& node, const LaunchShape& ls, int key_waves = 0,
-                                bool preload_weights = false, int row_blocks = 1);
+                                bool preload_weights = false, int row_blocks = 1, Partition part = Partition());
+// Element offset, inside the buffer of its storage root, of element e = (bidx * M + m) * K + k of a GEMM operand that is
+// stored [batch, M, K] with k minor-most, as an expression in one variable (index 0); false when the operand's
+// storage does not have that many elements
+bool operand_offset_expr(const graph::Program& prog, const hlo::Instr* operand, int64_t elements, LinExpr* out);
 // the input of a row program fused in front of a GEMM whose rows the GEMM loads as its left-operand fragments
 const hlo::Instr* prologue_primary(const graph::Program& prog, const std::vector<const hlo::Instr*>& row_members, int64_t M, int64_t K);
 // the GEMM `gemm3` reads nothing but the heads that the attention's second GEMM produces, merged by pure data movement

@@ -111,6 +111,17 @@ bool LinExpr::is_unit_stride_in(int var, int64_t extent) const {
   return n == 1;
 }
 
+bool LinExpr::evaluate(const std::vector<int64_t>& values, int64_t* out) const {
+  if (!opaque_.empty()) return false;
+  int64_t v = c_;
+  for (auto& t : terms_) {
+    if (t.var < 0 || static_cast<size_t>(t.var) >= values.size()) return false;
+    v += ((values[t.var] / t.div) % t.mod) * t.mul;
+  }
+  *out = v;
+  return true;
+}
+
 std::string LinExpr::str(const VarTable& vars) const {
   std::string s;
   auto add = [&](const std::string& p) {

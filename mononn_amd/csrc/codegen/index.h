@@ -91,6 +91,9 @@ class LinExpr {
   bool depends_on(int var) const;
 
   std::string str(const VarTable& vars) const;   // C expression (int arithmetic)
+  // value of the expression for given values of the loop variables (indexed like the variable table); false when
+  // the expression has run-time terms, which have no value on the host
+  bool evaluate(const std::vector<int64_t>& values, int64_t* out) const;
 
  private:
   friend LinExpr linearize(const std::vector<LinExpr>&, const std::vector<int64_t>&);

@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <functional>
 #include <set>
 #include <sstream>
 
@@ -63,6 +64,218 @@ Operand make_operand(const graph::Program& prog, const hlo::Instr* root, bool is
       break;
   }
   return o;
+}
+
+// ---- regional synchronisation ------------------------------------------------------------------------------------
+// Counterpart of RegionalSynchronizationAssignmentPass (regional_synchronization_assignment_pass.cc:35-72) on a part
+// with 8 L2s: which nodes deal their units to the XCDs by ownership, and which values then never leave the XCD that
+// wrote them.  Candidates come from the shapes (a k split over workgroups, the heads of an attention node, a GEMM in
+// front of either); whether a value really stays inside an XCD is decided element by element: the writer's epilogue
+// says where element (bidx, m, n) goes, the reader's operand map says which elements its partition fetches, and
+// every element a partition reads must have been written by the same partition.
+using NodeGenerator = std::function<NodeFunction(const Node&, const Partition&)>;
+
+// owner[e] = partition that writes element e of the root's buffer, -1 = nobody; false when the map has run-time terms
+bool owners_of(const WriteMap& w, const Partition& part, int64_t elements, std::vector<int8_t>& owner) {
+  owner.assign(static_cast<size_t>(elements), -1);
+  if (part.kind == Partition::kColumns && (w.batch != 1 || w.N % part.parts != 0)) return false;
+  if (part.kind == Partition::kHeads && w.batch % part.parts != 0) return false;
+  std::vector<int64_t> v(w.num_vars, 0);
+  auto set = [&](int var, int64_t value) {
+    if (var >= 0 && static_cast<size_t>(var) < v.size()) v[var] = value;
+  };
+  for (int64_t b = 0; b < w.batch; ++b)
+    for (int64_t m = 0; m < w.M; ++m)
+      for (int64_t n = 0; n < w.N; ++n) {
+        set(w.vb, b);
+        if (w.vm4 >= 0) set(w.vm4, m / 4), set(w.vr, m % 4), set(w.vnn, n);
+        else if (w.vn4 >= 0) set(w.vm, m), set(w.vn4, n / 4), set(w.vr, n % 4);
+        else set(w.vm, m), set(w.vnn, n);
+        int64_t off = 0;
+        if (!w.offset.evaluate(v, &off) || off < 0 || off >= elements) return false;
+        owner[static_cast<size_t>(off)] = static_cast<int8_t>(part.kind == Partition::kColumns ? n / (w.N / part.parts) : b / (w.batch / part.parts));
+      }
+  return true;
+}
+
+// every element of `root` that partition x of node `r` reads has owner x
+bool reads_own_partition(const graph::Program& prog, const Node& r, const Partition& part, const hlo::Instr* root, const std::vector<int8_t>& owner) {
+  const int64_t elements = static_cast<int64_t>(owner.size());
+  if (r.kind == NodeKind::kGemm && part.kind == Partition::kSplitK) {
+    const graph::GemmDesc& g = r.gemm;
+    const hlo::Instr* gi = r.members[0];
+    if (g.batch != 1 || !g.a_k_contig || g.split_k != part.parts || g.K % part.parts != 0 || r.members.size() != 1 || !r.prologue.empty()) return false;
+    if (prog.storage_root(gi->operands[0]) != root || prog.storage_root(gi->operands[1]) == root) return false;
+    LinExpr off;
+    if (g.M * g.K != elements || !operand_offset_expr(prog, gi->operands[0], elements, &off)) return false;
+    const int64_t ks = g.K / part.parts;
+    std::vector<int64_t> v(1);
+    for (int64_t e = 0; e < elements; ++e) {
+      v[0] = e;
+      int64_t at = 0;
+      if (!off.evaluate(v, &at) || at < 0 || at >= elements || owner[static_cast<size_t>(at)] != (e % g.K) / ks) return false;
+    }
+    return true;
+  }
+  if (r.kind == NodeKind::kAttention && part.kind == Partition::kHeads && r.gemm3_index == 0) {
+    const hlo::Instr* g1 = r.members[0];
+    const hlo::Instr* g2 = r.members[r.gemm2_index];
+    const graph::GemmDesc &d1 = r.gemm, &d2 = r.gemm2;
+    if (d1.batch % part.parts != 0 || d2.batch != d1.batch) return false;
+    // the node reads batch element b of an operand from [b * per_head, (b + 1) * per_head) of its buffer
+    int64_t per_head = 0;
+    int uses = 0;
+    if (prog.storage_root(g1->operands[0]) == root) ++uses, per_head = d1.M * d1.K, uses += (d1.a_packed || d1.a_batch_stride == per_head) ? 0 : 8;
+    if (prog.storage_root(g1->operands[1]) == root) ++uses, per_head = d1.N * d1.K, uses += (d1.b_tiled || d1.b_batch_stride == per_head) ? 0 : 8;
+    if (prog.storage_root(g2->operands[1]) == root) ++uses, per_head = d2.N * d2.K, uses += (d2.b_tiled || d2.b_batch_stride == per_head) ? 0 : 8;
+    if (uses != 1 || per_head * d1.batch != elements) return false;
+    for (size_t i = 0; i < r.members.size(); ++i) {
+      if (i == 0 || i == r.gemm2_index) continue;
+      for (auto* o : r.members[i]->operands)
+        if (prog.storage_root(o) == root) return false;   // also read by the row program or the epilogue
+    }
+    const int64_t heads_per_part = d1.batch / part.parts;
+    for (int64_t e = 0; e < elements; ++e)
+      if (owner[static_cast<size_t>(e)] != (e / per_head) / heads_per_part) return false;
+    return true;
+  }
+  return false;
+}
+
+void plan_regional_synchronization(const graph::Program& prog, const spec::GraphSpecification& spec, std::vector<Partition>& partition,
+                                   std::vector<NodeFunction>& fns, const NodeGenerator& generate) {
+  const size_t count = prog.nodes.size();
+  std::map<const hlo::Instr*, std::vector<size_t>> readers;
+  std::map<const hlo::Instr*, size_t> writer;
+  for (size_t i = 0; i < count; ++i) {
+    for (auto* r : prog.nodes[i].inputs) readers[r].push_back(i);
+    for (auto* o : prog.nodes[i].outputs) writer[prog.storage_root(o)] = i;
+  }
+  auto direct_tile = [&](const Node& n) {
+    auto it = spec.gemm_spec_list.find(n.name);
+    return n.kind == NodeKind::kGemm && it != spec.gemm_spec_list.end() && it->second.stages < 2 && gemm_uses_mfma(n.gemm) && n.gemm.batch == 1 && !n.gemm.is_conv &&
+           n.prologue.empty();
+  };
+  // candidates by shape
+  for (size_t i = 0; i < count; ++i) {
+    const Node& n = prog.nodes[i];
+    if (n.kind == NodeKind::kAttention && n.gemm3_index == 0) {
+      for (int p = 8; p >= 2; --p)
+        if (n.gemm.batch % p == 0) {
+          partition[i] = {Partition::kHeads, p};
+          break;
+        }
+    } else if (direct_tile(n) && n.gemm.split_k >= 2 && n.gemm.split_k <= 8) {
+      partition[i] = {Partition::kSplitK, n.gemm.split_k};
+    }
+  }
+  for (size_t i = 0; i < count; ++i) {
+    const Node& n = prog.nodes[i];
+    if (!direct_tile(n) || n.gemm.split_k > 1 || n.outputs.empty()) continue;
+    int parts = 0;
+    bool ok = true;
+    for (auto* o : n.outputs) {
+      auto b = prog.buffers.find(prog.storage_root(o));
+      auto rd = readers.find(prog.storage_root(o));
+      ok = ok && b != prog.buffers.end() && b->second.kind == graph::Buffer::kTemp && rd != readers.end() && !rd->second.empty();
+      if (!ok) break;
+      for (size_t j : rd->second) {
+        ok = ok && prog.nodes[j].stage == n.stage + 1 && partition[j].on() && (parts == 0 || parts == partition[j].parts);
+        if (ok) parts = partition[j].parts;
+      }
+    }
+    const spec::GemmSpec& g = spec.gemm_spec_list.at(n.name);
+    if (ok && parts > 0 && n.gemm.N % parts == 0 && n.gemm.N % g.tb_n == 0 && (n.gemm.N / parts) % g.tb_n == 0) partition[i] = {Partition::kColumns, parts};
+  }
+  // Column slices on fewer than 8 XCDs must not cost the stage a second round of units: the GEMMs of a stage that
+  // would go to the XCDs together (the projections in front of an attention node) stay round-robin when the units of
+  // one XCD no longer fit its workgroups although the stage fitted the grid before.
+  {
+    const int64_t grid = spec.runtime.grid_dim.x;
+    std::map<int, std::pair<int64_t, int64_t>> per_stage;   // stage -> (units of one XCD when partitioned, units dealt round-robin)
+    auto tiles = [&](const Node& n) {
+      const spec::GemmSpec& g = spec.gemm_spec_list.at(n.name);
+      return ((n.gemm.M + g.tb_m - 1) / g.tb_m) * ((n.gemm.N + g.tb_n - 1) / g.tb_n);
+    };
+    for (size_t i = 0; i < count; ++i)
+      if (partition[i].kind == Partition::kColumns) {
+        auto& ps = per_stage[prog.nodes[i].stage];
+        ps.first += tiles(prog.nodes[i]) / partition[i].parts;
+        ps.second += tiles(prog.nodes[i]);
+      }
+    for (size_t i = 0; i < count; ++i)
+      if (partition[i].kind == Partition::kColumns) {
+        const auto& ps = per_stage.at(prog.nodes[i].stage);
+        const int64_t rounds_regional = (ps.first + grid / 8 - 1) / (grid / 8), rounds_before = (ps.second + grid - 1) / grid;
+        if (rounds_regional > rounds_before) partition[i] = Partition();
+      }
+  }
+  std::vector<Partition> generated(count);
+  std::set<const hlo::Instr*> roots;
+  for (int round = 0; round < 4; ++round) {
+    for (size_t i = 0; i < count; ++i)
+      if (generated[i].kind != partition[i].kind || generated[i].parts != partition[i].parts) {
+        fns[i] = generate(prog.nodes[i], partition[i]);
+        generated[i] = partition[i];
+      }
+    // values whose every reader fetches what its own XCD wrote
+    roots.clear();
+    for (auto& kv : writer) {
+      const hlo::Instr* root = kv.first;
+      const size_t w = kv.second;
+      auto b = prog.buffers.find(root);
+      auto rd = readers.find(root);
+      if (!(partition[w].kind == Partition::kColumns || partition[w].kind == Partition::kHeads) || b == prog.buffers.end() || b->second.kind != graph::Buffer::kTemp ||
+          rd == readers.end() || rd->second.empty())
+        continue;
+      const WriteMap* wm = nullptr;
+      int maps = 0;
+      for (auto& m : fns[w].write_maps)
+        if (m.root == root) wm = &m, ++maps;
+      if (maps != 1) continue;
+      bool ok = true;
+      for (size_t j : rd->second) ok = ok && partition[j].on() && partition[j].parts == partition[w].parts && prog.nodes[j].stage > prog.nodes[w].stage;
+      std::vector<int8_t> owner;
+      ok = ok && owners_of(*wm, partition[w], root->shape.num_elements(), owner);
+      for (size_t j : rd->second) ok = ok && reads_own_partition(prog, prog.nodes[j], partition[j], root, owner);
+      if (ok) roots.insert(root);
+    }
+    // a partition that keeps nothing inside an XCD only costs parallelism: back to round-robin units
+    bool changed = false;
+    for (size_t i = 0; i < count; ++i) {
+      if (!partition[i].on()) continue;
+      const Node& n = prog.nodes[i];
+      bool in = false, out = !n.outputs.empty();
+      for (auto* r : n.inputs) in = in || roots.count(r) > 0;
+      bool any_out = false;
+      for (auto* o : n.outputs) {
+        out = out && roots.count(prog.storage_root(o)) > 0;
+        any_out = any_out || roots.count(prog.storage_root(o)) > 0;
+      }
+      const bool keep = partition[i].kind == Partition::kColumns ? out : partition[i].kind == Partition::kSplitK ? in : (in || any_out);
+      if (!keep) {
+        partition[i] = Partition();
+        changed = true;
+      }
+    }
+    if (!changed) break;
+    if (round == 3) {   // did not settle: nothing regional
+      roots.clear();
+      for (auto& p : partition) p = Partition();
+    }
+  }
+  for (size_t i = 0; i < count; ++i)
+    if (generated[i].kind != partition[i].kind || generated[i].parts != partition[i].parts) {
+      fns[i] = generate(prog.nodes[i], partition[i]);
+      generated[i] = partition[i];
+    }
+  // the writers of those values take ordinary stores: generated once more with the annotation in place
+  prog.regional_roots = roots;
+  for (size_t i = 0; i < count; ++i) {
+    bool writes = false;
+    for (auto* o : prog.nodes[i].outputs) writes = writes || roots.count(prog.storage_root(o)) > 0;
+    if (writes) fns[i] = generate(prog.nodes[i], partition[i]);
+  }
 }
 }  // namespace
 
@@ -143,13 +356,14 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     int fn_id = 0;
     std::vector<Operand> args;
     int64_t units;
+    int parts = 0;   // regional synchronisation: XCDs that take part in the node (unit u belongs to XCD u % 8); 0 = units dealt round-robin
   };
   std::map<std::string, int> fn_ids;
   std::set<int> preload_fns;   // functions with a companion that requests constant operands ahead of the barrier wait
   std::map<int, std::vector<std::string>> fn_arg_types;   // fn id -> pointer types of its arguments
   std::map<int, std::vector<Call>> by_stage;
   int smem = 0;
-  for (auto& n : prog.nodes) {
+  auto generate_node = [&](const Node& n, const Partition& part) {
     NodeFunction f;
     if (n.kind == NodeKind::kAttention) {
       // the fused node borrows a gemm_spec_list entry; of its fields wave_arrangement.k (key waves) and
@@ -178,7 +392,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
             << "gemm_spec_list[" << n.name << "]: threadblockshape.m " << g.tb_m << " is not a multiple of the " << rows_per_round << " query rows the workgroup's waves take per round";
         row_blocks = g.tb_m / rows_per_round;
       }
-      f = generate_attention(prog, n, ls, it->second.wave_k, spec.hip.operand_preload, row_blocks);
+      f = generate_attention(prog, n, ls, it->second.wave_k, spec.hip.operand_preload, row_blocks, part);
     } else if (n.kind == NodeKind::kGemm) {
       auto it = spec.gemm_spec_list.find(n.name);
       GemmTuning t;
@@ -209,6 +423,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
         t.bk = it->second.tb_k;
       }
       t.split_k = n.gemm.split_k;
+      t.part = part;
       t.preload_b = spec.hip.operand_preload;
       f = generate_gemm(prog, n, ls, t);
     } else {
@@ -244,6 +459,21 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       }
       f = generate_cluster(prog, n, ls, t);
     }
+    return f;
+  };
+  // Every node once with the units dealt round-robin (this also fills the specification with the defaults of nodes
+  // it does not mention); with regional synchronisation the plan then names the nodes whose units go to the XCDs by
+  // ownership and the values that stay inside an XCD, and those nodes are generated again.
+  prog.regional_roots.clear();
+  std::vector<NodeFunction> node_fns;
+  for (auto& n : prog.nodes) node_fns.push_back(generate_node(n, Partition()));
+  std::vector<Partition> partition(prog.nodes.size());
+  const bool regional = spec.hip.regional_synchronization && spec.hip.barrier == "flags_coherent" && hp.grid % 8 == 0 && hp.grid == spec.device.sm_count &&
+                        ls.waves_per_simd == 1 && !spec.hip.cooperative_launch;
+  if (regional) plan_regional_synchronization(prog, spec, partition, node_fns, generate_node);
+  for (size_t ni = 0; ni < prog.nodes.size(); ++ni) {
+    const Node& n = prog.nodes[ni];
+    NodeFunction& f = node_fns[ni];
     bool emit = (allow.empty() || allow.count(n.name)) && !reject.count(n.name);
     std::string fn;
     auto known = fn_by_text.find(f.text);
@@ -271,11 +501,14 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     rep.function = fn;
     rep.stage = n.stage;
     rep.units = f.num_units;
+    if (partition[ni].on())
+      rep.partition = std::string(partition[ni].kind == Partition::kColumns ? "columns/" : partition[ni].kind == Partition::kSplitK ? "split_k/" : "heads/") + std::to_string(partition[ni].parts);
     hp.nodes.push_back(rep);
     if (!emit) continue;
     smem = std::max(smem, f.smem_bytes);
     Call c;
     c.node = &n;
+    c.parts = partition[ni].on() ? partition[ni].parts : 0;
     c.fn = fn;
     c.units = f.num_units;
     c.fn_id = fn_ids.at(fn);
@@ -289,6 +522,35 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   MONONN_CHECK(smem <= spec.device.max_configurable_smem_size, kResourceExhausted)
       << "kernel needs " << smem << " bytes of LDS, device offers " << spec.device.max_configurable_smem_size;
 
+  // Barrier tiers.  A value that does not stay inside an XCD needs a barrier of the memory-side tier somewhere between
+  // its writer's stage and each reader's stage; every other barrier only has to order the workgroups of one XCD.
+  // Fewest memory-side barriers: readers by stage, a barrier right in front of a reader that has none yet in its range.
+  std::vector<bool> regional_before(by_stage.size(), false);
+  if (regional && !prog.regional_roots.empty() && allow.empty() && reject.empty()) {
+    std::map<int, int> index_of_stage;
+    for (auto& st : by_stage) index_of_stage.emplace(st.first, static_cast<int>(index_of_stage.size()));
+    std::vector<std::pair<int, int>> need;   // (reader's stage, first stage after the writer's): emitted stage indices
+    for (auto& st : by_stage)
+      for (auto& c : st.second)
+        for (auto* in : c.node->inputs) {
+          auto pr = prog.producer.find(in);
+          if (pr == prog.producer.end() || prog.regional_roots.count(in)) continue;
+          const int ws = index_of_stage.at(prog.nodes[pr->second].stage), rs = index_of_stage.at(c.node->stage);
+          MONONN_CHECK(ws < rs, kInternal) << c.node->name << " reads a value of its own or a later stage";
+          need.emplace_back(rs, ws + 1);
+        }
+    std::sort(need.begin(), need.end());
+    std::vector<bool> memory_side(by_stage.size(), false);
+    int last = -1;
+    for (auto& iv : need)
+      if (last < iv.second) {
+        last = iv.first;
+        memory_side[last] = true;
+      }
+    for (size_t b = 1; b < by_stage.size(); ++b) regional_before[b] = !memory_side[b];
+  }
+  bool any_regional = false;
+  for (bool r : regional_before) any_regional = any_regional || r;
   // The translation unit is kept in three parts so that the tuner can put many candidate kernels of
   // one node class into a single hipRTC compilation: preamble (defines + include), global
   // declarations (shared by all candidates), body (node functions + kernel).
@@ -305,6 +567,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     for (auto& kv : spec.gemm_spec_list) opaque = opaque || kv.second.stages >= 2;
     pre << "#define MONONN_OPAQUE_THREAD_ID " << (opaque ? 1 : 0) << "\n";
   }
+  if (any_regional) pre << "#define MONONN_REGIONAL_SYNC 1\n";
   pre << "#define MONONN_BARRIER_BUDGET_TICKS " << static_cast<long long>(spec.hip.barrier_timeout_ms) * 100000 << "ull   // wall clock: 100 MHz\n";
   pre << "#include \"headers.h\"\n\n";
   for (auto& c : hp.constants) {
@@ -316,6 +579,11 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     std::ostringstream d;
     d << "__device__ unsigned mononn_barrier_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];";
     hp.global_decls.push_back(d.str());
+    if (any_regional) {
+      std::ostringstream r;
+      r << "__device__ unsigned mononn_regional_flags[" << hp.max_grid << " * mononn_dev::kFlagStride];   // barrier tier over the workgroups of one XCD";
+      hp.global_decls.push_back(r.str());
+    }
     hp.global_decls.push_back("__device__ unsigned mononn_barrier_error[4];   // [0]: 0, or the ordinal (from 1) of the first barrier a wait gave up on");
   }
   hp.profiled = spec.hip.profile_stages;
@@ -356,6 +624,7 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     int first_unit, stage_total;
     bool new_stage;
     int rot;   // unit u of the stage runs on workgroup (u + rot) % grid
+    bool regional;   // the barrier in front of the stage is one of the regional tier
   };
   std::vector<Flat> flat;
   // A workgroup that had a unit in the previous stage reaches the barrier later than an idle one and has asked for
@@ -364,8 +633,9 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   int64_t prev_total = 0, prev_rot = 0;
   bool any_rot = false;
   for (auto& st : by_stage) {
+    // a node whose units belong to XCDs (unit % 8) starts at a multiple of 8 in the stage's unit range
     int64_t total = 0;
-    for (auto& c : st.second) total += c.units;
+    for (auto& c : st.second) total = (c.parts ? (total + 7) / 8 * 8 : total) + c.units;
     MONONN_CHECK(total < (int64_t(1) << 31), kResourceExhausted) << "stage has too many work units";
     int64_t rot = 0;
     if (spec.hip.stage_rotation && hp.grid % 8 == 0 && prev_total > 0 && total + (prev_total + 7) / 8 * 8 <= hp.grid)
@@ -376,7 +646,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     bool ns = true;
     for (auto& c : st.second) {
       hp.stage_nodes.back().push_back(c.node->name);
-      flat.push_back({&c, static_cast<int>(first), static_cast<int>(total), ns, static_cast<int>(rot)});
+      if (c.parts) first = (first + 7) / 8 * 8;
+      flat.push_back({&c, static_cast<int>(first), static_cast<int>(total), ns, static_cast<int>(rot), regional_before[hp.stage_nodes.size() - 1]});
       ns = false;
       first += c.units;
     }
@@ -384,6 +655,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     prev_rot = rot;
   }
   hp.num_barriers = by_stage.empty() ? 0 : static_cast<int>(by_stage.size()) - 1;
+  hp.regional_before = regional_before;
+  for (bool r : regional_before) hp.num_regional_barriers += r ? 1 : 0;
   auto base_expr = [&](const Operand& o) -> std::string {
     if (o.base < 0) return "(char*)" + o.abs;
     std::string b;
@@ -403,15 +676,23 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   src << "void* temp_buffer) {\n";
   src << "  extern __shared__ __attribute__((aligned(16))) char smem[];\n";
   src << "  mononn_dev::GridBarrier barrier;\n  barrier.init(mononn_barrier_flags, mononn_barrier_error);\n";
+  if (any_regional) src << "  barrier.init_regional(mononn_regional_flags);\n";
+  bool any_parts = false;
+  for (auto& f : flat) any_parts = any_parts || f.call->parts > 0;
   src << "  int stage = -1;\n";
   const bool lazy = !preload_fns.empty();
   if (lazy) {
     // The wait half of a barrier is put off until the workgroup's first unit of the new stage, behind the
     // requests for that unit's constant operands; a workgroup without a unit in a stage does not wait for it.
     src << "  bool pending = false;   // announced the end of the previous stage, not yet waited for the others\n";
+    // with two tiers: the latest announcement of each tier that the workgroup has not waited for (a barrier over all
+    // workgroups also covers every regional one before it)
+    if (any_regional) src << "  bool pending_memory = false, pending_regional = false;\n";
   }
   src << "  for (int c = 0; c < " << flat.size() << "; ++c) {\n";
   src << "    int fn = 0, units = 0, first = 0, total = 0" << (any_rot ? ", rot = 0" : "") << ";\n    bool new_stage = false;\n";
+  if (any_regional) src << "    bool regional = false;   // the barrier in front of the stage orders the workgroups of one XCD only\n";
+  if (any_parts) src << "    int parts = 0;   // > 0: unit u belongs to XCD u % 8, and only this many XCDs take part\n";
   src << "    char*";
   for (size_t i = 0; i < max_ptrs; ++i) src << (i ? ", *" : " ") << "p" << i << " = nullptr";
   src << ";\n";
@@ -421,6 +702,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
     src << "      case " << i << ": fn = " << f.call->fn_id << "; units = " << f.call->units << "; first = " << f.first_unit << "; total = "
         << f.stage_total << "; new_stage = " << (f.new_stage ? "true" : "false") << ";";
     if (f.rot) src << " rot = " << f.rot << ";";
+    if (f.regional && f.new_stage) src << " regional = true;";
+    if (f.call->parts) src << " parts = " << f.call->parts << ";";
     for (size_t a = 0; a < f.call->args.size(); ++a) src << " p" << a << " = " << base_expr(f.call->args[a]) << ";";
     src << " break;   // " << f.call->node->name.substr(0, 50) << "\n";
   }
@@ -434,7 +717,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       src << "      if (stage >= 0) {\n        __syncthreads();\n";
       src << "        if (threadIdx.x == 0) " << clk << " + 1] = wall_clock64();\n      }\n";
     }
-    src << "      if (stage >= 0) barrier.sync();\n      ++stage;\n";
+    if (any_regional) src << "      if (stage >= 0) {\n        if (regional) { barrier.arrive_regional(); barrier.wait_regional(); } else barrier.sync();\n      }\n      ++stage;\n";
+    else src << "      if (stage >= 0) barrier.sync();\n      ++stage;\n";
     if (hp.profiled) src << "      if (threadIdx.x == 0) " << clk << "] = wall_clock64();\n";
   } else {
     src << "      if (stage >= 0) {\n";
@@ -444,7 +728,13 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       src << "          if (pending) " << clk << "] = 0;\n";
       src << "          " << clk << " + 1] = pending ? 0 : wall_clock64();\n        }\n";
     }
-    src << "        barrier.arrive();\n        pending = true;\n      }\n      ++stage;\n";
+    if (any_regional) {
+      src << "        if (regional) { barrier.arrive_regional(); pending_regional = true; }\n";
+      src << "        else { barrier.arrive(); pending_memory = true; pending_regional = false; }\n";
+      src << "        pending = true;\n      }\n      ++stage;\n";
+    } else {
+      src << "        barrier.arrive();\n        pending = true;\n      }\n      ++stage;\n";
+    }
     if (hp.profiled) src << "      if (stage == 0 && threadIdx.x == 0) " << clk << "] = wall_clock64();\n";
   }
   src << "    }\n";
@@ -452,12 +742,14 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
   else src << "    for (int u = blockIdx.x; u < total; u += gridDim.x) {\n";
   src << "      const int unit = u - first;\n";
   src << "      if (unit < 0 || unit >= units) continue;\n";
+  if (any_parts) src << "      if (parts > 0 && (unit & 7) >= parts) continue;   // an XCD without a share of this node\n";
   // One dispatch switch; in the lazy form every case first requests what it can, then waits if a barrier is pending
   // (the wait is spelled out per case so that the requested registers flow straight into the function that uses
   // them instead of meeting at a join of all cases).
   std::string wait_text;
   if (lazy) {
-    wait_text = "if (pending) { barrier.wait(); pending = false;";
+    if (any_regional) wait_text = "if (pending) { if (pending_memory) barrier.wait(); if (pending_regional) barrier.wait_regional(); pending = pending_memory = pending_regional = false;";
+    else wait_text = "if (pending) { barrier.wait(); pending = false;";
     if (hp.profiled) wait_text += " if (threadIdx.x == 0) " + clk + "] = wall_clock64();";
     wait_text += " } ";
   }

@@ -43,6 +43,7 @@ struct NodeReport {
   std::string name, kind, function;
   int stage = 0;
   int64_t units = 0;
+  std::string partition;   // regional synchronisation: "columns/8", "split_k/8", "heads/6", or empty
 };
 
 struct HipProgram {
@@ -56,6 +57,10 @@ struct HipProgram {
   std::vector<ConstantInfo> constants;
   std::vector<NodeReport> nodes;
   int num_barriers = 0;
+  // of which barriers of the regional tier (over the workgroups of one XCD); regional_before[s]: the barrier in front
+  // of emitted stage s is one
+  int num_regional_barriers = 0;
+  std::vector<bool> regional_before;
   bool cooperative = false;   // launch through the cooperative-launch entry point
   int grid = 0, block = 0, smem = 0;
   int max_grid = 4096;       // barrier flag capacity

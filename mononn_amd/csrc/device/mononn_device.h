@@ -51,16 +51,6 @@ typedef int int4_t __attribute__((ext_vector_type(4)));
 #ifndef MONONN_OPAQUE_VALUE
 #define MONONN_OPAQUE_VALUE(v) asm volatile("" : "+v"(v))
 #endif
-// 16 bytes written through to the memory side with one instruction.  Agent-scope atomic stores stop at 8 bytes (two
-// instructions, two requests per lane); the cache policy bit they carry (sc1) is available on a plain 16-byte store
-// as well.  The store counts in vmcnt like any other, which is what the grid barrier's arrive() waits on.
-#ifndef MONONN_STORE16_AGENT
-// The compiler does not look inside an asm statement, so it places none of the wait states it would put between a
-// vector-ALU write of the data registers and a store that reads them, nor behind a store of more than 8 bytes whose
-// registers are overwritten next.  Without the idle cycles in front the first dword of some lanes arrived as garbage
-// (measured; identical on every run), with them no wrong value was seen.
-#define MONONN_STORE16_AGENT(p, v) asm volatile("s_nop 7\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory")
-#endif
 // an empty statement that requires `v` in accumulation registers at this point of the program
 #ifndef MONONN_PIN_ACC
 #define MONONN_PIN_ACC(v) asm volatile("" : "+a"(v))
@@ -105,12 +95,75 @@ __device__ __forceinline__ int wave_id() { return thread_id() / kWaveSize; }
 #define MONONN_BARRIER_BUDGET_TICKS 1000000000ull   // 10 s
 #endif
 
+// Regional tier (MONONN_REGIONAL_SYNC): the 8 XCDs of the part have an L2 each, and a launch of one workgroup per
+// compute unit deals the workgroups to them round-robin (workgroup b runs on XCD b % 8; checked at kernel start against
+// the hardware's XCC_ID, a mismatch is reported through the error word).  Where every value that crosses a stage
+// boundary is produced and consumed on the same XCD, the hand-over stays inside that L2: ordinary stores (acknowledged
+// by the L2), a flag array of its own published with a store that stops at the L2, and a wait that looks at the 32
+// flags of the workgroup's XCD only, with loads that miss the compute unit's L1 (nt) and hit the L2.  Measured in
+// isolation, store -> flag -> poll -> dependent load: 0.84 us against 3.1 us through the memory side.
+// Counterpart of the reference's regional synchronisation (regional_synchronization_assignment_pass.cc:35-72).
+#ifndef MONONN_REGIONAL_SYNC
+#define MONONN_REGIONAL_SYNC 0
+#endif
+constexpr int kXcds = 8;
+constexpr unsigned kErrorRegional = 0x40000000u;    // error word: a wait of the regional tier gave up
+constexpr unsigned kErrorPlacement = 0x80000000u;   // error word: a workgroup does not run on XCD blockIdx.x % 8
+
+// a load that is served by the L2 (the compute unit's L1 does not keep what it returns); an asm statement because no
+// builtin combines this cache policy with the ordering a spin loop needs (a load instruction reads no data register
+// that an earlier instruction writes, so there are no wait states for the compiler to place around it)
+#ifndef MONONN_LOAD_THROUGH_L2
+#define MONONN_LOAD_THROUGH_L2(v, p) asm volatile("global_load_dword %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory")
+#endif
+__device__ __forceinline__ unsigned load_through_l2(const unsigned* p) {
+  unsigned v;
+  MONONN_LOAD_THROUGH_L2(v, p);
+  return v;
+}
+
 struct GridBarrier {
   unsigned* flags;   // [gridDim.x * kFlagStride]
   unsigned* error;   // [0]: 0, or 1 + ordinal of the first barrier a wait gave up on
   unsigned epoch;    // last epoch this workgroup has published
   unsigned first;    // epoch at kernel start (for the ordinal in the error word)
   unsigned long long deadline;
+#if MONONN_REGIONAL_SYNC
+  unsigned* rflags;  // [gridDim.x * kFlagStride]: flags of the regional tier
+  unsigned repoch, rfirst;
+
+  __device__ __forceinline__ void init_regional(unsigned* f) {
+    rflags = f;
+    repoch = load_through_l2(&rflags[blockIdx.x * kFlagStride]);
+    rfirst = repoch;
+    const unsigned xcc = __builtin_amdgcn_s_getreg(6164) & (kXcds - 1);   // hwreg(HW_REG_XCC_ID, 0, 4)
+    if (threadIdx.x == 0 && xcc != (blockIdx.x & (kXcds - 1))) {
+      unsigned expected = 0;
+      __hip_atomic_compare_exchange_strong(error, &expected, kErrorPlacement | blockIdx.x, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  // the workgroup's part of the stage is in the XCD's L2 (every wave has its stores acknowledged), then the flag
+  __device__ __forceinline__ void arrive_regional() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    repoch += 1;
+    if (threadIdx.x == 0) __hip_atomic_store(&rflags[blockIdx.x * kFlagStride], repoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  __device__ __forceinline__ void wait_regional() {
+    for (int b = (blockIdx.x & (kXcds - 1)) + kXcds * threadIdx.x; b < (int)gridDim.x; b += kXcds * blockDim.x) {
+      unsigned spins = 0;
+      while ((int)(load_through_l2(&rflags[b * kFlagStride]) - repoch) < 0) {
+        __builtin_amdgcn_s_sleep(1);
+        if ((++spins & 63u) == 0u && wall_clock64() > deadline) {
+          unsigned expected = 0;
+          __hip_atomic_compare_exchange_strong(error, &expected, kErrorRegional | (repoch - rfirst), __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+    __syncthreads();
+  }
+#endif
 
   __device__ __forceinline__ void init(unsigned* f, unsigned* err) {
     flags = f;
@@ -216,6 +269,27 @@ __device__ __forceinline__ void st1(T* p, T v) {
 template <class T>
 __device__ __forceinline__ void st1(T* p, T v) { *p = v; }
 #endif
+#if MONONN_COHERENT_STORES
+// 16 bytes written through to the memory side with one instruction.  Agent-scope atomic stores stop at 8 bytes (two
+// instructions, two requests per lane); the cache policy they carry (sc1) is also available on a buffer store, which
+// the compiler knows as an ordinary store instruction: it places the wait states between whatever produced the data
+// registers (an MFMA, a conversion) and the store, and counts it in vmcnt, which is what the grid barrier's arrive()
+// waits on.  The descriptor spans the 2 GiB window that holds the address: its base, the upper bits of the address,
+// must be wave-uniform, so the lanes of a wave that straddle a window boundary take their turns in the loop.
+typedef unsigned store16_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store16_agent(void* p, store16_t v) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(p);
+  const unsigned window = static_cast<unsigned>(a >> 31), offset = static_cast<unsigned>(a) & 0x7fffffffu;
+  for (;;) {
+    const unsigned w0 = __builtin_amdgcn_readfirstlane(window);
+    if (window == w0) {
+      __builtin_amdgcn_raw_buffer_store_b128(v, __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(static_cast<unsigned long long>(w0) << 31), 0, -1, 0x00020000),
+                                             offset, 0, 16 /* sc1 */);
+      break;
+    }
+  }
+}
+#endif
 // N consecutive elements starting at an address aligned to N * sizeof(T) (N * sizeof(T) in {4, 8, 16})
 template <class T, int N>
 __device__ __forceinline__ void stN(T* p, const T (&v)[N]) {
@@ -231,10 +305,9 @@ __device__ __forceinline__ void stN(T* p, const T (&v)[N]) {
     st1(reinterpret_cast<unsigned long long*>(p), b);
   } else {
 #if MONONN_COHERENT_STORES
-    typedef unsigned v4u __attribute__((ext_vector_type(4)));
-    v4u b;
+    store16_t b;
     __builtin_memcpy(&b, v, 16);
-    MONONN_STORE16_AGENT(p, b);
+    store16_agent(p, b);
 #else
     unsigned long long b[2];
     __builtin_memcpy(b, v, 16);

@@ -145,6 +145,10 @@ struct Program {
   std::map<const hlo::Instr*, TileLayout> physical_tile;
   // GEMM results kept as S fp32 partial sums [S][elements] (split-K); readers add them up
   std::map<const hlo::Instr*, int> split_k;
+  // Storage roots whose every reader runs on the XCD that wrote the bytes it reads (an annotation of the code
+  // generator's regional synchronisation plan, empty otherwise): their writers use ordinary cached stores, the
+  // hand-over stays inside that XCD's L2
+  mutable std::set<const hlo::Instr*> regional_roots;
   std::vector<const hlo::Instr*> live_outs;                        // storage roots, root-tuple order
   std::map<const hlo::Instr*, int> producer;                       // storage root -> node id
   int num_stages = 0;

@@ -318,6 +318,42 @@ void decode_gemm_config(Instr* ins) {
   }
 }
 
+// __cublas$lt$matmul(a, b[, c][, bias]): what newer XLA versions print instead of __cublas$gemm.  Same
+// gemm_backend_config plus `epilogue`; operand c is present when beta != 0, the bias vector (one value per result
+// column) when the epilogue names it; the result may come as a (matrix, workspace) tuple.  The reference knows only
+// __cublas$gemm (core/op/custom_call.cc:96-100, :165-167) and applies alpha / beta as gemm_impl.cc:182-231 reads
+// them; the epilogue semantics here are cuBLASLt's as XLA's GEMM rewriter uses them, reconstructed without a dump of
+// such a module at hand: D = act(alpha * A.B + beta * C + bias), act = identity, max(x, 0) or tanh-GELU.
+void decode_lt_matmul_config(Instr* ins) {
+  decode_gemm_config(ins);
+  auto it = ins->attrs.find("backend_config");
+  Json top = Json::parse(it->second);
+  const Json& j = top.contains("gemm_backend_config") ? top.at("gemm_backend_config") : top;
+  std::string ep = "DEFAULT";
+  if (j.contains("epilogue")) {
+    const Json& e = j.at("epilogue");
+    static const char* by_number[] = {"DEFAULT", "BIAS", "RELU", "BIAS_RELU", "GELU", "BIAS_GELU", "GELU_AUX", "BIAS_GELU_AUX"};
+    if (e.is_string()) ep = e.as_string();
+    else {
+      const int64_t k = e.as_int();
+      MONONN_CHECK(k >= 0 && k < 8, kUnsupported) << ins->hlo_name << ": unknown epilogue number " << k;
+      ep = by_number[k];
+    }
+  }
+  MONONN_CHECK(ep == "DEFAULT" || ep == "BIAS" || ep == "RELU" || ep == "GELU" || ep == "BIAS_RELU" || ep == "BIAS_GELU", kUnsupported)
+      << ins->hlo_name << ": epilogue " << ep << " of __cublas$lt$matmul is not supported (an auxiliary output has no place in the one-result call)";
+  ins->gemm.epilogue = ep;
+  const size_t want = 2 + (ins->gemm.beta != 0 ? 1 : 0) + (ep.rfind("BIAS", 0) == 0 ? 1 : 0);
+  MONONN_CHECK(ins->operands.size() == want, kParseError)
+      << ins->hlo_name << ": __cublas$lt$matmul with beta " << ins->gemm.beta << " and epilogue " << ep << " takes " << want << " operands, got " << ins->operands.size();
+  if (ins->shape.is_tuple()) {
+    MONONN_CHECK(!ins->shape.tuple.empty() && !ins->shape.tuple[0].is_tuple(), kParseError) << ins->hlo_name << ": __cublas$lt$matmul yields (matrix, workspace)";
+    Shape arr = ins->shape.tuple[0];
+    ins->shape = arr;
+    ins->lt_tuple_result = true;
+  }
+}
+
 // window={size=16x16 stride=16x16 pad=1_1x1_1}: fields separated by blanks, dimensions by 'x'
 std::map<std::string, std::vector<std::string>> window_fields(const std::string& raw) {
   std::map<std::string, std::vector<std::string>> out;
@@ -597,6 +633,10 @@ void decode_attrs(Instr* ins, Module* mod) {
       MONONN_CHECK(ins->tuple_index == 0, kUnsupported) << ins->hlo_name << ": the scratch result of a convolution call cannot be used";
       ins->opcode = "bitcast";
     }
+    if (!ins->operands.empty() && ins->operands[0]->lt_tuple_result) {
+      MONONN_CHECK(ins->tuple_index == 0, kUnsupported) << ins->hlo_name << ": the workspace of a __cublas$lt$matmul call cannot be used";
+      ins->opcode = "bitcast";
+    }
   }
   if (op == "iota") ins->iota_dimension = std::strtoll(need("iota_dimension").c_str(), nullptr, 10);
   if (op == "slice") {
@@ -688,6 +728,8 @@ void decode_attrs(Instr* ins, Module* mod) {
     ins->custom_call_target = need("custom_call_target");
     if (ins->custom_call_target == "__cublas$gemm") {
       decode_gemm_config(ins);
+    } else if (ins->custom_call_target == "__cublas$lt$matmul") {
+      decode_lt_matmul_config(ins);
     } else if (ins->custom_call_target == "__cudnn$convForward") {
       decode_conv_config(ins);
     } else {
@@ -945,6 +987,119 @@ void fold_layout_transposes_into_gemms(Computation* comp, std::set<const Instr*>
 
 }  // namespace
 
+// The epilogue of a __cublas$lt$matmul call (bias vector, ReLU, tanh-GELU) becomes what the older dialect writes for
+// it: a kLoop fusion behind the call, computed in f32 and rounded to the result type.  The GEMM-epilogue fusion of the
+// compiler then runs it on the accumulator tile like any other element-wise consumer of a GEMM.
+void lower_lt_matmul_epilogues(Module* mod) {
+  int serial = 0;
+  for (size_t ci = 0; ci < mod->computations.size(); ++ci) {
+    Computation* comp = mod->computations[ci].get();
+    for (size_t at = 0; at < comp->instrs.size(); ++at) {
+      Instr* call = comp->instrs[at].get();
+      if (call->opcode != "custom-call" || call->custom_call_target != "__cublas$lt$matmul" || call->gemm.epilogue == "DEFAULT") continue;
+      const std::string ep = call->gemm.epilogue;
+      const bool has_bias = ep.rfind("BIAS", 0) == 0;
+      const bool relu = ep.find("RELU") != std::string::npos, gelu = ep.find("GELU") != std::string::npos;
+      Instr* bias = nullptr;
+      if (has_bias) {
+        bias = call->operands.back();
+        MONONN_CHECK(bias->shape.rank() == 1 && !call->shape.dims.empty() && bias->shape.dims[0] == call->shape.dims.back(), kInvalidArgument)
+            << call->hlo_name << ": the bias of __cublas$lt$matmul must be a vector with one value per result column";
+        unlink_user(bias, call);
+        call->operands.pop_back();
+      }
+      MONONN_CHECK(is_float(call->shape.dtype), kUnsupported) << call->hlo_name << ": epilogue on a non-float result";
+      auto body = std::make_unique<Computation>();
+      body->hlo_name = body->name = "lt_matmul_epilogue_" + std::to_string(serial++);
+      while (mod->by_name.count(body->name)) body->hlo_name = body->name = "lt_matmul_epilogue_" + std::to_string(serial++);
+      Computation* bc = body.get();
+      int counter = 0;
+      auto add = [&](const char* opcode, DType t, const std::vector<int64_t>& dims, std::vector<Instr*> operands) {
+        auto ins = std::make_unique<Instr>();
+        ins->hlo_name = ins->name = std::string(opcode == std::string("parameter") ? "param_" : "lt_") + std::to_string(counter++);
+        ins->opcode = opcode;
+        ins->shape.dtype = t;
+        ins->shape.dims = dims;
+        for (int i = static_cast<int>(dims.size()) - 1; i >= 0; --i) ins->shape.minor_to_major.push_back(i);
+        ins->operands = std::move(operands);
+        for (auto* o : ins->operands) o->users.push_back(ins.get());
+        ins->parent = bc;
+        ins->index_in_comp = static_cast<int>(bc->instrs.size());
+        bc->instrs.push_back(std::move(ins));
+        return bc->instrs.back().get();
+      };
+      const std::vector<int64_t>& dims = call->shape.dims;
+      const DType rt = call->shape.dtype;
+      Instr* p0 = add("parameter", rt, dims, {});
+      p0->parameter_number = 0;
+      bc->params.push_back(p0);
+      Instr* p1 = nullptr;
+      if (has_bias) {
+        p1 = add("parameter", bias->shape.dtype, bias->shape.dims, {});
+        p1->parameter_number = 1;
+        bc->params.push_back(p1);
+      }
+      auto constant = [&](const char* text) {
+        Instr* c = add("constant", DType::kF32, {}, {});
+        c->literal = text;
+        Instr* b = add("broadcast", DType::kF32, dims, {c});
+        return b;
+      };
+      auto f32 = [&](Instr* v) { return v->shape.dtype == DType::kF32 ? v : add("convert", DType::kF32, v->shape.dims, {v}); };
+      Instr* x = f32(p0);
+      if (has_bias) {
+        Instr* b = add("broadcast", DType::kF32, dims, {f32(p1)});
+        b->dimensions = {static_cast<int64_t>(dims.size()) - 1};
+        x = add("add", DType::kF32, dims, {x, b});
+      }
+      if (relu) x = add("maximum", DType::kF32, dims, {x, constant("0")});
+      if (gelu) {
+        // 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
+        Instr* x3 = add("multiply", DType::kF32, dims, {add("multiply", DType::kF32, dims, {x, x}), x});
+        Instr* inner = add("add", DType::kF32, dims, {x, add("multiply", DType::kF32, dims, {constant("0.044715"), x3})});
+        Instr* t = add("tanh", DType::kF32, dims, {add("multiply", DType::kF32, dims, {constant("0.7978845608028654"), inner})});
+        x = add("multiply", DType::kF32, dims, {add("multiply", DType::kF32, dims, {constant("0.5"), x}), add("add", DType::kF32, dims, {constant("1"), t})});
+      }
+      if (rt != DType::kF32) x = add("convert", rt, dims, {x});
+      x->is_root = true;
+      bc->root = x;
+      // the fusion takes the call's place for every user
+      auto fus = std::make_unique<Instr>();
+      Instr* f = fus.get();
+      f->hlo_name = f->name = call->name + "_epilogue";
+      f->opcode = "fusion";
+      f->fusion_kind = "kLoop";
+      f->called = bc;
+      f->shape = call->shape;
+      f->parent = comp;
+      std::vector<Instr*> users = call->users;
+      call->users.clear();
+      for (Instr* u : users)
+        for (auto& o : u->operands)
+          if (o == call) {
+            o = f;
+            if (std::find(f->users.begin(), f->users.end(), u) == f->users.end()) f->users.push_back(u);
+          }
+      f->operands = {call};
+      call->users.push_back(f);
+      if (has_bias) {
+        f->operands.push_back(bias);
+        bias->users.push_back(f);
+      }
+      if (comp->root == call) {
+        comp->root = f;
+        f->is_root = true;
+        call->is_root = false;
+      }
+      comp->instrs.insert(comp->instrs.begin() + static_cast<long>(at) + 1, std::move(fus));
+      for (size_t i = 0; i < comp->instrs.size(); ++i) comp->instrs[i]->index_in_comp = static_cast<int>(i);
+      mod->by_name[bc->name] = bc;
+      mod->computations.push_back(std::move(body));
+      comp = mod->computations[ci].get();
+    }
+  }
+}
+
 std::unique_ptr<Module> parse_module(const std::string& text) {
   auto mod = std::make_unique<Module>();
   Lexer lx(text);
@@ -1067,6 +1222,7 @@ std::unique_ptr<Module> parse_module(const std::string& text) {
     mod->computations.push_back(std::move(comp));
   }
   MONONN_CHECK(mod->entry != nullptr, kParseError) << "module has no ENTRY computation";
+  lower_lt_matmul_epilogues(mod.get());
   std::set<const Instr*> layout_transposes;
   for (auto& comp : mod->computations) {
     normalize_layouts(comp.get(), &layout_transposes);

@@ -51,6 +51,9 @@ struct GemmConfig {   // backend_config of __cublas$gemm (gemm_impl.cc:182-231)
   std::vector<int> lhs_batch, rhs_batch;
   int64_t batch_size = 1, lhs_stride = 0, rhs_stride = 0;
   std::string selected_algorithm;
+  // __cublas$lt$matmul only: DEFAULT, BIAS, RELU, GELU, BIAS_RELU, BIAS_GELU (the epilogue enum of the newer call);
+  // the parser turns it into a fusion behind the call, after which the field is documentation
+  std::string epilogue = "DEFAULT";
 };
 
 // __cudnn$convForward (attributes read by ir_parser_fused.cc:749-823, lowering conv_impl.cc:252-324):
@@ -96,7 +99,12 @@ struct Instr {
   bool is_conv() const { return opcode == "custom-call" && custom_call_target == "__cudnn$convForward"; }
   // a dense contraction with a decoded GemmConfig: the cuBLAS custom call, or a plain `dot` (what a stock XLA
   // prints before its GEMM rewriter has run)
-  bool is_gemm() const { return (opcode == "custom-call" && custom_call_target == "__cublas$gemm") || opcode == "dot"; }
+  bool is_gemm() const {
+    return (opcode == "custom-call" && (custom_call_target == "__cublas$gemm" || custom_call_target == "__cublas$lt$matmul")) || opcode == "dot";
+  }
+  // __cublas$lt$matmul written with a (result, workspace) tuple: the call carries the result's array shape and its
+  // get-tuple-element 0 aliases it, as with the convolution call
+  bool lt_tuple_result = false;
 
   std::vector<Instr*> users;           // within the same computation
   bool is_scalar_constant() const { return opcode == "constant" && shape.num_elements() == 1 && !literal_elided; }

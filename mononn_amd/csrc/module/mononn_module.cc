@@ -111,7 +111,9 @@ std::string MonoNNModule::summary() const {
   std::ostringstream os;
   os << "module " << module_name_ << " kernel " << kernel_name_ << "\n";
   if (program_) os << program_->summary();
-  os << "grid=" << hip_.grid << " block=" << hip_.block << " smem=" << hip_.smem << " barriers=" << hip_.num_barriers << "\n";
+  os << "grid=" << hip_.grid << " block=" << hip_.block << " smem=" << hip_.smem << " barriers=" << hip_.num_barriers;
+  if (hip_.num_regional_barriers > 0) os << " (" << hip_.num_regional_barriers << " of them over one XCD's workgroups)";
+  os << "\n";
   for (size_t i = 0; i < hip_.param_bytes.size(); ++i) os << "Parameter " << i << ": " << hip_.param_bytes[i] << " bytes.\n";
   for (size_t i = 0; i < hip_.liveout_bytes.size(); ++i) os << "Liveout(output) buffer " << i << " size: " << hip_.liveout_bytes[i] << " bytes.\n";
   os << "Temporary buffer size: " << hip_.temp_bytes << " bytes.\n";
@@ -429,7 +431,21 @@ void MonoNNModule::synchronize(void* stream) {
   size_t flag_bytes = 0;
   void* flags = dev_.global("mononn_barrier_flags", &flag_bytes);
   dev_.zero(flags, flag_bytes);
+  if (hip_.num_regional_barriers > 0) {
+    size_t regional_bytes = 0;
+    void* regional = dev_.global("mononn_regional_flags", &regional_bytes);
+    dev_.zero(regional, regional_bytes);
+  }
   dev_.zero(err, err_bytes);
+  // error word of the device runtime: bit 31 = a workgroup found itself on another XCD than its index modulo 8 says,
+  // bit 30 = the wait that gave up belongs to the regional tier
+  MONONN_CHECK((word[0] & 0x80000000u) == 0, kRuntimeError)
+      << "kernel " << kernel_name_ << ": workgroup " << (word[0] & 0x7fffffffu) << " does not run on XCD " << (word[0] & 7u)
+      << " (regional synchronisation assumes that a grid of one workgroup per compute unit is dealt to the 8 XCDs round-robin); the outputs of this launch are invalid";
+  MONONN_CHECK((word[0] & 0x40000000u) == 0, kRuntimeError)
+      << "kernel " << kernel_name_ << ": a workgroup gave up waiting at regional barrier " << (word[0] & 0x3fffffffu) << " of " << hip_.num_regional_barriers << " after "
+      << spec_.hip.barrier_timeout_ms << " ms (mononn_hip.barrier_timeout_ms): the grid of " << grid_
+      << " workgroups was not resident as a whole (another kernel running on the device?); the outputs of this launch are invalid";
   MONONN_FAIL(kRuntimeError) << "kernel " << kernel_name_ << ": a workgroup gave up waiting at grid barrier " << word[0] << " of " << hip_.num_barriers
                              << " after " << spec_.hip.barrier_timeout_ms << " ms (mononn_hip.barrier_timeout_ms): the grid of " << grid_
                              << " workgroups was not resident as a whole (another kernel running on the device?); the outputs of this launch are invalid";

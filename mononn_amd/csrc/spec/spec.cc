@@ -143,6 +143,7 @@ Json GraphSpecification::to_json() const {
   h["pack_left_operands"] = hip.pack_left_operands;
   h["attention_out_proj_fusion"] = hip.attention_out_proj_fusion;
   h["stage_rotation"] = hip.stage_rotation;
+  h["regional_synchronization"] = hip.regional_synchronization;
   j["mononn_hip"] = h;
   return j;
 }
@@ -230,7 +231,7 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
   s.codegen_reject_list = strings_from(j, "codegen_reject_list");
   if (j.contains("mononn_hip")) {
     const Json& h = j.at("mononn_hip");
-    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "layer_norm_folding", "barrier", "profile_stages", "cooperative_launch", "operand_preload", "pack_left_operands", "attention_out_proj_fusion", "stage_rotation", "barrier_timeout_ms", "opaque_thread_id"}, "mononn_hip");
+    check_keys(h, {"merge_dependent", "gemm_epilogue_fusion", "transpose_constant_b", "assign_operand_layouts", "fuse_attention", "gemm_prologue_fusion", "layer_norm_folding", "barrier", "profile_stages", "cooperative_launch", "operand_preload", "pack_left_operands", "attention_out_proj_fusion", "stage_rotation", "barrier_timeout_ms", "opaque_thread_id", "regional_synchronization"}, "mononn_hip");
     s.hip.merge_dependent = getb(h, "merge_dependent", true);
     s.hip.gemm_epilogue_fusion = getb(h, "gemm_epilogue_fusion", true);
     s.hip.transpose_constant_b = getb(h, "transpose_constant_b", true);
@@ -248,6 +249,7 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
     s.hip.pack_left_operands = getb(h, "pack_left_operands", true);
     s.hip.attention_out_proj_fusion = getb(h, "attention_out_proj_fusion", false);
     s.hip.stage_rotation = getb(h, "stage_rotation", true);
+    s.hip.regional_synchronization = getb(h, "regional_synchronization", false);
   }
   MONONN_CHECK(s.runtime.grid_dim.x >= 1 && s.runtime.grid_dim.y == 1 && s.runtime.grid_dim.z == 1, kSpecError) << "grid must be 1-D";
   MONONN_CHECK(s.runtime.block_dim.x >= 64 && s.runtime.block_dim.x % 64 == 0 && s.runtime.block_dim.x <= 1024 && s.runtime.block_dim.y == 1 && s.runtime.block_dim.z == 1,

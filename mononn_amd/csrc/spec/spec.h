@@ -105,6 +105,12 @@ struct HipOptions {       // "mononn_hip" section
   bool attention_out_proj_fusion = false;
   // a stage whose units fit beside those of the stage before it runs on the workgroups that stage left idle
   bool stage_rotation = true;
+  // Regional synchronisation (regional_synchronization_assignment_pass.cc:35-72 in the reference): chains of stages
+  // whose hand-overs can be kept inside one XCD (a GEMM's column slices feeding the k slices of the next GEMM; the
+  // heads of a projection feeding the attention and its output projection) are dealt to the XCDs by ownership, their
+  // intermediate results are written with ordinary stores and the barrier between them is one over the XCD's 32
+  // workgroups through its L2.  Takes effect on a grid of one workgroup per compute unit with the "flags_coherent" barrier.
+  bool regional_synchronization = false;
 };
 
 struct GraphSpecification {

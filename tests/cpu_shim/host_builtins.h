@@ -26,7 +26,9 @@
 #define __builtin_amdgcn_s_barrier() ((void)0)
 #define __builtin_amdgcn_readfirstlane(x) (x)
 #define MONONN_PIN_ACC(v) ((void)0) /* register placement only */
-#define MONONN_STORE16_AGENT(p, v) std::memcpy((void*)(p), &(v), 16) /* a GPU store instruction written in assembly */
+#define MONONN_LOAD_THROUGH_L2(v, p) ((v) = *(p)) /* a GPU load instruction written in assembly */
+#define __HIP_MEMORY_SCOPE_WORKGROUP 1
+#define __builtin_amdgcn_s_getreg(reg) (blockIdx.x & 7u) /* the only register read is the XCD number */
 #define MONONN_OPAQUE_VALUE(v) ((void)0) /* an empty asm with a GPU register constraint */
 /* buffer descriptor + 16-byte load at descriptor base + lane offset + wave offset */
 typedef const char* __amdgpu_buffer_rsrc_t;
@@ -36,6 +38,9 @@ inline host_uint4 __builtin_amdgcn_raw_buffer_load_b128(const char* rsrc, unsign
   host_uint4 v;
   std::memcpy(&v, rsrc + (size_t)voffset + (size_t)soffset, 16);
   return v;
+}
+inline void __builtin_amdgcn_raw_buffer_store_b128(host_uint4 v, const char* rsrc, unsigned voffset, unsigned soffset, int) {
+  std::memcpy(const_cast<char*>(rsrc) + (size_t)voffset + (size_t)soffset, &v, 16);
 }
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) (src)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
