@@ -300,6 +300,27 @@ class Computation:
                           attrs=f'custom_call_target="__cublas$gemm", backend_config="{cfg_s}"',
                           name_hint="cublas-batch-gemm" if batch > 1 else "cublas-gemm")
 
+    def lt_matmul(self, a: Value, b: Value, lhs_contract: int, rhs_contract: int, epilogue: str = "DEFAULT", bias: Optional[Value] = None,
+                  alpha: float = 1.0, beta: float = 0.0, addend: Optional[Value] = None, nested_config: bool = True) -> Value:
+        """`__cublas$lt$matmul` custom call as newer XLA versions print it: operands (a, b[, c][, bias]), the
+        `gemm_backend_config` of `gemm` plus `epilogue` (DEFAULT, BIAS, RELU, GELU, BIAS_RELU, BIAS_GELU)."""
+        r = len(a.dims)
+        assert r == 2 and len(b.dims) == 2, "unbatched matrices"
+        m_dim = 1 if lhs_contract == 0 else 0
+        n_dim = 1 if rhs_contract == 0 else 0
+        assert a.dims[lhs_contract] == b.dims[rhs_contract]
+        out_dims = [a.dims[m_dim], b.dims[n_dim]]
+        cfg = {"alpha_real": alpha, "alpha_imag": 0, "beta": beta,
+               "dot_dimension_numbers": {"lhs_contracting_dimensions": [str(lhs_contract)], "rhs_contracting_dimensions": [str(rhs_contract)],
+                                         "lhs_batch_dimensions": [], "rhs_batch_dimensions": []},
+               "epilogue": epilogue}
+        if nested_config:
+            cfg = {"gemm_backend_config": cfg}
+        cfg_s = json.dumps(cfg, separators=(",", ":")).replace('"', '\\"')
+        ops = [a, b] + ([addend] if addend is not None else []) + ([bias] if bias is not None else [])
+        return self._emit("custom-call", a.dtype, out_dims, ops,
+                          attrs=f'custom_call_target="__cublas$lt$matmul", backend_config="{cfg_s}"', name_hint="cublas-lt-matmul")
+
     def dot(self, a: Value, b: Value, lhs_contract: int, rhs_contract: int, batch_dims: Sequence[int] = ()) -> Value:
         """Plain `dot` with the same operand conventions as `gemm` (what XLA prints before its GEMM rewriter)."""
         r = len(a.dims)

@@ -23,7 +23,10 @@ from . import MonoNNModule
 from .hlo import models
 
 
-def stage_report(hlo_text: str, constants, inputs, outputs, spec_dir=None, launches=50, device=0):
+def stage_report(hlo_text: str, constants, inputs, outputs, spec_dir=None, launches=50, device=0, details=None):
+    """Rows of the report, one per stage.  `details`, when given, is filled with what the profiled build computed
+    (`outputs`, the live-outs of the last launch) and with its event-timed duration (`kernel_us`, the average over
+    `launches` back-to-back launches): the report's steps must add up to the kernel they describe."""
     base = MonoNNModule.from_spec_dir(hlo_text, spec_dir) if spec_dir else MonoNNModule.compile(hlo_text, build=False)
     spec = json.loads(base.get_tuning_spec())
     spec["mononn_hip"]["profile_stages"] = True
@@ -45,6 +48,11 @@ def stage_report(hlo_text: str, constants, inputs, outputs, spec_dir=None, launc
     for a in acc:
         for k in ("busy_us", "barrier_us", "mean_wg_us", "step_us"):
             a[k] /= launches
+    if details is not None:
+        details["outputs"] = m.run(inputs, outputs)
+        avg_ms, _ = m.time_raw(m.buffer_pointers(), warmup=5, iters=max(launches, 20))
+        m.synchronize()
+        details["kernel_us"] = avg_ms * 1e3
     m.close()
     return acc
 

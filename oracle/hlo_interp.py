@@ -488,6 +488,8 @@ class Evaluator:
                 return self._gemm(ins, x, dt)
             if target == "__cudnn$convForward":
                 return self._conv_forward(ins, x)
+            if target == "__cublas$lt$matmul":
+                return self._lt_matmul(ins, x, dt)
             raise NotImplementedError(f"custom-call target {target}")
         raise NotImplementedError(f"opcode {op}")
 
@@ -584,6 +586,46 @@ class Evaluator:
         with np.errstate(over="ignore"):
             return D.astype(dt, copy=False)
 
+
+    def _lt_matmul(self, ins: Instr, x, dt):
+        """__cublas$lt$matmul(a, b[, c][, bias]), the newer spelling of the cuBLAS call.  The reference accepts only
+        __cublas$gemm (core/op/custom_call.cc:96-100); alpha / beta / dimension numbers are read as for that call
+        (gemm_impl.cc:182-231), the `epilogue` field follows cuBLASLt as XLA's GEMM rewriter uses it:
+        D = act(alpha * A.B + beta * C + bias[column]), act = identity | max(., 0) | tanh-GELU, evaluated in fp32 and
+        rounded once to the result type.  Reconstructed without a dump of such a module: parity unpinned against XLA."""
+        cfg = json.loads(ins.attrs["backend_config"][1:-1].replace('\\"', '"'))
+        cfg = cfg.get("gemm_backend_config", cfg)
+        ep = cfg.get("epilogue", "DEFAULT")
+        if not isinstance(ep, str):
+            ep = ["DEFAULT", "BIAS", "RELU", "BIAS_RELU", "GELU", "BIAS_GELU", "GELU_AUX", "BIAS_GELU_AUX"][int(ep)]
+        if ep not in ("DEFAULT", "BIAS", "RELU", "GELU", "BIAS_RELU", "BIAS_GELU"):
+            raise NotImplementedError(f"__cublas$lt$matmul epilogue {ep}")
+        dn = cfg["dot_dimension_numbers"]
+        lc, rc = int(dn["lhs_contracting_dimensions"][0]), int(dn["rhs_contracting_dimensions"][0])
+        A, B = x[0].astype(np.float32), x[1].astype(np.float32)
+        r = A.ndim
+        A = np.swapaxes(A, -1, -2) if lc == r - 2 else A
+        B = np.swapaxes(B, -1, -2) if rc == r - 1 else B
+        D = np.einsum("...mk,...kn->...mn", A, B) * np.float32(cfg["alpha_real"])
+        nxt = 2
+        if float(cfg["beta"]) != 0.0:
+            D = D + np.float32(cfg["beta"]) * x[nxt].astype(np.float32)
+            nxt += 1
+        if ep.startswith("BIAS"):
+            D = D + x[nxt].astype(np.float32)[None, :]
+            nxt += 1
+        if len(x) != nxt:
+            raise ValueError("__cublas$lt$matmul: operand count does not match beta and epilogue")
+        if ep.endswith("RELU"):
+            D = np.maximum(D, np.float32(0))
+        if ep.endswith("GELU"):
+            D = np.float32(0.5) * D * (np.float32(1) + np.tanh(np.float32(0.7978845608028654) * (D + np.float32(0.044715) * D * D * D)))
+        out_sh = ins.shape.tuple_shapes[0] if ins.shape.tuple_shapes else ins.shape
+        with np.errstate(over="ignore"):
+            out = D.astype(self.np_dtype(out_sh.dtype))
+        if ins.shape.tuple_shapes:
+            return (out, np.zeros(ins.shape.tuple_shapes[1].dims, np.uint8))
+        return out
 
     def _conv_forward(self, ins: Instr, x):
         """cuDNN forward convolution custom call as the reference lowers it (conv_impl.cc:252-324, attributes

@@ -165,6 +165,34 @@ def test_gather_bit_exact(gpu_device):
     assert np.array_equal(got.view(np.uint16), t[i].view(np.uint16))
 
 
+@pytest.mark.parametrize("epilogue,beta", [("DEFAULT", 0.0), ("BIAS", 0.0), ("RELU", 0.0), ("GELU", 0.0), ("BIAS_RELU", 2.0), ("BIAS_GELU", 0.0), ("BIAS_GELU", 0.5)])
+def test_lt_matmul_cases(gpu_device, epilogue, beta):
+    """__cublas$lt$matmul (a, b[, c][, bias]) with every epilogue of its enum that has one result, on the MFMA tile with
+    the epilogue fused, against the oracle's own restatement of the call (core/op/custom_call.cc:96-100 knows only the
+    older spelling; gemm_impl.cc:182-231 for alpha / beta)."""
+    M, K, N = 128, 256, 384
+    mb = HloModuleBuilder("cluster_7__lt_test.1")
+    e = mb.entry
+    a = e.parameter("f16", (M, K), "a")
+    w = e.elided_constant("f16", (K, N), "w/kernel")
+    c = e.parameter("f16", (M, N), "c") if beta else None
+    bias = e.elided_constant("f16", (N,), "w/bias") if epilogue.startswith("BIAS") else None
+    e.set_tuple_root([e.lt_matmul(a, w, 1, 0, epilogue=epilogue, bias=bias, alpha=0.25, beta=beta, addend=c)])
+    rng = np.random.default_rng(11)
+    A = rng.normal(0, 1, (M, K)).astype(np.float16)
+    C = rng.normal(0, 1, (M, N)).astype(np.float16)
+    names = list(mb.constants)
+    consts = {names[0]: rng.normal(0, 1, (K, N)).astype(np.float16)}
+    if bias is not None:
+        consts[names[1]] = rng.normal(0, 2, (N,)).astype(np.float16)
+    inputs = [A] + ([C] if beta else [])
+    text = mb.text()
+    assert MonoNNModule.compile(text, build=False).launch_dims()["barriers"] == 0   # one stage: the epilogue runs in the tile
+    (got,), _ = run_module(text, inputs, consts, [{"dtype": "f16", "dims": [M, N]}])
+    want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
+    assert np.abs(got.astype(np.float32) - want).max() <= 2e-3 * np.abs(want).max() + 1e-3
+
+
 def _spec_with(hlo_text, gemm_overrides=None, hip=None, grid=None):
     """Default specification with some entries replaced; per-node maps are cleared so that nodes whose names
     change with the fusion decisions get fresh defaults."""

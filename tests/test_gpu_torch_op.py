@@ -3,6 +3,7 @@ import numpy as np
 import pytest
 
 from mononn_amd.hlo import models
+from oracle import hlo_interp
 
 pytestmark = pytest.mark.gpu
 
@@ -92,8 +93,18 @@ def test_perf_report_lists_every_stage(gpu_device, tmp_path):
     import csv
     from mononn_amd import perf_report
     fx = models.bert_encoder(L=2, B=1, S=64, H=256, NH=4, F=512, vocab=300, max_pos=64)
-    rows = perf_report.stage_report(fx.hlo_text, fx.make_constants(5, "baseline"), fx.make_inputs(5), fx.outputs, launches=5, device=gpu_device)
+    consts, inputs, details = fx.make_constants(5, "random"), fx.make_inputs(5), {}
+    rows = perf_report.stage_report(fx.hlo_text, consts, inputs, fx.outputs, launches=20, device=gpu_device, details=details)
     assert len(rows) == 15 and [r["stage"] for r in rows] == list(range(15))
+    # the profiled build computes what the module computes (mononn_module_tuner.cc:422-448 reports on the kernel it runs) ...
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0].astype(np.float64).ravel()
+    got = details["outputs"][0].astype(np.float64).ravel()
+    assert np.abs(got - want).max() <= 2e-2 and got @ want / (np.linalg.norm(got) * np.linalg.norm(want)) >= 0.9999
+    # ... and its steps add up to that kernel: first workgroup in to last workgroup out, against the event-timed launch
+    # period of the same build (which also holds the launch itself and the kernel's first and last instructions)
+    steps = sum(r["step_us"] for r in rows)
+    print(f"sum of steps {steps:.1f} us, event-timed kernel {details['kernel_us']:.1f} us", flush=True)
+    assert 0.80 * details["kernel_us"] <= steps <= 1.02 * details["kernel_us"], (steps, details["kernel_us"])
     assert all(r["busy_us"] > 0 and r["mean_wg_us"] > 0 and r["step_us"] > 0 for r in rows)
     assert all(r["barrier_us"] > 0 for r in rows[:-1])
     assert any("cublas_gemm" in r["nodes"] for r in rows)

@@ -430,6 +430,33 @@ def test_plain_dot_and_nested_backend_config_are_gemms():
     assert m1.get_source("main.hip") == m2.get_source("main.hip")
 
 
+def _lt_module(epilogue, beta=0.0, n_operands=None):
+    mb = HloModuleBuilder("cluster_5__lt.1")
+    e = mb.entry
+    a = e.parameter("f16", (128, 256), "a")
+    w = e.elided_constant("f16", (256, 512), "w/kernel")
+    c = e.parameter("f16", (128, 512), "c") if beta else None
+    bias = e.elided_constant("f16", (512,), "w/bias") if epilogue.startswith("BIAS") else None
+    e.set_tuple_root([e.lt_matmul(a, w, 1, 0, epilogue=epilogue, bias=bias, beta=beta, addend=c)])
+    return mb
+
+
+def test_lt_matmul_becomes_a_gemm_with_a_fused_epilogue():
+    # core/op/custom_call.cc:96-100 accepts __cublas$gemm only; the newer spelling lowers onto the same GEMM node with
+    # its epilogue enum as an element-wise cluster behind it, which the GEMM-epilogue fusion takes into the tile
+    plain = MonoNNModule.compile(_lt_module("DEFAULT").text(), build=False)
+    assert "gemm    cublas_lt_matmul_" in plain.summary() and "members=1" in plain.summary() and "f16_b1_m128_n512_k256_ak_bp" in plain.summary()
+    fused = MonoNNModule.compile(_lt_module("BIAS_GELU", beta=1.0).text(), build=False)
+    s = fused.summary()
+    assert "stages=1" in s and "members=2" in s            # one stage: bias, addend and GELU run in the GEMM's epilogue
+    src = fused.get_source("main.hip")
+    assert "fast_tanh" in src or "tanhf" in src
+    for bad, code in ((_lt_module("BIAS").text().replace('\\"epilogue\\":\\"BIAS\\"', '\\"epilogue\\":\\"BIAS_GELU_AUX\\"'), "UNSUPPORTED"),
+                      (_lt_module("BIAS").text().replace('\\"epilogue\\":\\"BIAS\\"', '\\"epilogue\\":\\"RELU\\"'), "PARSE_ERROR")):
+        with pytest.raises(MonoNNError, match=code):
+            MonoNNModule.compile(bad, build=False)
+
+
 def test_dump_contains_a_standalone_driver_and_the_constants(layer, tmp_path):
     # host_codegen.cc:31-73 counterpart: the dump can be run without the library
     m = MonoNNModule.compile(layer.hlo_text, build=True)

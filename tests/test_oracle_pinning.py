@@ -340,6 +340,58 @@ def test_dot_matches_einsum_and_the_gemm_call():
     assert np.array_equal(got_dot, got_gemm)
 
 
+@pytest.mark.parametrize("epilogue", ["DEFAULT", "BIAS", "RELU", "GELU", "BIAS_RELU", "BIAS_GELU"])
+def test_lt_matmul_matches_einsum_and_the_closed_forms(epilogue):
+    # the newer spelling of the cuBLAS call: D = act(alpha A.B + beta C + bias) against einsum in fp64 and torch's
+    # relu / tanh-approximated gelu as library routines (a dropped bias, a bias along the rows instead of the columns,
+    # the erf form of GELU or an activation applied before the addend all fail here)
+    rng = np.random.default_rng(47)
+    M, K, N = 24, 40, 56
+    A = rng.normal(0, 1, (M, K)).astype(np.float16)
+    B = rng.normal(0, 1, (N, K)).astype(np.float16)          # stored [N, K]: contracting dimension 1
+    C = rng.normal(0, 1, (M, N)).astype(np.float16)
+    bias = rng.normal(0, 2, (N,)).astype(np.float16)
+    mb = HloModuleBuilder("cluster_5__lt.1")
+    e = mb.entry
+    a, b, c = e.parameter("f16", A.shape, "a"), e.parameter("f16", B.shape, "b"), e.parameter("f16", C.shape, "c")
+    bv = e.parameter("f16", bias.shape, "bias") if epilogue.startswith("BIAS") else None
+    e.set_tuple_root([e.lt_matmul(a, b, 1, 1, epilogue=epilogue, bias=bv, alpha=0.5, beta=2.0, addend=c)])
+    feeds = [A, B, C] + ([bias] if bv is not None else [])
+    got = hlo_interp.evaluate(mb.text(), feeds, {}, "fp32")[0].astype(np.float64)
+    want = 0.5 * np.einsum("mk,nk->mn", A.astype(np.float64), B.astype(np.float64)) + 2.0 * C.astype(np.float64)
+    if bv is not None:
+        want = want + bias.astype(np.float64)[None, :]
+    t = torch.tensor(want)
+    if epilogue.endswith("RELU"):
+        want = torch.relu(t).numpy()
+    if epilogue.endswith("GELU"):
+        want = torch.nn.functional.gelu(t, approximate="tanh").numpy()
+    assert np.abs(got - want).max() < 3e-5
+    # as written (f16 result): one rounding of the fp32 value
+    got16 = hlo_interp.evaluate(mb.text(), feeds, {})[0]
+    assert got16.dtype == np.float16 and np.abs(got16.astype(np.float64) - want).max() <= 2.0 ** -11 * np.abs(want).max() + 1e-6
+
+
+def test_lt_matmul_with_a_workspace_tuple_and_numbered_epilogue():
+    # (matrix, workspace) result read through get-tuple-element, fields not nested, epilogue given by its enum number
+    text = """HloModule cluster_5__lt2.1
+
+ENTRY %main (a: f16[8,16], b: f16[16,4], bias: f16[4]) -> (f16[8,4]) {
+  %a = f16[8,16]{1,0} parameter(0)
+  %b = f16[16,4]{1,0} parameter(1)
+  %bias = f16[4]{0} parameter(2)
+  %lt = (f16[8,4]{1,0}, s8[256]{0}) custom-call(f16[8,16]{1,0} %a, f16[16,4]{1,0} %b, f16[4]{0} %bias), custom_call_target="__cublas$lt$matmul", backend_config="{\\"alpha_real\\":1,\\"alpha_imag\\":0,\\"beta\\":0,\\"dot_dimension_numbers\\":{\\"lhs_contracting_dimensions\\":[\\"1\\"],\\"rhs_contracting_dimensions\\":[\\"0\\"],\\"lhs_batch_dimensions\\":[],\\"rhs_batch_dimensions\\":[]},\\"epilogue\\":3}"
+  %d = f16[8,4]{1,0} get-tuple-element((f16[8,4]{1,0}, s8[256]{0}) %lt), index=0
+  ROOT %t = (f16[8,4]{1,0}) tuple(f16[8,4]{1,0} %d)
+}
+"""
+    rng = np.random.default_rng(48)
+    A, B, bias = rng.normal(0, 1, (8, 16)).astype(np.float16), rng.normal(0, 1, (16, 4)).astype(np.float16), rng.normal(0, 1, (4,)).astype(np.float16)
+    got = hlo_interp.evaluate(text, [A, B, bias], {}, "fp32")[0]
+    want = np.maximum(A.astype(np.float64) @ B.astype(np.float64) + bias.astype(np.float64), 0)   # 3 = BIAS_RELU
+    assert np.abs(got - want).max() < 1e-5
+
+
 @pytest.mark.parametrize("xd,size,stride,pad", [
     ((2, 9, 10, 8), (1, 3, 3, 1), (1, 2, 2, 1), ((0, 0), (1, 1), (1, 1), (0, 0))),
     ((1, 8, 8, 4), (1, 2, 2, 1), (1, 2, 2, 1), ((0, 0), (0, 0), (0, 0), (0, 0))),
