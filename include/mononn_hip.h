@@ -104,6 +104,9 @@ int mononn_module_load(mononn_module* m, int device);
  * load time.  Launches of such kernels must not overlap on one device (two partly resident grids would wait for
  * each other at their first grid barrier): use one stream, or build with "mononn_hip": {"cooperative_launch": true}
  * in the specification, which lets the runtime keep them apart.
+ * The outputs of a launch are known to be valid once mononn_module_synchronize has returned MONONN_OK for it: a
+ * caller that waits for the stream by other means (hipStreamSynchronize, an event, a framework's own stream
+ * order) does not see a barrier wait that gave up, and the error word stays set until that call reads and clears it.
  * Replaces: Launch(...) of profile_kernel (mononn_module_tuner.cc:135-139); the call is asynchronous
  *           on `stream` (a hipStream_t, NULL = default stream). */
 int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);
@@ -113,7 +116,8 @@ int mononn_launch(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, voi
  * the library's own device image instead of a buffer of the caller, and the call allocates nothing.  device_ptrs:
  * entry parameters in parameter order, then live-out buffers -- no temp slot.  A module whose temp arena is larger
  * is refused with MONONN_RESOURCE_EXHAUSTED.  Each GPU holds one such array from the first mononn_module_load on it
- * until the process ends; every call on a GPU, from any module, shares it, so calls that overlap on one GPU race.
+ * until the process ends (64 MiB of device memory per GPU for every process that loads a module, whether it uses
+ * this entry point or not); every call on a GPU, from any module, shares it, so calls that overlap on one GPU race.
  * Nothing in the arena has to start at zero: every temp address is written before it is read in the same launch.
  * No counterpart in the reference. */
 int mononn_launch_static_temp(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream);

@@ -61,7 +61,8 @@ namespace mononn_dev {
 constexpr int kWaveSize = 64;
 constexpr int kFlagStride = 64;   // 256 bytes between workgroup flags: measured fastest among 64 B .. 4 KiB
 
-// The thread's index in its workgroup, opaque to the compiler (MONONN_OPAQUE_THREAD_ID, the default): the kernel is
+// The thread's index in its workgroup, opaque to the compiler (MONONN_OPAQUE_THREAD_ID: the host compiler turns it on in
+// kernels that hold an LDS-staged GEMM tile or whose specification asks for it, off otherwise): the kernel is
 // one function holding every stage, and whatever the compiler can derive from threadIdx.x once -- lane and wave
 // numbers, address parts of every stage -- it computes ahead of the stage loop and keeps in registers through all
 // stages.  A stage with a large register tile then pushes those values out to scratch, and the stages that use

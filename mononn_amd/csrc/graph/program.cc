@@ -28,7 +28,7 @@ const Node* Program::node_of(const Instr* member) const {
 
 std::string GemmDesc::problem_hash() const {
   std::ostringstream os;
-  os << (f32 ? "f32_b" : "f16_b") << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_packed ? "_bp" : (b_k_contig ? "_bk" : "_bn"));
+  os << (f32 ? "f32_b" : bf16 ? "bf16_b" : "f16_b") << batch << "_m" << M << "_n" << N << "_k" << K << (a_k_contig ? "_ak" : "_am") << (b_packed ? "_bp" : (b_k_contig ? "_bk" : "_bn"));
   if (is_conv) os << "_conv" << conv.R << "x" << conv.S << "s" << conv.stride_h << "x" << conv.stride_w << "p" << conv.pad_h << "x" << conv.pad_w;
   return os.str();
 }

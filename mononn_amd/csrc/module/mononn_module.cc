@@ -181,8 +181,7 @@ static float half_bits_to_float(uint16_t b) {
 bool MonoNNModule::resolve_device_bytes(const codegen::ConstantInfo& ci, std::vector<char>* out) const {
   std::vector<char> s0, s1;
   if (ci.derived()) {
-    // f32[N]: sum over k of vector[k] * weight[k, n], accumulated in double (the weights as the host gave them,
-    // before any scaling)
+    // f32[N]: sum over k of vector[k] * weight[k, n], accumulated in double
     const std::vector<char>* w = raw_payload(ci.sums_weight, &s0);
     const std::vector<char>* v = raw_payload(ci.sums_vector, &s1);
     if (!w || !v) return false;
@@ -190,10 +189,19 @@ bool MonoNNModule::resolve_device_bytes(const codegen::ConstantInfo& ci, std::ve
     MONONN_CHECK(static_cast<int64_t>(w->size()) == K * N * 2, kInternal) << "sources of " << ci.name << " do not match";
     const uint16_t* wp = reinterpret_cast<const uint16_t*>(w->data());
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(v->data());
+    // The sums that go with the scaled weights (vector = the gamma those weights were multiplied by) are taken over
+    // the products as the MFMAs read them, rounded to half: the epilogue's x . W' - mean * colsum(W') is then
+    // (x - mean) . W' exactly, whatever the row's mean.  (Over the unrounded products an error of mean * sum of the
+    // rounding errors of a column stays behind, which grows with |mean| / sigma of the row.)
+    bool of_scaled_weights = false;
+    for (auto& other : hip_.constants) of_scaled_weights = of_scaled_weights || (other.name == ci.sums_weight && other.row_scale_by == ci.sums_vector);
     std::vector<double> acc(static_cast<size_t>(N), 0.0);
     for (int64_t k = 0; k < K; ++k) {
-      const double vk = half_bits_to_float(vp[k]);
-      for (int64_t n = 0; n < N; ++n) acc[n] += vk * half_bits_to_float(wp[k * N + n]);
+      const float vk = half_bits_to_float(vp[k]);
+      for (int64_t n = 0; n < N; ++n) {
+        const float w = half_bits_to_float(wp[k * N + n]);
+        acc[n] += of_scaled_weights ? static_cast<double>(static_cast<float>(static_cast<_Float16>(w * vk))) : static_cast<double>(vk) * w;
+      }
     }
     out->assign(static_cast<size_t>(N) * 4, 0);
     for (int64_t n = 0; n < N; ++n) {

@@ -24,8 +24,12 @@ _REGISTRY: Dict[int, "MonoNNFunction"] = {}
 class MonoNNFunction:
     """Callable view of a module whose constants are uploaded and which is loaded on `device`."""
 
-    def __init__(self, module: MonoNNModule, outputs: Sequence[dict], device: int = 0):
+    def __init__(self, module: MonoNNModule, outputs: Sequence[dict], device: int = 0, checked: bool = False):
+        """`checked`: every call waits for its launch through mononn_module_synchronize and raises when a grid-barrier
+        wait gave up (the outputs are then invalid).  Unchecked calls stay asynchronous on torch's current stream, and
+        such a failure only shows in the caller's next MonoNNModule.synchronize()."""
         self.module = module
+        self.checked = checked
         self.outputs = list(outputs)
         self.device = torch.device("cuda", device)
         info = module.buffer_info()
@@ -57,7 +61,10 @@ class MonoNNFunction:
             outs.append(t)
             ptrs.append(t.data_ptr())
         ptrs.append(0 if self._temp is None else self._temp.data_ptr())
-        self.module.launch_raw(ptrs, torch.cuda.current_stream(self.device).cuda_stream)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        self.module.launch_raw(ptrs, stream)
+        if self.checked:
+            self.module.synchronize(stream)
         return outs
 
 

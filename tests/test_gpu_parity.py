@@ -217,6 +217,44 @@ def _gemm_instr_names(hlo_text):
     return [n.replace(".", "_").replace("-", "_") for n in re.findall(r"%(cublas-gemm\.\d+) =", hlo_text)]
 
 
+def test_folded_layer_norm_on_rows_far_from_zero(gpu_device):
+    """LayerNorm folded into weights and epilogue, h.W = r (x.W' - mean colsum(W')) + beta^T W with W' = half(gamma o W):
+    the column sums must belong to the weights the MFMAs multiply, or an error of r * mean * (sum of a column's
+    rounding errors) stays behind.  Rows with |mean| = 40 sigma make that term visible: against the oracle the folded
+    kernel must be as close as the kernel that runs the LayerNorm as written."""
+    import json
+    from test_host_compiler import norm_gemm_module
+    text, _ = norm_gemm_module(True)
+    M, K, N = 64, 256, 128
+    rng = np.random.default_rng(71)
+    x = (rng.normal(0, 0.25, (M, K)) + rng.choice([-10.0, 10.0], (M, 1))).astype(np.float16)
+    m0 = MonoNNModule.compile(text, build=False)
+    names = [c["name"] for c in m0.constants() if c["needs_payload"]]
+    m0.close()
+    assert len(names) == 3
+    consts = {}
+    sizes = {c["name"]: c["bytes"] for c in MonoNNModule.compile(text, build=False).constants() if c["needs_payload"]}
+    vecs = sorted(n for n in sizes if sizes[n] == K * 2)
+    mats = [n for n in sizes if sizes[n] == K * N * 2]
+    consts[vecs[0]] = rng.uniform(0.5, 1.5, (K,)).astype(np.float16)        # gamma
+    consts[vecs[1]] = rng.normal(0, 0.5, (K,)).astype(np.float16)           # beta
+    consts[mats[0]] = rng.normal(0, 0.05, (K, N)).astype(np.float16)
+    want = hlo_interp.evaluate(text, [x], consts, "fp32")[0].astype(np.float64)
+    outs = [{"dtype": "f16", "dims": [M, N]}]
+    (plain,), m1 = run_module(text, [x], consts, outs)
+    spec = json.loads(MonoNNModule.compile(text, build=False).get_tuning_spec())
+    spec["mononn_hip"].update(gemm_prologue_fusion=True, layer_norm_folding=True)
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"] = {}, {}
+    (folded,), m2 = run_module(text, [x], consts, outs, json.dumps(spec))
+    assert "ln_stats[" in m2.get_source("main.hip")
+    err_plain = np.abs(plain.astype(np.float64) - want).max()
+    err_folded = np.abs(folded.astype(np.float64) - want).max()
+    print(f"rows at |mean| = 40 sigma: as written {err_plain:.3e}, folded {err_folded:.3e}", flush=True)
+    assert err_folded <= max(2 * err_plain, 4e-3 * np.abs(want).max())
+    m1.close()
+    m2.close()
+
+
 def test_fusion_variants_agree(gpu_device):
     """Every stage-fusion decision must leave the result unchanged (bit for bit where the arithmetic is the
     same, within fp16 rounding where a reduction order changes)."""

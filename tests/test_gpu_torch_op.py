@@ -43,6 +43,11 @@ def test_custom_op_matches_the_ctypes_path_bit_for_bit(gpu_device):
     with pytest.raises(AssertionError):
         fn(tin[0][:, :32], tin[1], tin[2])          # wrong size is refused before anything is launched
     fn.close()
+    # checked mode: every call waits for its launch and would raise on a barrier wait that gave up
+    checked = torch_op.MonoNNFunction(m, fx.outputs, gpu_device, checked=True)
+    (got4,) = torch_op.forward(checked, *tin)
+    assert np.array_equal(got4.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    checked.close()
     m.close()
 
 

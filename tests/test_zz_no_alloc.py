@@ -27,8 +27,13 @@ def _both_ways(m, fx, inputs, device):
     torch.cuda.synchronize()
     ptrs = [t.data_ptr() for t in bufs["params"]] + [t.data_ptr() for t in bufs["liveouts"]]
     stream = torch.cuda.current_stream().cuda_stream
+    # what the entry point exists for: the call takes no device memory (the driver's count of free bytes on the GPU
+    # is the same before the launch and after it has finished)
+    free_before, _ = torch.cuda.mem_get_info(device)
     m.launch_static_temp(ptrs, stream)                        # no temp slot: the library's static arena
     m.synchronize(stream)
+    free_after, _ = torch.cuda.mem_get_info(device)
+    assert free_after == free_before, f"launch_static_temp changed the free device memory by {free_before - free_after} bytes"
     got = bufs["liveouts"][0].cpu().numpy().view(np.float16).reshape(fx.outputs[0]["dims"])
     return got, want
 
