@@ -581,9 +581,11 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     // graph changes shape: the candidates are compared on GEMM stage + consumer stage together, against the
     // same pair of stages of the unsplit graph.
     double stitched_us = -1;
+    std::string why_not;   // why the last whole kernel was not built or timed; written beside its -1 in the log
     auto whole_kernel_us = [&](GraphSpecification s) -> double {
       s.codegen_allow_list.clear();
       s.hip.profile_stages = false;
+      why_not.clear();
       try {
         MonoNNModule m(params.hlo_text, s.to_json().dump(0), params.kernel_name);
         m.generate_code();
@@ -594,8 +596,18 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         return us;
       } catch (const Error& e) {
         if (verbose) std::fprintf(stderr, "[mononn tuner] %s   a whole kernel was not built: %.200s\n", ctx_str.c_str(), e.what());
+        why_not = e.what();
+        for (char& ch : why_not)
+          if (ch == '\n') ch = ' ';
+        if (why_not.size() > 160) why_not = why_not.substr(0, 160) + "...";
         return -1;
       }
+    };
+    // " <label>=<us>", with the reason in brackets behind a candidate that produced no kernel
+    auto timed = [&](const std::string& label, double us) {
+      char buf[64];
+      std::snprintf(buf, sizeof buf, "=%.2f", us);
+      return " " + label + buf + (us < 0 && !why_not.empty() ? " [" + why_not + "]" : std::string());
     };
     // ---- whole-kernel refinement ------------------------------------------------------------------------
     // A class is timed above in a kernel that holds nothing but its own stages, where every workgroup reaches
@@ -647,9 +659,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             else if (c.kind == "cluster_elewise") s.cluster_elewise_spec[n] = alt.spec.cluster_elewise_spec.at(n);
           }
           const double us = whole_kernel_us(s);
-          char buf[160];
-          std::snprintf(buf, sizeof buf, " %s=%.2f", alt.label.c_str(), us);
-          line += buf;
+          line += timed(alt.label, us);
           if (us > 0 && (best_alt_us < 0 || us < best_alt_us)) {
             best_alt_us = us;
             best_alt = &alt;
@@ -892,7 +902,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             GraphSpecification adopted = trials[i].spec;
             drop_unknown(adopted, trials[i].mod->program());
             const double with_split = whole_kernel_us(adopted);
-            log << " " << trials[i].label << "=" << with_split;
+            log << timed(trials[i].label, with_split);
             if (with_split > 0 && (best_with < 0 || with_split < best_with)) {
               best_with = with_split;
               best_spec = std::move(adopted);
@@ -926,8 +936,8 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
                 if (!changed) continue;
                 const double us = whole_kernel_us(s);
                 char buf[64];
-                std::snprintf(buf, sizeof buf, " tier%d_ilp%d=%.2f", tier, ilp, us);
-                line += buf;
+                std::snprintf(buf, sizeof buf, "tier%d_ilp%d", tier, ilp);
+                line += timed(buf, us);
                 if (us > 0 && (best_knobs_us < 0 || us < best_knobs_us)) {
                   best_knobs_us = us;
                   best_knobs = std::move(s);
@@ -1030,9 +1040,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
                 for (auto& n : groups.at({fam.first, pos[i]})) apply_gemm(s2, n, cd.t, g.K);
               const double us2 = whole_kernel_us(s2);
               char buf[112];
-              std::snprintf(buf, sizeof buf, " first%zu:tile%dx%d_waves%dx%dx%d(%lld units each)=%.2f", p, cd.t.bm, cd.t.bn, cd.t.wm, cd.t.wn, cd.t.wk,
-                            static_cast<long long>(cd.units), us2);
-              line += buf;
+              std::snprintf(buf, sizeof buf, "first%zu:tile%dx%d_waves%dx%dx%d(%lld units each)", p, cd.t.bm, cd.t.bn, cd.t.wm, cd.t.wn, cd.t.wk,
+                            static_cast<long long>(cd.units));
+              line += timed(buf, us2);
               if (us2 > 0 && (best_us2 < 0 || us2 < best_us2)) {
                 best_us2 = us2;
                 best_spec2 = std::move(s2);
@@ -1047,6 +1057,143 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             stitched = std::move(best_spec2);
             stitched_us = best_us2;
           }
+        }
+      }
+    }
+    // ---- stage-fusion decisions ------------------------------------------------------------------------
+    // Which stages exist is a tuning decision like any tile (the reference's per-node implementation alternatives,
+    // tuning_space_generator.cc:139-307, and its pass switches, config.cc:82-86): with the tiles settled, every decision
+    // of the specification's mononn_hip section that changes the stage list or the barrier tiers is tried on the whole
+    // kernel and kept when that kernel is faster.  A decision that merges nodes renames them: the new nodes start from
+    // the tile of the GEMM instruction they contain, and the GEMMs that changed get a short tile search of their own.
+    if (promising && !env::is_true("MONONN_TUNER_NO_FUSION_SEARCH") && !env::is_true("MONONN_TUNER_NO_REFINEMENT")) {
+      struct Decision {
+        const char* name;
+        void (*set)(spec::HipOptions&);
+        bool (*is_on)(const spec::HipOptions&);
+      };
+      const Decision decisions[] = {
+          {"regional_synchronization", [](spec::HipOptions& h) { h.regional_synchronization = true; }, [](const spec::HipOptions& h) { return h.regional_synchronization; }},
+          {"attention_out_proj_fusion", [](spec::HipOptions& h) { h.attention_out_proj_fusion = true; }, [](const spec::HipOptions& h) { return h.attention_out_proj_fusion; }},
+          {"layer_norm_folding", [](spec::HipOptions& h) { h.gemm_prologue_fusion = h.layer_norm_folding = true; }, [](const spec::HipOptions& h) { return h.layer_norm_folding; }},
+          {"gemm_prologue_fusion", [](spec::HipOptions& h) { h.gemm_prologue_fusion = true; }, [](const spec::HipOptions& h) { return h.gemm_prologue_fusion; }},
+      };
+      auto plain = [](GraphSpecification s) {
+        s.codegen_allow_list.clear();
+        s.hip.profile_stages = false;
+        return s;
+      };
+      // node name -> name of the GEMM instruction inside, and the nodes of a specification's graph
+      auto gemm_instr_of = [&](const GraphSpecification& s, std::map<std::string, std::string>* instr_of, std::map<std::string, graph::GemmDesc>* desc_of,
+                               std::set<std::string>* all_nodes, std::map<std::string, bool>* has_prologue) {
+        MonoNNModule probe(params.hlo_text, plain(s).to_json().dump(0), "mononn_probe");
+        probe.generate_code();
+        for (auto& n : probe.program().nodes) {
+          all_nodes->insert(n.name);
+          if (n.kind != graph::NodeKind::kGemm) continue;
+          (*instr_of)[n.name] = n.members[0]->name;
+          (*desc_of)[n.name] = n.gemm;
+          (*has_prologue)[n.name] = !n.prologue.empty();
+        }
+      };
+      if (stitched_us < 0) stitched_us = whole_kernel_us(stitched);
+      for (const Decision& d : decisions) {
+        if (d.is_on(stitched.hip) || stitched_us < 0) continue;
+        GraphSpecification s = stitched;
+        d.set(s.hip);
+        std::string line;
+        double best_d = -1;
+        GraphSpecification best_spec_d;
+        try {
+          std::map<std::string, std::string> old_instr, new_instr;
+          std::map<std::string, graph::GemmDesc> old_desc, new_desc;
+          std::map<std::string, bool> old_pro, new_pro;
+          std::set<std::string> old_nodes, new_nodes;
+          gemm_instr_of(stitched, &old_instr, &old_desc, &old_nodes, &old_pro);
+          // the graph under the decision: entries of nodes that no longer exist would be refused, so only the k splits
+          // stay (a split GEMM goes by the name of its instruction and shapes the nodes around it); where the decision
+          // takes such a GEMM away (a projection absorbed by its attention node), its split goes with it
+          GraphSpecification bare = s;
+          bare.cluster_reduce_spec.clear();
+          bare.cluster_elewise_spec.clear();
+          for (auto it = bare.gemm_spec_list.begin(); it != bare.gemm_spec_list.end();) it = it->second.split_k > 1 ? std::next(it) : bare.gemm_spec_list.erase(it);
+          for (;;) {
+            try {
+              gemm_instr_of(bare, &new_instr, &new_desc, &new_nodes, &new_pro);
+              break;
+            } catch (const Error&) {
+              if (bare.gemm_spec_list.empty()) throw;
+              new_instr.clear(), new_desc.clear(), new_nodes.clear(), new_pro.clear();
+              bare.gemm_spec_list.erase(bare.gemm_spec_list.begin());
+            }
+          }
+          auto drop = [&](auto& m) {
+            for (auto it = m.begin(); it != m.end();) it = new_nodes.count(it->first) ? std::next(it) : m.erase(it);
+          };
+          drop(s.gemm_spec_list);
+          drop(s.cluster_reduce_spec);
+          drop(s.cluster_elewise_spec);
+          std::map<std::string, std::string> entry_of_instr;   // GEMM instruction -> node that held it before
+          for (auto& kv : old_instr) entry_of_instr[kv.second] = kv.first;
+          std::vector<std::string> renamed;
+          for (auto& kv : new_instr) {
+            if (s.gemm_spec_list.count(kv.first)) continue;
+            renamed.push_back(kv.first);
+            auto from = entry_of_instr.find(kv.second);
+            if (from == entry_of_instr.end() || !stitched.gemm_spec_list.count(from->second)) continue;
+            // the tile moves with the instruction when the generator takes it for the new node
+            GraphSpecification with = s;
+            with.gemm_spec_list[kv.first] = stitched.gemm_spec_list.at(from->second);
+            try {
+              MonoNNModule probe(params.hlo_text, plain(with).to_json().dump(0), "mononn_probe");
+              probe.generate_code();
+              s = std::move(with);
+            } catch (const Error&) {
+            }
+          }
+          double us = whole_kernel_us(s);
+          line += timed("as_is", us);
+          if (us > 0) best_d = us, best_spec_d = s;
+          // the GEMMs whose node changed, by problem: a few tiles each, on the whole kernel
+          if (us > 0 && us < 1.15 * stitched_us && !renamed.empty()) {
+            std::map<std::string, std::vector<std::string>> families;
+            for (auto& n : renamed) families[new_desc.at(n).problem_hash() + (new_pro.at(n) ? "_pro" : "")].push_back(n);
+            for (auto& fam : families) {
+              const graph::GemmDesc& g = new_desc.at(fam.second[0]);
+              if (!codegen::gemm_uses_mfma(g)) continue;
+              std::vector<codegen::GemmTuning> tiles = gemm_candidates(g, cx.block / 64, std::max(budget, 1));
+              // nearest to the grid first: the tiles whose unit count fills the workgroups once
+              const int64_t grid = base.runtime.grid_dim.x;
+              std::stable_sort(tiles.begin(), tiles.end(), [&](const codegen::GemmTuning& a, const codegen::GemmTuning& b) {
+                auto units = [&](const codegen::GemmTuning& t) { return ((g.M + t.bm - 1) / t.bm) * ((g.N + t.bn - 1) / t.bn) * g.batch * std::max(1, g.split_k); };
+                auto badness = [&](int64_t u) { return u > grid ? (u - grid) * 4 : grid - u; };
+                return badness(units(a)) < badness(units(b));
+              });
+              if (tiles.size() > 6) tiles.resize(6);
+              for (auto& t : tiles) {
+                GraphSpecification s2 = best_spec_d;
+                for (auto& n : fam.second) {
+                  const int split = s2.gemm_spec_list.count(n) ? s2.gemm_spec_list.at(n).split_k : 1;
+                  apply_gemm(s2, n, t, g.K / std::max(1, g.split_k));
+                  s2.gemm_spec_list[n].split_k = split;
+                }
+                const double us2 = whole_kernel_us(s2);
+                char lbl[96];
+                std::snprintf(lbl, sizeof lbl, "%s:tile%dx%d_waves%dx%dx%d%s", fam.first.c_str(), t.bm, t.bn, t.wm, t.wn, t.wk, t.stages >= 2 ? "_lds" : "");
+                line += timed(lbl, us2);
+                if (us2 > 0 && us2 < best_d) best_d = us2, best_spec_d = std::move(s2);
+              }
+            }
+          }
+        } catch (const Error& e) {
+          line += std::string(" not applicable [") + e.what() + "]";
+        }
+        log << "  [" << ctx_str << "] fusion decision " << d.name << ", whole kernel: now " << stitched_us << " us;" << line
+            << (best_d > 0 && best_d < 0.997 * stitched_us ? "  -> adopted" : "  -> not adopted") << "\n";
+        if (verbose) std::fprintf(stderr, "[mononn tuner] %s fusion decision %s: now %.2f us;%s\n", ctx_str.c_str(), d.name, stitched_us, line.c_str());
+        if (best_d > 0 && best_d < 0.997 * stitched_us) {
+          stitched = std::move(best_spec_d);
+          stitched_us = best_d;
         }
       }
     }

@@ -46,6 +46,21 @@ def test_tuned_module_dump_tree_and_reload(gpu_device, encoder, tmp_path, monkey
     log = open(os.path.join(cluster, "tuning_log.log")).read()
     assert "Tuning result for each thread grid setting" in log and "gemm x" in log and " ms\n" in log
     assert "whole kernel" in log                         # the class winners were confirmed in the whole kernel
+    # the stage-fusion decisions were tried as whole-kernel alternatives (tuning_space_generator.cc:139-307: per-node
+    # implementation alternatives), each with a verdict, and the specification records what was kept
+    import re
+    verdicts = dict(re.findall(r"fusion decision (\w+), whole kernel: now [\d.]+ us;.*?-> (adopted|not adopted)", log))
+    for line in log.splitlines():
+        if "fusion decision" in line:
+            print(line[:500], flush=True)
+    hip = json.loads(tuned.get_tuning_spec())["mononn_hip"]
+    # (the prologue fusion is not a question of its own once the folding, which implies it, has been adopted)
+    assert {"regional_synchronization", "attention_out_proj_fusion", "layer_norm_folding"} <= set(verdicts), verdicts
+    assert "gemm_prologue_fusion" in verdicts or hip["gemm_prologue_fusion"] is True
+    for name, verdict in verdicts.items():
+        if verdict == "adopted":
+            assert hip[name] is True
+    assert not re.search(r"=-1\.00(?! \[)", log)         # a candidate that produced no kernel says why
     report = open(os.path.join(cluster, "performance_report.csv")).read().splitlines()
     assert len(report) > 10 and all(len(r.split(",")) == 3 for r in report[1:])
     # the tree is enough to get the same kernel back, bit for bit
