@@ -654,14 +654,15 @@ bool can_merge_clusters(const Program& prog, const std::vector<const Instr*>& pr
 bool gemm_uses_mfma(const graph::GemmDesc& g) {
   if (g.f32) return !g.is_conv && g.a_k_contig;   // f32 tiles take any k extent and either right-operand layout
   if (g.is_conv && !g.conv_fragment_loads()) return false;
-  // the left operand k-contiguous; the right one k-contiguous, packed, or a plain [K, N] matrix (gathered per lane)
-  if (!g.a_k_contig) return false;
+  // either operand k-contiguous, or a plain matrix with k as its slow dimension (gathered per lane); the right one
+  // also packed.  An m-contiguous left operand comes as plain memory only: no fragment order, no convolution map.
+  if (!g.a_k_contig && (g.a_packed || g.is_conv)) return false;
   // a k extent that is not a multiple of 32 is zero-filled in the last step, from plain row-major operands only
   return g.K % 32 == 0 || (!g.is_conv && !g.b_packed && !g.a_packed && g.split_k <= 1);
 }
 
 // the LDS-staged tile copies k-contiguous or fragment-order operands
-static bool gemm_lds_capable(const graph::GemmDesc& g) { return !g.f32 && gemm_uses_mfma(g) && (g.b_k_contig || g.b_packed) && g.K % 32 == 0; }
+static bool gemm_lds_capable(const graph::GemmDesc& g) { return !g.f32 && gemm_uses_mfma(g) && g.a_k_contig && (g.b_k_contig || g.b_packed) && g.K % 32 == 0; }
 
 GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus) {
   GemmTuning t;
@@ -761,7 +762,7 @@ void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const
   MONONN_CHECK(t.bm % (16 * t.wm) == 0 && t.bn % (16 * t.wn) == 0 && t.bm > 0 && t.bn > 0, kSpecError)
       << "GEMM tile " << t.bm << "x" << t.bn << " is not a multiple of 16 per wave";
   if (t.stages >= 2) {
-    MONONN_CHECK(g.b_k_contig || g.b_packed, kSpecError) << "an LDS-staged GEMM tile takes a k-contiguous or packed right operand";
+    MONONN_CHECK(g.a_k_contig && (g.b_k_contig || g.b_packed), kSpecError) << "an LDS-staged GEMM tile takes a k-contiguous left operand and a k-contiguous or packed right operand";
     MONONN_CHECK(!has_prologue && t.wk == 1 && g.K % 32 == 0, kSpecError) << "an LDS-staged GEMM tile takes no row-program prologue, no k split over waves and a k extent that is a multiple of 32";
     MONONN_CHECK(t.stages == 2 && t.bk >= 32 && t.bk % 32 == 0 && t.bk <= 128, kSpecError)
         << "LDS-staged GEMM tile: " << t.stages << " stages of " << t.bk << " k: two LDS buffers of 32, 64, 96 or 128 k";
@@ -1750,7 +1751,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
   if (g.bf16) {
     // the tiles move operands as 16-byte pieces whatever the 2-byte type; only the MFMA differs (last template argument)
-    MONONN_CHECK(!has_pro && !g.is_conv && !fold, kUnsupported) << gi->hlo_name << ": bf16 GEMMs take neither a row-program prologue nor a convolution's operand map";
+    MONONN_CHECK(!has_pro && !fold, kUnsupported) << gi->hlo_name << ": bf16 GEMMs take no row-program prologue";
     if (mfma) {
       pa = "reinterpret_cast<const half_t*>(" + pa + ")";
       pb = "reinterpret_cast<const half_t*>(" + pb + ")";
@@ -1858,11 +1859,11 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
       conv_struct = am.str();
       if (t.stages >= 2)
         call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", false, false, false, "
-             << t.bk << ", @NAME@_epi, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
+             << t.bk << ", @NAME@_epi, @NAME@_amap" << (g.bf16 ? ", true" : "") << ">(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
              << ", bidx, tile_m, tile_n, epi, smem, @NAME@_amap());";
       else
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", false, " << g.K
-             << ", @NAME@_epi, mononn_dev::NoPrologue, @NAME@_amap>(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
+             << ", @NAME@_epi, mononn_dev::NoPrologue, @NAME@_amap" << (g.bf16 ? ", false, mononn_dev::NoPreB, false, false, false, true" : "") << ">(" << pa << ", " << pb << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K
              << ", bidx, tile_m, tile_n, epi, smem, mononn_dev::NoPrologue(), @NAME@_amap());";
     } else {
       std::ostringstream b_expr;
@@ -1889,9 +1890,10 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
              << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
              << ", mononn_dev::RowMajorA, " << (preload ? "true, @NAME@_preb" : "false, mononn_dev::NoPreB") << ", " << (g.a_packed ? "true" : "false") << ", "
-             << (epi.along_m ? "true" : "false") << ", " << (b_along_n ? "true" : "false") << (g.bf16 ? ", true" : "") << ">("
-             << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", " << b_expr.str() << ", " << g.M
-             << ", " << g.N << ", " << g.K << ", " << (b_along_n ? g.N : g.K) << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
+             << (epi.along_m ? "true" : "false") << ", " << (b_along_n ? "true" : "false") << (g.bf16 || !g.a_k_contig ? (g.bf16 ? ", true" : ", false") : "")
+             << (!g.a_k_contig ? ", true" : "") << ">("
+             << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : g.a_k_contig ? KS : KS * g.M) << ", " << b_expr.str() << ", " << g.M
+             << ", " << g.N << ", " << (g.a_k_contig ? g.K : g.M) << ", " << (b_along_n ? g.N : g.K) << ", bidx, tile_m, tile_n, epi, smem, " << (has_pro ? "pro" : "mononn_dev::NoPrologue()")
              << ", mononn_dev::RowMajorA()" << (preload ? ", &pre_b" : "");
       call << ");";
       if (preload) {

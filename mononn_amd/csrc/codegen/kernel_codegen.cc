@@ -252,7 +252,20 @@ void plan_regional_synchronization(const graph::Program& prog, const spec::Graph
         out = out && roots.count(prog.storage_root(o)) > 0;
         any_out = any_out || roots.count(prog.storage_root(o)) > 0;
       }
-      const bool keep = partition[i].kind == Partition::kColumns ? out : partition[i].kind == Partition::kSplitK ? in : (in || any_out);
+      bool keep = partition[i].kind == Partition::kColumns ? out : partition[i].kind == Partition::kSplitK ? in : (in || any_out);
+      // column slices only pay when the barrier behind their stage becomes regional: every value of that stage that
+      // a reader of this node takes must stay inside its XCD (the three projections in front of an attention node
+      // go to the XCDs together or not at all)
+      if (keep && partition[i].kind == Partition::kColumns)
+        for (auto* o : n.outputs) {
+          auto rd = readers.find(prog.storage_root(o));
+          if (rd == readers.end()) continue;
+          for (size_t j : rd->second)
+            for (auto* r : prog.nodes[j].inputs) {
+              auto w = writer.find(r);
+              if (w != writer.end() && prog.nodes[w->second].stage == n.stage && !roots.count(r)) keep = false;
+            }
+        }
       if (!keep) {
         partition[i] = Partition();
         changed = true;

@@ -585,8 +585,11 @@ __device__ __forceinline__ void gemm_b_preload(const half_t* B, int N, int tile_
 // B_ALONG_N: the right operand is stored [K, ldb] with n contiguous (a run-time [K, N] matrix, weights passed as
 // kernel parameters): a lane gathers its eight k values of one column with eight 2-byte loads.  Slower per byte
 // than the k-contiguous layouts, but the contraction stays on the MFMAs.
+// A_ALONG_M: likewise the left operand stored [K, lda] with m contiguous (gemm_impl.cc:408-469 takes either operand
+// in either order): a lane gathers the eight k values of its row.
 template <int BM, int BN, int WM, int WN, int WK, int K, bool PACKED_B, int KTOTAL, class Epi, class Pro = NoPrologue, class AMap = RowMajorA,
-          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false, bool B_ALONG_N = false, bool BF16 = false>
+          bool PRE_B = false, class Pre = NoPreB, bool PACKED_A = false, bool D_ALONG_M = false, bool B_ALONG_N = false, bool BF16 = false,
+          bool A_ALONG_M = false>
 __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int M, int N, int lda, int ldb,
                                           int batch, int tile_m, int tile_n, Epi& epi, char* smem, const Pro& pro = Pro(),
                                           const AMap& amap = AMap(), const Pre* pb = nullptr) {
@@ -603,6 +606,7 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   static_assert(!RAGGED_K || (!PACKED_A && !PACKED_B && !PRE_B && AMap::kRowMajor && K == KTOTAL && !Pro::enabled),
                 "a k extent that is not a multiple of 32 is taken from plain k-contiguous operands only");
   static_assert(!B_ALONG_N || (!PACKED_B && !PRE_B), "an n-contiguous right operand is neither packed nor requested ahead");
+  static_assert(!A_ALONG_M || (!PACKED_A && AMap::kRowMajor && !Pro::enabled), "an m-contiguous left operand is plain memory: no fragment order, row map or row program");
   const int lane = lane_id();
   const int wave = wave_id();
   const int wk = wave % WK;
@@ -627,6 +631,8 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
       const int mt_max = M / 16 - 1;
       mt = mt < mt_max ? mt : mt_max;
       a_ptr[i] = A + ((long)mt * (KTOTAL / 32) * 64 + lane) * 8;
+    } else if constexpr (A_ALONG_M) {
+      a_ptr[i] = A + m + (long)kq * lda;
     } else {
       a_ptr[i] = A + (long)m * lda + kq;
     }
@@ -647,10 +653,10 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
   }
   constexpr int B_STEP = PACKED_B ? 64 * 8 : 32;   // halves between consecutive k steps (k-contiguous layouts)
   // eight k values of one column of an n-contiguous operand, zero past the end of k
-  auto load_along_n = [&](const half_t* p, int k0) {
+  auto load_along_n = [&](const half_t* p, int k0, int ld) {
     half8_t v;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = (!RAGGED_K || k0 + e < K) ? p[(long)e * ldb] : half_t(0);
+    for (int e = 0; e < 8; ++e) v[e] = (!RAGGED_K || k0 + e < K) ? p[(long)e * ld] : half_t(0);
     return v;
   };
 
@@ -675,13 +681,14 @@ __device__ __forceinline__ void gemm_tile(const half_t* A, const half_t* B, int 
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         if (PRE_B && c == 0) b[buf][s][j] = pb->v[s * TN + j];
-        else if constexpr (B_ALONG_N) b[buf][s][j] = load_along_n(b_ptr[j] + (long)ks * 32 * ldb, ks * 32 + kq);
+        else if constexpr (B_ALONG_N) b[buf][s][j] = load_along_n(b_ptr[j] + (long)ks * 32 * ldb, ks * 32 + kq, ldb);
         else if constexpr (RAGGED_K) b[buf][s][j] = load_ragged(b_ptr[j] + (long)ks * B_STEP, ks * 32 + kq);
         else b[buf][s][j] = *reinterpret_cast<const half8_t*>(b_ptr[j] + (long)ks * B_STEP);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        if constexpr (RAGGED_K) a[buf][s][i] = load_ragged(a_ptr[i] + (long)ks * A_STEP, ks * 32 + kq);
+        if constexpr (A_ALONG_M) a[buf][s][i] = load_along_n(a_ptr[i] + (long)ks * 32 * lda, ks * 32 + kq, lda);
+        else if constexpr (RAGGED_K) a[buf][s][i] = load_ragged(a_ptr[i] + (long)ks * A_STEP, ks * 32 + kq);
         else if constexpr (AMap::kRowMajor) a[buf][s][i] = *reinterpret_cast<const half8_t*>(a_ptr[i] + (long)ks * A_STEP);
         else a[buf][s][i] = *reinterpret_cast<const half8_t*>(amap(A, a_row[i], ks * 32 + kq, lda));
       }
@@ -1264,8 +1271,8 @@ __device__ __forceinline__ void gemm_naive_element(const T* A, const T* B, int K
 
 // Correctness fallback for convolutions the fragment loads do not cover (padding, channel counts that break the
 // 16-byte pieces): one thread per output element.  Input N,H,W,C, filter K,R,S,C, output N,P,Q,K.
-template <class Epi>
-__device__ __forceinline__ void conv_naive_element(const half_t* in, const half_t* flt, int H, int W, int C, int R, int S, int P, int Q,
+template <class T, class Epi>
+__device__ __forceinline__ void conv_naive_element(const T* in, const T* flt, int H, int W, int C, int R, int S, int P, int Q,
                                                    int stride_h, int stride_w, int pad_h, int pad_w, int m, int k_out, Epi& epi) {
   const int n = m / (P * Q), pq = m % (P * Q), p = pq / Q, q = pq % Q;
   float acc = 0.f;
@@ -1275,8 +1282,8 @@ __device__ __forceinline__ void conv_naive_element(const half_t* in, const half_
     for (int s = 0; s < S; ++s) {
       const int w = q * stride_w + s - pad_w;
       if (w < 0 || w >= W) continue;
-      const half_t* x = in + (((long)n * H + h) * W + w) * C;
-      const half_t* f = flt + (((long)k_out * R + r) * S + s) * C;
+      const T* x = in + (((long)n * H + h) * W + w) * C;
+      const T* f = flt + (((long)k_out * R + r) * S + s) * C;
       for (int c = 0; c < C; ++c) acc += (float)x[c] * (float)f[c];
     }
   }

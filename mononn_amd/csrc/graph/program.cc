@@ -118,6 +118,7 @@ struct Builder {
     GemmDesc d;
     d.is_conv = true;
     d.conv = c;
+    d.bf16 = g->operands[0]->shape.dtype == hlo::DType::kBF16;   // the same tiles on the bf16 forms of the MFMAs
     d.batch = 1;
     d.M = c.N * c.P * c.Q;
     d.N = c.K;

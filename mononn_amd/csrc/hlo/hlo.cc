@@ -395,7 +395,8 @@ void decode_conv_config(Instr* ins) {
   MONONN_CHECK(fg.empty() || std::strtoll(fg.c_str(), nullptr, 10) == 1, kUnsupported) << ins->hlo_name << ": grouped convolution is not supported";
   const hlo::Shape &in = ins->operands[0]->shape, &flt = ins->operands[1]->shape, &out = ins->shape.tuple[0];
   MONONN_CHECK(in.rank() == 4 && flt.rank() == 4 && out.rank() == 4, kUnsupported) << ins->hlo_name << ": only 2-d convolutions are supported";
-  MONONN_CHECK(in.dtype == DType::kF16 && flt.dtype == DType::kF16 && out.dtype == DType::kF16, kUnsupported) << ins->hlo_name << ": only f16 convolutions are supported";
+  MONONN_CHECK(is_half_float(in.dtype) && flt.dtype == in.dtype && out.dtype == in.dtype, kUnsupported)
+      << ins->hlo_name << ": a convolution's input, filter and output must all be f16 or all be bf16";
   ConvConfig& c = ins->conv;
   c.N = in.dims[0], c.H = in.dims[1], c.W = in.dims[2], c.C = in.dims[3];
   c.K = flt.dims[0], c.R = flt.dims[1], c.S = flt.dims[2];

@@ -116,7 +116,7 @@ std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int w
   }
   // large problems: operand tiles staged through LDS once per workgroup (the reference's tiles with shared-memory
   // stages, tile_description.cc:84-258); four waves as 2 x 2, per-wave blocks of up to 128 x 128
-  if (waves == 4 && g.K % 32 == 0 && g.K >= 128 && g.split_k <= 1 && g.M >= 128 && g.N >= 128 && (g.b_k_contig || g.b_packed)) {
+  if (waves == 4 && g.K % 32 == 0 && g.K >= 128 && g.split_k <= 1 && g.M >= 128 && g.N >= 128 && g.a_k_contig && (g.b_k_contig || g.b_packed)) {
     struct Shape { int bm, bn, bk; };
     for (const Shape& sh : {Shape{256, 256, 32}, Shape{192, 256, 32}, Shape{256, 192, 32}, Shape{256, 128, 64}, Shape{128, 256, 64}, Shape{192, 128, 64},
                             Shape{128, 192, 64}, Shape{128, 128, 64}}) {
@@ -345,6 +345,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         trials.push_back(std::move(t));
       };
       add("default", filled);
+      // MONONN_TUNER_ONLY_FUSION_DECISIONS (with a seed specification): the seed's tiles stand, only the stage-fusion
+      // decisions are searched (large models, whose class search takes many minutes)
+      if (seed && env::is_true("MONONN_TUNER_ONLY_FUSION_DECISIONS")) continue;
       if (c.kind == "gemm") {
         for (auto& t : gemm_candidates(c.sample->gemm, cx.block / 64, budget)) {
           GraphSpecification s = filled;

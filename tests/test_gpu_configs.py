@@ -136,18 +136,18 @@ def test_gpt2_full_size_properties(gpu_device):
     m.close()
 
 
-def _conv_module(xd, fd, stride, pad, bias):
+def _conv_module(xd, fd, stride, pad, bias, dtype="f16"):
     from mononn_amd.hlo.builder import HloModuleBuilder
     mb = HloModuleBuilder("cluster_9__conv.1")
     e = mb.entry
-    x = e.parameter("f16", xd, "x")
-    f = e.parameter("f16", fd, "f")
+    x = e.parameter(dtype, xd, "x")
+    f = e.parameter(dtype, fd, "f")
     y = e.conv_forward(x, f, stride=stride, pad=pad)
     if bias:
-        b = e.parameter("f16", (fd[0],), "b")
+        b = e.parameter(dtype, (fd[0],), "b")
 
         def body(fz, py, pb):
-            return fz.convert(fz.add(fz.convert(py, "f32"), fz.broadcast(fz.convert(pb, "f32"), py.dims, [3])), "f16")
+            return fz.convert(fz.add(fz.convert(py, "f32"), fz.broadcast(fz.convert(pb, "f32"), py.dims, [3])), dtype)
         y = e.fusion("kLoop", [y, b], body)
     e.set_tuple_root([y])
     return mb.text(), y.dims
@@ -173,6 +173,33 @@ def test_convolution_parity(gpu_device, xd, fd, stride, pad, bias):
     m.close()
     want = hlo_interp.evaluate(text, args, {}, "fp32")[0]
     _check(got, want, f"conv {xd} * {fd} stride {stride} pad {pad}")
+
+
+@pytest.mark.parametrize("xd,fd,stride,pad,bias", [
+    ((2, 64, 64, 8), (64, 16, 16, 8), (16, 16), (0, 0), True),      # patch embedding on the bf16 MFMA tile, gathered rows
+    ((4, 128, 128, 8), (256, 16, 16, 8), (16, 16), (0, 0), True),   # [256, 2048] x [2048, 256]: large enough for the LDS-staged tile
+    ((2, 9, 10, 4), (6, 3, 3, 4), (2, 1), (1, 1), False),           # padding: per-element path in bf16
+])
+def test_bf16_convolution_parity(gpu_device, xd, fd, stride, pad, bias):
+    """The convolution call on bf16 pixels and filters (conv_impl.cc:51 instantiates half only; bf16 is this build's
+    own): same implicit GEMM, bf16 form of the MFMAs, against the oracle's as-written evaluation (every bf16
+    instruction rounded) within one bf16 spacing of the largest value."""
+    from mononn_amd import MonoNNModule, bf16
+    text, out_dims = _conv_module(xd, fd, stride, pad, bias, dtype="bf16")
+    rng = np.random.default_rng(43)
+    args = [bf16.to_bits(rng.normal(0, 1, xd)), bf16.to_bits(rng.normal(0, 0.05, fd))]
+    if bias:
+        args.append(bf16.to_bits(rng.normal(0, 0.5, (fd[0],))))
+    m = MonoNNModule.compile(text)
+    m.load(gpu_device)
+    got = bf16.from_bits(m.run(args, [{"dtype": "bf16", "dims": list(out_dims)}])[0]).astype(np.float64)
+    m.close()
+    want = hlo_interp.evaluate(text, args, {}, "fp32")[0].astype(np.float64)
+    err, scale = np.abs(got - want).max(), np.abs(want).max()
+    print(f"bf16 conv {xd} * {fd}: max_abs_err={err:.3e} at scale {scale:.3e}", flush=True)
+    # the convolution's result rounded to bf16 once, the bias added in f32 and rounded again: two half spacings, and a
+    # bf16 spacing is at most 2^-7 of the value
+    assert err <= 2.0 ** -7 * scale + 1e-3, (err, scale)
 
 
 def test_vit_encoder_parity(gpu_device):

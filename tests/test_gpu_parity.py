@@ -60,7 +60,11 @@ def gemm_module(M, N, K, batch=(), lhs_c=None, rhs_c=None, alpha=1.0, b_const=Fa
     dict(M=197, N=64, K=197, batch=(2, 3), rhs_c=3),              # odd row length: fragments start at unaligned addresses
     dict(M=33, N=20, K=17, rhs_c=1),                              # K below one MFMA step
     dict(M=64, N=48, K=40),                                       # K not a multiple of 32 and B stored [K,N]: zero-filled gather
-    dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                     # A stored [K,M]
+    dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                     # A stored [K,M]: gathered per lane onto the MFMAs (gemm_impl.cc:408-469 takes either order)
+    dict(M=128, N=96, K=256, lhs_c=0),                            # A stored [K,M] and B stored [K,N]: both gathered
+    dict(M=100, N=52, K=72, lhs_c=0, rhs_c=1),                    # A stored [K,M], ragged M / N, K off the MFMA step
+    dict(M=64, N=128, K=128, lhs_c=1, batch=(3,)),                # batched, A stored [b,K,M]
+    dict(M=128, N=256, K=256, lhs_c=0, b_const=True),             # A stored [K,M] against constant weights (left as given: not packed)
     dict(M=128, N=256, K=256, b_const=True, as_dot=True),         # plain `dot` with a constant right operand
     dict(M=48, N=80, K=64, batch=(3,), rhs_c=2, as_dot=True),     # batched `dot`, both operands k-contiguous
     dict(M=200, N=136, K=256, dtype="f32", rhs_c=1),              # f32 on v_mfma_f32_16x16x4_f32, both operands k-contiguous
@@ -224,21 +228,14 @@ def test_folded_layer_norm_on_rows_far_from_zero(gpu_device):
     kernel must be as close as the kernel that runs the LayerNorm as written."""
     import json
     from test_host_compiler import norm_gemm_module
-    text, _ = norm_gemm_module(True)
+    text, declared = norm_gemm_module(True)
     M, K, N = 64, 256, 128
     rng = np.random.default_rng(71)
     x = (rng.normal(0, 0.25, (M, K)) + rng.choice([-10.0, 10.0], (M, 1))).astype(np.float16)
-    m0 = MonoNNModule.compile(text, build=False)
-    names = [c["name"] for c in m0.constants() if c["needs_payload"]]
-    m0.close()
-    assert len(names) == 3
-    consts = {}
-    sizes = {c["name"]: c["bytes"] for c in MonoNNModule.compile(text, build=False).constants() if c["needs_payload"]}
-    vecs = sorted(n for n in sizes if sizes[n] == K * 2)
-    mats = [n for n in sizes if sizes[n] == K * N * 2]
-    consts[vecs[0]] = rng.uniform(0.5, 1.5, (K,)).astype(np.float16)        # gamma
-    consts[vecs[1]] = rng.normal(0, 0.5, (K,)).astype(np.float16)           # beta
-    consts[mats[0]] = rng.normal(0, 0.05, (K, N)).astype(np.float16)
+    by_role = {v["role"]: k for k, v in declared.items()}
+    consts = {by_role["ln/gamma"]: rng.uniform(0.5, 1.5, (K,)).astype(np.float16),
+              by_role["ln/beta"]: rng.normal(0, 0.5, (K,)).astype(np.float16),
+              by_role["w/kernel"]: rng.normal(0, 0.05, (K, N)).astype(np.float16)}
     want = hlo_interp.evaluate(text, [x], consts, "fp32")[0].astype(np.float64)
     outs = [{"dtype": "f16", "dims": [M, N]}]
     (plain,), m1 = run_module(text, [x], consts, outs)
@@ -430,7 +427,7 @@ def _bf16_check(got_bits, want32, what, steps=4.0, atol=2e-2):
     dict(M=100, N=52, K=96, rhs_c=1),                              # ragged M / N
     dict(M=64, N=48, K=40, rhs_c=1),                               # K off the MFMA step: zero-filled last step
     dict(M=256, N=1001, K=128, rhs_c=1, b_const=True),             # odd N: four columns per store where they fit
-    dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                      # A stored [K,M]: per-element fallback
+    dict(M=40, N=24, K=64, lhs_c=0, rhs_c=1),                      # A stored [K,M]: gathered per lane
 ])
 def test_bf16_gemm_cases(gpu_device, case):
     from mononn_amd import bf16
@@ -442,8 +439,7 @@ def test_bf16_gemm_cases(gpu_device, case):
     consts = {n: b for n in mb.constants}
     inputs = [a] if case.get("b_const") else [a, b]
     (got,), m = run_module(text, inputs, consts, [{"dtype": "bf16", "dims": d_dims}])
-    if not (case.get("lhs_c") == 0):
-        assert ", true>(reinterpret_cast<const half_t*>(" in m.get_source("main.hip")
+    assert ", true>(reinterpret_cast<const half_t*>(" in m.get_source("main.hip")
     want = hlo_interp.evaluate(text, inputs, consts, "fp32")[0]
     # one rounding of an exactly accumulated sum: half a bf16 spacing, a little more for the summation order
     _bf16_check(got, want, f"bf16 gemm {case}", steps=1.0, atol=2e-3 * float(np.abs(want).max()))
