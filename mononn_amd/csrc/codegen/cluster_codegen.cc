@@ -664,7 +664,7 @@ bool gemm_uses_mfma(const graph::GemmDesc& g) {
 // the LDS-staged tile copies k-contiguous or fragment-order operands
 static bool gemm_lds_capable(const graph::GemmDesc& g) { return !g.f32 && gemm_uses_mfma(g) && g.a_k_contig && (g.b_k_contig || g.b_packed) && g.K % 32 == 0; }
 
-GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus) {
+GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus, bool allow_lds_tile) {
   GemmTuning t;
   int waves = ls.waves();
   // Large problems: every wave owns a 64x64 (else 32x32) block of the result over the whole k range, no exchange
@@ -680,7 +680,7 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
   // units x tile area / throughput of a compute unit that is busy with such a tile, relative to 256 x 256 (measured
   // on [6144, 1024] x [1024, 4096] with both operands in fragment order: 1.0 PFLOP/s-equivalent for 256 x 256,
   // which fills the chip only 1.5 times there; 0.87 for 192 x 256, which fills it twice).
-  if (gemm_lds_capable(g) && g.K >= 128 && waves == 4 && ls.waves_per_simd == 1 && g.split_k <= 1) {
+  if (allow_lds_tile && gemm_lds_capable(g) && g.K >= 128 && waves == 4 && ls.waves_per_simd == 1 && g.split_k <= 1) {
     struct Cand { int bm, bn, bk; double eff; };
     double best = 0;
     const int cus = std::max(num_cus, 1);
@@ -709,6 +709,7 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
     }
   }
   for (int per_wave : {64, 32}) {
+    if (!allow_lds_tile) break;             // a row program in front: the waves split k so that a wave's fragments of its rows fit its registers
     if (g.f32 && per_wave > 32) continue;   // 16 fragments of a 64 x 64 block leave no room for a chunk in flight
     int wm = 1, wn = waves;
     while (wn > wm) {
@@ -728,6 +729,10 @@ GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, 
   }
   int wk = 1;
   while (!g.f32 && wk * 2 <= waves && g.K / 32 >= wk * 2 * 2 && g.K >= 256 * wk) wk *= 2;
+  // with a row program in front a wave holds the fragments of its rows over its whole k range: as many waves along k
+  // as divide the k steps
+  if (!allow_lds_tile && !g.f32)
+    while (wk * 2 <= waves && (g.K / 32) % (wk * 2) == 0) wk *= 2;
   t.wk = wk;
   int rest = waves / wk;
   t.wm = 1;
@@ -1724,8 +1729,22 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fold_stats_offset = (fold_exchange_offset + rb + 15) / 16 * 16;
   }
   const bool mfma = gemm_uses_mfma(g);
-  const bool has_pro = !prologue.empty();
+  bool has_pro = !prologue.empty();
   MONONN_CHECK(!has_pro || mfma, kUnsupported) << gi->hlo_name << ": a row-program prologue needs the MFMA path";
+  // A folded LayerNorm on the LDS-staged tile: no row program runs at all, the tile itself adds up the row sums of
+  // the fragments it multiplies (mononn_dev::gemm_tile_lds, LN_STATS); the statistics live behind the operand
+  // buffers and the rows of the epilogue.  Nobody can ask such a GEMM for the normalised rows.
+  const bool lds_fold = fold && has_pro && t.stages >= 2;
+  const Instr* lds_fold_primary = nullptr;
+  if (lds_fold) {
+    MONONN_CHECK(!prologue_stores, kSpecError) << gi->hlo_name << ": an LDS-staged tile cannot store the rows of the LayerNorm folded into it (other stages read them)";
+    MONONN_CHECK(g.split_k <= 1 && !g.bf16 && !g.is_conv, kSpecError) << gi->hlo_name << ": a folded LayerNorm needs the whole k range in one f16 GEMM";
+    lds_fold_primary = prologue_primary(prog, prologue, g.M, g.K);
+    MONONN_CHECK(lds_fold_primary != nullptr, kUnsupported) << gi->hlo_name << ": no [M,K] f16 input to take the place of the left operand";
+    has_pro = false;
+    const int rows_bytes = ls.waves() * 32 * (t.bn / t.wn + 4) * 4;
+    fold_stats_offset = (std::max(2 * (t.bm + t.bn) * t.bk * 2, rows_bytes) + 15) / 16 * 16;
+  }
   if (mfma) validate_gemm_tuning(g, ls, t, has_pro);
   PointerTable ptrs;
   // the two operands come first in the pointer list; with a prologue the left operand is the row
@@ -1745,7 +1764,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     for (auto* o : outputs)
       if (std::find(pouts.begin(), pouts.end(), o) == pouts.end()) epi_outputs.push_back(o);
   } else {
-    pa = ptrs.input(prog.storage_root(gi->operands[0]));
+    pa = ptrs.input(lds_fold ? lds_fold_primary : prog.storage_root(gi->operands[0]));
     pb = ptrs.input(prog.storage_root(gi->operands[1]));
   }
   const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
@@ -1884,8 +1903,18 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         for (auto* o : epi_outputs) rows_lds = rows_lds && !prog.physical_tile.count(prog.storage_root(o)) && !prog.physical_perm.count(prog.storage_root(o));
         call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", "
              << (g.a_packed ? "true" : "false") << ", " << (g.b_packed ? "true" : "false") << ", " << (epi.along_m ? "true" : "false") << ", " << t.bk
-             << ", @NAME@_epi" << (g.bf16 || rows_lds ? std::string(", mononn_dev::RowMajorA, ") + (g.bf16 ? "true" : "false") + (rows_lds ? ", true" : "") : std::string()) << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
+             << ", @NAME@_epi"
+             << (g.bf16 || rows_lds || lds_fold ? std::string(", mononn_dev::RowMajorA, ") + (g.bf16 ? "true" : "false") + (rows_lds || lds_fold ? (rows_lds ? ", true" : ", false") : "") + (lds_fold ? ", true" : "")
+                                                : std::string())
+             << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
              << b_expr.str() << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
+        if (lds_fold) {
+          char eps[48];
+          std::snprintf(eps, sizeof eps, "%.9gf", fold->eps);
+          std::string e = eps;
+          if (e.find_first_of(".e") == std::string::npos) e.insert(e.size() - 1, ".0");
+          call << ", mononn_dev::RowMajorA(), " << e << ", reinterpret_cast<float*>(smem + " << fold_stats_offset << ")";
+        }
       } else
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
              << (g.b_packed ? "true" : "false") << ", " << g.K << ", @NAME@_epi, " << (has_pro ? "@NAME@_pro" : "mononn_dev::NoPrologue")
@@ -1928,6 +1957,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
     if (t.stages >= 2) smem = std::max(2 * (t.bm + t.bn) * t.bk * 2, rows_lds ? ls.waves() * 32 * (t.bn / t.wn + 4) * 4 : 0);
+    if (lds_fold) smem = fold_stats_offset + t.bm * 8;
     smem = std::max(smem, pro.smem);
   } else {
     const int64_t total = g.batch * g.M * g.N;
@@ -2626,7 +2656,9 @@ bool can_fuse_prologue(const Program& prog, const std::vector<const Instr*>& row
     if (!d.a_k_contig || d.batch != 1 || d.K % 32 != 0) return false;
     d.b_k_contig = true;   // constant weights are packed / activations re-laid out before real generation
     LaunchShape ls;
-    GemmTuning t = default_gemm_tuning(d, ls, 256);
+    // the dry run takes the direct tile: the row program runs on the fragments a wave holds in registers (a folded
+    // LayerNorm may later get an LDS-staged tile, which needs no row program at all)
+    GemmTuning t = default_gemm_tuning(d, ls, 256, false);
     auto outs = external_outputs(prog, gemm_members);
     if (outs.empty()) return false;
     gen_gemm(prog, gemm_members, outs, d, ls, t, row_members, true);

@@ -114,7 +114,9 @@ bool can_fuse_out_proj(const graph::Program& prog, const hlo::Instr* gemm2, cons
                        const std::vector<const hlo::Instr*>& epilogue_members, const hlo::Instr* gemm3, const graph::GemmDesc& d3, int heads);
 int default_attention_key_waves(const graph::GemmDesc& first_gemm, const LaunchShape& ls);
 
-GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus);
+// allow_lds_tile false: the direct tile with k split over the waves whatever the problem size (a GEMM with a row
+// program in front that is not a folded LayerNorm: that program runs on the fragments a wave holds in registers)
+GemmTuning default_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, int num_cus, bool allow_lds_tile = true);
 // throws Error(kSpecError) when the tile / wave arrangement cannot be generated for this GEMM
 void validate_gemm_tuning(const graph::GemmDesc& g, const LaunchShape& ls, const GemmTuning& t, bool has_prologue = false);
 bool gemm_uses_mfma(const graph::GemmDesc& g);

@@ -978,10 +978,15 @@ __device__ __forceinline__ float16_t mfma_32x32x16(half8_t a, half8_t b, float16
 }
 
 // BK: k extent of one LDS buffer (a multiple of 32); K a multiple of 32.
+// LN_STATS: the left operand's rows are the input of a LayerNorm that has been folded into weights and epilogue: while
+// a wave multiplies, it also adds up x and x * x of the fragments it reads (v_dot2_f32_f16 between the MFMAs: a
+// lane holds 8 values of one row), and in front of the epilogue leaves (mean, rsqrt(var + ln_eps)) of its rows in
+// ln_stats[row of the tile][2] (LDS) for the epilogue's rank-1 correction.  The waves that share rows write the same
+// values; a wave reads only rows it has written itself.
 template <int BM, int BN, int WM, int WN, int K, int KTOTAL, bool PACKED_A, bool PACKED_B, bool D_ALONG_M, int BK, class Epi,
-          class AMap = RowMajorA, bool BF16 = false, bool ROWS_LDS = false>
+          class AMap = RowMajorA, bool BF16 = false, bool ROWS_LDS = false, bool LN_STATS = false>
 __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, int M, int N, int lda, int ldb, int batch, int tile_m,
-                                              int tile_n, Epi& epi, char* smem, const AMap& amap = AMap()) {
+                                              int tile_n, Epi& epi, char* smem, const AMap& amap = AMap(), float ln_eps = 0.f, float* ln_stats = nullptr) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;             // 32 x 32 fragments per wave
   constexpr int KSTP = BK / 16;                                    // MFMA steps per k tile
@@ -1131,6 +1136,9 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   const lds_char_t* a_frag = lds + (wm * TM * KSTP) * 1024 + lane * 16;
   const lds_char_t* b_frag = lds + (ABLK + wn * TN * KSTP) * 1024 + lane * 16;
   half8_t fa[2][TM], fb[2][TN];
+  float ln_s1[LN_STATS ? TM : 1], ln_s2[LN_STATS ? TM : 1];
+#pragma unroll
+  for (int i = 0; i < (LN_STATS ? TM : 1); ++i) ln_s1[i] = ln_s2[i] = 0.f;
   auto read_one = [&](int buf, int ks, int rb, int r) {
     if (r < TM) fa[rb][r] = *reinterpret_cast<const lds_half8_t*>(a_frag + buf * STAGE_BYTES + (r * KSTP + ks) * 1024);
     else fb[rb][r - TM] = *reinterpret_cast<const lds_half8_t*>(b_frag + buf * STAGE_BYTES + ((r - TM) * KSTP + ks) * 1024);
@@ -1154,6 +1162,16 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
 #pragma unroll
       for (int c = l0 + ((l1 - l0) * q) / Q; c < l0 + ((l1 - l0) * (q + 1)) / Q; ++c) load_one(t + 3, set, c);
       const int i = q / TN, j = q % TN;
+      if constexpr (LN_STATS) {
+        if (j == 0) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const half2_t h = {fa[rb][i][2 * e], fa[rb][i][2 * e + 1]};
+            ln_s1[i] = __builtin_amdgcn_fdot2(h, half2_t{(half_t)1, (half_t)1}, ln_s1[i], false);
+            ln_s2[i] = __builtin_amdgcn_fdot2(h, h, ln_s2[i], false);
+          }
+        }
+      }
       acc[i][j] = D_ALONG_M ? mfma_32x32x16<BF16>(fa[rb][i], fb[rb][j], acc[i][j]) : mfma_32x32x16<BF16>(fb[rb][j], fa[rb][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1206,6 +1224,23 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   // k loop ends: as many registers again as the tile itself, paid for by spilling everything else that is live in
   // the loop.  Pinning the rows that are not yet due (an empty statement that wants them in accumulation
   // registers) keeps the move to one row at a time.
+  if constexpr (LN_STATS) {
+    // the two lanes that hold the two k pieces of a row put their sums together; the variance is E[x^2] - mean^2
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const float s1 = ln_s1[i] + __shfl_xor(ln_s1[i], 32, kWaveSize), s2 = ln_s2[i] + __shfl_xor(ln_s2[i], 32, kWaveSize);
+      const float mean = s1 * (1.0f / K);
+      const float var = s2 * (1.0f / K) - mean * mean;
+      if (lane < 32) {
+        float* dst = ln_stats + ((wm * TM + i) * 32 + lane) * 2;
+        dst[0] = mean;
+        dst[1] = rsqrtf((var > 0.f ? var : 0.f) + ln_eps);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
   typedef __attribute__((address_space(3))) float4_t lds_float4_t;
   lds_char_t* const rows_lds = lds + wave * (32 * PITCH * 4);   // this wave's 32 rows
   if constexpr (ROWS_LDS) __syncthreads();   // the other waves may still be reading the last operand tiles
