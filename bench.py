@@ -404,7 +404,8 @@ def main():
         "config": {"workload": "BERT-base encoder, 12 layers + embedding gather, batch 1, seq 128, fp16 weights "
                                "N(0,0.02), one launch of the monolithic persistent kernel per forward",
                    "tuning_spec": used_spec, "grid": dims["grid"], "block": dims["block"], "lds_bytes": dims["smem"],
-                   "grid_barriers": dims["barriers"]},
+                   "grid_barriers": dims["barriers"],
+                   "barrier_tiers": {"memory_side": dims["barriers"] - dims["regional_barriers"], "one_xcd": dims["regional_barriers"]}},
         "latency_us": {"kernel_avg": round(kern_us, 2), "kernel_p10": round(float(each_us[len(each_us) // 10]), 2),
                        "kernel_median": round(float(each_us[len(each_us) // 2]), 2),
                        "kernel_p90": round(float(each_us[(len(each_us) * 9) // 10]), 2),

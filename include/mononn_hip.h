@@ -82,6 +82,11 @@ int mononn_module_buffer_info(const mononn_module* m, int* n_params, const int64
  * (temp_buffer argument, mononn_engine/module/mononn_module.cc:91-143). */
 int mononn_module_owns_temp(const mononn_module* m);
 int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int* smem, int* barriers);
+/* How many of those barriers belong to the regional tier: barriers over the workgroups of one XCD, through its L2
+ * ("mononn_hip": {"regional_synchronization": true}); the others go through the memory side and order the whole grid.
+ * Replaces: the split the reference makes between global and regional synchronisation
+ *           (mononn_engine/optimization/regional_synchronization_assignment_pass.cc:35-72). */
+int mononn_module_regional_barriers(const mononn_module* m, int* regional);
 
 /* Non-scalar constants of the module ("buffer_for_<node>" globals that the host fills before
  * launch: mononn_engine/codegen/graph_codegen.cc:71-86, :448-459).  needs_payload is 1 for a constant the

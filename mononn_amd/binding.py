@@ -55,6 +55,7 @@ def _load_library() -> ctypes.CDLL:
     lib.mononn_module_buffer_info.argtypes = [c.c_void_p, P(c.c_int), P(P(c.c_int64)), P(c.c_int), P(P(c.c_int64)),
                                               P(c.c_int64)]
     lib.mononn_module_launch_dims.argtypes = [c.c_void_p, P(c.c_int), P(c.c_int), P(c.c_int), P(c.c_int)]
+    lib.mononn_module_regional_barriers.argtypes = [c.c_void_p, P(c.c_int)]
     lib.mononn_module_owns_temp.argtypes = [c.c_void_p]
     lib.mononn_module_num_constants.argtypes = [c.c_void_p]
     lib.mononn_module_constant_info.argtypes = [c.c_void_p, c.c_int, P(c.c_char_p), P(c.c_char_p), P(c.c_int64), P(c.c_int)]
@@ -81,7 +82,7 @@ _lib = _load_library()
 EXPORTED_SYMBOLS = [
     "mononn_last_error", "mononn_version", "mononn_compile", "mononn_tune", "mononn_compile_from_spec_dir",
     "mononn_module_destroy", "mononn_module_kernel_name", "mononn_module_spec_json", "mononn_module_source",
-    "mononn_module_code_object", "mononn_module_summary", "mononn_module_buffer_info", "mononn_module_launch_dims", "mononn_module_owns_temp",
+    "mononn_module_code_object", "mononn_module_summary", "mononn_module_buffer_info", "mononn_module_launch_dims", "mononn_module_regional_barriers", "mononn_module_owns_temp",
     "mononn_module_num_constants", "mononn_module_constant_info", "mononn_module_set_constant", "mononn_module_load",
     "mononn_launch", "mononn_launch_static_temp", "mononn_static_temp_bytes", "mononn_module_synchronize", "mononn_module_global", "mononn_time_kernel", "mononn_module_stage_clock", "mononn_module_stage_name", "mononn_module_dump", "mononn_device_count", "mononn_device_info"]
 
@@ -185,7 +186,9 @@ class MonoNNModule:
     def launch_dims(self) -> dict:
         g, b, s, nb = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
         _check(_lib.mononn_module_launch_dims(self._h, ctypes.byref(g), ctypes.byref(b), ctypes.byref(s), ctypes.byref(nb)))
-        return {"grid": g.value, "block": b.value, "smem": s.value, "barriers": nb.value}
+        rb = ctypes.c_int()
+        _check(_lib.mononn_module_regional_barriers(self._h, ctypes.byref(rb)))
+        return {"grid": g.value, "block": b.value, "smem": s.value, "barriers": nb.value, "regional_barriers": rb.value}
 
     def constants(self) -> List[dict]:
         out = []

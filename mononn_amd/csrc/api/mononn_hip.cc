@@ -178,6 +178,13 @@ int mononn_module_launch_dims(const mononn_module* m, int* grid, int* block, int
   });
 }
 
+int mononn_module_regional_barriers(const mononn_module* m, int* regional) {
+  return guarded([&] {
+    require(m != nullptr && regional != nullptr, "NULL argument");
+    *regional = m->impl->hip_program().num_regional_barriers;
+  });
+}
+
 int mononn_module_num_constants(const mononn_module* m) { return m ? static_cast<int>(m->impl->hip_program().constants.size()) : 0; }
 
 int mononn_module_constant_info(const mononn_module* m, int index, const char** hlo_name, const char** role, int64_t* bytes,

@@ -202,6 +202,35 @@ def test_bf16_convolution_parity(gpu_device, xd, fd, stride, pad, bias):
     assert err <= 2.0 ** -7 * scale + 1e-3, (err, scale)
 
 
+def test_layer_norm_folded_into_lds_staged_tiles(gpu_device):
+    """Pre-LN decoder, 2048 rows: the LayerNorm in front of the feed-forward GEMM is folded into an LDS-staged tile, which
+    adds up the row sums of the fragments it multiplies (no row program, no stage); the other folded LayerNorms sit on
+    direct tiles.  Against the oracle, and no further from it than the kernel that runs every LayerNorm as a stage."""
+    import json
+    from mononn_amd import MonoNNModule
+    fx = models.gpt2(L=2, B=4, S=512, H=768, NH=12, F=3072, vocab=1000, max_pos=512)
+    consts = fx.make_constants(1244, "random")
+    inputs = fx.make_inputs(1244)
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    spec["mononn_hip"].update(gemm_prologue_fusion=True, layer_norm_folding=True)
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}, {}
+    folded = MonoNNModule.compile(fx.hlo_text, json.dumps(spec))
+    src = folded.get_source("main.hip")
+    assert "mononn_dev::RowMajorA, false, false, true>(" in src and "ln_stats" in src        # LN_STATS on an LDS-staged tile
+    plain = MonoNNModule.compile(fx.hlo_text)
+    assert folded.launch_dims()["barriers"] < plain.launch_dims()["barriers"]
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    errs = {}
+    for name, m in (("folded", folded), ("as written", plain)):
+        m.set_constants(consts)
+        m.load(gpu_device)
+        got = m.run(inputs, fx.outputs)[0]
+        m.close()
+        _check(got, want, f"gpt2 L=2 b4 s512, LayerNorm {name}")
+        errs[name] = np.abs(got.astype(np.float64) - want).max()
+    assert errs["folded"] <= 2 * errs["as written"] + 1e-3
+
+
 def test_vit_encoder_parity(gpu_device):
     fx = models.vit(L=2, B=2, image=64, patch=16, H=256, NH=4, F=512)
     consts = fx.make_constants(1238, "random")
