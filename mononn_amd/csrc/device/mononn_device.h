@@ -97,8 +97,12 @@ __device__ __forceinline__ int wave_id() { return thread_id() / kWaveSize; }
 #endif
 
 // Regional tier (MONONN_REGIONAL_SYNC): the 8 XCDs of the part have an L2 each, and a launch of one workgroup per
-// compute unit deals the workgroups to them round-robin (workgroup b runs on XCD b % 8; checked at kernel start against
-// the hardware's XCC_ID, a mismatch is reported through the error word).  Where every value that crosses a stage
+// compute unit deals the workgroups to them round-robin: workgroup b runs on XCD (b + s) % 8, where the start s is the
+// same for every workgroup of a launch and depends on the hardware queue the launch went through (0 in a process with
+// one stream; measured 7 and 5 on the null stream once a second and a fourth stream existed).  So the 32 workgroups
+// with equal b % 8 share an XCD whatever s is, which is all the regional tier relies on; every workgroup leaves its
+// XCC_ID beside its flag, and the first regional wait of a workgroup compares the 32 it polls with its own (a mismatch
+// is reported through the error word).  Where every value that crosses a stage
 // boundary is produced and consumed on the same XCD, the hand-over stays inside that L2: ordinary stores (acknowledged
 // by the L2), a flag array of its own published with a store that stops at the L2, and a wait that looks at the 32
 // flags of the workgroup's XCD only, with loads that miss the compute unit's L1 (nt) and hit the L2.  Measured in
@@ -109,7 +113,7 @@ __device__ __forceinline__ int wave_id() { return thread_id() / kWaveSize; }
 #endif
 constexpr int kXcds = 8;
 constexpr unsigned kErrorRegional = 0x40000000u;    // error word: a wait of the regional tier gave up
-constexpr unsigned kErrorPlacement = 0x80000000u;   // error word: a workgroup does not run on XCD blockIdx.x % 8
+constexpr unsigned kErrorPlacement = 0x80000000u;   // error word: two workgroups with equal blockIdx.x % 8 run on different XCDs
 
 // a load that is served by the L2 (the compute unit's L1 does not keep what it returns); an asm statement because no
 // builtin combines this cache policy with the ordering a spin loop needs (a load instruction reads no data register
@@ -132,16 +136,17 @@ struct GridBarrier {
 #if MONONN_REGIONAL_SYNC
   unsigned* rflags;  // [gridDim.x * kFlagStride]: flags of the regional tier
   unsigned repoch, rfirst;
+  unsigned xcc;          // the XCD this workgroup runs on
+  bool placement_seen;   // this workgroup has compared its XCD with that of the workgroups it polls
 
   __device__ __forceinline__ void init_regional(unsigned* f) {
     rflags = f;
     repoch = load_through_l2(&rflags[blockIdx.x * kFlagStride]);
     rfirst = repoch;
-    const unsigned xcc = __builtin_amdgcn_s_getreg(6164) & (kXcds - 1);   // hwreg(HW_REG_XCC_ID, 0, 4)
-    if (threadIdx.x == 0 && xcc != (blockIdx.x & (kXcds - 1))) {
-      unsigned expected = 0;
-      __hip_atomic_compare_exchange_strong(error, &expected, kErrorPlacement | blockIdx.x, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    xcc = __builtin_amdgcn_s_getreg(6164) & (kXcds - 1);   // hwreg(HW_REG_XCC_ID, 0, 4)
+    placement_seen = false;
+    // beside the flag, in its line: in the L2 before the first flag of this launch is (arrive_regional waits for it)
+    if (threadIdx.x == 0) __hip_atomic_store(&rflags[blockIdx.x * kFlagStride + 1], xcc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   // the workgroup's part of the stage is in the XCD's L2 (every wave has its stores acknowledged), then the flag
   __device__ __forceinline__ void arrive_regional() {
@@ -161,7 +166,16 @@ struct GridBarrier {
           break;
         }
       }
+      if (!placement_seen) {
+        const unsigned theirs = load_through_l2(&rflags[b * kFlagStride + 1]) & (kXcds - 1);
+        if (theirs != xcc) {
+          unsigned expected = 0;
+          __hip_atomic_compare_exchange_strong(error, &expected, kErrorPlacement | (theirs << 24) | (xcc << 20) | ((unsigned)b & 0xfffffu), __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
     }
+    placement_seen = true;
     __syncthreads();
   }
 #endif

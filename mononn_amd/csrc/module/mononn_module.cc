@@ -445,11 +445,11 @@ void MonoNNModule::synchronize(void* stream) {
     dev_.zero(regional, regional_bytes);
   }
   dev_.zero(err, err_bytes);
-  // error word of the device runtime: bit 31 = a workgroup found itself on another XCD than its index modulo 8 says,
+  // error word of the device runtime: bit 31 = two workgroups with the same index modulo 8 found themselves on different XCDs (bits 24-26 and 20-22),
   // bit 30 = the wait that gave up belongs to the regional tier
   MONONN_CHECK((word[0] & 0x80000000u) == 0, kRuntimeError)
-      << "kernel " << kernel_name_ << ": workgroup " << (word[0] & 0x7fffffffu) << " does not run on XCD " << (word[0] & 7u)
-      << " (regional synchronisation assumes that a grid of one workgroup per compute unit is dealt to the 8 XCDs round-robin); the outputs of this launch are invalid";
+      << "kernel " << kernel_name_ << ": workgroup " << (word[0] & 0xfffffu) << " runs on XCD " << ((word[0] >> 24) & 7u) << ", a workgroup with the same index modulo 8 on XCD "
+      << ((word[0] >> 20) & 7u) << " (regional synchronisation assumes that a grid of one workgroup per compute unit is dealt to the 8 XCDs round-robin); the outputs of this launch are invalid";
   MONONN_CHECK((word[0] & 0x40000000u) == 0, kRuntimeError)
       << "kernel " << kernel_name_ << ": a workgroup gave up waiting at regional barrier " << (word[0] & 0x3fffffffu) << " of " << hip_.num_regional_barriers << " after "
       << spec_.hip.barrier_timeout_ms << " ms (mononn_hip.barrier_timeout_ms): the grid of " << grid_

@@ -188,7 +188,11 @@ def test_regional_barrier_hands_over_complete_data(gpu_device):
     """Integer-valued f16 data (every product and sum exact) through GEMM -> regional barrier -> k-split GEMM ->
     memory-side barrier -> sum, 40 launches with fresh inputs: a store that is still on its way when the regional flag
     is seen, a reader that looks into another XCD's slice, or a line left from the launch before is a wrong value.
-    Every consumer workgroup reads tiles that 4 to 8 other workgroups (compute units) of its XCD wrote."""
+    Every consumer workgroup reads tiles that 4 to 8 other workgroups (compute units) of its XCD wrote.
+    From launch 20 on a second stream exists and has run a kernel: the hardware then starts dealing the workgroups of
+    a launch on this stream at another XCD (measured: workgroup b on XCD (b + 7) % 8 instead of b % 8), which must not
+    matter, because workgroups with equal b % 8 still share an XCD."""
+    import torch
     mb, (M, K, F, N) = exchange_module()
     rng = np.random.default_rng(5)
     w1 = rng.integers(-1, 2, (K, F)) * (rng.random((K, F)) < 0.05)
@@ -199,6 +203,11 @@ def test_regional_barrier_hands_over_complete_data(gpu_device):
     m.set_constants({names[0]: w1.astype(np.float16), names[1]: w2.astype(np.float16)})
     m.load(gpu_device)
     for launch in range(40):
+        if launch == 20:
+            side = torch.cuda.Stream(device=torch.device("cuda", gpu_device))
+            with torch.cuda.stream(side):
+                torch.zeros(100 * 1024, device=torch.device("cuda", gpu_device)).add_(1.0)
+            side.synchronize()
         x = rng.integers(-3, 4, (M, K))
         h = x @ w1
         want = h @ w2 + 1
