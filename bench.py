@@ -32,7 +32,7 @@ SPEC_DIR = os.path.join(ROOT, "mononn_amd", "specs", "bert_base_b1_s128")
 # HBM-side bytes of one launch of the kernel built from SPEC_DIR: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of
 # this script, each scaled by what the same counter reads for the 256 MiB --calibration-copy (summary under
 # profiles/).  Counters cannot be read inside a timed run, so the figure is carried here.
-MEASURED_TRAFFIC_BYTES = 451_087_059   # 372,282,922 fetched + 78,804,137 written
+MEASURED_TRAFFIC_BYTES = 451_033_377   # 372,229,281 fetched + 78,804,096 written
 
 
 def algorithmic_bytes(fx) -> int:
