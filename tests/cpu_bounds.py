@@ -2,11 +2,13 @@
 
 Bounds check of generated kernels on the CPU: the generated translation unit of a module (its main.hip and the
 device prelude it includes, unchanged) is compiled for the host with tests/cpu_shim/host_builtins.h pre-included and
-run thread by thread with every buffer placed against inaccessible guard pages, once flush with the page before it (catches reads in front of a
-buffer) and once flush with the page behind it (catches reads past its end).  An out-of-range access ends the run
+run thread by thread with every buffer (parameters, live-outs, the temp arena and every constant of the module, which
+the generated source declares as arrays of the code object) placed against inaccessible guard pages, once flush with the
+page before it (catches reads in front of a buffer) and once flush with the page behind it (catches reads past its end).  An out-of-range access ends the run
 with the buffer, the offset and the thread that made it."""
 import json
 import os
+import re
 import subprocess
 import tempfile
 
@@ -23,6 +25,7 @@ DRIVER = r"""
 #include <unistd.h>
 Dim3 threadIdx, blockIdx, gridDim, blockDim;
 extern "C" { alignas(16) char smem[160 << 10]; }
+%(const_decls)s
 #include "main.hip"
 
 struct Buf { const char* name; size_t bytes; char* base; char* lo; char* hi; };
@@ -52,6 +55,7 @@ int main(int argc, char** argv) {
     for (size_t k = 0; k < sizes[i]; ++k) base[k] = char(k * 7 + i);     // finite halves, small integers as indices
     bufs[i] = {names[i], sizes[i], base, r, r + body + 2 * kGuard};
   }
+%(const_binds)s
   struct sigaction sa = {};
   sa.sa_sigaction = on_fault;
   sa.sa_flags = SA_SIGINFO;
@@ -87,14 +91,23 @@ def check_module(hlo_text, spec_json=None, workdir=None, opt="-O0", shrink=None)
         sizes.append(b)
     names.append("temp arena")
     sizes.append(max(info["temp"], 16))
+    # constants: `__device__ ... unsigned char buffer_for_<name>[bytes];` becomes a pointer into a guarded mapping
+    consts = re.findall(r"^__device__ __attribute__\(\(aligned\(256\)\)\) unsigned char (buffer_for_\w+)\[(\d+)\];$", src, flags=re.M)
+    src = re.sub(r"^__device__ __attribute__\(\(aligned\(256\)\)\) unsigned char (buffer_for_\w+)\[(\d+)\];$", r"// \1: \2 bytes, guarded by the driver", src, flags=re.M)
+    n_args = len(names)
+    for cname, cbytes in consts:
+        names.append(cname)
+        sizes.append(int(cbytes))
     if shrink:
         sizes[names.index(shrink[0])] -= shrink[1]
+    const_decls = "\n".join(f"unsigned char* {cname};" for cname, _ in consts)
+    const_binds = "\n".join(f"  {cname} = reinterpret_cast<unsigned char*>(bufs[{n_args + i}].base);" for i, (cname, _) in enumerate(consts))
     tmp = workdir or tempfile.mkdtemp(prefix="mononn_cpu_bounds_")
     open(os.path.join(tmp, "main.hip"), "w").write(src)
     open(os.path.join(tmp, "headers.h"), "w").write(m.get_source("headers.h"))
     drv = DRIVER % {"nbuf": len(names), "names": ", ".join(json.dumps(n) for n in names), "sizes": ", ".join(f"{s}ul" for s in sizes),
                     "grid": dims["grid"], "block": dims["block"], "kernel": m.kernel_name,
-                    "args": ", ".join(f"bufs[{i}].base" for i in range(len(names)))}
+                    "args": ", ".join(f"bufs[{i}].base" for i in range(n_args)), "const_decls": const_decls, "const_binds": const_binds}
     open(os.path.join(tmp, "driver.cpp"), "w").write(drv)
     exe = os.path.join(tmp, "driver")
     cp = subprocess.run([CLANG, "-x", "c++", "-std=c++17", opt, "-w", "-include", os.path.join(HERE, "cpu_shim", "host_builtins.h"), "-I", tmp,
