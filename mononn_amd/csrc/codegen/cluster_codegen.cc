@@ -204,10 +204,13 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
   if (info.row_program) {
     const int64_t ROWS = info.rows, R = info.row_len;
     const bool block_tier = t.locality_tier == 2;
-    // 8 rows per wave, 8 lanes per row, 16-byte runs per lane: rows of whole runs that fit the registers
+    // G = 8, 4 or 2 rows per wave (reduce_implementation 1, 2, 3), 64 / G lanes per row, 16-byte runs per lane: rows of
+    // whole runs that fit the registers.  Lane l works on row l % G of the wave's G rows.
     const int group_run = 16 / hlo::dtype_bytes(outputs[0]->shape.dtype);
-    const bool row_groups = !block_tier && t.reduce_implementation == 1 && R % group_run == 0 && R / group_run >= 8 && (R / group_run + 7) / 8 * group_run <= 160;
-    const int stride = block_tier ? ls.block_size : row_groups ? 8 : 64;
+    const int G = t.reduce_implementation == 1 ? 8 : t.reduce_implementation == 2 ? 4 : t.reduce_implementation == 3 ? 2 : 1;
+    const int GL = 64 / G;   // lanes per row
+    const bool row_groups = !block_tier && G > 1 && R % group_run == 0 && R / group_run >= GL && (R / group_run + GL - 1) / GL * group_run <= 160;
+    const int stride = block_tier ? ls.block_size : row_groups ? GL : 64;
     int row = vars.add("row", ROWS);
     std::vector<const Instr*> row_outs, full_outs;
     for (auto* o : outputs) {
@@ -217,13 +220,13 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       else MONONN_FAIL(kUnsupported) << o->hlo_name << ": output with " << n << " elements does not fit a " << ROWS << " x " << R << " row space";
     }
     cb.line("const int lane = mononn_dev::lane_id();");
-    cb.line(std::string("const int tid = ") + (block_tier ? "(int)threadIdx.x;" : row_groups ? "lane >> 3;" : "lane;"));
+    cb.line(std::string("const int tid = ") + (block_tier ? "(int)threadIdx.x;" : row_groups ? "lane / " + S(G) + ";" : "lane;"));
     if (block_tier) {
       cb.line("const int row = unit;");
       cb.open("");
     } else if (row_groups) {
-      cb.line("const int row = (unit * " + S(NW) + " + mononn_dev::wave_id()) * 8 + (lane & 7);");
-      cb.open("if (row < " + S(ROWS) + ")");   // the 8 lanes of a row agree
+      cb.line("const int row = (unit * " + S(NW) + " + mononn_dev::wave_id()) * " + S(G) + " + (lane & " + S(G - 1) + ");");
+      cb.open("if (row < " + S(ROWS) + ")");   // the lanes of a row agree
     } else {
       cb.line("const int row = unit * " + S(NW) + " + mononn_dev::wave_id();");
       cb.open("if (row < " + S(ROWS) + ")");
@@ -231,7 +234,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
     auto all_reduce = [&](const Instr* r, const std::string& acc) {
       std::string T = hlo::dtype_ctype(r->shape.dtype);
       if (block_tier) cb.line(acc + " = mononn_dev::block_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ", reinterpret_cast<" + T + "*>(smem));");
-      else if (row_groups) cb.line(acc + " = mononn_dev::lane_group8_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
+      else if (row_groups) cb.line(acc + " = mononn_dev::lane_group_all_reduce<" + S(G) + ">(" + acc + ", " + Emitter::reducer_functor(r) + ");");
       else cb.line(acc + " = mononn_dev::wave_all_reduce(" + acc + ", " + Emitter::reducer_functor(r) + ");");
     };
     // Tuple-valued reductions: N accumulators, the reducer computation inlined for every element and, as a local
@@ -289,7 +292,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
         return comb + "(" + args + ");";
       };
       cb.line("#pragma unroll");
-      cb.open("for (int off = 32; off >= " + S(row_groups ? 8 : 1) + "; off >>= 1)");
+      cb.open("for (int off = 32; off >= " + S(row_groups ? G : 1) + "; off >>= 1)");
       cb.line(call([&](size_t i) { return "mononn_dev::lane_xor(" + ta.acc[i] + ", off)"; }));
       cb.close();
       if (!block_tier) return;
@@ -457,7 +460,7 @@ NodeFunction gen_cluster(const Program& prog, const std::vector<const Instr*>& m
       }
     }
     cb.close();
-    int64_t units = block_tier ? ROWS : row_groups ? (ROWS + 8 * NW - 1) / (8 * NW) : (ROWS + NW - 1) / NW;
+    int64_t units = block_tier ? ROWS : row_groups ? (ROWS + G * NW - 1) / (G * NW) : (ROWS + NW - 1) / NW;
     return finish(T * V <= 32 || row_groups ? hoist_row_loads(cb.text()) : cb.text(), ptrs, tables_of(em), units, block_tier ? NW * 8 * static_cast<int>(max_tuple) : 0);
   }
 

@@ -397,12 +397,21 @@ __device__ __forceinline__ T wave_all_reduce(T v, Op op) {
   }
 }
 
-// Reduction over the 8 lanes that share (lane % 8): a wave that works on 8 rows at once keeps row r in lanes r, r + 8,
-// ..., r + 56.  One rotation by 8 inside the row of 16 lanes on the vector ALU, two LDS-crossbar permutes.
-template <class T, class Op>
-__device__ __forceinline__ T lane_group8_all_reduce(T v, Op op) {
-  if constexpr (sizeof(T) == 4) v = op(v, dpp_move<0x128>(v));   // row_ror:8
-  else v = op(v, __shfl_xor(v, 8, kWaveSize));
+// Reduction over the 64 / G lanes that share (lane % G), G = 8, 4 or 2: a wave that works on G rows at once keeps row r
+// in lanes r, r + G, ..., r + 64 - G.  Rotations by G .. 8 inside the row of 16 lanes on the vector ALU (a rotation by
+// half the distance already covered doubles the set of lanes a value stands for, like the butterfly does), then two
+// LDS-crossbar permutes.
+template <int G, class T, class Op>
+__device__ __forceinline__ T lane_group_all_reduce(T v, Op op) {
+  static_assert(G == 8 || G == 4 || G == 2, "8, 4 or 2 rows per wave");
+  if constexpr (sizeof(T) == 4) {
+    v = op(v, dpp_move<0x128>(v));                          // row_ror:8
+    if constexpr (G <= 4) v = op(v, dpp_move<0x124>(v));    // row_ror:4
+    if constexpr (G <= 2) v = op(v, dpp_move<0x122>(v));    // row_ror:2
+  } else {
+#pragma unroll
+    for (int off = 8; off >= G; off >>= 1) v = op(v, __shfl_xor(v, off, kWaveSize));
+  }
   v = op(v, __shfl_xor(v, 16, kWaveSize));
   v = op(v, __shfl_xor(v, 32, kWaveSize));
   return v;

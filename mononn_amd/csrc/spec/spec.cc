@@ -197,7 +197,7 @@ GraphSpecification GraphSpecification::from_json(const Json& j) {
       e.locality_tier = geti(kv.second, "locality_tier", 1);
       e.reduce_implementation = geti(kv.second, "reduce_implementation", 0);
       MONONN_CHECK(e.locality_tier == 1 || e.locality_tier == 2, kSpecError) << "locality_tier of " << kv.first << " must be 1 or 2";
-      MONONN_CHECK(e.reduce_implementation == 0 || e.reduce_implementation == 1, kSpecError) << "reduce_implementation of " << kv.first << " must be 0 or 1";
+      MONONN_CHECK(e.reduce_implementation >= 0 && e.reduce_implementation <= 3, kSpecError) << "reduce_implementation of " << kv.first << " must be 0 ... 3";
       s.cluster_reduce_spec[kv.first] = e;
     }
   if (j.contains("gemm_spec_list"))

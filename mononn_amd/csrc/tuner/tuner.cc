@@ -400,6 +400,11 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
             s.cluster_reduce_spec[n].reduce_implementation = 1;
           }
           add("tier1_rows8", s);
+          // 4 and 2 rows per wave: the same scheme for row counts that leave most waves idle at 8 rows each
+          for (int impl : {2, 3}) {
+            for (auto& n : c.nodes) s.cluster_reduce_spec[n].reduce_implementation = impl;
+            add(impl == 2 ? "tier1_rows4" : "tier1_rows2", s);
+          }
         }
       } else if (c.kind == "cluster_elewise") {
         for (int ilp : {2, 4, 8}) {
