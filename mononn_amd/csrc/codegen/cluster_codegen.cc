@@ -1736,11 +1736,11 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   MONONN_CHECK(!has_pro || mfma, kUnsupported) << gi->hlo_name << ": a row-program prologue needs the MFMA path";
   // A folded LayerNorm on the LDS-staged tile: no row program runs at all, the tile itself adds up the row sums of
   // the fragments it multiplies (mononn_dev::gemm_tile_lds, LN_STATS); the statistics live behind the operand
-  // buffers and the rows of the epilogue.  Nobody can ask such a GEMM for the normalised rows.
+  // buffers and the rows of the epilogue.  Where later stages read the normalised rows (prologue_stores), the column
+  // tiles of a row block store a share of them each, from the statistics and a second look at the operand rows.
   const bool lds_fold = fold && has_pro && t.stages >= 2;
   const Instr* lds_fold_primary = nullptr;
   if (lds_fold) {
-    MONONN_CHECK(!prologue_stores, kSpecError) << gi->hlo_name << ": an LDS-staged tile cannot store the rows of the LayerNorm folded into it (other stages read them)";
     MONONN_CHECK(g.split_k <= 1 && !g.bf16 && !g.is_conv, kSpecError) << gi->hlo_name << ": a folded LayerNorm needs the whole k range in one f16 GEMM";
     lds_fold_primary = prologue_primary(prog, prologue, g.M, g.K);
     MONONN_CHECK(lds_fold_primary != nullptr, kUnsupported) << gi->hlo_name << ": no [M,K] f16 input to take the place of the left operand";
@@ -1769,6 +1769,39 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   } else {
     pa = ptrs.input(lds_fold ? lds_fold_primary : prog.storage_root(gi->operands[0]));
     pb = ptrs.input(prog.storage_root(gi->operands[1]));
+    if (lds_fold) {
+      auto pouts = external_outputs(prog, prologue);
+      epi_outputs.clear();
+      for (auto* o : outputs)
+        if (std::find(pouts.begin(), pouts.end(), o) == pouts.end()) epi_outputs.push_back(o);
+    }
+  }
+  // rows of a LayerNorm folded into an LDS-staged tile, for the stages that read them: ((x - mean) * r) * gamma + beta
+  // as two fused multiply-adds per element, like the folded direct tile stores them
+  std::string rows_struct, rows_init;
+  if (lds_fold && prologue_stores) {
+    auto pouts = external_outputs(prog, prologue);
+    MONONN_CHECK(pouts.size() == 1 && pouts[0]->shape.dtype == DType::kF16 && pouts[0]->shape.dims == std::vector<int64_t>({g.M, g.K}), kUnsupported)
+        << gi->hlo_name << ": the folded LayerNorm must produce exactly the f16 [M,K] rows";
+    const Instr* H = pouts[0];
+    VarTable rv;
+    const int vm = rv.add("m", g.M), vr = rv.add("run", g.K / 8);
+    Index idx;
+    idx.push_back(LinExpr::variable(vm, g.M));
+    idx.push_back(LinExpr::variable(vr, g.K / 8).scaled(8));
+    const LinExpr off = physical_offset(prog, H, idx, &rv);
+    const std::string pg = ptrs.input(fold->gamma), pbt = ptrs.input(fold->beta), ph = ptrs.output(H);
+    rows_struct = "struct @NAME@_rows {\n  static constexpr bool enabled = true;\n  const _Float16* gamma;\n  const _Float16* beta;\n  _Float16* out;\n"
+                  "  __device__ __forceinline__ void operator()(int m, int k, half8_t x, float mean, float rs) const {\n"
+                  "    const int run = k >> 3;\n"
+                  "    const half8_t gam = *reinterpret_cast<const half8_t*>(gamma + k), bet = *reinterpret_cast<const half8_t*>(beta + k);\n"
+                  "    const float nmr = -mean * rs;\n"
+                  "    _Float16 hn[8];\n"
+                  "#pragma unroll\n"
+                  "    for (int e = 0; e < 8; ++e) hn[e] = (_Float16)fmaf(fmaf((float)x[e], rs, nmr), (float)gam[e], (float)bet[e]);\n"
+                  "    mononn_dev::stN<_Float16, 8>(out + " + off.str(rv) + ", hn);\n"
+                  "  }\n};\n";
+    rows_init = "@NAME@_rows rows{" + pg + ", " + pbt + ", " + ph + "};";
   }
   const size_t first_epi = ptrs.entries.size();   // 1 when both operands are the same buffer
   if (g.bf16) {
@@ -1808,6 +1841,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   if (g.split_k <= 1) fb.line(epi.init_line);
   if (fold) fb.line("epi.ln_stats = reinterpret_cast<const float*>(smem + " + S(fold_stats_offset) + ");");
   if (has_pro) fb.line(pro.init_line);
+  if (!rows_struct.empty()) fb.line(rows_init);
   int64_t units = 0;
   int smem = 0;
   if (mfma) {
@@ -1907,7 +1941,8 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
         call << "mononn_dev::gemm_tile_lds<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << KS << ", " << g.K << ", "
              << (g.a_packed ? "true" : "false") << ", " << (g.b_packed ? "true" : "false") << ", " << (epi.along_m ? "true" : "false") << ", " << t.bk
              << ", @NAME@_epi"
-             << (g.bf16 || rows_lds || lds_fold ? std::string(", mononn_dev::RowMajorA, ") + (g.bf16 ? "true" : "false") + (rows_lds || lds_fold ? (rows_lds ? ", true" : ", false") : "") + (lds_fold ? ", true" : "")
+             << (g.bf16 || rows_lds || lds_fold ? std::string(", mononn_dev::RowMajorA, ") + (g.bf16 ? "true" : "false") + (rows_lds || lds_fold ? (rows_lds ? ", true" : ", false") : "") + (lds_fold ? ", true" : "") +
+                                                      (!rows_struct.empty() ? ", @NAME@_rows" : "")
                                                 : std::string())
              << ">(" << pa << " + (long)bidx * " << g.a_batch_stride << " + ksplit * " << (g.a_packed ? KS / 32 * 512 : KS) << ", "
              << b_expr.str() << ", " << g.M << ", " << g.N << ", " << g.K << ", " << g.K << ", bidx, tile_m, tile_n, epi, smem";
@@ -1917,6 +1952,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
           std::string e = eps;
           if (e.find_first_of(".e") == std::string::npos) e.insert(e.size() - 1, ".0");
           call << ", mononn_dev::RowMajorA(), " << e << ", reinterpret_cast<float*>(smem + " << fold_stats_offset << ")";
+          if (!rows_struct.empty()) call << ", rows, " << tiles_n;
         }
       } else
         call << "mononn_dev::gemm_tile<" << t.bm << ", " << t.bn << ", " << t.wm << ", " << t.wn << ", " << t.wk << ", " << KS << ", "
@@ -1985,7 +2021,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
   }
   std::vector<std::string> globals = epi.globals;
   for (auto& gl : pro.globals) globals.push_back(gl);
-  NodeFunction f = finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + epi.struct_text + conv_struct);
+  NodeFunction f = finish(fb.text(), ptrs, globals, units, smem, pro.struct_text + rows_struct + epi.struct_text + conv_struct);
   f.write_maps = epi.writes;
   if (preload) {
     const std::string tail = ", char* smem) {";

@@ -411,8 +411,8 @@ HipProgram generate_program(const graph::Program& prog, spec::GraphSpecification
       GemmTuning t;
       if (it == spec.gemm_spec_list.end()) {
         // a row program in front of the GEMM runs on register-held fragments: direct tile, unless it is a LayerNorm
-        // folded away entirely and nobody else wants its rows
-        const bool lds_ok = n.prologue.empty() || (n.ln_fold.on() && !n.prologue_stores);
+        // folded away entirely (the LDS-staged tile computes its statistics and, if asked, stores its rows)
+        const bool lds_ok = n.prologue.empty() || n.ln_fold.on();
         t = default_gemm_tuning(n.gemm, ls, spec.device.sm_count, lds_ok);
         if (!n.prologue.empty() && t.stages < 2) t = default_gemm_tuning(n.gemm, ls, spec.device.sm_count, false);
         spec::GemmSpec g;

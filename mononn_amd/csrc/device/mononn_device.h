@@ -1000,16 +1000,25 @@ __device__ __forceinline__ float16_t mfma_32x32x16(half8_t a, half8_t b, float16
   else return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// No rows to store behind a folded LayerNorm (the default of gemm_tile_lds' last template argument).
+struct NoRowStore {
+  static constexpr bool enabled = false;
+};
+
 // BK: k extent of one LDS buffer (a multiple of 32); K a multiple of 32.
 // LN_STATS: the left operand's rows are the input of a LayerNorm that has been folded into weights and epilogue: while
 // a wave multiplies, it also adds up x and x * x of the fragments it reads (v_dot2_f32_f16 between the MFMAs: a
 // lane holds 8 values of one row), and in front of the epilogue leaves (mean, rsqrt(var + ln_eps)) of its rows in
 // ln_stats[row of the tile][2] (LDS) for the epilogue's rank-1 correction.  The waves that share rows write the same
 // values; a wave reads only rows it has written itself.
+// Rows (with LN_STATS): other stages read the normalised rows, so this GEMM also stores them: the column tiles of a
+// row block share the k range (tile_n of tiles_n takes a block of 16-byte runs), the waves that share rows split
+// them, and rows(m, k, x[m][k .. k + 7], mean, rsqrt) normalises and stores one run.
 template <int BM, int BN, int WM, int WN, int K, int KTOTAL, bool PACKED_A, bool PACKED_B, bool D_ALONG_M, int BK, class Epi,
-          class AMap = RowMajorA, bool BF16 = false, bool ROWS_LDS = false, bool LN_STATS = false>
+          class AMap = RowMajorA, bool BF16 = false, bool ROWS_LDS = false, bool LN_STATS = false, class Rows = NoRowStore>
 __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, int M, int N, int lda, int ldb, int batch, int tile_m,
-                                              int tile_n, Epi& epi, char* smem, const AMap& amap = AMap(), float ln_eps = 0.f, float* ln_stats = nullptr) {
+                                              int tile_n, Epi& epi, char* smem, const AMap& amap = AMap(), float ln_eps = 0.f, float* ln_stats = nullptr,
+                                              const Rows& rows = Rows(), int tiles_n = 1) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;             // 32 x 32 fragments per wave
   constexpr int KSTP = BK / 16;                                    // MFMA steps per k tile
@@ -1263,6 +1272,31 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if constexpr (Rows::enabled) {
+      static_assert(AMap::kRowMajor, "the rows are read back as the left operand stores them: row-major or in fragment order");
+      static_assert(32 % WN == 0, "the waves that share rows split them evenly");
+      constexpr int RUNS = K / 8;                              // 16-byte runs of a row
+      constexpr int ROWS_W = TM * 32 / WN;                     // rows of this wave
+      const int per_tile = (RUNS + tiles_n - 1) / tiles_n;     // runs of this column tile: [run0, run0 + per_tile)
+      const int run0 = tile_n * per_tile;
+      for (int idx = lane; idx < ROWS_W * per_tile; idx += kWaveSize) {
+        const int run = run0 + idx % per_tile;
+        const int rw = idx / per_tile;                                              // 0 .. ROWS_W - 1
+        const int row_in_tile = (wm * TM + rw / (32 / WN)) * 32 + wn * (32 / WN) + rw % (32 / WN);
+        const int m = tile_m * BM + row_in_tile;
+        if (run < RUNS && m < M) {
+          // fragment order: [row / 16][k / 32][(k % 32 / 8) * 16 + row % 16][8 halves]
+          const long at = PACKED_A ? (((long)(m >> 4) * (KTOTAL / 32) + (run >> 2)) * 512 + ((run & 3) * 16 + (m & 15)) * 8) : (long)m * lda + run * 8;
+          const half8_t x = *reinterpret_cast<const half8_t*>(A + at);
+          rows(m, run * 8, x, ln_stats[row_in_tile * 2], ln_stats[row_in_tile * 2 + 1]);
+        }
+      }
+      // the accumulators stay where they are while the rows are stored (see the epilogue below)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) MONONN_PIN_ACC(acc[i][j]);
+    }
   }
   typedef __attribute__((address_space(3))) float4_t lds_float4_t;
   lds_char_t* const rows_lds = lds + wave * (32 * PITCH * 4);   // this wave's 32 rows

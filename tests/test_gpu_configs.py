@@ -231,6 +231,44 @@ def test_layer_norm_folded_into_lds_staged_tiles(gpu_device):
     assert errs["folded"] <= 2 * errs["as written"] + 1e-3
 
 
+def test_post_ln_encoder_folded_on_lds_staged_tiles_stores_the_rows(gpu_device):
+    """Post-LN encoder: the residual of the next sub-layer reads the normalised rows, so a GEMM that has its LayerNorm
+    folded in also owes them to a later stage.  On LDS-staged tiles the column tiles of a row block store a share of the
+    rows each, from the statistics the tile has computed and a second look at its left operand (which the stage before
+    wrote in MFMA fragment order).  Against the oracle and against the kernel that runs every LayerNorm as a stage."""
+    import json
+    from mononn_amd import MonoNNModule
+    fx = models.bert_encoder(L=2, B=4, S=128, H=256, NH=4, F=1024, vocab=300, max_pos=128)
+    consts = fx.make_constants(1245, "random")
+    inputs = fx.make_inputs(1245)
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    spec["mononn_hip"].update(gemm_prologue_fusion=True, layer_norm_folding=True)
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}, {}
+    probe = MonoNNModule.compile(fx.hlo_text, json.dumps(spec), build=False)
+    assert "+row-prologue(stores)" in probe.summary()
+    spec = json.loads(probe.get_tuning_spec())
+    for name, entry in spec["gemm_spec_list"].items():
+        if name.startswith("fusion_"):      # the GEMMs with a LayerNorm folded in
+            c = entry["cutlass_config"]
+            c["threadblockshape"], c["warpshape"] = dict(m=128, n=128, k=64), dict(m=64, n=64, k=256)
+            c["wave_arrangement"], c["stages"] = dict(m=2, n=2, k=1), 2
+    folded = MonoNNModule.compile(fx.hlo_text, json.dumps(spec))
+    src = folded.get_source("main.hip")
+    assert src.count("_rows {") == 2 and "_rows>(" in src and "ln_stats" in src
+    plain = MonoNNModule.compile(fx.hlo_text)
+    assert folded.launch_dims()["barriers"] < plain.launch_dims()["barriers"]
+    want = hlo_interp.evaluate(fx.hlo_text, inputs, consts, "fp32")[0]
+    errs = {}
+    for name, m in (("folded", folded), ("as written", plain)):
+        m.set_constants(consts)
+        m.load(gpu_device)
+        got = m.run(inputs, fx.outputs)[0]
+        m.close()
+        _check(got, want, f"post-LN encoder, LayerNorm {name}")
+        errs[name] = np.abs(got.astype(np.float64) - want).max()
+    assert errs["folded"] <= 2 * errs["as written"] + 1e-3
+
+
 def test_vit_encoder_parity(gpu_device):
     fx = models.vit(L=2, B=2, image=64, patch=16, H=256, NH=4, F=512)
     consts = fx.make_constants(1238, "random")
