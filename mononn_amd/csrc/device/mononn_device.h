@@ -1168,9 +1168,10 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   const lds_char_t* a_frag = lds + (wm * TM * KSTP) * 1024 + lane * 16;
   const lds_char_t* b_frag = lds + (ABLK + wn * TN * KSTP) * 1024 + lane * 16;
   half8_t fa[2][TM], fb[2][TN];
-  float ln_s1[LN_STATS ? TM : 1], ln_s2[LN_STATS ? TM : 1];
+  // two running sums each (even and odd pairs of a fragment), so that consecutive v_dot2 do not wait for one another
+  float ln_s1[LN_STATS ? TM : 1][2], ln_s2[LN_STATS ? TM : 1][2];
 #pragma unroll
-  for (int i = 0; i < (LN_STATS ? TM : 1); ++i) ln_s1[i] = ln_s2[i] = 0.f;
+  for (int i = 0; i < (LN_STATS ? TM : 1); ++i) ln_s1[i][0] = ln_s1[i][1] = ln_s2[i][0] = ln_s2[i][1] = 0.f;
   auto read_one = [&](int buf, int ks, int rb, int r) {
     if (r < TM) fa[rb][r] = *reinterpret_cast<const lds_half8_t*>(a_frag + buf * STAGE_BYTES + (r * KSTP + ks) * 1024);
     else fb[rb][r - TM] = *reinterpret_cast<const lds_half8_t*>(b_frag + buf * STAGE_BYTES + ((r - TM) * KSTP + ks) * 1024);
@@ -1199,8 +1200,8 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const half2_t h = {fa[rb][i][2 * e], fa[rb][i][2 * e + 1]};
-            ln_s1[i] = __builtin_amdgcn_fdot2(h, half2_t{(half_t)1, (half_t)1}, ln_s1[i], false);
-            ln_s2[i] = __builtin_amdgcn_fdot2(h, h, ln_s2[i], false);
+            ln_s1[i][e & 1] = __builtin_amdgcn_fdot2(h, half2_t{(half_t)1, (half_t)1}, ln_s1[i][e & 1], false);
+            ln_s2[i][e & 1] = __builtin_amdgcn_fdot2(h, h, ln_s2[i][e & 1], false);
           }
         }
       }
@@ -1260,7 +1261,8 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
     // the two lanes that hold the two k pieces of a row put their sums together; the variance is E[x^2] - mean^2
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const float s1 = ln_s1[i] + __shfl_xor(ln_s1[i], 32, kWaveSize), s2 = ln_s2[i] + __shfl_xor(ln_s2[i], 32, kWaveSize);
+      const float p1 = ln_s1[i][0] + ln_s1[i][1], p2 = ln_s2[i][0] + ln_s2[i][1];
+      const float s1 = p1 + __shfl_xor(p1, 32, kWaveSize), s2 = p2 + __shfl_xor(p2, 32, kWaveSize);
       const float mean = s1 * (1.0f / K);
       const float var = s2 * (1.0f / K) - mean * mean;
       if (lane < 32) {
