@@ -308,6 +308,17 @@ def test_fusion_variants_agree(gpu_device):
     for name in ("weights requested inside the tile", "small grid"):
         (other,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants[name])
         assert np.array_equal(other.view(np.uint16), base.view(np.uint16)), f"{name}: when an operand is requested must not change any bit"
+    # MFMA accumulators stored as they are (fp32 partial sums of a k-split GEMM, per-head partial sums of the projection
+    # inside the attention stage): the 16-byte write-through store of the default barrier against the two plain
+    # 8-byte stores of the fenced one, bit for bit
+    import json
+    for name in ("split-K", "output projection inside the attention stage"):
+        fenced_spec = json.loads(variants[name])
+        fenced_spec["mononn_hip"]["barrier"] = "flags"
+        (a,), _ = run_module(fx.hlo_text, inputs, consts, fx.outputs, variants[name])
+        (b,), mb = run_module(fx.hlo_text, inputs, consts, fx.outputs, json.dumps(fenced_spec))
+        assert "#define MONONN_COHERENT_STORES 1" not in mb.get_source("main.hip")
+        assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), f"{name}: the store instruction must not change any bit"
 
 
 def test_repeated_launches_are_bit_identical(gpu_device):
