@@ -252,6 +252,17 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         }
       }
     }
+    // the stage-fusion decisions of the seed are where the search starts (its entries name the nodes of that graph)
+    if (seed && (seed->hip.gemm_prologue_fusion != base.hip.gemm_prologue_fusion || seed->hip.layer_norm_folding != base.hip.layer_norm_folding ||
+                 seed->hip.attention_out_proj_fusion != base.hip.attention_out_proj_fusion || seed->hip.regional_synchronization != base.hip.regional_synchronization)) {
+      base.hip.gemm_prologue_fusion = base.hip.gemm_prologue_fusion || seed->hip.gemm_prologue_fusion;
+      base.hip.layer_norm_folding = base.hip.layer_norm_folding || seed->hip.layer_norm_folding;
+      base.hip.attention_out_proj_fusion = seed->hip.attention_out_proj_fusion;
+      base.hip.regional_synchronization = seed->hip.regional_synchronization;
+      def_holder = std::make_unique<MonoNNModule>(params.hlo_text, base.to_json().dump(0), params.kernel_name);
+      def_holder->generate_code();
+      log << "  [" << ctx_str << "] stage-fusion decisions taken from the seed specification\n";
+    }
     // MONONN_TUNER_KEEP_SEED_SPLIT_K=<F>: the seed's k splits by at least F are in place from the start.  With
     // LayerNorm folding a split and a fold exclude each other at one LayerNorm (the row program that adds the partial
     // sums up stays a stage), and the split-K search below only compares a GEMM and its consumer, so which of the
@@ -346,8 +357,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       };
       add("default", filled);
       // MONONN_TUNER_ONLY_FUSION_DECISIONS (with a seed specification): the seed's tiles stand, only the stage-fusion
-      // decisions are searched (large models, whose class search takes many minutes)
-      if (seed && env::is_true("MONONN_TUNER_ONLY_FUSION_DECISIONS")) continue;
+      // decisions are searched (large models, whose class search takes many minutes); with
+      // MONONN_TUNER_ROW_PROGRAMS_TOO the row-program classes are searched as well (few candidates each)
+      if (seed && env::is_true("MONONN_TUNER_ONLY_FUSION_DECISIONS") && !(c.kind == "cluster_reduce" && env::is_true("MONONN_TUNER_ROW_PROGRAMS_TOO"))) continue;
       if (c.kind == "gemm") {
         for (auto& t : gemm_candidates(c.sample->gemm, cx.block / 64, budget)) {
           GraphSpecification s = filled;
