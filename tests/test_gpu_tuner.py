@@ -3,6 +3,7 @@ computes the same function as the default one, leave the reference's dump tree b
 to rebuild the same kernel (TF_MONONN_EXISTING_TUNING_SPEC_DIR contract, README.md:145-149)."""
 import json
 import os
+import re
 
 import numpy as np
 import pytest
@@ -82,11 +83,18 @@ def test_tuned_module_dump_tree_and_reload(gpu_device, encoder, tmp_path, monkey
     assert t_tuned <= 1.05 * t_def
 
 
-def test_tuning_from_a_seed_specification(gpu_device, encoder, tmp_path, monkeypatch):
-    fx, consts, inputs, want = encoder
-    first = str(tmp_path / "first")
+@pytest.fixture(scope="module")
+def first_run(gpu_device, encoder, tmp_path_factory):
+    """Dump directory of an unseeded tuning run (shared by the tests that start from a seed)."""
+    fx, _, _, _ = encoder
+    first = str(tmp_path_factory.mktemp("seed") / "first")
     MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, first, budget=2).close()
-    monkeypatch.setenv("MONONN_TUNER_SEED_SPEC_DIR", first)
+    return first
+
+
+def test_tuning_from_a_seed_specification(gpu_device, encoder, first_run, tmp_path, monkeypatch):
+    fx, consts, inputs, want = encoder
+    monkeypatch.setenv("MONONN_TUNER_SEED_SPEC_DIR", first_run)
     second = str(tmp_path / "second")
     tuned = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, second, budget=2)
     log = open(os.path.join(second, "cluster_0", "tuning_log.log")).read()
@@ -94,6 +102,26 @@ def test_tuning_from_a_seed_specification(gpu_device, encoder, tmp_path, monkeyp
     tuned.set_constants(consts)
     tuned.load(gpu_device)
     _check(tuned.run(inputs, fx.outputs)[0], want)
+
+
+def test_row_programs_and_fusion_decisions_from_a_seed(gpu_device, encoder, first_run, tmp_path, monkeypatch):
+    """A run that keeps the seed's tiles and searches only the row programs and the stage-fusion decisions: it starts
+    from the seed's decisions, and the rows-per-wave variants are among what it tries."""
+    fx, consts, inputs, want = encoder
+    monkeypatch.setenv("MONONN_TUNER_SEED_SPEC_DIR", first_run)
+    monkeypatch.setenv("MONONN_TUNER_ONLY_FUSION_DECISIONS", "1")
+    monkeypatch.setenv("MONONN_TUNER_ROW_PROGRAMS_TOO", "1")
+    out = str(tmp_path / "rows")
+    again = MonoNNModuleTuner.tune(fx.hlo_text, gpu_device, out, budget=2)
+    log = open(os.path.join(out, "cluster_0", "tuning_log.log")).read()
+    assert "tier1_rows2=" in log and "tier1_rows4=" in log and "fusion decision" in log
+    assert not re.search(r"gemm x\d+ \([^)]*\): best \S+ [\d.]+ us per stage; default=[\d.]+ \S", log), "GEMM classes keep the seed's tiles"
+    seed_hip = json.loads(open(os.path.join(first_run, "cluster_0", "best_tuning_spec.json")).read())["mononn_hip"]
+    if any(seed_hip[k] for k in ("gemm_prologue_fusion", "layer_norm_folding", "attention_out_proj_fusion", "regional_synchronization")):
+        assert "stage-fusion decisions taken from the seed specification" in log
+    again.set_constants(consts)
+    again.load(gpu_device)
+    _check(again.run(inputs, fx.outputs)[0], want)
 
 
 def test_launch_contexts_can_be_named(gpu_device, encoder, tmp_path, monkeypatch):
