@@ -1996,7 +1996,7 @@ NodeFunction gen_gemm(const Program& prog, const std::vector<const Instr*>& memb
     fb.line(call.str());
     if (t.wk > 1) smem = ls.waves() * (t.bm / t.wm / 16) * (t.bn / t.wn / 16) * 64 * 16;
     if (t.stages >= 2) smem = std::max(2 * (t.bm + t.bn) * t.bk * 2, rows_lds ? ls.waves() * 32 * (t.bn / t.wn + 4) * 4 : 0);
-    if (lds_fold) smem = fold_stats_offset + t.bm * 8 * 3;   // statistics, and the partial sums of the two wave columns behind them
+    if (lds_fold) smem = fold_stats_offset + t.bm * 8;
     smem = std::max(smem, pro.smem);
   } else {
     const int64_t total = g.batch * g.M * g.N;

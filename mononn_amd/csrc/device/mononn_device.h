@@ -1009,11 +1009,8 @@ struct NoRowStore {
 // LN_STATS: the left operand's rows are the input of a LayerNorm that has been folded into weights and epilogue: while
 // a wave multiplies, it also adds up x and x * x of the fragments it reads (v_dot2_f32_f16 between the MFMAs: a
 // lane holds 8 values of one row), and in front of the epilogue leaves (mean, rsqrt(var + ln_eps)) of its rows in
-// ln_stats[row of the tile][2] (LDS) for the epilogue's rank-1 correction.  The WN waves that share rows take the k
-// steps in turn (step s belongs to wave s % WN when WN is 2), leave their partial sums behind the statistics
-// (ln_stats + 2 * BM floats on, [wave column][row][2]), and after a workgroup barrier every wave adds the WN partial
-// sums of its rows up; the waves that share rows then write the same values, and a wave reads only rows it has
-// written itself.
+// ln_stats[row of the tile][2] (LDS) for the epilogue's rank-1 correction.  The waves that share rows write the same
+// values; a wave reads only rows it has written itself.
 // Rows (with LN_STATS): other stages read the normalised rows, so this GEMM also stores them: the column tiles of a
 // row block share the k range (tile_n of tiles_n takes a block of 16-byte runs), the waves that share rows split
 // them, and rows(m, k, x[m][k .. k + 7], mean, rsqrt) normalises and stores one run.
@@ -1035,7 +1032,6 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
   static_assert(ABLK % NW == 0 && BBLK % NW == 0, "the waves share the copy of a k tile evenly");
   static_assert(!PACKED_A || AMap::kRowMajor, "a fragment-order left operand takes no row map");
   constexpr int ACPY = ABLK / NW, BCPY = BBLK / NW;                // copies per lane and k tile
-  constexpr bool kShareStats = LN_STATS && WN == 2 && KSTEPS % 2 == 0;   // the two waves that share rows split the statistics' k steps
   constexpr int CPY = ACPY + BCPY;
   const int lane = lane_id();
   const int wave = wave_id();
@@ -1200,7 +1196,7 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
       for (int c = l0 + ((l1 - l0) * q) / Q; c < l0 + ((l1 - l0) * (q + 1)) / Q; ++c) load_one(t + 3, set, c);
       const int i = q / TN, j = q % TN;
       if constexpr (LN_STATS) {
-        if (j == 0 && (!kShareStats || rb == wn)) {   // rb is the parity of the k step
+        if (j == 0) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const half2_t h = {fa[rb][i][2 * e], fa[rb][i][2 * e + 1]};
@@ -1266,36 +1262,13 @@ __device__ __forceinline__ void gemm_tile_lds(const half_t* A, const half_t* B, 
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const float p1 = ln_s1[i][0] + ln_s1[i][1], p2 = ln_s2[i][0] + ln_s2[i][1];
-      float s1 = p1 + __shfl_xor(p1, 32, kWaveSize), s2 = p2 + __shfl_xor(p2, 32, kWaveSize);
-      if constexpr (kShareStats) {
-        float* part = ln_stats + 2 * BM;
-        if (lane < 32) {
-          part[((wn * BM) + (wm * TM + i) * 32 + lane) * 2] = s1;
-          part[((wn * BM) + (wm * TM + i) * 32 + lane) * 2 + 1] = s2;
-        }
-        continue;
-      }
+      const float s1 = p1 + __shfl_xor(p1, 32, kWaveSize), s2 = p2 + __shfl_xor(p2, 32, kWaveSize);
       const float mean = s1 * (1.0f / K);
       const float var = s2 * (1.0f / K) - mean * mean;
       if (lane < 32) {
         float* dst = ln_stats + ((wm * TM + i) * 32 + lane) * 2;
         dst[0] = mean;
         dst[1] = rsqrtf((var > 0.f ? var : 0.f) + ln_eps);
-      }
-    }
-    if constexpr (kShareStats) {
-      __syncthreads();   // the partial sums of both wave columns are in LDS
-      const float* part = ln_stats + 2 * BM;
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = (wm * TM + i) * 32 + r32;
-        const float s1 = part[row * 2] + part[(BM + row) * 2], s2 = part[row * 2 + 1] + part[(BM + row) * 2 + 1];
-        const float mean = s1 * (1.0f / K);
-        const float var = s2 * (1.0f / K) - mean * mean;
-        if (lane < 32) {
-          ln_stats[row * 2] = mean;
-          ln_stats[row * 2 + 1] = rsqrtf((var > 0.f ? var : 0.f) + ln_eps);
-        }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
