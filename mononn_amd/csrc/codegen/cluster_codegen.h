@@ -30,8 +30,9 @@ struct LaunchShape {
 struct ClusterTuning {
   int ilp_factor = 1;        // independent elements per thread per trip (element-wise clusters)
   int locality_tier = 1;     // row programs: 1 = one wave per row, 2 = one workgroup per row
-  // row programs of tier 1: 0 = a wave on one row; 1 = a wave on 8 consecutive rows at once, 8 lanes per row (every
-  // load and store instruction then covers whole 128-byte lines of 8 rows, and one trip moves 8 rows' worth of bytes)
+  // row programs of tier 1: 0 = a wave on one row; 1 / 2 / 3 = a wave on 8 / 4 / 2 consecutive rows at once, 8 / 16 / 32
+  // lanes per row (every load and store instruction then covers whole 128-byte lines of those rows, and one trip
+  // moves that many rows' worth of bytes)
   int reduce_implementation = 0;
 };
 

@@ -49,7 +49,7 @@ struct ClusterReduceSpec {
   std::string name;
   int ilp_factor = 1;
   int locality_tier = 1;          // 1 = wave per row, 2 = workgroup per row (reference: warp / block)
-  int reduce_implementation = 0;
+  int reduce_implementation = 0;  // tier 1: rows a wave takes at once, 0 = one, 1 / 2 / 3 = 8 / 4 / 2
 };
 
 struct GemmSpec {
