@@ -4,7 +4,8 @@ Bounds check of generated kernels on the CPU: the generated translation unit of 
 device prelude it includes, unchanged) is compiled for the host with tests/cpu_shim/host_builtins.h pre-included and
 run thread by thread with every buffer (parameters, live-outs, the temp arena and every constant of the module, which
 the generated source declares as arrays of the code object) placed against inaccessible guard pages, once flush with the
-page before it (catches reads in front of a buffer) and once flush with the page behind it (catches reads past its end).  An out-of-range access ends the run
+page before it (catches reads in front of a buffer) and once flush with the page behind it (catches reads past its end).
+The workgroup's LDS is a buffer of exactly the kernel's dynamic LDS size whose end sits against a guard page.  An out-of-range access ends the run
 with the buffer, the offset and the thread that made it."""
 import json
 import os
@@ -24,7 +25,7 @@ DRIVER = r"""
 #include <sys/mman.h>
 #include <unistd.h>
 Dim3 threadIdx, blockIdx, gridDim, blockDim;
-extern "C" { alignas(16) char smem[160 << 10]; }
+char* mononn_lds;   // the kernel's `smem`: launch_dims()["smem"] bytes, the last of them in front of a guard page
 %(const_decls)s
 #include "main.hip"
 
@@ -56,6 +57,8 @@ int main(int argc, char** argv) {
     bufs[i] = {names[i], sizes[i], base, r, r + body + 2 * kGuard};
   }
 %(const_binds)s
+  mononn_lds = bufs[%(lds_index)d].lo + kGuard + ((((std::max<size_t>(sizes[%(lds_index)d], 1) + page - 1) / page * page) - sizes[%(lds_index)d]) & ~size_t(15));
+  bufs[%(lds_index)d].base = mononn_lds;
   struct sigaction sa = {};
   sa.sa_sigaction = on_fault;
   sa.sa_flags = SA_SIGINFO;
@@ -98,6 +101,11 @@ def check_module(hlo_text, spec_json=None, workdir=None, opt="-O0", shrink=None)
     for cname, cbytes in consts:
         names.append(cname)
         sizes.append(int(cbytes))
+    names.append("LDS")
+    sizes.append(max(dims["smem"], 16))
+    lds_decl = "extern __shared__ __attribute__((aligned(16))) char smem[];"
+    assert lds_decl in src, "the kernel's LDS declaration has changed"
+    src = src.replace(lds_decl, "char* const smem = mononn_lds;")
     if shrink:
         sizes[names.index(shrink[0])] -= shrink[1]
     const_decls = "\n".join(f"unsigned char* {cname};" for cname, _ in consts)
@@ -107,7 +115,7 @@ def check_module(hlo_text, spec_json=None, workdir=None, opt="-O0", shrink=None)
     open(os.path.join(tmp, "headers.h"), "w").write(m.get_source("headers.h"))
     drv = DRIVER % {"nbuf": len(names), "names": ", ".join(json.dumps(n) for n in names), "sizes": ", ".join(f"{s}ul" for s in sizes),
                     "grid": dims["grid"], "block": dims["block"], "kernel": m.kernel_name,
-                    "args": ", ".join(f"bufs[{i}].base" for i in range(n_args)), "const_decls": const_decls, "const_binds": const_binds}
+                    "args": ", ".join(f"bufs[{i}].base" for i in range(n_args)), "const_decls": const_decls, "const_binds": const_binds, "lds_index": len(names) - 1}
     open(os.path.join(tmp, "driver.cpp"), "w").write(drv)
     exe = os.path.join(tmp, "driver")
     cp = subprocess.run([CLANG, "-x", "c++", "-std=c++17", opt, "-w", "-include", os.path.join(HERE, "cpu_shim", "host_builtins.h"), "-I", tmp,
