@@ -139,6 +139,10 @@ std::vector<codegen::GemmTuning> gemm_candidates(const graph::GemmDesc& g, int w
   return out;
 }
 
+// barrier time budget of the kernels the tuner times (candidates of a class, whole-kernel candidates); the module it
+// hands back keeps the specification's own
+constexpr int kTrialBarrierTimeoutMs = 1000;
+
 struct ClassInfo {
   std::string function;                 // de-duplicated device function name under the default spec
   std::vector<std::string> nodes;       // node names sharing it
@@ -352,6 +356,9 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       auto add = [&](const std::string& label, GraphSpecification s) {
         s.codegen_allow_list = c.nodes;
         s.hip.profile_stages = true;
+        // a candidate's stages take microseconds: one whose grid turns out not to be resident must not spin at its
+        // first barrier for the full budget of a production launch
+        s.hip.barrier_timeout_ms = std::min(s.hip.barrier_timeout_ms, kTrialBarrierTimeoutMs);
         Trial t;
         t.label = label;
         t.spec = std::move(s);
@@ -479,8 +486,20 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
       auto res = runtime::compile_hip(files, "main.hip", props.arch);
       runtime::DeviceModule dm;
       dm.load(params.device, res.code_object, trials[live[0]].mod->kernel_name());
-      size_t fb = 0;
-      dm.zero(dm.global("mononn_barrier_flags", &fb), fb);
+      size_t fb = 0, eb = 0;
+      void* const flags = dm.global("mononn_barrier_flags", &fb);
+      void* const error_word = dm.global("mononn_barrier_error", &eb);
+      dm.zero(flags, fb);
+      // A barrier wait that gave up leaves the workgroups at different epochs: the candidate is out, and the flags
+      // start from zero again so that the candidates behind it (same translation unit, same flags) are not held up
+      auto gave_up = [&]() {
+        unsigned word[4] = {0, 0, 0, 0};
+        dm.download(word, error_word, sizeof(word));
+        if (word[0] == 0) return false;
+        dm.zero(flags, fb);
+        dm.zero(error_word, eb);
+        return true;
+      };
       for (size_t i : live) {
         Trial& t = trials[i];
         const codegen::HipProgram& hp = t.mod->hip_program();
@@ -503,6 +522,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           int count = 0;
           for (int it = 0; it < warm + iters; ++it) {
             dm.launch(hp.grid, hp.block, hp.smem, args.data(), nullptr);
+            if (it == 0 && gave_up()) MONONN_FAIL(kRuntimeError) << "a grid-barrier wait gave up (the grid was not resident as a whole)";
             if (it < warm) continue;
             dm.download(ticks.data(), clk, cb);
             // A stage is charged from the moment the last workgroup finished the stage before it (the first stage:
@@ -527,6 +547,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           }
           t.us = count ? total / count : -1;
           t.total_us = count ? total / iters : -1;
+          if (gave_up()) MONONN_FAIL(kRuntimeError) << "a grid-barrier wait gave up (the grid was not resident as a whole)";
         } catch (const Error& e) {
           t.error = e.what();
           t.us = -1;
@@ -608,6 +629,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
     auto whole_kernel_us = [&](GraphSpecification s) -> double {
       s.codegen_allow_list.clear();
       s.hip.profile_stages = false;
+      s.hip.barrier_timeout_ms = std::min(s.hip.barrier_timeout_ms, kTrialBarrierTimeoutMs);
       why_not.clear();
       try {
         MonoNNModule m(params.hlo_text, s.to_json().dump(0), params.kernel_name);
@@ -755,6 +777,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         {
           GraphSpecification s = stitched;
           s.hip.profile_stages = true;
+          s.hip.barrier_timeout_ms = std::min(s.hip.barrier_timeout_ms, kTrialBarrierTimeoutMs);
           s.codegen_allow_list.clear();
           MonoNNModule probe(params.hlo_text, s.to_json().dump(0), "mononn_probe");
           try {
@@ -789,6 +812,7 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
           if (g.K % (32 * S) != 0 || g.K / S < 256) continue;
           GraphSpecification s0 = stitched;
           s0.hip.profile_stages = true;
+          s0.hip.barrier_timeout_ms = std::min(s0.hip.barrier_timeout_ms, kTrialBarrierTimeoutMs);
           s0.codegen_allow_list.clear();
           for (auto& n : c.nodes) s0.gemm_spec_list.erase(n);
           for (auto& n : base_consumers) {
