@@ -24,6 +24,18 @@ def test_the_check_itself_reports_an_access_past_a_buffer():
         assert not ok and "OUT OF BOUNDS: " + which in msg, msg
     ok, msg = check_module(models.bert_layer().hlo_text, shrink=("temp arena", 64))
     assert not ok and "temp arena" in msg
+    # the constants of the module (arrays of the code object) and the workgroup's LDS are guarded like the arguments
+    import re
+    from mononn_amd import MonoNNModule
+    layer = models.bert_layer().hlo_text
+    m = MonoNNModule.compile(layer, build=False)
+    weights = [(n, int(b)) for n, b in re.findall(r"unsigned char (buffer_for_\w+)\[(\d+)\];", m.get_source("main.hip")) if int(b) >= 4096]
+    assert weights
+    for name, _ in weights[:2]:
+        ok, msg = check_module(layer, shrink=(name, 16))
+        assert not ok and "OUT OF BOUNDS: " + name in msg, msg
+    ok, msg = check_module(layer, shrink=("LDS", m.launch_dims()["smem"] // 2))
+    assert not ok and "OUT OF BOUNDS: LDS" in msg, msg
 
 
 @pytest.mark.parametrize("case", GEMM_CASES)
