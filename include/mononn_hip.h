@@ -142,7 +142,8 @@ int mononn_module_synchronize(mononn_module* m, void* stream);
 int mononn_module_global(const mononn_module* m, const char* symbol, void** device_ptr, size_t* bytes);
 
 /* Time `iters` launches after `warmup` with HIP events on `stream`; avg_ms receives the mean,
- * each_ms (may be NULL, else iters floats) the individual launches.
+ * each_ms (may be NULL, else iters floats) the individual launches.  One launch checked like
+ * mononn_module_synchronize comes first: a kernel whose grid-barrier waits give up is an error here, not a time.
  * Replaces: the CUPTI gpu__time_duration range of profile_in_batch
  *           (mononn_engine/module/mononn_module_tuner.cc:250-372, tuning/profiler/cupti_profiling_session.h:20-78). */
 int mononn_time_kernel(mononn_module* m, void* const* device_ptrs, size_t n_ptrs, void* stream, int warmup,
