@@ -498,6 +498,12 @@ std::unique_ptr<MonoNNModule> MonoNNModuleTuner::tune(const TuneParams& params) 
         if (word[0] == 0) return false;
         dm.zero(flags, fb);
         dm.zero(error_word, eb);
+        try {
+          size_t rb = 0;
+          void* regional = dm.global("mononn_regional_flags", &rb);   // only in kernels with a regional tier
+          dm.zero(regional, rb);
+        } catch (const Error&) {
+        }
         return true;
       };
       for (size_t i : live) {
