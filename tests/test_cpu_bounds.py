@@ -174,3 +174,25 @@ def test_bf16_encoder_and_gemms():
             c["stages"] = 2
     ok, msg = check_module(fx.hlo_text, json.dumps(spec), opt="-O1")
     assert ok, "LDS-staged tiles: " + msg
+
+
+def test_folded_layer_norm_on_lds_staged_tiles_that_store_their_rows():
+    """Post-LN encoder, LayerNorms folded into LDS-staged tiles: the GEMMs that owe the normalised rows to a later stage
+    re-read their left operand (stored in fragment order by the stage before) and store a share of the rows per column tile."""
+    import json
+    from mononn_amd import MonoNNModule
+    fx = models.bert_encoder(L=2, B=4, S=128, H=256, NH=4, F=1024, vocab=300, max_pos=128)
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, build=False).get_tuning_spec())
+    spec["mononn_hip"].update(gemm_prologue_fusion=True, layer_norm_folding=True)
+    spec["gemm_spec_list"], spec["cluster_reduce_spec"], spec["cluster_elewise_spec"] = {}, {}, {}
+    spec = json.loads(MonoNNModule.compile(fx.hlo_text, json.dumps(spec), build=False).get_tuning_spec())
+    for name, entry in spec["gemm_spec_list"].items():
+        if name.startswith("fusion_"):
+            c = entry["cutlass_config"]
+            c["threadblockshape"], c["warpshape"] = dict(m=128, n=128, k=64), dict(m=64, n=64, k=256)
+            c["wave_arrangement"], c["stages"] = dict(m=2, n=2, k=1), 2
+    src = MonoNNModule.compile(fx.hlo_text, json.dumps(spec), build=False).get_source("main.hip")
+    assert src.count("_rows {") == 2 and "_rows>(" in src
+    ok, msg = check_module(fx.hlo_text, json.dumps(spec))
+    assert ok, msg
+
